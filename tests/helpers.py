@@ -1,0 +1,98 @@
+"""Shared checks for the parity tests (host side, numpy only)."""
+import numpy as np
+
+
+def ordered_int(a):
+    """float32 array -> int64 whose integer order is the float order
+    (-0 and +0 both map to 0), so |difference| is a distance in ulps."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.int32).astype(np.int64)
+    return np.where(u < 0, -(u & 0x7FFFFFFF), u)
+
+
+def ulp_diff(a, b):
+    """Element-wise distance in float32 ulps; NaN vs NaN counts as 0,
+    NaN vs number as a huge distance."""
+    a = np.asarray(a, dtype=np.float32)
+    b = np.asarray(b, dtype=np.float32)
+    d = np.abs(ordered_int(a) - ordered_int(b))
+    an, bn = np.isnan(a), np.isnan(b)
+    d = np.where(an & bn, 0, d)
+    d = np.where(an ^ bn, 1 << 40, d)
+    return d
+
+
+def half_ulp_diff(a, b):
+    """Distance in binary16 ulps between two float16 (or uint16-bit) arrays."""
+    def oi(h):
+        h = np.asarray(h)
+        if h.dtype == np.float16:
+            h = h.view(np.uint16)
+        s = h.astype(np.int64)
+        return np.where(s & 0x8000, -(s & 0x7FFF), s)
+    return np.abs(oi(a) - oi(b))
+
+
+def topk_brute(x, k, axis=-1, largest=True):
+    """Stable-sort brute force of the tie rule (value order, then lower index);
+    NaN ranks as the largest value.  Returns (values, int32 indices)."""
+    x = np.asarray(x)
+    xm = np.moveaxis(x, axis, -1)
+    xf = xm.astype(np.float32)
+    nan = np.isnan(xf)
+    key = np.where(nan, np.inf, xf) + np.float32(0.0)  # -0 -> +0
+    # rank NaN strictly above +inf through a second key
+    n = xf.shape[-1]
+    idx = np.broadcast_to(np.arange(n), xf.shape)
+    if largest:
+        order = np.lexsort((idx, -key, ~nan), axis=-1)
+    else:
+        order = np.lexsort((idx, key, nan), axis=-1)
+    order = order[..., :k]
+    vals = np.take_along_axis(xm, order, axis=-1)
+    return np.moveaxis(vals, -1, axis), np.moveaxis(order.astype(np.int32), -1, axis)
+
+
+def check_topk_invariants(x, vals, idx, k, largest=True):
+    """Structural properties any correct top-k along the last axis has,
+    whatever the data: values are copies of x[idx], ordered, indices unique,
+    nothing left out beats the k-th, equal values in increasing index order."""
+    x = np.asarray(x, dtype=np.float32)
+    rows = x.reshape(-1, x.shape[-1])
+    v = np.asarray(vals, dtype=np.float32).reshape(rows.shape[0], k)
+    ix = np.asarray(idx).reshape(rows.shape[0], k)
+    for r in range(rows.shape[0]):
+        assert ix[r].min() >= 0 and ix[r].max() < rows.shape[1]
+        assert len(set(ix[r].tolist())) == k
+        assert np.array_equal(rows[r][ix[r]].view(np.uint32), v[r].view(np.uint32))
+        s = v[r] if largest else -v[r]
+        assert np.all(s[:-1] >= s[1:])
+        same = s[:-1] == s[1:]
+        assert np.all(ix[r][1:][same] > ix[r][:-1][same])
+        rest = np.ones(rows.shape[1], bool)
+        rest[ix[r]] = False
+        if rest.any():
+            rs = rows[r][rest] if largest else -rows[r][rest]
+            assert rs.max() <= s[-1]
+            tied = np.nonzero(rest & ((rows[r] if largest else -rows[r]) == s[-1]))[0]
+            if tied.size:
+                last_sel = ix[r][s == s[-1]].max()
+                assert tied.min() > last_sel
+
+
+def reference_float_tolerance_ok(out, exp):
+    """The reference harness's own three-band float32 tolerance
+    (tests/setup.hpp:241-263): a floor every result must also meet."""
+    out = np.asarray(out, dtype=np.float32).ravel()
+    exp = np.asarray(exp, dtype=np.float32).ravel()
+    a = np.abs(exp)
+    thr = np.where(a > 1.0, a * 0.01, np.where(a > 1e-3, np.maximum(0.003, a * 0.02), 0.002))
+    return bool(np.all(~np.isnan(out)) and np.all(np.abs(out - exp) <= thr))
+
+
+def reference_half_tolerance_ok(out, exp):
+    """tests/setup.hpp:215-233: |d| <= max(0.02, 2 %) on the widened halves."""
+    out = np.asarray(out).view(np.float16).astype(np.float32).ravel()
+    exp = np.asarray(exp).view(np.float16).astype(np.float32).ravel()
+    a = np.abs(exp)
+    thr = np.where(a > 1.0, a * 0.02, 0.02)
+    return bool(np.all(~np.isnan(out)) and np.all(np.abs(out - exp) <= thr))
