@@ -1,0 +1,136 @@
+/*
+ * vkop_hip.h -- C ABI of the MI355X (gfx950) softmax / top-k post-processing
+ * library (libvkop_hip.so, built from vkop_amd/csrc).
+ *
+ * This is the boundary the reference's two operators sit on once their Vulkan
+ * plumbing is taken away: where `Softmax::execute` (ops/Softmax.hpp:61-141) and
+ * `Topk::execute` (ops/Topk.hpp:95-218) bind storage buffers, fill push
+ * constants and call `Operator::submit` (ops/Operator.hpp:225-238), a HIP build
+ * calls one function of this header with device pointers and a stream.
+ *
+ * Conventions
+ *  - plain C: pointers, sizes, ints; no C++ or framework types.
+ *  - every function returns an int status (0 = VKOP_HIP_OK) unless it returns a
+ *    size; no exception crosses the boundary; vkop_hip_last_error() gives the
+ *    calling thread's last failure text.
+ *  - `in`, `out*`, `workspace` are DEVICE pointers; `stream` is a hipStream_t
+ *    passed as void* (NULL = the default stream).  Calls only enqueue work.
+ *  - tensors are dense row-major with `ndim` (1..4) extents in `shape`, the
+ *    layout of the reference's storage-buffer tensors (core/Tensor.hpp:722-729,
+ *    765-801); `axis` may be negative (ops/Softmax.hpp:111-113).
+ *  - dtype VKOP_HIP_F16 means IEEE binary16 bits in uint16_t, the reference's
+ *    Tensor<uint16_t> (core/Tensor.hpp:116-198).  Arithmetic is float32 either way.
+ *  - a workspace must have been cleared once with vkop_hip_workspace_init()
+ *    before its first use; calls leave it ready for the next call.  Two calls
+ *    that are in flight at the same time must not share a workspace.
+ */
+#ifndef VKOP_HIP_H_
+#define VKOP_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum vkop_hip_status {
+    VKOP_HIP_OK = 0,
+    VKOP_HIP_ERR_INVALID = 1,     /* bad argument: null pointer, dtype, rank, axis, k */
+    VKOP_HIP_ERR_DEVICE = 2,      /* a HIP runtime call failed */
+    VKOP_HIP_ERR_WORKSPACE = 3,   /* workspace missing or smaller than *_workspace_bytes() */
+    VKOP_HIP_ERR_UNSUPPORTED = 4  /* valid request this build does not cover (k too large) */
+};
+
+enum vkop_hip_dtype { VKOP_HIP_F32 = 0, VKOP_HIP_F16 = 1 };
+
+/* Largest k the top-k entry points accept (the reference asserts k < 256,
+ * ops/Topk.hpp:103). */
+#define VKOP_HIP_MAX_K 2048
+
+/* ---- device, memory, streams: replaces VulkanDevice / VulkanBuffer /
+ * VulkanCommandPool + staging (vulkan/, core/Tensor.hpp:765-832) for this path. */
+int vkop_hip_init(int device);
+int vkop_hip_shutdown(void);
+const char *vkop_hip_last_error(void);
+/* name: caller buffer of name_len bytes; any out pointer may be NULL. */
+int vkop_hip_device_info(char *name, size_t name_len, int *compute_units,
+                         size_t *memory_bytes);
+
+int vkop_hip_malloc(void **ptr, size_t bytes);
+int vkop_hip_free(void *ptr);
+/* Host pointers may be pageable; the copy is ordered on `stream` and has
+ * completed on return (Tensor::copyToGPU / copyToCPU block the same way). */
+int vkop_hip_memcpy_h2d(void *dst_device, const void *src_host, size_t bytes, void *stream);
+int vkop_hip_memcpy_d2h(void *dst_host, const void *src_device, size_t bytes, void *stream);
+int vkop_hip_memcpy_d2d(void *dst_device, const void *src_device, size_t bytes, void *stream);
+
+int vkop_hip_stream_create(void **stream);
+int vkop_hip_stream_destroy(void *stream);
+int vkop_hip_stream_sync(void *stream);
+
+/* Timeline points (VulkanCommandBuffer's timeline semaphore wait/signal,
+ * core/runtime.cpp:421-446) and timing. */
+int vkop_hip_event_create(void **event);
+int vkop_hip_event_destroy(void *event);
+int vkop_hip_event_record(void *event, void *stream);
+int vkop_hip_event_sync(void *event);
+int vkop_hip_stream_wait_event(void *stream, void *event);
+int vkop_hip_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* Recorded work: everything enqueued on `stream` between begin and end is
+ * recorded instead of run, the way Operator::onExecute only records into a
+ * VulkanCommandBuffer between begin() and end() (ops/Operator.hpp:124-134) and
+ * Runtime::Run submits the recorded buffers (core/runtime.cpp:435-440).
+ * vkop_hip_graph_launch submits the recording; it may be launched any number
+ * of times.  Implemented with HIP stream capture. */
+int vkop_hip_graph_begin(void *stream);
+int vkop_hip_graph_end(void *stream, void **graph);
+int vkop_hip_graph_launch(void *graph, void *stream);
+int vkop_hip_graph_destroy(void *graph);
+
+/* Clears a workspace with a fill kernel (safe to capture in a HIP graph). */
+int vkop_hip_workspace_init(void *workspace, size_t bytes, void *stream);
+
+/* ---- Softmax: ops/Softmax.hpp:61-141 over shaders/softmax2.comp:50-184 and
+ * shaders/softmax.comp:31-207.  out has the shape and dtype of in; in == out is
+ * allowed.  nan_where != 0 replaces NaN results by nan_value (the shader's
+ * `nan_optimization`, shaders/softmax2.comp:177-181), on every axis. */
+size_t vkop_hip_softmax_workspace_bytes(int dtype, const int *shape, int ndim, int axis);
+int vkop_hip_softmax(const void *in, void *out, int dtype, const int *shape,
+                     int ndim, int axis, int nan_where, float nan_value,
+                     void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- TopK: ops/Topk.hpp:95-218 over shaders/topk.comp:110-262.
+ * out_values: dtype of in, out_indices: int32 positions along `axis`; both have
+ * the shape of in with [axis] = k.  Always sorted (descending for largest != 0,
+ * ascending otherwise); ties: lower index first; NaN ranks above +inf.
+ * `sorted` is accepted for signature parity (the reference parses and ignores
+ * it, ops/Topk.hpp:73-75).  1 <= k <= min(extent of axis, VKOP_HIP_MAX_K). */
+size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k);
+int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices,
+                  int dtype, const int *shape, int ndim, int axis, int k,
+                  int largest, int sorted, void *workspace,
+                  size_t workspace_bytes, void *stream);
+
+/* ---- Fused post-proc: TOPK applied to the SOFTMAX output, the pair
+ * benchmark/main.cpp:85-101 registers through Runtime::RegisterPostProcess
+ * (core/runtime.cpp:480-520).  Result = top-k (value order, then lower index)
+ * of the softmax tensor, without writing that tensor.  out_probs may be NULL;
+ * when given it receives the full softmax tensor as well. */
+size_t vkop_hip_softmax_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k);
+int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
+                          int32_t *out_indices, int dtype, const int *shape,
+                          int ndim, int axis, int k, int largest,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---- Max along an axis, (.., n, ..) -> (.., ..): the per-anchor class max
+ * between softmax and top-k in the detection-style post-proc
+ * (example/yolo/main.cpp:60-127; ops/Reduce.hpp covers only 4-D images). */
+int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape,
+                        int ndim, int axis, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VKOP_HIP_H_ */

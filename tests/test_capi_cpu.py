@@ -1,0 +1,70 @@
+"""CPU-only checks of the C-ABI library: it loads, it exports every function the
+header declares, and argument errors are reported without touching a GPU."""
+import ctypes
+import os
+import subprocess
+
+import pytest
+
+from vkop_amd import capi
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(capi.LIB_PATH):
+        capi.build()
+    return capi.lib()
+
+
+def test_exports_every_declared_symbol(lib):
+    declared = capi.declared_symbols()
+    assert len(declared) >= 25
+    for name in declared:
+        assert hasattr(lib, name), name
+    # and the binding knows a signature for each of them
+    assert sorted(lib._signatures) == declared
+    out = subprocess.check_output(["nm", "-D", "--defined-only", capi.LIB_PATH]).decode()
+    exported = {line.split()[-1] for line in out.splitlines() if " T " in line}
+    assert set(declared) <= exported
+
+
+def test_no_oracle_or_torch_linked_into_product():
+    out = subprocess.check_output(["ldd", capi.LIB_PATH]).decode()
+    assert "oracle" not in out and "torch" not in out
+    assert "amdhip64" in out
+
+
+def test_argument_errors_need_no_gpu(lib):
+    shape = (ctypes.c_int * 2)(4, 1000)
+    dummy = ctypes.c_void_p(256)
+    f = lib.vkop_hip_softmax
+    assert f(dummy, dummy, 7, shape, 2, 1, 0, 0.0, None, 0, None) == capi.ERR_INVALID
+    assert "dtype" in capi.last_error()
+    assert f(dummy, dummy, capi.F32, shape, 5, 1, 0, 0.0, None, 0, None) == capi.ERR_INVALID
+    assert f(dummy, dummy, capi.F32, shape, 2, 2, 0, 0.0, None, 0, None) == capi.ERR_INVALID
+    assert f(dummy, dummy, capi.F32, shape, 2, -3, 0, 0.0, None, 0, None) == capi.ERR_INVALID
+    assert f(None, dummy, capi.F32, shape, 2, 1, 0, 0.0, None, 0, None) == capi.ERR_INVALID
+    assert f(dummy, dummy, capi.F32, None, 2, 1, 0, 0.0, None, 0, None) == capi.ERR_INVALID
+    t = lib.vkop_hip_topk
+    assert t(dummy, dummy, dummy, capi.F32, shape, 2, -1, 0, 1, 1, None, 0, None) == capi.ERR_INVALID
+    assert t(dummy, dummy, dummy, capi.F32, shape, 2, -1, 1001, 1, 1, None, 0, None) == capi.ERR_INVALID
+    assert "exceeds" in capi.last_error()
+    big = (ctypes.c_int * 2)(1, 100000)
+    assert t(dummy, dummy, dummy, capi.F32, big, 2, -1, capi.MAX_K + 1, 1, 1, None, 0, None) == capi.ERR_UNSUPPORTED
+    s = lib.vkop_hip_softmax_topk
+    need = lib.vkop_hip_softmax_topk_workspace_bytes(capi.F32, shape, 2, -1, 5)
+    assert need > 0
+    assert s(dummy, None, dummy, dummy, capi.F32, shape, 2, -1, 5, 1, None, 0, None) == capi.ERR_WORKSPACE
+    assert s(dummy, None, dummy, dummy, capi.F32, shape, 2, -1, 5, 1, dummy, need - 1, None) == capi.ERR_WORKSPACE
+    assert lib.vkop_hip_reduce_max(dummy, dummy, capi.F32, (ctypes.c_int * 2)(3, 0), 2, 1, None) == capi.ERR_INVALID
+    # empty tensors are a no-op, not an error
+    empty = (ctypes.c_int * 2)(0, 1000)
+    assert f(None, None, capi.F32, empty, 2, 1, 0, 0.0, None, 0, None) == capi.OK
+
+
+def test_workspace_queries_are_pure(lib):
+    shape = (ctypes.c_int * 2)(64, 128256)
+    a = lib.vkop_hip_softmax_topk_workspace_bytes(capi.F32, shape, 2, -1, 50)
+    b = lib.vkop_hip_softmax_topk_workspace_bytes(capi.F32, shape, 2, -1, 50)
+    assert a == b and a % 256 == 0
+    assert lib.vkop_hip_softmax_topk_workspace_bytes(9, shape, 2, -1, 50) == 0

@@ -1,0 +1,331 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle, on the GPU.
+
+Bars: top-k indices and values bit-exact; float32 softmax within 2 ulp of the
+oracle (correctly rounded exp terms, double sum); float16 within 1e-3 relative
+(in practice 1 half ulp).  The distance to libtorch's own CPU softmax is
+reported through the reference harness's tolerance, not gated tighter: libtorch
+sums in ISA-dependent float lanes and is itself many ulp from an exact sum on
+long rows.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import (check_topk_invariants, half_ulp_diff, reference_float_tolerance_ok,
+                     reference_half_tolerance_ok, ulp_diff)
+from vkop_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from vkop_amd import capi, ops as _ops
+    capi.lib()              # raises if the HIP library is not built: no fallback
+    capi.init(0)
+    return _ops
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        a = a.view(np.float16)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def assert_softmax_close(got, x, axis, what=""):
+    exp = oracle.softmax(x, axis)
+    if got.dtype == np.float16:
+        assert half_ulp_diff(got, exp).max() <= 1, what
+        g, e = got.astype(np.float32), exp.astype(np.float32)
+        ok = np.abs(g - e) <= 1e-3 * np.abs(e) + 6e-8
+        assert ok.all(), what
+    else:
+        d = ulp_diff(got, exp)
+        assert d.max() <= 2, "%s: %d ulp" % (what, d.max())
+
+
+# ------------------------------------------------------------------ softmax --
+
+@pytest.mark.parametrize("tag", ["f32", "f16"])
+@pytest.mark.parametrize("case", range(6))
+def test_softmax_reference_test_shapes(ops, golden, case, tag):
+    """tests/SoftmaxTest.cpp:193-231: same shapes, axes, seed-42 inputs."""
+    x = golden["softmax%d_%s_in" % (case, tag)]
+    axis = int(golden["softmax%d_axis" % case])
+    xin = x.view(np.float16) if tag == "f16" else x
+    got = host(ops.softmax(dev(xin), axis))
+    assert got.shape == x.shape
+    assert_softmax_close(got, xin, axis, "case %d %s" % (case, tag))
+    exp = golden["softmax%d_%s_out" % (case, tag)]
+    if tag == "f16":
+        assert reference_half_tolerance_ok(got, exp)
+    else:
+        assert reference_float_tolerance_ok(got, exp)
+        assert ulp_diff(got, exp).max() <= 8
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 5, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 4097, 20001])
+def test_softmax_ragged_lengths(ops, n):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal((3, n)) * 3).astype(np.float32)
+    assert_softmax_close(host(ops.softmax(dev(x))), x, -1, "n=%d" % n)
+    xh = x.astype(np.float16)
+    assert_softmax_close(host(ops.softmax(dev(xh))), xh, -1, "n=%d half" % n)
+
+
+@pytest.mark.parametrize("shape,axis", [((5, 7, 9), 0), ((5, 7, 9), 1), ((5, 7, 9), 2), ((2, 3, 4, 5), 0), ((2, 3, 4, 5), 1),
+                                        ((2, 3, 4, 5), -2), ((300,), 0), ((4, 2500, 3), 1), ((3, 70, 130), 1), ((2, 5, 64), 1)])
+def test_softmax_axes(ops, shape, axis):
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal(shape) * 2).astype(np.float32)
+    assert_softmax_close(host(ops.softmax(dev(x), axis)), x, axis, str((shape, axis)))
+
+
+def test_softmax_special_values_and_nan_option(ops):
+    x = np.zeros((5, 130), np.float32)
+    x[0, 7] = np.nan
+    x[1, 9] = np.inf
+    x[2, :] = -np.inf
+    x[3, 3] = -np.inf
+    x[4, 100] = 300.0
+    with np.errstate(invalid="ignore"):
+        exp = oracle.softmax(x)
+        expn = oracle.softmax(x, nan_where=1, nan_value=0.125)
+    got = host(ops.softmax(dev(x)))
+    assert np.array_equal(np.isnan(got), np.isnan(exp))
+    assert ulp_diff(got, exp).max() <= 2
+    assert got[4, 100] == 1.0 and np.count_nonzero(got[4]) == 1 and got[3, 3] == 0.0
+    gotn = host(ops.softmax(dev(x), nan_where=True, nan_value=0.125))
+    assert not np.isnan(gotn).any() and ulp_diff(gotn, expn).max() <= 2
+    # all-equal rows give exactly 1/n
+    c = np.full((2, 777), -3.5, np.float32)
+    assert np.all(host(ops.softmax(dev(c))) == np.float32(1.0 / 777))
+
+
+def test_softmax_in_place(ops):
+    x = synth.classifier_logits(16, 1000, seed=3)
+    xd = dev(x)
+    ops.softmax(xd, out=xd)
+    assert_softmax_close(host(xd), x, -1)
+
+
+def test_softmax_workloads(ops):
+    x2 = synth.classifier_logits(256, 1000, synth.SEEDS["C2"])
+    assert_softmax_close(host(ops.softmax(dev(x2))), x2, -1, "C2 f32")
+    x2h = x2.astype(np.float16)
+    assert_softmax_close(host(ops.softmax(dev(x2h))), x2h, -1, "C2 f16")
+    x3 = synth.llm_logits(64, 128256, synth.SEEDS["C3"])
+    got = host(ops.softmax(dev(x3)))
+    assert_softmax_close(got, x3, -1, "C3")
+    assert np.abs(got.astype(np.float64).sum(-1) - 1).max() < 1e-5
+    x4 = synth.grid_values(8, 262144, synth.SEEDS["C4"])
+    assert_softmax_close(host(ops.softmax(dev(x4))), x4, -1, "C4")
+    x5 = synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"])
+    assert_softmax_close(host(ops.softmax(dev(x5), 1)), x5, 1, "C5")
+
+
+# -------------------------------------------------------------------- top-k --
+
+def assert_topk_exact(ops, x, k, axis=-1, largest=True):
+    v, ix = ops.topk(dev(x), k, axis, largest)
+    v, ix = host(v), host(ix)
+    ev, eix = oracle.topk(x, k, axis, largest)
+    assert ix.dtype == np.int32 and ix.shape == eix.shape
+    assert np.array_equal(ix, eix), (x.shape, k, axis, largest)
+    bits = np.uint16 if x.dtype == np.float16 else np.uint32
+    assert np.array_equal(v.view(bits), ev.view(bits))
+    return v, ix
+
+
+@pytest.mark.parametrize("tag", ["f32", "f16"])
+@pytest.mark.parametrize("case", range(5))
+def test_topk_reference_test_shapes(ops, golden, case, tag):
+    """tests/TopkTest.cpp:91-128: same shapes, k, seed-56 inputs; libtorch's
+    values always, its indices on rows without ties."""
+    x = golden["topk%d_%s_in" % (case, tag)]
+    k = int(golden["topk%d_k" % case])
+    xin = x.view(np.float16) if tag == "f16" else x
+    v, ix = assert_topk_exact(ops, xin, k, int(golden["topk%d_axis" % case]))
+    ev, eix = golden["topk%d_%s_val" % (case, tag)], golden["topk%d_%s_idx" % (case, tag)]
+    assert np.array_equal(v.view(ev.dtype) if tag == "f16" else v.view(np.uint32), ev if tag == "f16" else ev.view(np.uint32))
+    for r in range(x.shape[0]):
+        top = np.sort(xin[r].astype(np.float32))[::-1][:k + 1]
+        if len(np.unique(top)) == len(top):
+            assert np.array_equal(ix[r], eix[r])
+
+
+@pytest.mark.parametrize("shape,axis,k", [((4, 300), 1, 17), ((4, 300), 0, 3), ((3, 40, 5), 1, 40), ((2, 3, 64, 4), 2, 9),
+                                          ((500,), 0, 1), ((6, 64), -1, 64), ((2, 5000), -1, 2048), ((3, 1), -1, 1),
+                                          ((2, 70000), -1, 100), ((5, 257), -1, 256)])
+def test_topk_ties_axes_smallest(ops, shape, axis, k):
+    rng = np.random.default_rng(31)
+    for largest in (True, False):
+        x = (rng.integers(-6, 7, size=shape).astype(np.float32) / np.float32(4))
+        x.ravel()[rng.integers(0, x.size, 3)] = -0.0
+        assert_topk_exact(ops, x, k, axis, largest)
+        xr = rng.standard_normal(shape).astype(np.float32)
+        assert_topk_exact(ops, xr, k, axis, largest)
+        assert_topk_exact(ops, xr.astype(np.float16), k, axis, largest)
+
+
+def test_topk_nan_inf(ops):
+    x = np.random.default_rng(2).standard_normal((4, 500)).astype(np.float32)
+    x[0, [3, 77]] = np.nan
+    x[1, 5] = np.inf
+    x[1, 6] = -np.inf
+    x[2, :] = np.nan
+    x[3, 10] = -np.nan
+    for largest in (True, False):
+        v, ix = ops.topk(dev(x), 9, -1, largest)
+        ev, eix = oracle.topk(x, 9, -1, largest)
+        assert np.array_equal(host(ix), eix)
+        assert np.array_equal(np.isnan(host(v)), np.isnan(ev))
+
+
+def test_topk_workloads(ops, golden):
+    x4 = synth.grid_values(8, 262144, synth.SEEDS["C4"])
+    v, ix = assert_topk_exact(ops, x4, 1024)
+    check_topk_invariants(x4, v, ix, 1024)
+    x3 = synth.llm_logits(64, 128256, synth.SEEDS["C3"])
+    assert_topk_exact(ops, x3, 50)
+    x2 = synth.classifier_logits(256, 1000, synth.SEEDS["C2"])
+    assert_topk_exact(ops, x2, 5)
+    assert_topk_exact(ops, x2.astype(np.float16), 5)
+    # libtorch values on the down-sized grid workload
+    v, _ = assert_topk_exact(ops, golden["c4_in"], int(golden["c4_k"]))
+    assert np.array_equal(v.view(np.uint32), golden["c4_val"].view(np.uint32))
+
+
+# -------------------------------------------------------------------- fused --
+
+def assert_fused(ops, x, k, axis=-1, largest=True):
+    v, ix, p = ops.softmax_topk(dev(x), k, axis, largest, return_probs=True)
+    v, ix, p = host(v), host(ix), host(p)
+    # (1) exactly the top-k of the softmax tensor the same call wrote
+    ev, eix = oracle.topk(p, k, axis, largest)
+    bits = np.uint16 if x.dtype == np.float16 else np.uint32
+    assert np.array_equal(ix, eix), (x.shape, k)
+    assert np.array_equal(v.view(bits), ev.view(bits))
+    # (2) that tensor is the softmax, to the softmax bar
+    assert_softmax_close(p, x, axis)
+    # (3) without the tensor the result is the same
+    v2, ix2 = ops.softmax_topk(dev(x), k, axis, largest)
+    assert np.array_equal(host(ix2), ix) and np.array_equal(host(v2).view(bits), v.view(bits))
+    # (4) against the oracle's own fused result: values to the softmax bar,
+    # indices wherever the oracle's probabilities around the cut are distinct
+    ov, oix, op = oracle.softmax_topk(x, k, axis, largest, return_probs=True)
+    if x.dtype == np.float32:
+        assert ulp_diff(v, ov).max() <= 2
+        pm = np.moveaxis(op, axis, -1).reshape(-1, x.shape[axis])
+        im, om = np.moveaxis(ix, axis, -1).reshape(-1, k), np.moveaxis(oix, axis, -1).reshape(-1, k)
+        xm = np.moveaxis(x, axis, -1).reshape(-1, x.shape[axis])
+        for r in range(pm.shape[0]):
+            top = np.sort(xm[r])[::-1][:k + 1] if largest else np.sort(xm[r])[:k + 1]
+            ptop = np.sort(pm[r])[::-1][:k + 1] if largest else np.sort(pm[r])[:k + 1]
+            if len(np.unique(top)) == len(top) and len(np.unique(ptop)) == len(ptop) and not np.isnan(ptop).any():
+                assert np.array_equal(im[r], om[r]), r
+    return v, ix
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c2h"])
+def test_fused_downsized_workloads(ops, golden, name):
+    x, k = golden[name + "_in"], int(golden[name + "_k"])
+    if name == "c2h":
+        x = x.view(np.float16)
+    v, ix = assert_fused(ops, x, k)
+    ev, eix = golden[name + "_val"], golden[name + "_idx"]
+    if name == "c2h":
+        assert reference_half_tolerance_ok(v, ev)
+    else:
+        assert reference_float_tolerance_ok(v, ev)
+        for r in range(x.shape[0]):
+            if len(np.unique(ev[r])) == k:
+                assert np.array_equal(ix[r], eix[r])
+
+
+@pytest.mark.parametrize("shape,axis,k", [((7, 33), -1, 5), ((3, 50, 11), 1, 7), ((2, 3, 64, 4), 2, 64), ((1, 5), -1, 5),
+                                          ((2, 20000), -1, 300), ((4, 1), -1, 1), ((9, 777), -1, 1)])
+def test_fused_shapes_and_ties(ops, shape, axis, k):
+    rng = np.random.default_rng(41)
+    for largest in (True, False):
+        assert_fused(ops, rng.standard_normal(shape).astype(np.float32) * 2, k, axis, largest)
+        # grid data: many equal logits, hence many equal probabilities
+        assert_fused(ops, rng.integers(-8, 9, size=shape).astype(np.float32) / np.float32(2), k, axis, largest)
+        assert_fused(ops, (rng.standard_normal(shape) * 2).astype(np.float16), k, axis, largest)
+
+
+def test_fused_probability_collisions(ops):
+    """Distinct logits whose probabilities round to the same float: the
+    reference order (top-k of the softmax tensor) puts the lower index first
+    even when its logit is the smaller one."""
+    n = 4096
+    x = np.full((2, n), -20.0, np.float32)
+    x[:, 100] = 12.0                                # max; ulp(x - 12) = 2^-20 near 0 logits
+    base = np.float32(1.0)
+    x[0, 900] = base                                # larger logit, higher index
+    x[0, 50] = np.nextafter(base, np.float32(0))    # smaller logit, lower index
+    x[1, 2000:2100] = np.float32(0.25) + np.arange(100, dtype=np.float32) * np.float32(2.0 ** -24)
+    assert_fused(ops, x, 3)
+    assert_fused(ops, x, 60)
+    # underflow: most probabilities are exactly zero and tie by index
+    y = np.random.default_rng(3).standard_normal((2, 3000)).astype(np.float32)
+    y[:, 17] = 200.0
+    assert_fused(ops, y, 10)
+    assert_fused(ops, y.astype(np.float16) , 10)
+
+
+def test_fused_nan_rows(ops):
+    x = np.random.default_rng(4).standard_normal((3, 900)).astype(np.float32)
+    x[0, 400] = np.nan
+    x[1, 2] = np.inf
+    v, ix = ops.softmax_topk(dev(x), 6)
+    v, ix = host(v), host(ix)
+    assert np.isnan(v[0]).all() and np.isnan(v[1]).all()
+    assert ix[0].tolist() == list(range(6)) and ix[1].tolist() == list(range(6))
+    ov, oix = oracle.softmax_topk(x, 6)
+    assert np.array_equal(ix, oix) and ulp_diff(v, ov).max() <= 2
+
+
+def test_fused_headline_workload(ops):
+    """[64,128256] float32, k=50: every row against the oracle."""
+    x = synth.llm_logits(64, 128256, synth.SEEDS["C3"])
+    v, ix = ops.softmax_topk(dev(x), 50)
+    v, ix = host(v), host(ix)
+    ov, oix = oracle.softmax_topk(x, 50)
+    assert np.array_equal(ix, oix)
+    assert ulp_diff(v, ov).max() <= 2
+    # run to run: bit-identical
+    v2, ix2 = ops.softmax_topk(dev(x), 50)
+    assert np.array_equal(host(ix2), ix) and np.array_equal(host(v2).view(np.uint32), v.view(np.uint32))
+
+
+def test_detection_style_chain(ops, golden):
+    """softmax over the class axis -> per-anchor class max -> top-k anchors."""
+    for x, k in ((golden["c5_in"], int(golden["c5_k"])), (synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"]), 300)):
+        p = ops.softmax(dev(x), 1)
+        m = ops.reduce_max(p, 1)
+        v, ix = ops.topk(m, k)
+        p, m, v, ix = host(p), host(m), host(v), host(ix)
+        assert np.array_equal(m.view(np.uint32), p.max(axis=1).view(np.uint32))
+        ev, eix = oracle.topk(m, k)
+        assert np.array_equal(ix, eix) and np.array_equal(v.view(np.uint32), ev.view(np.uint32))
+        assert ulp_diff(m, oracle.reduce_max(oracle.softmax(x, 1), 1)).max() <= 2
+    assert reference_float_tolerance_ok(host(ops.reduce_max(ops.softmax(dev(golden["c5_in"]), 1), 1)), golden["c5_max"])
+
+
+def test_workspace_too_small_is_an_error(ops):
+    from vkop_amd import capi
+    x = dev(synth.classifier_logits(4, 1000, 1))
+    v = torch.empty((4, 5), device="cuda")
+    ix = torch.empty((4, 5), dtype=torch.int32, device="cuda")
+    with pytest.raises(capi.VkopHipError) as e:
+        capi.softmax_topk(x.data_ptr(), 0, v.data_ptr(), ix.data_ptr(), capi.F32, (4, 1000), -1, 5, 1, 0, 0, 0)
+    assert e.value.code == capi.ERR_WORKSPACE

@@ -1,0 +1,112 @@
+// Device-side building blocks shared by the softmax / top-k kernels (gfx950,
+// wave64).  Header only; every function is __device__ __forceinline__.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vkop {
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------- loads ----
+
+// Element of a float or half (uint16_t bits) tensor, widened to float.
+template <typename T> __device__ __forceinline__ float load_elem(const T *p, size_t i);
+template <> __device__ __forceinline__ float load_elem<float>(const float *p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float load_elem<uint16_t>(const uint16_t *p, size_t i) {
+    return __half2float(__ushort_as_half(p[i]));
+}
+
+// Round-to-nearest-even store of a float into a float or half tensor.
+template <typename T> __device__ __forceinline__ void store_elem(T *p, size_t i, float v);
+template <> __device__ __forceinline__ void store_elem<float>(float *p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void store_elem<uint16_t>(uint16_t *p, size_t i, float v) {
+    p[i] = __half_as_ushort(__float2half_rn(v));
+}
+
+// Value as the tensor type would hold it (float stays, half is rounded to
+// binary16 and widened again).
+template <typename T> __device__ __forceinline__ float round_to_storage(float v);
+template <> __device__ __forceinline__ float round_to_storage<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_to_storage<uint16_t>(float v) {
+    return __half2float(__float2half_rn(v));
+}
+
+// ------------------------------------------------------------ ordering ----
+
+// Maps a float to a uint32 whose unsigned order is the ranking top-k uses:
+// NaN (either sign) above +inf, -0 == +0, otherwise the numeric order.
+__device__ __forceinline__ uint32_t order_key(float v) {
+    if (v != v) return 0xFFFFFFFFu;
+    uint32_t u = __float_as_uint(v + 0.0f);  // -0 + +0 = +0
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Composite of key and position: larger composite = ranks earlier; among equal
+// keys the lower index is the larger composite.  Never 0 for idx < 2^32-1.
+__device__ __forceinline__ uint64_t composite(uint32_t key, uint32_t idx) {
+    return (static_cast<uint64_t>(key) << 32) | static_cast<uint64_t>(0xFFFFFFFFu - idx);
+}
+__device__ __forceinline__ uint32_t composite_index(uint64_t c) {
+    return 0xFFFFFFFFu - static_cast<uint32_t>(c);
+}
+
+// ---------------------------------------------------------- reductions ----
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+
+// Block-wide max / sum through a small LDS array (one slot per wave).  Every
+// thread of the block must call; the result is returned to all of them.
+// `scratch` needs NT / 64 slots and is reusable after the call returns.
+template <int NT> __device__ __forceinline__ float block_max(float v, float *scratch) {
+    constexpr int NW = NT / kWave;
+    v = wave_max(v);
+    if constexpr (NW == 1) return v;
+    __syncthreads();  // scratch may still be read from a previous call
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) r = fmaxf(r, scratch[w]);
+    return r;
+}
+template <int NT> __device__ __forceinline__ double block_sum(double v, double *scratch) {
+    constexpr int NW = NT / kWave;
+    v = wave_sum(v);
+    if constexpr (NW == 1) return v;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    double r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) r += scratch[w];  // fixed order: run-to-run stable
+    return r;
+}
+
+// --------------------------------------------------------------- softmax ----
+
+// One softmax term: exp of the single-precision difference, <= 1 ulp.
+__device__ __forceinline__ float softmax_term(float x, float m) { return expf(x - m); }
+
+}  // namespace vkop

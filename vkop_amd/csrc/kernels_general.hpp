@@ -1,0 +1,185 @@
+// General kernels: correct for every shape, axis, dtype and k the C ABI accepts.
+// One workgroup per line (or one thread per line for the strided variants).
+// The streaming kernels in kernels_rows.hpp take over for the shapes that
+// matter for throughput; these stay as the path for everything else and as the
+// exact fallback.
+#pragma once
+
+#include "device_utils.hpp"
+#include "select.hpp"
+
+namespace vkop {
+
+// A line of the (outer, n, inner) view: element j lives at base + j * inner.
+struct LineGeom {
+    uint32_t outer, n, inner;
+    __device__ __forceinline__ size_t base(uint32_t line) const {
+        const uint32_t o = line / inner, i = line - o * inner;
+        return static_cast<size_t>(o) * n * inner + i;
+    }
+};
+
+struct LineStats {
+    float m;  // max of the line (NaN ignored)
+    float s;  // sum of exp(x - m), rounded once from double
+};
+
+// max and sum of exp(x - max) of one line, by all NT threads of the block.
+template <typename T, int NT>
+__device__ __forceinline__ LineStats line_stats(const T *x, size_t base, uint32_t n, uint32_t stride,
+                                                float *fscratch, double *dscratch) {
+    const uint32_t tid = threadIdx.x;
+    float m = -INFINITY;
+    for (uint32_t j = tid; j < n; j += NT) m = fmaxf(m, load_elem(x, base + static_cast<size_t>(j) * stride));
+    m = block_max<NT>(m, fscratch);
+    // four independent float partial sums per thread keep every running sum
+    // short; the cross-thread combine is in double, in a fixed order
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    uint32_t j = tid;
+    for (; j + 3u * NT < n; j += 4u * NT) {
+        a0 += softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m);
+        a1 += softmax_term(load_elem(x, base + static_cast<size_t>(j + NT) * stride), m);
+        a2 += softmax_term(load_elem(x, base + static_cast<size_t>(j + 2u * NT) * stride), m);
+        a3 += softmax_term(load_elem(x, base + static_cast<size_t>(j + 3u * NT) * stride), m);
+    }
+    for (; j < n; j += NT) a0 += softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m);
+    double s = (static_cast<double>(a0) + static_cast<double>(a1)) + (static_cast<double>(a2) + static_cast<double>(a3));
+    s = block_sum<NT>(s, dscratch);
+    return LineStats{m, static_cast<float>(s)};
+}
+
+// Probability of one element given its line's statistics: the single formula
+// every kernel uses, so separately computed results agree bit for bit.
+__device__ __forceinline__ float softmax_prob(float x, LineStats st) { return softmax_term(x, st.m) / st.s; }
+
+// ---- softmax, one workgroup per line ---------------------------------------
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void softmax_lines_kernel(const T *in, T *out, LineGeom g, int nan_where,
+                                                           float nan_value, LineStats *stats_out) {
+    __shared__ float fscratch[NT / kWave];
+    __shared__ double dscratch[NT / kWave];
+    const uint32_t line = blockIdx.x;
+    const size_t base = g.base(line);
+    const LineStats st = line_stats<T, NT>(in, base, g.n, g.inner, fscratch, dscratch);
+    if (stats_out != nullptr && threadIdx.x == 0) stats_out[line] = st;
+    if (out == nullptr) return;
+    for (uint32_t j = threadIdx.x; j < g.n; j += NT) {
+        const size_t at = base + static_cast<size_t>(j) * g.inner;
+        float p = round_to_storage<T>(softmax_prob(load_elem(in, at), st));
+        if (nan_where && p != p) p = nan_value;
+        store_elem(out, at, p);
+    }
+}
+
+// ---- softmax along a non-last axis, one thread per line --------------------
+// Threads run along `inner` (contiguous), so each step over j is a coalesced
+// row of the (n, inner) slab.
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void softmax_strided_kernel(const T *in, T *out, LineGeom g, int nan_where,
+                                                             float nan_value) {
+    const uint32_t line = blockIdx.x * NT + threadIdx.x;
+    if (line >= g.outer * g.inner) return;
+    const size_t base = g.base(line);
+    float m = -INFINITY;
+    for (uint32_t j = 0; j < g.n; j++) m = fmaxf(m, load_elem(in, base + static_cast<size_t>(j) * g.inner));
+    double s = 0.0;
+    for (uint32_t j = 0; j < g.n; j++)
+        s += static_cast<double>(softmax_term(load_elem(in, base + static_cast<size_t>(j) * g.inner), m));
+    const LineStats st{m, static_cast<float>(s)};
+    for (uint32_t j = 0; j < g.n; j++) {
+        const size_t at = base + static_cast<size_t>(j) * g.inner;
+        float p = round_to_storage<T>(softmax_prob(load_elem(in, at), st));
+        if (nan_where && p != p) p = nan_value;
+        store_elem(out, at, p);
+    }
+}
+
+// ---- max along an axis ------------------------------------------------------
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void reduce_max_strided_kernel(const T *__restrict__ in, T *out, LineGeom g) {
+    const uint32_t line = blockIdx.x * NT + threadIdx.x;
+    if (line >= g.outer * g.inner) return;
+    const size_t base = g.base(line);
+    float m = -INFINITY;
+    bool nan = false;
+    for (uint32_t j = 0; j < g.n; j++) {
+        const float v = load_elem(in, base + static_cast<size_t>(j) * g.inner);
+        nan |= (v != v);
+        m = fmaxf(m, v);
+    }
+    store_elem(out, line, nan ? __uint_as_float(0x7FC00000u) : m);
+}
+
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void reduce_max_lines_kernel(const T *__restrict__ in, T *out, LineGeom g) {
+    __shared__ float fscratch[NT / kWave];
+    const uint32_t line = blockIdx.x;
+    const size_t base = g.base(line);
+    float m = -INFINITY;
+    float nan = 0.f;
+    for (uint32_t j = threadIdx.x; j < g.n; j += NT) {
+        const float v = load_elem(in, base + static_cast<size_t>(j) * g.inner);
+        if (v != v) nan = 1.f;
+        m = fmaxf(m, v);
+    }
+    m = block_max<NT>(m, fscratch);
+    nan = block_max<NT>(nan, fscratch);
+    if (threadIdx.x == 0) store_elem(out, line, nan != 0.f ? __uint_as_float(0x7FC00000u) : m);
+}
+
+// ---- top-k, one workgroup per line -----------------------------------------
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void topk_lines_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                        int32_t *__restrict__ indices, LineGeom g, uint32_t k,
+                                                        int largest) {
+    __shared__ SelectShared sh;
+    const uint32_t line = blockIdx.x;
+    const size_t base = g.base(line);
+    const uint32_t flip = largest ? 0u : 0xFFFFFFFFu;
+    select_topk_line<NT>(sh, g.n, k, [&](uint32_t j) {
+        return order_key(load_elem(in, base + static_cast<size_t>(j) * g.inner)) ^ flip;
+    });
+    const uint32_t o = line / g.inner, i = line - o * g.inner;
+    const size_t obase = static_cast<size_t>(o) * k * g.inner + i;
+    for (uint32_t r = threadIdx.x; r < k; r += NT) {
+        const uint32_t idx = composite_index(sh.sel[r]);
+        values[obase + static_cast<size_t>(r) * g.inner] = in[base + static_cast<size_t>(idx) * g.inner];  // bit copy
+        indices[obase + static_cast<size_t>(r) * g.inner] = static_cast<int32_t>(idx);
+    }
+}
+
+// ---- top-k of the softmax of a line, from precomputed line statistics -------
+// The key of element j is its probability as the output tensor would store it,
+// so the result is exactly top-k (value order, then lower index) of the softmax
+// tensor, including probabilities that collide after rounding.
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void softmax_topk_lines_kernel(const T *__restrict__ in,
+                                                                const LineStats *__restrict__ stats,
+                                                                T *__restrict__ values, int32_t *__restrict__ indices,
+                                                                LineGeom g, uint32_t k, int largest) {
+    __shared__ SelectShared sh;
+    const uint32_t line = blockIdx.x;
+    const size_t base = g.base(line);
+    const LineStats st = stats[line];
+    const uint32_t flip = largest ? 0u : 0xFFFFFFFFu;
+    select_topk_line<NT>(sh, g.n, k, [&](uint32_t j) {
+        const float p = softmax_prob(load_elem(in, base + static_cast<size_t>(j) * g.inner), st);
+        return order_key(round_to_storage<T>(p)) ^ flip;
+    });
+    const uint32_t o = line / g.inner, i = line - o * g.inner;
+    const size_t obase = static_cast<size_t>(o) * k * g.inner + i;
+    for (uint32_t r = threadIdx.x; r < k; r += NT) {
+        const uint32_t idx = composite_index(sh.sel[r]);
+        const float p = softmax_prob(load_elem(in, base + static_cast<size_t>(idx) * g.inner), st);
+        store_elem(values, obase + static_cast<size_t>(r) * g.inner, p);
+        indices[obase + static_cast<size_t>(r) * g.inner] = static_cast<int32_t>(idx);
+    }
+}
+
+// ---- workspace clear ---------------------------------------------------------
+__global__ void fill_zero_kernel(uint32_t *p, size_t words) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+}  // namespace vkop

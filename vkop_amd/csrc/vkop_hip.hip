@@ -1,0 +1,398 @@
+// C ABI of the softmax / top-k library (declared in include/vkop_hip.h):
+// argument checking, kernel selection and launches.  No kernel code lives here.
+#include "../../include/vkop_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "kernels_general.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define VKOP_HIP_TRY(expr)                                                                        \
+    do {                                                                                          \
+        hipError_t e_ = (expr);                                                                   \
+        if (e_ != hipSuccess) return fail(VKOP_HIP_ERR_DEVICE, "%s: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+
+// (outer, n, inner) view of a dense tensor around `axis`.
+struct View {
+    vkop::LineGeom g;
+    uint64_t elems;
+};
+
+int make_view(const int *shape, int ndim, int axis, View *v) {
+    if (shape == nullptr) return fail(VKOP_HIP_ERR_INVALID, "shape is null");
+    if (ndim < 1 || ndim > 4) return fail(VKOP_HIP_ERR_INVALID, "rank %d outside 1..4", ndim);
+    if (axis < 0) axis += ndim;
+    if (axis < 0 || axis >= ndim) return fail(VKOP_HIP_ERR_INVALID, "axis outside the tensor's rank %d", ndim);
+    uint64_t outer = 1, inner = 1;
+    for (int d = 0; d < ndim; d++) {
+        if (shape[d] < 0) return fail(VKOP_HIP_ERR_INVALID, "negative extent %d at dim %d", shape[d], d);
+        if (d < axis) outer *= static_cast<uint64_t>(shape[d]);
+        if (d > axis) inner *= static_cast<uint64_t>(shape[d]);
+    }
+    const uint64_t n = static_cast<uint64_t>(shape[axis]);
+    const uint64_t elems = outer * n * inner;
+    if (outer * inner >= (1ull << 31) || elems >= (1ull << 40))
+        return fail(VKOP_HIP_ERR_UNSUPPORTED, "tensor too large (%llu elements)", static_cast<unsigned long long>(elems));
+    v->g.outer = static_cast<uint32_t>(outer);
+    v->g.n = static_cast<uint32_t>(n);
+    v->g.inner = static_cast<uint32_t>(inner);
+    v->elems = elems;
+    return VKOP_HIP_OK;
+}
+
+int check_dtype(int dtype) {
+    if (dtype != VKOP_HIP_F32 && dtype != VKOP_HIP_F16) return fail(VKOP_HIP_ERR_INVALID, "unknown dtype %d", dtype);
+    return VKOP_HIP_OK;
+}
+
+int check_k(const View &v, int k) {
+    if (k < 1) return fail(VKOP_HIP_ERR_INVALID, "k = %d must be at least 1", k);
+    if (static_cast<uint64_t>(k) > v.g.n)
+        return fail(VKOP_HIP_ERR_INVALID, "k = %d exceeds the axis extent %u", k, v.g.n);
+    if (k > VKOP_HIP_MAX_K) return fail(VKOP_HIP_ERR_UNSUPPORTED, "k = %d exceeds VKOP_HIP_MAX_K = %d", k, VKOP_HIP_MAX_K);
+    return VKOP_HIP_OK;
+}
+
+int launched(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(VKOP_HIP_ERR_DEVICE, "launch of %s failed: %s", what, hipGetErrorString(e));
+    return VKOP_HIP_OK;
+}
+
+constexpr int kLineThreads = 256;
+constexpr size_t kAlign = 256;
+inline size_t align_up(size_t b) { return (b + kAlign - 1) / kAlign * kAlign; }
+
+// ---------------------------------------------------------------- softmax ----
+template <typename T>
+int softmax_impl(const T *in, T *out, const View &v, int nan_where, float nan_value, hipStream_t st) {
+    const uint32_t lines = v.g.outer * v.g.inner;
+    if (v.g.inner == 1 || v.g.n >= 2048) {
+        vkop::softmax_lines_kernel<T, kLineThreads>
+            <<<lines, kLineThreads, 0, st>>>(in, out, v.g, nan_where, nan_value, nullptr);
+        return launched("softmax_lines_kernel");
+    }
+    const uint32_t blocks = (lines + kLineThreads - 1) / kLineThreads;
+    vkop::softmax_strided_kernel<T, kLineThreads><<<blocks, kLineThreads, 0, st>>>(in, out, v.g, nan_where, nan_value);
+    return launched("softmax_strided_kernel");
+}
+
+// ------------------------------------------------------------------ top-k ----
+template <typename T>
+int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, hipStream_t st) {
+    const uint32_t lines = v.g.outer * v.g.inner;
+    vkop::topk_lines_kernel<T, kLineThreads>
+        <<<lines, kLineThreads, 0, st>>>(in, values, indices, v.g, static_cast<uint32_t>(k), largest);
+    return launched("topk_lines_kernel");
+}
+
+// ------------------------------------------------------------------ fused ----
+size_t fused_ws_bytes(const View &v) {
+    return align_up(static_cast<size_t>(v.g.outer) * v.g.inner * sizeof(vkop::LineStats));
+}
+
+template <typename T>
+int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, void *ws,
+               hipStream_t st) {
+    const uint32_t lines = v.g.outer * v.g.inner;
+    auto *stats = static_cast<vkop::LineStats *>(ws);
+    vkop::softmax_lines_kernel<T, kLineThreads><<<lines, kLineThreads, 0, st>>>(in, probs, v.g, 0, 0.f, stats);
+    if (int rc = launched("softmax_lines_kernel")) return rc;
+    vkop::softmax_topk_lines_kernel<T, kLineThreads>
+        <<<lines, kLineThreads, 0, st>>>(in, stats, values, indices, v.g, static_cast<uint32_t>(k), largest);
+    return launched("softmax_topk_lines_kernel");
+}
+
+template <typename T> int reduce_max_impl(const T *in, T *out, const View &v, hipStream_t st) {
+    const uint32_t lines = v.g.outer * v.g.inner;
+    if (v.g.inner == 1) {
+        vkop::reduce_max_lines_kernel<T, kLineThreads><<<lines, kLineThreads, 0, st>>>(in, out, v.g);
+        return launched("reduce_max_lines_kernel");
+    }
+    const uint32_t blocks = (lines + kLineThreads - 1) / kLineThreads;
+    vkop::reduce_max_strided_kernel<T, kLineThreads><<<blocks, kLineThreads, 0, st>>>(in, out, v.g);
+    return launched("reduce_max_strided_kernel");
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *vkop_hip_last_error(void) { return g_err; }
+
+int vkop_hip_init(int device) {
+    int count = 0;
+    VKOP_HIP_TRY(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(VKOP_HIP_ERR_INVALID, "device %d of %d", device, count);
+    VKOP_HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    VKOP_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(VKOP_HIP_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
+                    prop.gcnArchName);
+    VKOP_HIP_TRY(hipFree(nullptr));  // force context creation here, not inside the first timed call
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_shutdown(void) {
+    VKOP_HIP_TRY(hipDeviceSynchronize());
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_device_info(char *name, size_t name_len, int *compute_units, size_t *memory_bytes) {
+    int dev = 0;
+    VKOP_HIP_TRY(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    VKOP_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    if (name != nullptr && name_len > 0) std::snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+    if (compute_units != nullptr) *compute_units = prop.multiProcessorCount;
+    if (memory_bytes != nullptr) *memory_bytes = prop.totalGlobalMem;
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_malloc(void **ptr, size_t bytes) {
+    if (ptr == nullptr) return fail(VKOP_HIP_ERR_INVALID, "ptr is null");
+    *ptr = nullptr;
+    if (bytes == 0) return VKOP_HIP_OK;
+    VKOP_HIP_TRY(hipMalloc(ptr, bytes));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_free(void *ptr) {
+    if (ptr == nullptr) return VKOP_HIP_OK;
+    VKOP_HIP_TRY(hipFree(ptr));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return VKOP_HIP_OK;
+    if (dst == nullptr || src == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null pointer in h2d copy");
+    VKOP_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    VKOP_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return VKOP_HIP_OK;
+    if (dst == nullptr || src == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null pointer in d2h copy");
+    VKOP_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    VKOP_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return VKOP_HIP_OK;
+    if (dst == nullptr || src == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null pointer in d2d copy");
+    VKOP_HIP_TRY(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_stream_create(void **stream) {
+    if (stream == nullptr) return fail(VKOP_HIP_ERR_INVALID, "stream is null");
+    hipStream_t s;
+    VKOP_HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+    *stream = s;
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_stream_destroy(void *stream) {
+    if (stream == nullptr) return VKOP_HIP_OK;
+    VKOP_HIP_TRY(hipStreamDestroy(as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_stream_sync(void *stream) {
+    VKOP_HIP_TRY(hipStreamSynchronize(as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_event_create(void **event) {
+    if (event == nullptr) return fail(VKOP_HIP_ERR_INVALID, "event is null");
+    hipEvent_t e;
+    VKOP_HIP_TRY(hipEventCreate(&e));
+    *event = e;
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_event_destroy(void *event) {
+    if (event == nullptr) return VKOP_HIP_OK;
+    VKOP_HIP_TRY(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_event_record(void *event, void *stream) {
+    if (event == nullptr) return fail(VKOP_HIP_ERR_INVALID, "event is null");
+    VKOP_HIP_TRY(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_event_sync(void *event) {
+    if (event == nullptr) return fail(VKOP_HIP_ERR_INVALID, "event is null");
+    VKOP_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_stream_wait_event(void *stream, void *event) {
+    if (event == nullptr) return fail(VKOP_HIP_ERR_INVALID, "event is null");
+    VKOP_HIP_TRY(hipStreamWaitEvent(as_stream(stream), static_cast<hipEvent_t>(event), 0));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_event_elapsed_ms(void *start, void *stop, float *ms) {
+    if (start == nullptr || stop == nullptr || ms == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null argument");
+    VKOP_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_graph_begin(void *stream) {
+    if (stream == nullptr) return fail(VKOP_HIP_ERR_INVALID, "recording needs a stream created by vkop_hip_stream_create");
+    VKOP_HIP_TRY(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_graph_end(void *stream, void **graph) {
+    if (stream == nullptr || graph == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null argument");
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    VKOP_HIP_TRY(hipStreamEndCapture(as_stream(stream), &g));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) return fail(VKOP_HIP_ERR_DEVICE, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    *graph = exec;
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_graph_launch(void *graph, void *stream) {
+    if (graph == nullptr) return fail(VKOP_HIP_ERR_INVALID, "graph is null");
+    VKOP_HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), as_stream(stream)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_graph_destroy(void *graph) {
+    if (graph == nullptr) return VKOP_HIP_OK;
+    VKOP_HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_workspace_init(void *workspace, size_t bytes, void *stream) {
+    if (bytes == 0) return VKOP_HIP_OK;
+    if (workspace == nullptr) return fail(VKOP_HIP_ERR_INVALID, "workspace is null");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 3u) != 0 || (bytes & 3u) != 0)
+        return fail(VKOP_HIP_ERR_INVALID, "workspace address and size must be multiples of 4");
+    const size_t words = bytes / 4;
+    const unsigned blocks = static_cast<unsigned>((words + 255) / 256);
+    vkop::fill_zero_kernel<<<blocks, 256, 0, as_stream(stream)>>>(static_cast<uint32_t *>(workspace), words);
+    return launched("fill_zero_kernel");
+}
+
+size_t vkop_hip_softmax_workspace_bytes(int dtype, const int *shape, int ndim, int axis) {
+    View v;
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
+    return 0;
+}
+
+int vkop_hip_softmax(const void *in, void *out, int dtype, const int *shape, int ndim, int axis, int nan_where,
+                     float nan_value, void *workspace, size_t workspace_bytes, void *stream) {
+    (void)workspace;
+    (void)workspace_bytes;
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (v.elems == 0) return VKOP_HIP_OK;
+    if (in == nullptr || out == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    if (dtype == VKOP_HIP_F32)
+        return softmax_impl(static_cast<const float *>(in), static_cast<float *>(out), v, nan_where, nan_value,
+                            as_stream(stream));
+    return softmax_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, nan_where, nan_value,
+                        as_stream(stream));
+}
+
+size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
+    View v;
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
+    (void)k;
+    return 0;
+}
+
+int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape, int ndim,
+                  int axis, int k, int largest, int sorted, void *workspace, size_t workspace_bytes, void *stream) {
+    (void)sorted;  // results are always sorted, which satisfies sorted == 0 too
+    (void)workspace;
+    (void)workspace_bytes;
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (v.elems == 0 && k == 0) return VKOP_HIP_OK;
+    if (int rc = check_k(v, k)) return rc;
+    if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
+    if (in == nullptr || out_values == nullptr || out_indices == nullptr)
+        return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    if (dtype == VKOP_HIP_F32)
+        return topk_impl(static_cast<const float *>(in), static_cast<float *>(out_values), out_indices, v, k, largest,
+                         as_stream(stream));
+    return topk_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_values), out_indices, v, k,
+                     largest, as_stream(stream));
+}
+
+size_t vkop_hip_softmax_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
+    View v;
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
+    (void)k;
+    return fused_ws_bytes(v);
+}
+
+int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int32_t *out_indices, int dtype,
+                          const int *shape, int ndim, int axis, int k, int largest, void *workspace,
+                          size_t workspace_bytes, void *stream) {
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (v.elems == 0 && k == 0) return VKOP_HIP_OK;
+    if (int rc = check_k(v, k)) return rc;
+    if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
+    if (in == nullptr || out_values == nullptr || out_indices == nullptr)
+        return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    const size_t need = fused_ws_bytes(v);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
+    if (dtype == VKOP_HIP_F32)
+        return fused_impl(static_cast<const float *>(in), static_cast<float *>(out_probs),
+                          static_cast<float *>(out_values), out_indices, v, k, largest, workspace, as_stream(stream));
+    return fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_probs),
+                      static_cast<uint16_t *>(out_values), out_indices, v, k, largest, workspace, as_stream(stream));
+}
+
+int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape, int ndim, int axis, void *stream) {
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
+    if (v.g.n == 0) return fail(VKOP_HIP_ERR_INVALID, "max over an empty axis");
+    if (in == nullptr || out == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    if (dtype == VKOP_HIP_F32)
+        return reduce_max_impl(static_cast<const float *>(in), static_cast<float *>(out), v, as_stream(stream));
+    return reduce_max_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, as_stream(stream));
+}
+
+}  // extern "C"

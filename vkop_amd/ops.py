@@ -1,0 +1,105 @@
+"""Operator front-ends over torch device tensors.
+
+torch is used for device memory and streams only; every computation goes
+through the C ABI (vkop_amd.capi).  Inputs must be contiguous CUDA/HIP tensors
+of float32 or float16; results are new tensors on the same device, enqueued on
+torch's current stream.
+"""
+import torch
+
+from . import capi
+
+_DTYPES = {torch.float32: capi.F32, torch.float16: capi.F16}
+
+
+def _prep(x):
+    if not isinstance(x, torch.Tensor) or not x.is_cuda:
+        raise TypeError("expected a tensor on the GPU (there is no CPU path)")
+    if x.dtype not in _DTYPES:
+        raise TypeError("float32 or float16 expected, got %s" % x.dtype)
+    if x.dim() < 1 or x.dim() > 4:
+        raise ValueError("rank %d outside 1..4" % x.dim())
+    return x.contiguous(), _DTYPES[x.dtype]
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+class Workspace:
+    """Scratch device memory an operator keeps between calls, like the
+    ping-pong temporaries the reference's Topk owns (ops/Topk.hpp:46-55,221-224).
+    Cleared once when (re)allocated; calls leave it ready for the next call.
+    One workspace serves one stream at a time."""
+
+    def __init__(self):
+        self.buf = None
+
+    def get(self, nbytes):
+        nbytes = int(nbytes)
+        if nbytes == 0:
+            return 0, 0
+        if self.buf is None or self.buf.numel() < nbytes:
+            self.buf = torch.empty(nbytes + 256, dtype=torch.uint8, device="cuda")
+            self._off = (-self.buf.data_ptr()) % 256
+            self._size = (self.buf.numel() - self._off) // 4 * 4
+            capi.workspace_init(self.buf.data_ptr() + self._off, self._size, _stream())
+        return self.buf.data_ptr() + self._off, self._size
+
+
+_default_ws = Workspace()
+
+
+def softmax(x, axis=-1, nan_where=False, nan_value=0.0, out=None, workspace=None):
+    """ops/Softmax.hpp:61-141 -- same shape and dtype as x."""
+    x, dt = _prep(x)
+    if out is None:
+        out = torch.empty_like(x)
+    ws = workspace or _default_ws
+    ptr, size = ws.get(capi.softmax_workspace_bytes(dt, x.shape, axis))
+    capi.softmax(x.data_ptr(), out.data_ptr(), dt, x.shape, axis, int(bool(nan_where)), nan_value, ptr, size, _stream())
+    return out
+
+
+def _out_shape(x, axis, k):
+    shape = list(x.shape)
+    shape[axis if axis >= 0 else axis + x.dim()] = int(k)
+    return shape
+
+
+def topk(x, k, axis=-1, largest=True, sorted=True, workspace=None):
+    """ops/Topk.hpp:95-218 -- (values like x, int32 indices), [axis] = k."""
+    x, dt = _prep(x)
+    shape = _out_shape(x, axis, k)
+    values = torch.empty(shape, dtype=x.dtype, device=x.device)
+    indices = torch.empty(shape, dtype=torch.int32, device=x.device)
+    ws = workspace or _default_ws
+    ptr, size = ws.get(capi.topk_workspace_bytes(dt, x.shape, axis, k))
+    capi.topk(x.data_ptr(), values.data_ptr(), indices.data_ptr(), dt, x.shape, axis, k, int(bool(largest)),
+              int(bool(sorted)), ptr, size, _stream())
+    return values, indices
+
+
+def softmax_topk(x, k, axis=-1, largest=True, return_probs=False, workspace=None):
+    """The registered post-proc pair of benchmark/main.cpp:85-101 in one call:
+    top-k of softmax(x) along `axis`, without materialising the softmax tensor
+    unless return_probs is set."""
+    x, dt = _prep(x)
+    shape = _out_shape(x, axis, k)
+    values = torch.empty(shape, dtype=x.dtype, device=x.device)
+    indices = torch.empty(shape, dtype=torch.int32, device=x.device)
+    probs = torch.empty_like(x) if return_probs else None
+    ws = workspace or _default_ws
+    ptr, size = ws.get(capi.softmax_topk_workspace_bytes(dt, x.shape, axis, k))
+    capi.softmax_topk(x.data_ptr(), probs.data_ptr() if return_probs else 0, values.data_ptr(), indices.data_ptr(),
+                      dt, x.shape, axis, k, int(bool(largest)), ptr, size, _stream())
+    return (values, indices, probs) if return_probs else (values, indices)
+
+
+def reduce_max(x, axis):
+    x, dt = _prep(x)
+    shape = list(x.shape)
+    del shape[axis if axis >= 0 else axis + x.dim()]
+    out = torch.empty(shape, dtype=x.dtype, device=x.device)
+    capi.reduce_max(x.data_ptr(), out.data_ptr(), dt, x.shape, axis, _stream())
+    return out
