@@ -106,7 +106,31 @@ template <int NT> __device__ __forceinline__ double block_sum(double v, double *
 
 // --------------------------------------------------------------- softmax ----
 
-// One softmax term: exp of the single-precision difference, <= 1 ulp.
-__device__ __forceinline__ float softmax_term(float x, float m) { return expf(x - m); }
+// exp(d) rounded to float, evaluated in double (fp64 FMA runs at the same rate
+// as scalar fp32 FMA on this chip): the relative error before the final
+// rounding is below 2^-36, so the result is the correctly rounded float except
+// within that distance of a rounding midpoint, where it is the other
+// neighbour.  d <= -104 (including -inf) gives 0; NaN gives NaN.
+__device__ __forceinline__ float exp_accurate(float d) {
+    if (d <= -104.0f) return 0.0f;
+    if (d > 89.0f) return __uint_as_float(0x7F800000u);
+    const double x = static_cast<double>(d);
+    const double n = rint(x * 1.4426950408889634074);
+    const double r = fma(-n, 0.69314718055994530942, x);  // |r| <= 0.3466
+    double p = 1.0 / 362880.0;
+    p = fma(p, r, 1.0 / 40320.0);
+    p = fma(p, r, 1.0 / 5040.0);
+    p = fma(p, r, 1.0 / 720.0);
+    p = fma(p, r, 1.0 / 120.0);
+    p = fma(p, r, 1.0 / 24.0);
+    p = fma(p, r, 1.0 / 6.0);
+    p = fma(p, r, 0.5);
+    p = fma(p, r, 1.0);
+    p = fma(p, r, 1.0);
+    return static_cast<float>(ldexp(p, static_cast<int>(n)));
+}
+
+// One softmax term: exp of the single-precision difference x - m.
+__device__ __forceinline__ float softmax_term(float x, float m) { return exp_accurate(x - m); }
 
 }  // namespace vkop

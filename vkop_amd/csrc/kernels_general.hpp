@@ -20,8 +20,9 @@ struct LineGeom {
 };
 
 struct LineStats {
-    float m;  // max of the line (NaN ignored)
-    float s;  // sum of exp(x - m), rounded once from double
+    float m;      // max of the line (NaN ignored)
+    float pad;
+    double rinv;  // 1 / sum of exp(x - m), the sum taken in double
 };
 
 // max and sum of exp(x - max) of one line, by all NT threads of the block.
@@ -32,25 +33,25 @@ __device__ __forceinline__ LineStats line_stats(const T *x, size_t base, uint32_
     float m = -INFINITY;
     for (uint32_t j = tid; j < n; j += NT) m = fmaxf(m, load_elem(x, base + static_cast<size_t>(j) * stride));
     m = block_max<NT>(m, fscratch);
-    // four independent float partial sums per thread keep every running sum
-    // short; the cross-thread combine is in double, in a fixed order
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    // every term is a float (as the softmax definition rounds it); the sum of
+    // the terms is exact to double rounding, in a fixed order
+    double a0 = 0.0, a1 = 0.0;
     uint32_t j = tid;
-    for (; j + 3u * NT < n; j += 4u * NT) {
-        a0 += softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m);
-        a1 += softmax_term(load_elem(x, base + static_cast<size_t>(j + NT) * stride), m);
-        a2 += softmax_term(load_elem(x, base + static_cast<size_t>(j + 2u * NT) * stride), m);
-        a3 += softmax_term(load_elem(x, base + static_cast<size_t>(j + 3u * NT) * stride), m);
+    for (; j + NT < n; j += 2u * NT) {
+        a0 += static_cast<double>(softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m));
+        a1 += static_cast<double>(softmax_term(load_elem(x, base + static_cast<size_t>(j + NT) * stride), m));
     }
-    for (; j < n; j += NT) a0 += softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m);
-    double s = (static_cast<double>(a0) + static_cast<double>(a1)) + (static_cast<double>(a2) + static_cast<double>(a3));
-    s = block_sum<NT>(s, dscratch);
-    return LineStats{m, static_cast<float>(s)};
+    if (j < n) a0 += static_cast<double>(softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m));
+    const double s = block_sum<NT>(a0 + a1, dscratch);
+    return LineStats{m, 0.f, 1.0 / s};
 }
 
 // Probability of one element given its line's statistics: the single formula
-// every kernel uses, so separately computed results agree bit for bit.
-__device__ __forceinline__ float softmax_prob(float x, LineStats st) { return softmax_term(x, st.m) / st.s; }
+// every kernel uses, so separately computed results agree bit for bit.  The
+// term is rounded to float first, then scaled in double and rounded once.
+__device__ __forceinline__ float softmax_prob(float x, LineStats st) {
+    return static_cast<float>(static_cast<double>(softmax_term(x, st.m)) * st.rinv);
+}
 
 // ---- softmax, one workgroup per line ---------------------------------------
 template <typename T, int NT>
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(NT) void softmax_strided_kernel(const T *in, T *out
     double s = 0.0;
     for (uint32_t j = 0; j < g.n; j++)
         s += static_cast<double>(softmax_term(load_elem(in, base + static_cast<size_t>(j) * g.inner), m));
-    const LineStats st{m, static_cast<float>(s)};
+    const LineStats st{m, 0.f, 1.0 / s};
     for (uint32_t j = 0; j < g.n; j++) {
         const size_t at = base + static_cast<size_t>(j) * g.inner;
         float p = round_to_storage<T>(softmax_prob(load_elem(in, at), st));
