@@ -216,9 +216,24 @@ def assert_fused(ops, x, k, axis=-1, largest=True):
     assert np.array_equal(v.view(bits), ev.view(bits))
     # (2) that tensor is the softmax, to the softmax bar
     assert_softmax_close(p, x, axis)
-    # (3) without the tensor the result is the same
+    # (3) without the tensor (the single-pass streaming kernel where it applies):
+    # same ranking; its row sum is built from chunk partials, so a value may
+    # round the other way
     v2, ix2 = ops.softmax_topk(dev(x), k, axis, largest)
-    assert np.array_equal(host(ix2), ix) and np.array_equal(host(v2).view(bits), v.view(bits))
+    v2, ix2 = host(v2), host(ix2)
+    same = np.array_equal(ix2, ix)
+    if x.dtype == np.float16:
+        assert half_ulp_diff(v2, v).max() <= 1
+    else:
+        assert ulp_diff(v2, v).max() <= 1
+    if not same:
+        # only a probability tie that the 1-ulp difference opens or closes may
+        # reorder: the ranking must still be exact for the values it returned
+        pm = np.moveaxis(p, axis, -1).reshape(-1, x.shape[axis])
+        i2 = np.moveaxis(ix2, axis, -1).reshape(-1, k)
+        i1 = np.moveaxis(ix, axis, -1).reshape(-1, k)
+        for r in range(pm.shape[0]):
+            assert sorted(pm[r][i2[r]].tolist()) == sorted(pm[r][i1[r]].tolist()), r
     # (4) against the oracle's own fused result: values to the softmax bar,
     # indices wherever the oracle's probabilities around the cut are distinct
     ov, oix, op = oracle.softmax_topk(x, k, axis, largest, return_probs=True)

@@ -8,7 +8,10 @@
 #include <cstdio>
 #include <cstring>
 
+#include <cstdlib>
+
 #include "kernels_general.hpp"
+#include "kernels_rows.hpp"
 
 namespace {
 
@@ -95,9 +98,130 @@ int softmax_impl(const T *in, T *out, const View &v, int nan_where, float nan_va
     return launched("softmax_strided_kernel");
 }
 
+// ------------------------------------------------- streaming rows kernel ----
+// Launch shape of rows_topk_kernel: NT threads, V 128-bit loads per thread,
+// G chunks per row of `per` elements each.
+struct RowsCfg {
+    bool ok = false;
+    int nt = 0, v = 0;
+    uint32_t g = 0, per = 0;
+};
+
+RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
+    RowsCfg c;
+    if (v.g.inner != 1 || k > vkop::kFastMaxK || v.g.n == 0 || v.g.outer == 0) return c;
+    const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
+    const uint32_t n = v.g.n, rows = v.g.outer;
+    static const int shapes_f32[][2] = {{256, 1}, {256, 2}, {256, 4}, {1024, 2}, {1024, 4}, {1024, 8}};
+    static const int shapes_f16[][2] = {{256, 1}, {256, 2}, {256, 4}, {1024, 2}, {1024, 4}, {1024, 4}};
+    const auto *shapes = dtype == VKOP_HIP_F32 ? shapes_f32 : shapes_f16;
+    int forced_nt = 0, forced_v = 0, forced_g = 0;
+    if (const char *env = std::getenv("VKOP_HIP_ROWS_CFG")) {  // tuning aid: "NT,V,G"
+        if (std::sscanf(env, "%d,%d,%d", &forced_nt, &forced_v, &forced_g) != 3) forced_nt = 0;
+    }
+    const uint32_t nvec = (n + vec - 1) / vec;
+    auto fits = [&](int nt, int vv, uint32_t g) {
+        if (g < 1 || g > 64 || static_cast<uint64_t>(g) * (k + 1) > vkop::kMergeSlots) return false;
+        const uint32_t per = (nvec + g - 1) / g * vec;
+        return per <= static_cast<uint32_t>(nt) * vv * vec && static_cast<uint64_t>(rows) * g < (1ull << 31);
+    };
+    if (forced_nt) {
+        if (!fits(forced_nt, forced_v, static_cast<uint32_t>(forced_g))) return c;
+        c.nt = forced_nt, c.v = forced_v, c.g = static_cast<uint32_t>(forced_g);
+    } else {
+        // largest per-workgroup chunk that still leaves >= 1024 workgroups; if the
+        // tensor is too small for that, the smallest shape that covers a row
+        int pick = -1;
+        for (int i = 0; i < 6; i++) {
+            const uint32_t cap = static_cast<uint32_t>(shapes[i][0]) * shapes[i][1] * vec;
+            const uint32_t g = (n + cap - 1) / cap;
+            if (!fits(shapes[i][0], shapes[i][1], g)) continue;
+            if (pick < 0) pick = i;
+            if (static_cast<uint64_t>(rows) * g >= 1024) pick = i;
+        }
+        if (pick < 0) return c;
+        c.nt = shapes[pick][0], c.v = shapes[pick][1];
+        const uint32_t cap = static_cast<uint32_t>(c.nt) * c.v * vec;
+        c.g = (n + cap - 1) / cap;
+    }
+    c.per = (nvec + c.g - 1) / c.g * vec;
+    c.ok = true;
+    return c;
+}
+
+struct RowsLayout {
+    size_t tickets = 0, partials = 0, cands = 0, stats = 0, total = 0;
+};
+
+// One layout serves the streaming kernel and the general two-kernel path, so
+// the size does not depend on which of them a call ends up taking.
+RowsLayout rows_layout(const View &v, int k, const RowsCfg &c) {
+    RowsLayout l;
+    const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
+    size_t off = 0;
+    l.tickets = off;
+    off += align_up(lines * sizeof(uint32_t));
+    l.stats = off;
+    off += align_up(lines * sizeof(vkop::LineStats));
+    if (c.ok) {
+        l.partials = off;
+        off += align_up(lines * c.g * sizeof(vkop::ChunkPartial));
+        l.cands = off;
+        off += align_up(lines * c.g * static_cast<size_t>(k + 1) * sizeof(uint64_t));
+    }
+    l.total = off;
+    return l;
+}
+
+template <typename T, bool SOFTMAX>
+int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, const RowsCfg &c, void *ws,
+                const RowsLayout &l, hipStream_t st) {
+    vkop::RowsWorkspace w;
+    auto *base = static_cast<unsigned char *>(ws);
+    w.tickets = reinterpret_cast<uint32_t *>(base + l.tickets);
+    w.partials = reinterpret_cast<vkop::ChunkPartial *>(base + l.partials);
+    w.cands = reinterpret_cast<uint64_t *>(base + l.cands);
+    w.kc = static_cast<uint32_t>(k + 1);
+    const uint32_t vec = 16 / sizeof(T);
+    const bool aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
+    const uint32_t blocks = v.g.outer * c.g;
+#define VKOP_ROWS_CASE(NT, V)                                                                                   \
+    if (c.nt == NT && c.v == V) {                                                                               \
+        if (aligned)                                                                                            \
+            vkop::rows_topk_kernel<T, NT, V, SOFTMAX, true>                                                     \
+                <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w);   \
+        else                                                                                                    \
+            vkop::rows_topk_kernel<T, NT, V, SOFTMAX, false>                                                    \
+                <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w);   \
+        return launched("rows_topk_kernel");                                                                    \
+    }
+    VKOP_ROWS_CASE(256, 1)
+    VKOP_ROWS_CASE(256, 2)
+    VKOP_ROWS_CASE(256, 4)
+    VKOP_ROWS_CASE(512, 2)
+    VKOP_ROWS_CASE(512, 4)
+    VKOP_ROWS_CASE(1024, 1)
+    VKOP_ROWS_CASE(1024, 2)
+    VKOP_ROWS_CASE(1024, 4)
+    if constexpr (sizeof(T) == 4) {
+        VKOP_ROWS_CASE(256, 8)
+        VKOP_ROWS_CASE(1024, 8)
+    }
+#undef VKOP_ROWS_CASE
+    return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_topk_kernel for %d threads x %d loads", c.nt, c.v);
+}
+
 // ------------------------------------------------------------------ top-k ----
 template <typename T>
-int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, hipStream_t st) {
+int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int dtype, void *ws,
+              size_t ws_bytes, hipStream_t st) {
+    const RowsCfg c = largest ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
+    if (c.ok) {
+        const RowsLayout l = rows_layout(v, k, c);
+        if (ws == nullptr || ws_bytes < l.total)
+            return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, l.total);
+        return launch_rows<T, false>(in, values, indices, v, k, c, ws, l, st);
+    }
     const uint32_t lines = v.g.outer * v.g.inner;
     vkop::topk_lines_kernel<T, kLineThreads>
         <<<lines, kLineThreads, 0, st>>>(in, values, indices, v.g, static_cast<uint32_t>(k), largest);
@@ -105,15 +229,16 @@ int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, in
 }
 
 // ------------------------------------------------------------------ fused ----
-size_t fused_ws_bytes(const View &v) {
-    return align_up(static_cast<size_t>(v.g.outer) * v.g.inner * sizeof(vkop::LineStats));
-}
-
 template <typename T>
-int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, void *ws,
-               hipStream_t st) {
+int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, int dtype,
+               void *ws, hipStream_t st) {
+    const RowsCfg c = choose_rows_cfg(v, k, dtype);
+    const RowsLayout l = rows_layout(v, k, c);
+    if (c.ok && largest && probs == nullptr) return launch_rows<T, true>(in, values, indices, v, k, c, ws, l, st);
+    // general path: line statistics (and the softmax tensor when asked for), then
+    // an exact select keyed by the probabilities those statistics define
     const uint32_t lines = v.g.outer * v.g.inner;
-    auto *stats = static_cast<vkop::LineStats *>(ws);
+    auto *stats = reinterpret_cast<vkop::LineStats *>(static_cast<unsigned char *>(ws) + l.stats);
     vkop::softmax_lines_kernel<T, kLineThreads><<<lines, kLineThreads, 0, st>>>(in, probs, v.g, 0, 0.f, stats);
     if (int rc = launched("softmax_lines_kernel")) return rc;
     vkop::softmax_topk_lines_kernel<T, kLineThreads>
@@ -328,16 +453,14 @@ int vkop_hip_softmax(const void *in, void *out, int dtype, const int *shape, int
 
 size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
-    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
-    (void)k;
-    return 0;
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return 0;
+    const RowsCfg c = choose_rows_cfg(v, k, dtype);
+    return c.ok ? rows_layout(v, k, c).total : 0;
 }
 
 int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape, int ndim,
                   int axis, int k, int largest, int sorted, void *workspace, size_t workspace_bytes, void *stream) {
     (void)sorted;  // results are always sorted, which satisfies sorted == 0 too
-    (void)workspace;
-    (void)workspace_bytes;
     View v;
     if (int rc = check_dtype(dtype)) return rc;
     if (int rc = make_view(shape, ndim, axis, &v)) return rc;
@@ -348,16 +471,15 @@ int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dt
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
     if (dtype == VKOP_HIP_F32)
         return topk_impl(static_cast<const float *>(in), static_cast<float *>(out_values), out_indices, v, k, largest,
-                         as_stream(stream));
+                         dtype, workspace, workspace_bytes, as_stream(stream));
     return topk_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_values), out_indices, v, k,
-                     largest, as_stream(stream));
+                     largest, dtype, workspace, workspace_bytes, as_stream(stream));
 }
 
 size_t vkop_hip_softmax_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
-    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
-    (void)k;
-    return fused_ws_bytes(v);
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return 0;
+    return rows_layout(v, k, choose_rows_cfg(v, k, dtype)).total;
 }
 
 int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int32_t *out_indices, int dtype,
@@ -371,16 +493,18 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
     if (in == nullptr || out_values == nullptr || out_indices == nullptr)
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
-    const size_t need = fused_ws_bytes(v);
+    const size_t need = rows_layout(v, k, choose_rows_cfg(v, k, dtype)).total;
     if (workspace == nullptr || workspace_bytes < need)
         return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
         return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
     if (dtype == VKOP_HIP_F32)
         return fused_impl(static_cast<const float *>(in), static_cast<float *>(out_probs),
-                          static_cast<float *>(out_values), out_indices, v, k, largest, workspace, as_stream(stream));
+                          static_cast<float *>(out_values), out_indices, v, k, largest, dtype, workspace,
+                          as_stream(stream));
     return fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_probs),
-                      static_cast<uint16_t *>(out_values), out_indices, v, k, largest, workspace, as_stream(stream));
+                      static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, workspace,
+                      as_stream(stream));
 }
 
 int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape, int ndim, int axis, void *stream) {
