@@ -1,6 +1,6 @@
-// Streaming kernel for contiguous rows (the reduced axis is the last one).
+// Streaming kernels for contiguous rows (the reduced axis is the last one).
 //
-// rows_topk_kernel makes one pass over the input.  A row is split into G
+// rows_chunk_kernel makes the one pass over the input.  A row is split into G
 // chunks, one workgroup per chunk, so a few long rows still fill the chip.
 // Each workgroup
 //   1. pulls its chunk into registers with 128-bit loads (V per thread),
@@ -9,14 +9,17 @@
 //      c-th largest per-lane maximum, then the minimum over the waves -- and
 //      appends the few elements above it to an LDS list,
 //   4. ranks that list exactly (key, then lower index) and writes its k+1 best,
-//      in order, plus (max, sum) to the workspace,
-//   5. takes a ticket; the workgroup that arrives last for a row merges the G
-//      partial results the same way, computes the probabilities of the winners
-//      only, orders equal probabilities by index and writes the row's result.
+//      in order, plus (max, sum) to the workspace.
+// rows_merge_kernel (one workgroup per row; run inside the chunk kernel when
+// G == 1) merges the G partial results the same way, computes the
+// probabilities of the winners only, orders equal probabilities by index and
+// writes the row's result.  There are no atomics or fences between workgroups:
+// the kernel boundary publishes the partial results, and the outcome does not
+// depend on scheduling.
 // Whatever the shortcut cannot prove exact (too many elements at a threshold,
-// a probability tie across the k-th place, NaN/inf rows) is redone by the same
-// workgroup with the exact radix select of select.hpp, so the result is always
-// top-k (probability, then lower index) of the row's softmax.
+// a probability tie across the k-th place, NaN/inf rows) is redone by the
+// merging workgroup with the exact radix select of select.hpp, so the result
+// is always top-k (probability, then lower index) of the row's softmax.
 #pragma once
 
 #include "device_utils.hpp"
@@ -25,15 +28,17 @@
 
 namespace vkop {
 
-constexpr int kFastCap = 1024;      // LDS slots for elements above a threshold
-constexpr int kFastMaxK = 255;      // k + 1 <= 256 ranks are kept in LDS
-constexpr int kMergeSlots = 4096;   // G * (k + 1) the merge can take in registers
+constexpr int kFastCap = 1024;     // LDS slots for elements above a threshold
+constexpr int kFastMaxK = 255;     // k + 1 <= 256 ranks are kept in LDS
+constexpr int kMergeThreads = 1024;
+constexpr int kMergeSlots = 4096;  // G * (k + 1) the merge takes in registers
 
 // ---- wave-level helpers (all 64 lanes must be active) -----------------------
 
 // max over the wave, returned wave-uniform: four DPP-fused steps inside each
 // row of 16 lanes, then the four row results through scalar registers.
-#define VKOP_DPP_U32(a, ctrl) static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(a), ctrl, 0xF, 0xF, true))
+#define VKOP_DPP_U32(a, ctrl) \
+    static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(a), ctrl, 0xF, 0xF, true))
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     v = max(v, VKOP_DPP_U32(v, 0xB1));   // quad_perm 1,0,3,2
     v = max(v, VKOP_DPP_U32(v, 0x4E));   // quad_perm 2,3,0,1
@@ -55,27 +60,17 @@ __device__ __forceinline__ uint32_t float_to_ordered(float v) {
 __device__ __forceinline__ float ordered_to_float(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
 }
-
 __device__ __forceinline__ float wave_max_f32_uniform(float v) {
     return ordered_to_float(wave_max_u32(float_to_ordered(v)));
 }
 
-// c-th largest (1-based, 1 <= c <= 64) of the 64 lane values, wave-uniform.
-// Equal values count separately.  Small c: knock the maximum out c-1 times;
-// otherwise a bitwise descent with ballots.
-__device__ __forceinline__ uint32_t wave_kth_largest_u32(uint32_t v, uint32_t c) {
-    if (c <= 8) {
-        uint32_t m = wave_max_u32(v);
-        for (uint32_t r = 1; r < c; r++) {
-            const uint64_t holders = __ballot(v == m);
-            const int first = __ffsll(static_cast<long long>(holders)) - 1;
-            if (static_cast<int>(threadIdx.x & (kWave - 1)) == first) v = 0u;
-            m = wave_max_u32(v);
-        }
-        return m;
-    }
+// A lower bound, wave-uniform, of the c-th largest (1 <= c <= 64) of the 64 lane
+// values that at least c lanes reach: bitwise descent over the top `bits` bits
+// with ballots (the low bits stay zero, which only lowers the bound).  Returns
+// 0 when fewer than c lanes are non-zero.
+__device__ __forceinline__ uint32_t wave_cth_largest_floor(uint32_t v, uint32_t c, int bits) {
     uint32_t prefix = 0;
-    for (int bit = 31; bit >= 0; bit--) {
+    for (int bit = 31; bit > 31 - bits; bit--) {
         const uint32_t trial = prefix | (1u << bit);
         if (static_cast<uint32_t>(__popcll(__ballot(v >= trial))) >= c) prefix = trial;
     }
@@ -93,7 +88,6 @@ struct ChunkPartial {
 };
 
 struct RowsWorkspace {
-    uint32_t *tickets;       // [rows], zero between calls
     ChunkPartial *partials;  // [rows][G]
     uint64_t *cands;         // [rows][G][kc]
     uint32_t kc;             // slots per chunk (k + 1)
@@ -123,14 +117,14 @@ union RowsSharedUnion {
 
 // Fast term for the running sum: exp2((x - m) * log2 e) on the hardware
 // exponential unit.  Only ever summed; every probability that is output uses
-// exp_accurate, and the terms of the chunk's largest elements are replaced by
+// exp_accurate, and the terms of a chunk's largest elements are replaced by
 // accurate ones before the sum leaves the workgroup.
 __device__ __forceinline__ float fast_term(float x, float m) {
     return __builtin_amdgcn_exp2f((x - m) * 1.44269504088896341f);
 }
 
 // Exact ranking of sh.cand[0..C): sh.rank[i] = number of larger composites.
-// All NT threads call; ends with a barrier.
+// All NT threads call with the same C; ends with a barrier.
 template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uint32_t C) {
     const uint32_t tid = threadIdx.x;
     if (C == 0) return;
@@ -162,7 +156,7 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
 // key of its e-th element (0 = no element), lane_max_key the largest of them.
 // On return sh.cand[0..sh.count) holds the composite of every element whose key
 // reaches the block threshold -- at least min(want, elements in the block) of
-// them -- unless sh.count > kFastCap (too many; list truncated).
+// them -- unless sh.count > kFastCap (too many; the list is truncated).
 template <int NT, int E, typename KeyAt, typename IdxAt>
 __device__ __forceinline__ void block_threshold_gather(RowsShared &sh, uint32_t lane_max_key, uint32_t want,
                                                        KeyAt key_at, IdxAt idx_at) {
@@ -185,7 +179,7 @@ __device__ __forceinline__ void block_threshold_gather(RowsShared &sh, uint32_t 
         }
     }
     const uint32_t cw = min(c, valid);
-    const uint32_t tw = (c == 0) ? 0u : (cw == 0 ? 0xFFFFFFFFu : wave_kth_largest_u32(lane_max_key, cw));
+    const uint32_t tw = (c == 0) ? 0u : (cw == 0 ? 0xFFFFFFFFu : wave_cth_largest_floor(lane_max_key, cw, 24));
     if (lane == 0) sh.wave_key[wave] = tw;
     __syncthreads();
     uint32_t thr = sh.wave_key[0];
@@ -222,154 +216,34 @@ template <> struct Vec128<uint16_t> {
     }
 };
 
-// SOFTMAX = true : fused softmax -> top-k (values are probabilities)
-// SOFTMAX = false: plain top-k, largest first (values are copies of the input)
-// ALIGNED: every row start is 16-byte aligned and n is a multiple of the vector
-// width, so chunks are read with 128-bit loads.
-// Launch: rows * G workgroups of NT threads; per = elements per chunk
-// (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
-template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED>
-__global__ __launch_bounds__(NT) void rows_topk_kernel(const T *__restrict__ in, T *__restrict__ values,
-                                                       int32_t *__restrict__ indices, uint32_t n, uint32_t k,
-                                                       uint32_t G, uint32_t per, RowsWorkspace ws) {
-    constexpr int VEC = Vec128<T>::N;
-    constexpr int E = V * VEC;
-    constexpr int NW = NT / kWave;
-    __shared__ RowsSharedUnion smem;
-    __shared__ float fscratch[NW];
-    __shared__ double dscratch[NW];
-    __shared__ uint32_t s_ticket, s_slow;
+// ---- merge of one row's chunk results (all NT threads of a workgroup) --------
+// EM = candidate slots each thread takes (EM * NT >= G * ws.kc).
+template <typename T, int NT, int EM, bool SOFTMAX>
+__device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch, double *dscratch, const T *rowp,
+                                          T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
+                                          const ChunkPartial *pp, const uint64_t *rc, uint32_t kc) {
     RowsShared &sh = smem.fast;
-
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
-    const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
-    const T *rowp = in + static_cast<size_t>(row) * n;
-    const uint32_t want = k + 1;  // one extra: the merge needs the (k+1)-th to prove the cut
+    const uint32_t want = k + 1;
+    const uint32_t kk = min(k, n);
+    const uint32_t slots = G * kc;
 
-    // ---- 1. chunk -> registers ------------------------------------------------
-    float x[E];
-    if constexpr (ALIGNED) {
-        Vec128<T> q[V];
+    // candidates first: their loads do not depend on the row statistics
+    uint64_t mc[EM];
+    uint32_t lmk = 0;
 #pragma unroll
-        for (int i = 0; i < V; i++) {
-            const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
-            if (e0 < c1) q[i].load(rowp + e0);
+    for (int e = 0; e < EM; e++) {
+        const uint32_t t = static_cast<uint32_t>(e) * NT + tid;
+        uint64_t c = 0;
+        if (t < slots) {
+            const uint32_t g = t / kc, j = t - g * kc;
+            if (j < pp[g].count) c = rc[t];
         }
-#pragma unroll
-        for (int i = 0; i < V; i++) {
-            const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
-#pragma unroll
-            for (int c = 0; c < VEC; c++) x[i * VEC + c] = (e0 < c1) ? q[i].get(c) : -INFINITY;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < V; i++) {
-#pragma unroll
-            for (int c = 0; c < VEC; c++) {
-                const uint32_t e = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC + c;
-                x[i * VEC + c] = (e < c1) ? load_elem(rowp, e) : -INFINITY;
-            }
-        }
+        mc[e] = c;
+        lmk = max(lmk, static_cast<uint32_t>(c >> 32));
     }
-    auto index_of = [&](int e) -> uint32_t {
-        return c0 + (static_cast<uint32_t>(e / VEC) * NT + tid) * VEC + static_cast<uint32_t>(e % VEC);
-    };
-
-    // ---- 2. max and sum of exp ------------------------------------------------
-    float lmax = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < E; e++) lmax = fmaxf(lmax, x[e]);
-    float m_g = -INFINITY;
-    if constexpr (SOFTMAX) {
-        const float wm = wave_max_f32_uniform(lmax);
-        if (lane == 0) sh.wave_m[wave] = wm;
-        __syncthreads();
-        m_g = sh.wave_m[0];
-#pragma unroll
-        for (int w = 1; w < NW; w++) m_g = fmaxf(m_g, sh.wave_m[w]);
-        // a chunk without a finite element sums against 0: its terms are all 0
-        // (or NaN, which must survive), never -inf - -inf
-        const float ref = (m_g > -INFINITY) ? m_g : 0.f;
-        float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-        for (int e = 0; e < E; e += 2) {
-            a0 += fast_term(x[e], ref);
-            a1 += fast_term(x[e + 1], ref);
-        }
-        const double wsum = wave_sum(static_cast<double>(a0) + static_cast<double>(a1));
-        if (lane == 0) sh.wave_s[wave] = wsum;
-    }
-
-    // ---- 3. threshold and gather ------------------------------------------------
-    const bool any_valid = (c0 + tid * VEC) < c1;
-    uint32_t lkey = any_valid ? order_key(lmax) : 0u;
-    if constexpr (!SOFTMAX) {
-        // fmaxf drops NaN, but NaN ranks first in a plain top-k: take the max of
-        // the keys instead (a softmax row with a NaN goes to the exact path anyway)
-        lkey = 0u;
-#pragma unroll
-        for (int e = 0; e < E; e++) lkey = max(lkey, index_of(e) < c1 ? order_key(x[e]) : 0u);
-    }
-    block_threshold_gather<NT, E>(
-        sh, lkey, want, [&](int e) -> uint32_t { return index_of(e) < c1 ? order_key(x[e]) : 0u; },
-        [&](int e) -> uint32_t { return index_of(e); });
-    const uint32_t C = sh.count;
-    const bool overflow = C > kFastCap;
-
-    // ---- 4. exact ranking of the gathered elements, emit the best `want` -------
-    uint64_t *out_c = ws.cands + (static_cast<size_t>(row) * G + chunk) * ws.kc;
-    uint32_t emitted = 0;
-    if (!overflow) {
-        block_rank<NT>(sh, C);
-        emitted = min(C, want);
-        for (uint32_t t = tid; t < C; t += NT) {
-            const uint32_t r = sh.rank[t];
-            if (r < emitted) {
-                const uint64_t cmp = sh.cand[t];
-                out_c[r] = cmp;
-                if constexpr (SOFTMAX) {
-                    // replace this element's fast term by the accurate one (the
-                    // difference of two nearby floats is exact)
-                    const float xv = ordered_to_float(static_cast<uint32_t>(cmp >> 32));
-                    const float ref = (m_g > -INFINITY) ? m_g : 0.f;
-                    sh.prob[r] = exp_accurate(xv - ref) - fast_term(xv, ref);
-                }
-            }
-        }
-    }
-    __syncthreads();
-    if (wave == 0) {
-        double acc = 0.0;
-        if constexpr (SOFTMAX) {
-            const float ref = (m_g > -INFINITY) ? m_g : 0.f;
-            (void)ref;
-            if (lane < NW) acc = sh.wave_s[lane];
-            for (uint32_t r = lane; r < emitted; r += kWave) acc += static_cast<double>(sh.prob[r]);
-            acc = wave_sum(acc);  // same tree every time: run-to-run stable
-        }
-        if (lane == 0) {
-            ChunkPartial p;
-            p.s = acc;
-            p.m = m_g;
-            p.count = emitted;
-            p.flags = overflow ? 1u : 0u;
-            p.pad[0] = p.pad[1] = p.pad[2] = 0;
-            ws.partials[static_cast<size_t>(row) * G + chunk] = p;
-        }
-    }
-
-    // ---- 5. ticket: the last workgroup of the row merges -----------------------
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) s_ticket = (G == 1) ? 0u : atomicAdd(&ws.tickets[row], 1u);
-    __syncthreads();
-    if (s_ticket != G - 1) return;
-    __threadfence();
-    if (tid == 0 && G > 1) ws.tickets[row] = 0;  // ready for the next call
 
     // row statistics: lane g of wave 0 takes chunk g (G <= 64), fixed reduction tree
-    const ChunkPartial *pp = ws.partials + static_cast<size_t>(row) * G;
     if (wave == 0) {
         float mg = -INFINITY;
         double sg = 0.0;
@@ -388,6 +262,7 @@ __global__ __launch_bounds__(NT) void rows_topk_kernel(const T *__restrict__ in,
         bool bad = __ballot(flg != 0u) != 0ull;
         if (SOFTMAX && !(S > 0.0 && S < 1e300)) bad = true;  // NaN / inf rows
         if (SOFTMAX && !(M > -INFINITY && M < INFINITY)) bad = true;
+        if (slots > static_cast<uint32_t>(EM) * NT) bad = true;
         if (lane == 0) {
             sh.row_m = M;
             sh.row_rinv = 1.0 / S;
@@ -400,27 +275,7 @@ __global__ __launch_bounds__(NT) void rows_topk_kernel(const T *__restrict__ in,
     bool slow = sh.row_slow != 0u;
     const uint32_t total = sh.row_total;
 
-    const uint32_t kk = min(k, n);
-    const uint32_t slots = G * ws.kc;
-    constexpr int EM = kMergeSlots / NT;  // merge elements per thread
-    if (slots > static_cast<uint32_t>(kMergeSlots)) slow = true;
     if (!slow) {
-        // gather the chunk lists and rank them again
-        uint64_t mc[EM];
-        uint32_t lmk = 0;
-        const uint64_t *rc = ws.cands + static_cast<size_t>(row) * G * ws.kc;
-#pragma unroll
-        for (int e = 0; e < EM; e++) {
-            const uint32_t t = static_cast<uint32_t>(e) * NT + tid;
-            uint64_t c = 0;
-            if (t < slots) {
-                const uint32_t g = t / ws.kc, j = t - g * ws.kc;
-                if (j < pp[g].count) c = rc[t];
-            }
-            mc[e] = c;
-            lmk = max(lmk, static_cast<uint32_t>(c >> 32));
-        }
-        __syncthreads();  // chunk stage is done with sh
         block_threshold_gather<NT, EM>(
             sh, lmk, min(want, total), [&](int e) -> uint32_t { return static_cast<uint32_t>(mc[e] >> 32); },
             [&](int e) -> uint32_t { return composite_index(mc[e]); });
@@ -446,12 +301,7 @@ __global__ __launch_bounds__(NT) void rows_topk_kernel(const T *__restrict__ in,
             }
         }
     }
-    if (tid == 0) s_slow = slow ? 1u : 0u;
-    __syncthreads();
-    slow = s_slow != 0u;
 
-    T *ov = values + static_cast<size_t>(row) * k;
-    int32_t *oi = indices + static_cast<size_t>(row) * k;
     if (!slow) {
         for (uint32_t r = tid; r < kk; r += NT) {
             const uint32_t idx = sh.pidx[r];
@@ -496,6 +346,164 @@ __global__ __launch_bounds__(NT) void rows_topk_kernel(const T *__restrict__ in,
             oi[r] = static_cast<int32_t>(idx);
         }
     }
+}
+
+// SOFTMAX = true : fused softmax -> top-k (values are probabilities)
+// SOFTMAX = false: plain top-k, largest first (values are copies of the input)
+// ALIGNED: every row start is 16-byte aligned and n is a multiple of the vector
+// width, so chunks are read with 128-bit loads.
+// Launch: rows * G workgroups of NT threads; per = elements per chunk
+// (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
+// With G == 1 the workgroup also merges (no second kernel).
+template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED>
+__global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                        int32_t *__restrict__ indices, uint32_t n, uint32_t k,
+                                                        uint32_t G, uint32_t per, RowsWorkspace ws) {
+    constexpr int VEC = Vec128<T>::N;
+    constexpr int E = V * VEC;
+    constexpr int NW = NT / kWave;
+    __shared__ RowsSharedUnion smem;
+    __shared__ float fscratch[NW];
+    __shared__ double dscratch[NW];
+    RowsShared &sh = smem.fast;
+
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
+    const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
+    const T *rowp = in + static_cast<size_t>(row) * n;
+    const uint32_t want = k + 1;  // one extra: the merge needs the (k+1)-th to prove the cut
+
+    // ---- 1. chunk -> registers ------------------------------------------------
+    float x[E];
+    if constexpr (ALIGNED) {
+        Vec128<T> q[V];
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
+            if (e0 < c1) q[i].load(rowp + e0);
+        }
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) x[i * VEC + c] = (e0 < c1) ? q[i].get(c) : -INFINITY;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const uint32_t e = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC + c;
+                x[i * VEC + c] = (e < c1) ? load_elem(rowp, e) : -INFINITY;
+            }
+        }
+    }
+    auto index_of = [&](int e) -> uint32_t {
+        return c0 + (static_cast<uint32_t>(e / VEC) * NT + tid) * VEC + static_cast<uint32_t>(e % VEC);
+    };
+
+    // ---- 2. max and sum of exp ------------------------------------------------
+    float lmax = -INFINITY;
+#pragma unroll
+    for (int e = 0; e < E; e++) lmax = fmaxf(lmax, x[e]);
+    float m_g = -INFINITY, ref = 0.f;
+    if constexpr (SOFTMAX) {
+        const float wm = wave_max_f32_uniform(lmax);
+        if (lane == 0) sh.wave_m[wave] = wm;
+        __syncthreads();
+        m_g = sh.wave_m[0];
+#pragma unroll
+        for (int w = 1; w < NW; w++) m_g = fmaxf(m_g, sh.wave_m[w]);
+        // a chunk without a finite element sums against 0: its terms are all 0
+        // (or NaN, which must survive), never -inf - -inf
+        ref = (m_g > -INFINITY) ? m_g : 0.f;
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int e = 0; e < E; e += 2) {
+            a0 += fast_term(x[e], ref);
+            a1 += fast_term(x[e + 1], ref);
+        }
+        const double wsum = wave_sum(static_cast<double>(a0) + static_cast<double>(a1));
+        if (lane == 0) sh.wave_s[wave] = wsum;
+    }
+
+    // ---- 3. threshold and gather ------------------------------------------------
+    const bool any_valid = (c0 + tid * VEC) < c1;
+    uint32_t lkey = any_valid ? order_key(lmax) : 0u;
+    if constexpr (!SOFTMAX) {
+        // fmaxf drops NaN, but NaN ranks first in a plain top-k: take the max of
+        // the keys instead (a softmax row with a NaN goes to the exact path anyway)
+        lkey = 0u;
+#pragma unroll
+        for (int e = 0; e < E; e++) lkey = max(lkey, index_of(e) < c1 ? order_key(x[e]) : 0u);
+    }
+    block_threshold_gather<NT, E>(
+        sh, lkey, want, [&](int e) -> uint32_t { return index_of(e) < c1 ? order_key(x[e]) : 0u; },
+        [&](int e) -> uint32_t { return index_of(e); });
+    const uint32_t C = sh.count;
+    const bool overflow = C > kFastCap;
+
+    // ---- 4. exact ranking of the gathered elements, emit the best `want` -------
+    uint64_t *out_c = ws.cands + (static_cast<size_t>(row) * G + chunk) * ws.kc;
+    uint32_t emitted = 0;
+    if (!overflow) {
+        block_rank<NT>(sh, C);
+        emitted = min(C, want);
+        for (uint32_t t = tid; t < C; t += NT) {
+            const uint32_t r = sh.rank[t];
+            if (r < emitted) {
+                const uint64_t cmp = sh.cand[t];
+                out_c[r] = cmp;
+                if constexpr (SOFTMAX) {
+                    // replace this element's fast term by the accurate one (the
+                    // difference of two nearby floats is exact)
+                    const float xv = ordered_to_float(static_cast<uint32_t>(cmp >> 32));
+                    sh.prob[r] = exp_accurate(xv - ref) - fast_term(xv, ref);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        double acc = 0.0;
+        if constexpr (SOFTMAX) {
+            if (lane < NW) acc = sh.wave_s[lane];
+            for (uint32_t r = lane; r < emitted; r += kWave) acc += static_cast<double>(sh.prob[r]);
+            acc = wave_sum(acc);  // same tree every time: run-to-run stable
+        }
+        if (lane == 0) {
+            ChunkPartial p;
+            p.s = acc;
+            p.m = m_g;
+            p.count = emitted;
+            p.flags = overflow ? 1u : 0u;
+            p.pad[0] = p.pad[1] = p.pad[2] = 0;
+            ws.partials[static_cast<size_t>(row) * G + chunk] = p;
+        }
+    }
+    if (G != 1) return;
+
+    // ---- single-chunk rows: merge right here --------------------------------------
+    __syncthreads();  // this workgroup's own global writes, and sh is free again
+    constexpr int EM1 = (kFastMaxK + 1 + NT - 1) / NT;
+    merge_row<T, NT, EM1, SOFTMAX>(smem, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
+                                   indices + static_cast<size_t>(row) * k, n, k, 1u, ws.partials + row,
+                                   ws.cands + static_cast<size_t>(row) * ws.kc, ws.kc);
+}
+
+// One workgroup of kMergeThreads per row.
+template <typename T, bool SOFTMAX>
+__global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                                   int32_t *__restrict__ indices, uint32_t n,
+                                                                   uint32_t k, uint32_t G, RowsWorkspace ws) {
+    __shared__ RowsSharedUnion smem;
+    __shared__ float fscratch[kMergeThreads / kWave];
+    __shared__ double dscratch[kMergeThreads / kWave];
+    const uint32_t row = blockIdx.x;
+    merge_row<T, kMergeThreads, kMergeSlots / kMergeThreads, SOFTMAX>(
+        smem, fscratch, dscratch, in + static_cast<size_t>(row) * n, values + static_cast<size_t>(row) * k,
+        indices + static_cast<size_t>(row) * k, n, k, G, ws.partials + static_cast<size_t>(row) * G,
+        ws.cands + static_cast<size_t>(row) * G * ws.kc, ws.kc);
 }
 
 }  // namespace vkop

@@ -150,7 +150,7 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
 }
 
 struct RowsLayout {
-    size_t tickets = 0, partials = 0, cands = 0, stats = 0, total = 0;
+    size_t partials = 0, cands = 0, stats = 0, total = 0;
 };
 
 // One layout serves the streaming kernel and the general two-kernel path, so
@@ -159,8 +159,6 @@ RowsLayout rows_layout(const View &v, int k, const RowsCfg &c) {
     RowsLayout l;
     const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
     size_t off = 0;
-    l.tickets = off;
-    off += align_up(lines * sizeof(uint32_t));
     l.stats = off;
     off += align_up(lines * sizeof(vkop::LineStats));
     if (c.ok) {
@@ -178,7 +176,6 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
                 const RowsLayout &l, hipStream_t st) {
     vkop::RowsWorkspace w;
     auto *base = static_cast<unsigned char *>(ws);
-    w.tickets = reinterpret_cast<uint32_t *>(base + l.tickets);
     w.partials = reinterpret_cast<vkop::ChunkPartial *>(base + l.partials);
     w.cands = reinterpret_cast<uint64_t *>(base + l.cands);
     w.kc = static_cast<uint32_t>(k + 1);
@@ -188,13 +185,14 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
 #define VKOP_ROWS_CASE(NT, V)                                                                                   \
     if (c.nt == NT && c.v == V) {                                                                               \
         if (aligned)                                                                                            \
-            vkop::rows_topk_kernel<T, NT, V, SOFTMAX, true>                                                     \
+            vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, true>                                                    \
                 <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w);   \
         else                                                                                                    \
-            vkop::rows_topk_kernel<T, NT, V, SOFTMAX, false>                                                    \
+            vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, false>                                                   \
                 <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w);   \
-        return launched("rows_topk_kernel");                                                                    \
+        launched_one = true;                                                                                    \
     }
+    bool launched_one = false;
     VKOP_ROWS_CASE(256, 1)
     VKOP_ROWS_CASE(256, 2)
     VKOP_ROWS_CASE(256, 4)
@@ -205,10 +203,18 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
     VKOP_ROWS_CASE(1024, 4)
     if constexpr (sizeof(T) == 4) {
         VKOP_ROWS_CASE(256, 8)
+        VKOP_ROWS_CASE(512, 8)
         VKOP_ROWS_CASE(1024, 8)
     }
 #undef VKOP_ROWS_CASE
-    return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_topk_kernel for %d threads x %d loads", c.nt, c.v);
+    if (!launched_one) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
+    if (int rc = launched("rows_chunk_kernel")) return rc;
+    if (c.g > 1) {
+        vkop::rows_merge_kernel<T, SOFTMAX><<<v.g.outer, vkop::kMergeThreads, 0, st>>>(
+            in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, w);
+        return launched("rows_merge_kernel");
+    }
+    return VKOP_HIP_OK;
 }
 
 // ------------------------------------------------------------------ top-k ----
