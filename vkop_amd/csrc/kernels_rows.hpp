@@ -3,24 +3,34 @@
 // rows_chunk_kernel makes the one pass over the input.  A row is split into G
 // chunks, one workgroup per chunk, so a few long rows still fill the chip.
 // Each workgroup
-//   1. pulls its chunk into registers with 128-bit loads (V per thread),
-//   2. reduces max and sum of exp(x - max) (wave DPP + one LDS hop),
-//   3. finds a threshold that at least k+1 of its elements reach -- per wave the
-//      c-th largest per-lane maximum, then the minimum over the waves -- and
-//      appends the few elements above it to an LDS list,
-//   4. ranks that list exactly (key, then lower index) and writes its k+1 best,
-//      in order, plus (max, sum) to the workspace.
+//   1. issues all of its 128-bit loads (V per thread) at once,
+//   2. consumes the vectors in the order they arrive: per vector its maximum and
+//      the sum of exp(x - ref), where ref is the maximum of the wave's FIRST
+//      vector (any reference is valid for a partial sum; taking it from the
+//      first vector lets the exponentials overlap the rest of the stream),
+//   3. publishes per-lane maxima to LDS; one wave finds, by a ballot descent over
+//      them, a threshold that at least k+1 elements of the chunk reach,
+//   4. compacts the few 128-bit vectors holding an element above the threshold
+//      (ballot + popcount, no atomics) straight into the wave's own segment of
+//      the workspace: the vector as loaded plus a header (index of its first
+//      element, its maximum as an order key),
+//   5. writes one partial (sum, reference, maximum) and one record count per wave.
 // rows_merge_kernel (one workgroup per row; run inside the chunk kernel when
-// G == 1) merges the G partial results the same way, computes the
-// probabilities of the winners only, orders equal probabilities by index and
-// writes the row's result.  There are no atomics or fences between workgroups:
-// the kernel boundary publishes the partial results, and the outcome does not
-// depend on scheduling.
-// Whatever the shortcut cannot prove exact (too many elements at a threshold,
-// a probability tie across the k-th place, NaN/inf rows) is redone by the
-// merging workgroup with the exact radix select of select.hpp, so the result
-// is always top-k (probability, then lower index) of the row's softmax.
+// G == 1) combines the partial sums, finds the (k+1)-th largest record header,
+// unpacks the few records above it, ranks their elements exactly (key, then
+// lower index), replaces the summed fast terms of the ranked elements by
+// accurate ones, computes the probabilities of the winners only, orders equal
+// probabilities by index and writes the row's result.
+// There are no atomics or fences between workgroups: the kernel boundary
+// publishes the partial results, and every order of summation is fixed, so
+// results are bit-identical from run to run.
+// Whatever the shortcut cannot prove exact (a segment overflows, a partial sum
+// overflows, a probability tie across the k-th place, NaN/inf rows) is redone
+// by the merging workgroup with the exact radix select of select.hpp, so the
+// result is always top-k (probability, then lower index) of the row's softmax.
 #pragma once
+
+#include <type_traits>
 
 #include "device_utils.hpp"
 #include "kernels_general.hpp"
@@ -28,10 +38,11 @@
 
 namespace vkop {
 
-constexpr int kFastCap = 1024;     // LDS slots for elements above a threshold
-constexpr int kFastMaxK = 255;     // k + 1 <= 256 ranks are kept in LDS
-constexpr int kMergeThreads = 1024;
-constexpr int kMergeSlots = 4096;  // G * (k + 1) the merge takes in registers
+constexpr int kFastCap = 1024;       // LDS slots for elements above the merge threshold
+constexpr int kFastMaxK = 255;       // k + 1 <= 256 ranks are kept in LDS
+constexpr int kMergeThreads = 256;   // rows_merge_kernel workgroup
+constexpr int kMergeRecsMax = 4096;  // record slots per row the merge takes in registers
+constexpr int kMergeWavesMax = 256;  // chunk-kernel waves per row the merge can combine
 
 // ---- wave-level helpers (all 64 lanes must be active) -----------------------
 
@@ -50,6 +61,30 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     const uint32_t r3 = __builtin_amdgcn_readlane(static_cast<int>(v), 48);
     return max(max(r0, r1), max(r2, r3));
 }
+
+// Sum of a double over the wave, returned wave-uniform.  Same four in-row steps
+// (every lane of a row ends with the same bits, because each step adds the same
+// two partial sums in either order), then the four rows in a fixed order.
+__device__ __forceinline__ double wave_sum_f64_uniform(double v) {
+    auto step = [](double a, auto tag) {
+        constexpr int ctrl = decltype(tag)::value;
+        const uint64_t u = static_cast<uint64_t>(__double_as_longlong(a));
+        const uint32_t lo = VKOP_DPP_U32(static_cast<uint32_t>(u), ctrl);
+        const uint32_t hi = VKOP_DPP_U32(static_cast<uint32_t>(u >> 32), ctrl);
+        return a + __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
+    };
+    v = step(v, std::integral_constant<int, 0xB1>{});
+    v = step(v, std::integral_constant<int, 0x4E>{});
+    v = step(v, std::integral_constant<int, 0x141>{});
+    v = step(v, std::integral_constant<int, 0x140>{});
+    const uint64_t u = static_cast<uint64_t>(__double_as_longlong(v));
+    auto row = [&](int l) {
+        const uint32_t lo = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(u)), l);
+        const uint32_t hi = __builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(u >> 32)), l);
+        return __longlong_as_double(static_cast<long long>((static_cast<uint64_t>(hi) << 32) | lo));
+    };
+    return (row(0) + row(16)) + (row(32) + row(48));
+}
 #undef VKOP_DPP_U32
 
 // Bijective order-preserving float <-> uint32 (no NaN / -0 canonicalisation).
@@ -64,49 +99,79 @@ __device__ __forceinline__ float wave_max_f32_uniform(float v) {
     return ordered_to_float(wave_max_u32(float_to_ordered(v)));
 }
 
-// A lower bound, wave-uniform, of the c-th largest (1 <= c <= 64) of the 64 lane
-// values that at least c lanes reach: bitwise descent over the top `bits` bits
-// with ballots (the low bits stay zero, which only lowers the bound).  Returns
-// 0 when fewer than c lanes are non-zero.
-__device__ __forceinline__ uint32_t wave_cth_largest_floor(uint32_t v, uint32_t c, int bits) {
+constexpr uint32_t kKeyNegInf = 0x007FFFFFu;  // order key of -inf, the smallest key of a real element
+
+// Number of lanes below the caller among those set in `mask`.
+__device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+// Float threshold equivalent to an order-key threshold: x passes iff
+// !(x < thr_f).  Keys at or below the key of -inf mean "everything passes".
+__device__ __forceinline__ float key_threshold_to_float(uint32_t thr) {
+    return thr <= kKeyNegInf ? -INFINITY : ordered_to_float(thr);
+}
+
+// One wave finds a lower bound of the `want`-th largest of NW * 64 keys held in
+// LDS (key 0 = no element): bitwise descent over the top `bits` bits, counting
+// with ballots; the untouched low bits stay zero, which only lowers the bound.
+// Returns 0 (= take everything) when fewer than `want` keys are non-zero in
+// those bits.  Called by all 64 lanes of one wave.
+template <int NW>
+__device__ __forceinline__ uint32_t block_kth_largest_floor(const uint32_t *keys, uint32_t want, int bits) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    uint32_t kv[NW];
+#pragma unroll
+    for (int w = 0; w < NW; w++) kv[w] = keys[w * kWave + lane];
     uint32_t prefix = 0;
     for (int bit = 31; bit > 31 - bits; bit--) {
         const uint32_t trial = prefix | (1u << bit);
-        if (static_cast<uint32_t>(__popcll(__ballot(v >= trial))) >= c) prefix = trial;
+        uint32_t cnt = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) cnt += static_cast<uint32_t>(__popcll(__ballot(kv[w] >= trial)));
+        if (cnt >= want) prefix = trial;
     }
     return prefix;
 }
 
 // ---- workspace ---------------------------------------------------------------
 
-struct ChunkPartial {
-    double s;        // sum of exp(x - m) over the chunk
-    float m;         // chunk max
-    uint32_t count;  // candidates written (<= k + 1), in rank order
-    uint32_t flags;  // bit 0: the chunk could not bound its candidates -> exact path
-    uint32_t pad[3];
+struct SumPartial {  // one per wave of the chunk kernel
+    double s;   // sum of exp(x - ref) over the wave's elements
+    float ref;  // reference of that sum: the maximum of the wave's first vectors, or 0 if that is -inf
+    float m;    // the maximum of the wave's elements
+};
+
+struct WaveMeta {  // one per wave
+    uint32_t count;  // records the wave wanted to write; > segment size means overflow
+    float thr;       // chunk threshold: every element with !(x < thr) is in a record
 };
 
 struct RowsWorkspace {
-    ChunkPartial *partials;  // [rows][G]
-    uint64_t *cands;         // [rows][G][kc]
-    uint32_t kc;             // slots per chunk (k + 1)
+    SumPartial *sums;    // [rows][G][waves per chunk]
+    WaveMeta *meta;      // [rows][G][waves per chunk]
+    uint4 *recs;         // [rows][G][waves per chunk][seg][2]: a 128-bit vector as loaded, then its
+                         // header (index of its first element, its maximum as an order key, 0, 0)
+    uint32_t seg;        // records per wave (power of two)
+    uint32_t seg_shift;  // log2(seg)
 };
 
 struct RowsShared {
     uint64_t cand[kFastCap];
+    uint16_t cand_src[kFastCap];  // the chunk-kernel wave the element was summed in
     uint32_t rank[kFastCap];
     float prob[kFastMaxK + 1];
     uint32_t pidx[kFastMaxK + 1];
-    uint32_t wave_key[16];
-    uint32_t wave_valid[16];
-    float wave_m[16];
-    double wave_s[16];
+    double corr[kFastMaxK + 1];
+    double scale[kMergeWavesMax];  // exp(ref - M) per wave partial
+    float ref[kMergeWavesMax];
+    uint32_t cnt[kMergeWavesMax];  // records per wave
+    uint32_t lane_key[1024];
+    uint32_t thr;
     uint32_t count;
-    // row statistics published by wave 0 of the merging workgroup
-    float row_m;
-    uint32_t row_total, row_slow;
-    double row_rinv;
+    uint32_t flag;
+    double total;
 };
 
 union RowsSharedUnion {
@@ -117,8 +182,8 @@ union RowsSharedUnion {
 
 // Fast term for the running sum: exp2((x - m) * log2 e) on the hardware
 // exponential unit.  Only ever summed; every probability that is output uses
-// exp_accurate, and the terms of a chunk's largest elements are replaced by
-// accurate ones before the sum leaves the workgroup.
+// exp_accurate, and the merge replaces the fast terms of the row's largest
+// elements (the ones it ranks) by accurate ones.
 __device__ __forceinline__ float fast_term(float x, float m) {
     return __builtin_amdgcn_exp2f((x - m) * 1.44269504088896341f);
 }
@@ -128,18 +193,32 @@ __device__ __forceinline__ float fast_term(float x, float m) {
 template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uint32_t C) {
     const uint32_t tid = threadIdx.x;
     if (C == 0) return;
-    for (uint32_t t = tid; t < C; t += NT) sh.rank[t] = 0;
-    __syncthreads();
     if (C <= NT) {
         const uint32_t parts = NT / C;                  // >= 1
         const uint32_t span = (C + parts - 1) / parts;  // entries per part
         const uint32_t part = tid / C, i = tid - part * C;
+        if (parts > 1) {
+            for (uint32_t t = tid; t < C; t += NT) sh.rank[t] = 0;
+            __syncthreads();
+        }
         if (part < parts) {
             const uint64_t mine = sh.cand[i];
             const uint32_t j0 = part * span, j1 = min(j0 + span, C);
             uint32_t cnt = 0;
-            for (uint32_t j = j0; j < j1; j++) cnt += (sh.cand[j] > mine) ? 1u : 0u;
-            if (cnt) atomicAdd(&sh.rank[i], cnt);
+            uint32_t j = j0;
+            for (; j + 8 <= j1; j += 8) {  // eight independent reads in flight
+                uint64_t o[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) o[u] = sh.cand[j + u];
+#pragma unroll
+                for (int u = 0; u < 8; u++) cnt += (o[u] > mine) ? 1u : 0u;
+            }
+            for (; j < j1; j++) cnt += (sh.cand[j] > mine) ? 1u : 0u;
+            if (parts > 1) {
+                if (cnt) atomicAdd(&sh.rank[i], cnt);
+            } else {
+                sh.rank[i] = cnt;
+            }
         }
     } else {
         for (uint32_t i = tid; i < C; i += NT) {
@@ -152,59 +231,21 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
     __syncthreads();
 }
 
-// Threshold + gather.  Every thread holds E elements; key_at(e) is the order
-// key of its e-th element (0 = no element), lane_max_key the largest of them.
-// On return sh.cand[0..sh.count) holds the composite of every element whose key
-// reaches the block threshold -- at least min(want, elements in the block) of
-// them -- unless sh.count > kFastCap (too many; the list is truncated).
-template <int NT, int E, typename KeyAt, typename IdxAt>
-__device__ __forceinline__ void block_threshold_gather(RowsShared &sh, uint32_t lane_max_key, uint32_t want,
-                                                       KeyAt key_at, IdxAt idx_at) {
-    constexpr int NW = NT / kWave;
-    const uint32_t tid = threadIdx.x, wave = tid / kWave, lane = tid & (kWave - 1);
-    const uint32_t valid = static_cast<uint32_t>(__popcll(__ballot(lane_max_key != 0u)));
-    if (lane == 0) sh.wave_valid[wave] = valid;
-    if (tid == 0) sh.count = 0;
-    __syncthreads();
-    // smallest c such that taking min(c, valid lanes) lanes from every wave
-    // reaches `want`; none (c = 0) means: take everything
-    uint32_t c = 0;
-    for (uint32_t t = (want + NW - 1) / NW; t <= kWave; t++) {
-        uint32_t got = 0;
-#pragma unroll
-        for (int w = 0; w < NW; w++) got += min(t, sh.wave_valid[w]);
-        if (got >= want) {
-            c = t;
-            break;
-        }
-    }
-    const uint32_t cw = min(c, valid);
-    const uint32_t tw = (c == 0) ? 0u : (cw == 0 ? 0xFFFFFFFFu : wave_cth_largest_floor(lane_max_key, cw, 24));
-    if (lane == 0) sh.wave_key[wave] = tw;
-    __syncthreads();
-    uint32_t thr = sh.wave_key[0];
-#pragma unroll
-    for (int w = 1; w < NW; w++) thr = min(thr, sh.wave_key[w]);
-    thr = max(thr, 1u);  // key 0 is "no element"
-    if (lane_max_key >= thr) {
-#pragma unroll
-        for (int e = 0; e < E; e++) {
-            const uint32_t key = key_at(e);
-            if (key >= thr) {
-                const uint32_t pos = atomicAdd(&sh.count, 1u);
-                if (pos < kFastCap) sh.cand[pos] = composite(key, idx_at(e));
-            }
-        }
-    }
-    __syncthreads();
-}
-
 template <typename T> struct Vec128;
 template <> struct Vec128<float> {
     static constexpr int N = 4;
-    float4 v;
-    __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const float4 *>(p); }
-    __device__ __forceinline__ float get(int c) const { return c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w; }
+    uint4 v;
+    __device__ __forceinline__ void load(const float *p) { v = *reinterpret_cast<const uint4 *>(p); }
+    __device__ __forceinline__ float get(int c) const {
+        return __uint_as_float(c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w);
+    }
+    __device__ __forceinline__ void set(int c, float f) {
+        const uint32_t u = __float_as_uint(f);
+        if (c == 0) v.x = u;
+        else if (c == 1) v.y = u;
+        else if (c == 2) v.z = u;
+        else v.w = u;
+    }
 };
 template <> struct Vec128<uint16_t> {
     static constexpr int N = 8;
@@ -214,86 +255,158 @@ template <> struct Vec128<uint16_t> {
         const uint32_t w = (c >> 1) == 0 ? v.x : (c >> 1) == 1 ? v.y : (c >> 1) == 2 ? v.z : v.w;
         return __half2float(__ushort_as_half(static_cast<uint16_t>((c & 1) ? (w >> 16) : (w & 0xFFFFu))));
     }
+    __device__ __forceinline__ void set(int c, float f) {  // f is a widened half: exact
+        const uint32_t h = __half_as_ushort(__float2half_rn(f));
+        uint32_t &w = (c >> 1) == 0 ? v.x : (c >> 1) == 1 ? v.y : (c >> 1) == 2 ? v.z : v.w;
+        w = (c & 1) ? ((w & 0x0000FFFFu) | (h << 16)) : ((w & 0xFFFF0000u) | h);
+    }
 };
 
 // ---- merge of one row's chunk results (all NT threads of a workgroup) --------
-// EM = candidate slots each thread takes (EM * NT >= G * ws.kc).
+// waves = chunk-kernel waves of this row (G * waves per chunk, <= NT and
+// <= kMergeWavesMax); EM = record slots each thread takes (EM * NT >= waves * seg).
 template <typename T, int NT, int EM, bool SOFTMAX>
 __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch, double *dscratch, const T *rowp,
-                                          T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
-                                          const ChunkPartial *pp, const uint64_t *rc, uint32_t kc) {
+                                          T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t waves,
+                                          const SumPartial *sums, const WaveMeta *meta, const uint4 *recs,
+                                          uint32_t seg, uint32_t seg_shift) {
+    constexpr int NW = NT / kWave;
+    constexpr int VEC = Vec128<T>::N;
     RowsShared &sh = smem.fast;
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t want = k + 1;
     const uint32_t kk = min(k, n);
-    const uint32_t slots = G * kc;
+    const uint32_t slots = waves << seg_shift;
+    const bool fits = slots <= static_cast<uint32_t>(EM) * NT && waves <= static_cast<uint32_t>(NT) &&
+                      waves <= static_cast<uint32_t>(kMergeWavesMax);
 
-    // candidates first: their loads do not depend on the row statistics
-    uint64_t mc[EM];
+    // ---- A. per-wave metadata and the row's sum from the partials -----------------
+    bool bad = !fits;
+    SumPartial p0{0.0, 0.f, -INFINITY};
+    if (fits && tid < waves) {
+        const WaveMeta mt = meta[tid];
+        p0 = sums[tid];
+        sh.cnt[tid] = min(mt.count, seg);
+        sh.ref[tid] = p0.ref;
+        bad = mt.count > seg;
+    }
+    const float M = block_max<NT>(p0.m, fscratch);  // (barrier: sh.cnt is published)
+    double acc = 0.0;
+    if (fits && tid < waves) {
+        const double sc = exp(static_cast<double>(p0.ref) - static_cast<double>(M));
+        sh.scale[tid] = sc;
+        if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
+    }
+    const double s_base = block_sum<NT>(acc, dscratch);  // (barrier: sh.scale is published)
+
+    // ---- B. record headers: the maximum of every live record ------------------------
+    // Thread t takes the slots q = e * NT + t of the list ordered by (position in
+    // segment, wave): the live records, which sit at the low positions of every
+    // segment, are then spread evenly over the threads.
+    uint32_t rkey[EM], ridx[EM], rslot[EM];
     uint32_t lmk = 0;
+    {
+        const uint32_t wv = fits ? waves : 1u;
+        const uint32_t dj = NT / wv, dw = NT - dj * wv;  // one step of e in (j, w)
+        uint32_t j = tid / wv, w = tid - j * wv;
 #pragma unroll
-    for (int e = 0; e < EM; e++) {
-        const uint32_t t = static_cast<uint32_t>(e) * NT + tid;
-        uint64_t c = 0;
-        if (t < slots) {
-            const uint32_t g = t / kc, j = t - g * kc;
-            if (j < pp[g].count) c = rc[t];
+        for (int e = 0; e < EM; e++) {
+            // never a branch around a load: dead slots read slot 0 and are masked
+            const bool live = fits && j < sh.cnt[w];
+            const uint32_t t = live ? ((w << seg_shift) + j) : 0u;
+            const uint4 hdr = recs[2 * t + 1];
+            rkey[e] = live ? hdr.y : 0u;
+            ridx[e] = hdr.x;
+            rslot[e] = t;
+            lmk = max(lmk, rkey[e]);
+            j += dj;
+            w += dw;
+            if (w >= wv) {
+                w -= wv;
+                j++;
+            }
         }
-        mc[e] = c;
-        lmk = max(lmk, static_cast<uint32_t>(c >> 32));
     }
 
-    // row statistics: lane g of wave 0 takes chunk g (G <= 64), fixed reduction tree
-    if (wave == 0) {
-        float mg = -INFINITY;
-        double sg = 0.0;
-        uint32_t cnt = 0, flg = 0;
-        if (lane < G) {
-            mg = pp[lane].m;
-            sg = pp[lane].s;
-            cnt = pp[lane].count;
-            flg = pp[lane].flags;
-        }
-        const float M = wave_max_f32_uniform(mg);
-        double term = 0.0;
-        if (SOFTMAX && sg != 0.0) term = sg * exp(static_cast<double>(mg) - static_cast<double>(M));
-        const double S = wave_sum(term);
-        const uint32_t tot = wave_sum(cnt);
-        bool bad = __ballot(flg != 0u) != 0ull;
-        if (SOFTMAX && !(S > 0.0 && S < 1e300)) bad = true;  // NaN / inf rows
-        if (SOFTMAX && !(M > -INFINITY && M < INFINITY)) bad = true;
-        if (slots > static_cast<uint32_t>(EM) * NT) bad = true;
-        if (lane == 0) {
-            sh.row_m = M;
-            sh.row_rinv = 1.0 / S;
-            sh.row_total = tot;
-            sh.row_slow = bad ? 1u : 0u;
-        }
+    // ---- C. threshold: the (k+1)-th largest lane maximum --------------------------
+    sh.lane_key[tid] = lmk;
+    if (tid == 0) {
+        sh.count = 0;
+        sh.flag = 0;
     }
     __syncthreads();
-    LineStats st{sh.row_m, 0.f, sh.row_rinv};
-    bool slow = sh.row_slow != 0u;
-    const uint32_t total = sh.row_total;
+    if (bad) sh.flag = 1;  // every writer stores the same value
+    if (wave == 0) {
+        const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
+        if (lane == 0) sh.thr = max(t, 1u);  // key 0 is "no element"
+    }
+    __syncthreads();
+    const uint32_t thr = sh.thr;
+    bool slow = sh.flag != 0u;
+    if (SOFTMAX && !(s_base > 0.0 && s_base < 1e300)) slow = true;  // NaN / inf rows, overflowed partials
+    if (SOFTMAX && !(M > -INFINITY && M < INFINITY)) slow = true;
 
     if (!slow) {
-        block_threshold_gather<NT, EM>(
-            sh, lmk, min(want, total), [&](int e) -> uint32_t { return static_cast<uint32_t>(mc[e] >> 32); },
-            [&](int e) -> uint32_t { return composite_index(mc[e]); });
+        // ---- D. unpack the few records reaching the threshold ------------------------
+        // (a thread rarely holds more than one: the loop is a round trip or two)
+#pragma unroll
+        for (int e = 0; e < EM; e++) {
+            if (rkey[e] < thr) continue;
+            const uint32_t t = rslot[e];
+            const uint32_t idx0 = ridx[e];
+            Vec128<T> q;
+            q.v = recs[2 * t];
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const uint32_t key = idx0 + c < n ? order_key(q.get(c)) : 0u;
+                if (key >= thr) {
+                    const uint32_t pos = atomicAdd(&sh.count, 1u);
+                    if (pos < kFastCap) {
+                        sh.cand[pos] = composite(key, idx0 + c);
+                        sh.cand_src[pos] = static_cast<uint16_t>(t >> seg_shift);
+                    }
+                }
+            }
+        }
+        __syncthreads();
         const uint32_t C2 = sh.count;
         if (C2 > kFastCap) {
             slow = true;
         } else {
+            // ---- E. exact ranks; accurate terms for the ranked elements ----------------
             block_rank<NT>(sh, C2);
+            const uint32_t ranked = min(C2, static_cast<uint32_t>(kFastMaxK + 1));
             for (uint32_t t = tid; t < C2; t += NT) {
                 const uint32_t r = sh.rank[t];
-                if (r <= kk && r <= static_cast<uint32_t>(kFastMaxK)) {
-                    const uint32_t idx = composite_index(sh.cand[t]);
-                    sh.pidx[r] = idx;
-                    if constexpr (SOFTMAX) sh.prob[r] = round_to_storage<T>(softmax_prob(load_elem(rowp, idx), st));
+                if (r < ranked) {
+                    const uint64_t cmp = sh.cand[t];
+                    const uint32_t key = static_cast<uint32_t>(cmp >> 32);
+                    sh.pidx[r] = composite_index(cmp);
+                    sh.prob[r] = ordered_to_float(key);  // the logit, for now
+                    double cr = 0.0;
+                    if (SOFTMAX && key != 0xFFFFFFFFu) {
+                        const uint32_t sp = sh.cand_src[t];
+                        const float xv = ordered_to_float(key);
+                        // what the element should contribute, exp(fl(x - M)), minus what
+                        // its wave added for it, exp2(fl(fl(x - ref) * log2 e)) * exp(ref - M)
+                        cr = static_cast<double>(exp_accurate(xv - M)) -
+                             static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
+                    }
+                    sh.corr[r] = cr;
                 }
             }
             __syncthreads();
+            if (wave == 0) {
+                double c = 0.0;
+                for (uint32_t r = lane; r < ranked; r += kWave) c += sh.corr[r];
+                c = wave_sum_f64_uniform(c);  // same tree every time: run-to-run stable
+                if (lane == 0) sh.total = s_base + c;
+            }
+            __syncthreads();
             if constexpr (SOFTMAX) {
+                const LineStats st{M, 0.f, 1.0 / sh.total};
+                if (tid <= kk && tid < ranked) sh.prob[tid] = round_to_storage<T>(softmax_prob(sh.prob[tid], st));
+                __syncthreads();
                 // Probabilities are non-increasing along the rank order, so equal
                 // ones are neighbours.  A tie that reaches past the k-th place
                 // cannot be settled from the candidates.
@@ -318,7 +431,7 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
                 store_elem(ov, pos, p);
                 oi[pos] = static_cast<int32_t>(idx);
             } else {
-                ov[r] = rowp[idx];
+                ov[r] = rowp[idx];  // bit copy (keeps the sign of a zero)
                 oi[r] = static_cast<int32_t>(idx);
             }
         }
@@ -329,7 +442,7 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
     __syncthreads();  // smem changes owner
     if constexpr (SOFTMAX) {
         // redo the statistics the way the general kernels define them
-        st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch);
+        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch);
         select_topk_line<NT>(smem.exact, n, kk, [&](uint32_t j) {
             return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
         });
@@ -354,156 +467,179 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
 // width, so chunks are read with 128-bit loads.
 // Launch: rows * G workgroups of NT threads; per = elements per chunk
 // (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
-// With G == 1 the workgroup also merges (no second kernel).
-template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED>
+// SINGLE: G == 1 and the workgroup also merges (no second kernel); otherwise the
+// kernel needs only a few KB of LDS.
+struct ChunkShared {
+    uint32_t lane_key[1024];
+    uint32_t thr;
+};
+
+template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, bool SINGLE>
 __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                         int32_t *__restrict__ indices, uint32_t n, uint32_t k,
                                                         uint32_t G, uint32_t per, RowsWorkspace ws) {
     constexpr int VEC = Vec128<T>::N;
-    constexpr int E = V * VEC;
     constexpr int NW = NT / kWave;
-    __shared__ RowsSharedUnion smem;
-    __shared__ float fscratch[NW];
-    __shared__ double dscratch[NW];
-    RowsShared &sh = smem.fast;
+    __shared__ std::conditional_t<SINGLE, RowsSharedUnion, ChunkShared> smem;
+    __shared__ float fscratch[SINGLE ? NW : 1];
+    __shared__ double dscratch[SINGLE ? NW : 1];
+    uint32_t *lane_keys;
+    uint32_t *thr_slot;
+    if constexpr (SINGLE) {
+        lane_keys = smem.fast.lane_key;
+        thr_slot = &smem.fast.thr;
+    } else {
+        lane_keys = smem.lane_key;
+        thr_slot = &smem.thr;
+    }
 
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
     const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
     const T *rowp = in + static_cast<size_t>(row) * n;
     const uint32_t want = k + 1;  // one extra: the merge needs the (k+1)-th to prove the cut
+    const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
+    const uint32_t went = (row * G + chunk) * NW + wave;  // this wave's slot in the row-major wave list
 
-    // ---- 1. chunk -> registers ------------------------------------------------
-    float x[E];
-    if constexpr (ALIGNED) {
-        Vec128<T> q[V];
+    // ---- 1. all loads in flight -----------------------------------------------------
+    Vec128<T> q[V];
 #pragma unroll
-        for (int i = 0; i < V; i++) {
-            const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
-            if (e0 < c1) q[i].load(rowp + e0);
+    for (int i = 0; i < V; i++) {
+        const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+        // never a branch around a load (the compiler would wait for each one in
+        // turn): out-of-chunk lanes read the row's first element(s) instead and
+        // are masked wherever the data is used
+        q[i].v = make_uint4(0, 0, 0, 0);
+        if constexpr (ALIGNED) {
+            q[i].load(rowp + (e0 < c1 ? e0 : 0u));
+        } else {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < c1 ? e0 + c : 0u));
         }
+    }
+
+    // The rest of the kernel exists twice: for a chunk that fills every lane of
+    // every vector (no masking anywhere) and for a ragged one.
+    auto body = [&](auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        auto in_range = [&](uint32_t e) { return FULL || e < c1; };
+
+        // ---- 2. per vector, in arrival order: maximum and sum of exp(x - ref) -----------
+        // vmax[i]: float max of vector i (NaN dropped) for the softmax variant; for the
+        // plain top-k the max of the order keys, so that NaN (which ranks first) counts.
+        float vmax[V];
+        uint32_t vkey[V];
+        // Every term is added in double (fp64 adds run at the fp32 rate here): a
+        // dominant term must not swallow the low bits of what the lane adds after it.
+        float lmax = -INFINITY, ref = 0.f;
+        double acc = 0.0;
+        uint32_t lkey = 0u;
 #pragma unroll
         for (int i = 0; i < V; i++) {
-            const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
-#pragma unroll
-            for (int c = 0; c < VEC; c++) x[i * VEC + c] = (e0 < c1) ? q[i].get(c) : -INFINITY;
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+            float xv[VEC];
+            float vm = -INFINITY;
+            uint32_t vk = 0u;
 #pragma unroll
             for (int c = 0; c < VEC; c++) {
-                const uint32_t e = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC + c;
-                x[i * VEC + c] = (e < c1) ? load_elem(rowp, e) : -INFINITY;
+                xv[c] = in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY;
+                vm = fmaxf(vm, xv[c]);
+                if constexpr (!SOFTMAX) vk = max(vk, in_range(ALIGNED ? e0 : e0 + c) ? order_key(xv[c]) : 0u);
             }
-        }
-    }
-    auto index_of = [&](int e) -> uint32_t {
-        return c0 + (static_cast<uint32_t>(e / VEC) * NT + tid) * VEC + static_cast<uint32_t>(e % VEC);
-    };
-
-    // ---- 2. max and sum of exp ------------------------------------------------
-    float lmax = -INFINITY;
-#pragma unroll
-    for (int e = 0; e < E; e++) lmax = fmaxf(lmax, x[e]);
-    float m_g = -INFINITY, ref = 0.f;
-    if constexpr (SOFTMAX) {
-        const float wm = wave_max_f32_uniform(lmax);
-        if (lane == 0) sh.wave_m[wave] = wm;
-        __syncthreads();
-        m_g = sh.wave_m[0];
-#pragma unroll
-        for (int w = 1; w < NW; w++) m_g = fmaxf(m_g, sh.wave_m[w]);
-        // a chunk without a finite element sums against 0: its terms are all 0
-        // (or NaN, which must survive), never -inf - -inf
-        ref = (m_g > -INFINITY) ? m_g : 0.f;
-        float a0 = 0.f, a1 = 0.f;
-#pragma unroll
-        for (int e = 0; e < E; e += 2) {
-            a0 += fast_term(x[e], ref);
-            a1 += fast_term(x[e + 1], ref);
-        }
-        const double wsum = wave_sum(static_cast<double>(a0) + static_cast<double>(a1));
-        if (lane == 0) sh.wave_s[wave] = wsum;
-    }
-
-    // ---- 3. threshold and gather ------------------------------------------------
-    const bool any_valid = (c0 + tid * VEC) < c1;
-    uint32_t lkey = any_valid ? order_key(lmax) : 0u;
-    if constexpr (!SOFTMAX) {
-        // fmaxf drops NaN, but NaN ranks first in a plain top-k: take the max of
-        // the keys instead (a softmax row with a NaN goes to the exact path anyway)
-        lkey = 0u;
-#pragma unroll
-        for (int e = 0; e < E; e++) lkey = max(lkey, index_of(e) < c1 ? order_key(x[e]) : 0u);
-    }
-    block_threshold_gather<NT, E>(
-        sh, lkey, want, [&](int e) -> uint32_t { return index_of(e) < c1 ? order_key(x[e]) : 0u; },
-        [&](int e) -> uint32_t { return index_of(e); });
-    const uint32_t C = sh.count;
-    const bool overflow = C > kFastCap;
-
-    // ---- 4. exact ranking of the gathered elements, emit the best `want` -------
-    uint64_t *out_c = ws.cands + (static_cast<size_t>(row) * G + chunk) * ws.kc;
-    uint32_t emitted = 0;
-    if (!overflow) {
-        block_rank<NT>(sh, C);
-        emitted = min(C, want);
-        for (uint32_t t = tid; t < C; t += NT) {
-            const uint32_t r = sh.rank[t];
-            if (r < emitted) {
-                const uint64_t cmp = sh.cand[t];
-                out_c[r] = cmp;
-                if constexpr (SOFTMAX) {
-                    // replace this element's fast term by the accurate one (the
-                    // difference of two nearby floats is exact)
-                    const float xv = ordered_to_float(static_cast<uint32_t>(cmp >> 32));
-                    sh.prob[r] = exp_accurate(xv - ref) - fast_term(xv, ref);
+            vmax[i] = vm;
+            vkey[i] = vk;
+            lmax = fmaxf(lmax, vm);
+            lkey = max(lkey, vk);
+            if constexpr (SOFTMAX) {
+                if (i == 0) {
+                    // reference of the wave's partial sum: the maximum of its first
+                    // vectors; 0 if they hold no finite element (terms are then 0, or
+                    // NaN, which must survive -- never -inf - -inf)
+                    const float wm0 = wave_max_f32_uniform(vm);
+                    ref = (wm0 > -INFINITY) ? wm0 : 0.f;
                 }
+#pragma unroll
+                for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(xv[c], ref));
             }
         }
-    }
-    __syncthreads();
-    if (wave == 0) {
-        double acc = 0.0;
-        if constexpr (SOFTMAX) {
-            if (lane < NW) acc = sh.wave_s[lane];
-            for (uint32_t r = lane; r < emitted; r += kWave) acc += static_cast<double>(sh.prob[r]);
-            acc = wave_sum(acc);  // same tree every time: run-to-run stable
-        }
-        if (lane == 0) {
-            ChunkPartial p;
-            p.s = acc;
-            p.m = m_g;
-            p.count = emitted;
-            p.flags = overflow ? 1u : 0u;
-            p.pad[0] = p.pad[1] = p.pad[2] = 0;
-            ws.partials[static_cast<size_t>(row) * G + chunk] = p;
-        }
-    }
-    if (G != 1) return;
+        if constexpr (SOFTMAX) lkey = in_range(e_first) ? order_key(lmax) : 0u;
 
-    // ---- single-chunk rows: merge right here --------------------------------------
-    __syncthreads();  // this workgroup's own global writes, and sh is free again
-    constexpr int EM1 = (kFastMaxK + 1 + NT - 1) / NT;
-    merge_row<T, NT, EM1, SOFTMAX>(smem, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
-                                   indices + static_cast<size_t>(row) * k, n, k, 1u, ws.partials + row,
-                                   ws.cands + static_cast<size_t>(row) * ws.kc, ws.kc);
+        // ---- 3. lane maxima -> LDS; one wave finds the chunk threshold ---------------------
+        lane_keys[tid] = lkey;
+        __syncthreads();
+        if (wave == blockIdx.x % NW) {  // not always wave 0: spreads this serial step over the SIMDs
+            const uint32_t t = block_kth_largest_floor<NW>(lane_keys, want, 16);
+            if (lane == 0) *thr_slot = t;
+        }
+        const float wm = wave_max_f32_uniform(lmax);
+        double wsum = 0.0;
+        if constexpr (SOFTMAX) wsum = wave_sum_f64_uniform(acc);
+        __syncthreads();
+        const uint32_t thr = *thr_slot;
+        const float thr_f = key_threshold_to_float(thr);
+
+        // ---- 4. compaction of the vectors reaching the threshold ----------------------------
+        uint4 *rec_out = ws.recs + (static_cast<size_t>(went) << (ws.seg_shift + 1));
+        const uint32_t last_slot = ws.seg - 1;
+        uint32_t wcount = 0;  // wave-uniform
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+            bool hit;
+            if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
+            else hit = (vkey[i] >= (thr > 1u ? thr : 1u)) && in_range(e0);
+            const uint64_t mask = __ballot(hit);
+            if (mask != 0ull) {
+                if (hit) {
+                    // past the end of the segment everything lands in the last slot;
+                    // the count then exceeds the segment and the row takes the exact path
+                    const uint32_t pos = min(wcount + lanes_below(mask), last_slot);
+                    rec_out[2 * pos] = q[i].v;
+                    rec_out[2 * pos + 1] = make_uint4(e0, SOFTMAX ? order_key(vmax[i]) : vkey[i], 0u, 0u);
+                }
+                wcount += static_cast<uint32_t>(__popcll(mask));
+            }
+        }
+
+        // ---- 5. partials ---------------------------------------------------------------------
+        if (lane == 0) {
+            ws.sums[went] = SumPartial{wsum, ref, wm};
+            ws.meta[went] = WaveMeta{wcount, thr_f};
+        }
+    };
+    if (c1 - c0 == static_cast<uint32_t>(NT) * V * VEC) body(std::true_type{});
+    else body(std::false_type{});
+
+    if constexpr (SINGLE) {
+        // ---- single-chunk rows: merge right here ----------------------------------
+        __syncthreads();  // this workgroup's own global writes
+        constexpr int EM1 = (kFastCap / VEC + NT - 1) / NT;
+        const size_t w0 = static_cast<size_t>(row) * NW;
+        merge_row<T, NT, EM1, SOFTMAX>(smem, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
+                                       indices + static_cast<size_t>(row) * k, n, k, NW, ws.sums + w0, ws.meta + w0,
+                                       ws.recs + (w0 << (ws.seg_shift + 1)), ws.seg, ws.seg_shift);
+    } else {
+        (void)values;
+        (void)indices;
+        (void)fscratch;
+        (void)dscratch;
+    }
 }
 
-// One workgroup of kMergeThreads per row.
+// One workgroup of kMergeThreads per row; waves = G * (waves per chunk workgroup).
 template <typename T, bool SOFTMAX>
 __global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                                    int32_t *__restrict__ indices, uint32_t n,
-                                                                   uint32_t k, uint32_t G, RowsWorkspace ws) {
+                                                                   uint32_t k, uint32_t waves, RowsWorkspace ws) {
     __shared__ RowsSharedUnion smem;
     __shared__ float fscratch[kMergeThreads / kWave];
     __shared__ double dscratch[kMergeThreads / kWave];
     const uint32_t row = blockIdx.x;
-    merge_row<T, kMergeThreads, kMergeSlots / kMergeThreads, SOFTMAX>(
+    const size_t w0 = static_cast<size_t>(row) * waves;
+    merge_row<T, kMergeThreads, kMergeRecsMax / kMergeThreads, SOFTMAX>(
         smem, fscratch, dscratch, in + static_cast<size_t>(row) * n, values + static_cast<size_t>(row) * k,
-        indices + static_cast<size_t>(row) * k, n, k, G, ws.partials + static_cast<size_t>(row) * G,
-        ws.cands + static_cast<size_t>(row) * G * ws.kc, ws.kc);
+        indices + static_cast<size_t>(row) * k, n, k, waves, ws.sums + w0, ws.meta + w0,
+        ws.recs + (w0 << (ws.seg_shift + 1)), ws.seg, ws.seg_shift);
 }
 
 }  // namespace vkop

@@ -105,7 +105,18 @@ struct RowsCfg {
     bool ok = false;
     int nt = 0, v = 0;
     uint32_t g = 0, per = 0;
+    uint32_t seg = 0, seg_shift = 0;  // candidate slots per wave of a chunk workgroup
 };
+
+// Slots per wave: four times the wave's quota of the k+1 wanted elements (about
+// 1.5 quotas are used on identically distributed data), at least 32, power of two.
+uint32_t rows_seg(int nt, int k) {
+    const uint32_t nw = static_cast<uint32_t>(nt) / 64u;
+    const uint32_t quota = (static_cast<uint32_t>(k) + 1u + nw - 1u) / nw;
+    uint32_t seg = 32;
+    while (seg < 4u * quota) seg <<= 1;
+    return seg;
+}
 
 RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     RowsCfg c;
@@ -121,9 +132,16 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     }
     const uint32_t nvec = (n + vec - 1) / vec;
     auto fits = [&](int nt, int vv, uint32_t g) {
-        if (g < 1 || g > 64 || static_cast<uint64_t>(g) * (k + 1) > vkop::kMergeSlots) return false;
-        const uint32_t per = (nvec + g - 1) / g * vec;
-        return per <= static_cast<uint32_t>(nt) * vv * vec && static_cast<uint64_t>(rows) * g < (1ull << 31);
+        const uint32_t nw = static_cast<uint32_t>(nt) / 64u;
+        const uint64_t slots = static_cast<uint64_t>(g) * nw * rows_seg(nt, k);
+        if (g < 1 || g > 64) return false;
+        if (g > 1 && static_cast<uint64_t>(g) * nw > static_cast<uint64_t>(vkop::kMergeWavesMax)) return false;
+        if (g > 1 && slots > vkop::kMergeRecsMax) return false;
+        // a single-chunk row is merged by its own workgroup: (1024 / vec) records per nt threads, rounded up
+        const uint64_t own = (static_cast<uint64_t>(vkop::kFastCap) / vec + nt - 1) / nt * nt;
+        if (g == 1 && slots > own) return false;
+        const uint64_t cap = static_cast<uint64_t>(nt) * vv * vec;
+        return cap * g >= n && static_cast<uint64_t>(rows) * g < (1ull << 31);
     };
     if (forced_nt) {
         if (!fits(forced_nt, forced_v, static_cast<uint32_t>(forced_g))) return c;
@@ -144,28 +162,36 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
         const uint32_t cap = static_cast<uint32_t>(c.nt) * c.v * vec;
         c.g = (n + cap - 1) / cap;
     }
-    c.per = (nvec + c.g - 1) / c.g * vec;
+    // chunks are whole multiples of the workgroup's capacity wherever the row allows
+    // it, so that all but the last chunk of a row run the unmasked code
+    c.per = static_cast<uint32_t>(c.nt) * c.v * vec;
+    if (static_cast<uint64_t>(c.per) * (c.g - 1) >= n) c.per = (nvec + c.g - 1) / c.g * vec;
+    c.seg = rows_seg(c.nt, k);
+    while ((1u << c.seg_shift) < c.seg) c.seg_shift++;
     c.ok = true;
     return c;
 }
 
 struct RowsLayout {
-    size_t partials = 0, cands = 0, stats = 0, total = 0;
+    size_t sums = 0, meta = 0, recs = 0, stats = 0, total = 0;
 };
 
 // One layout serves the streaming kernel and the general two-kernel path, so
 // the size does not depend on which of them a call ends up taking.
-RowsLayout rows_layout(const View &v, int k, const RowsCfg &c) {
+RowsLayout rows_layout(const View &v, const RowsCfg &c) {
     RowsLayout l;
     const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
     size_t off = 0;
     l.stats = off;
     off += align_up(lines * sizeof(vkop::LineStats));
     if (c.ok) {
-        l.partials = off;
-        off += align_up(lines * c.g * sizeof(vkop::ChunkPartial));
-        l.cands = off;
-        off += align_up(lines * c.g * static_cast<size_t>(k + 1) * sizeof(uint64_t));
+        const size_t entries = lines * c.g * (static_cast<size_t>(c.nt) / 64);
+        l.sums = off;
+        off += align_up(entries * sizeof(vkop::SumPartial));
+        l.meta = off;
+        off += align_up(entries * sizeof(vkop::WaveMeta));
+        l.recs = off;
+        off += align_up(entries * c.seg * 32);
     }
     l.total = off;
     return l;
@@ -176,20 +202,23 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
                 const RowsLayout &l, hipStream_t st) {
     vkop::RowsWorkspace w;
     auto *base = static_cast<unsigned char *>(ws);
-    w.partials = reinterpret_cast<vkop::ChunkPartial *>(base + l.partials);
-    w.cands = reinterpret_cast<uint64_t *>(base + l.cands);
-    w.kc = static_cast<uint32_t>(k + 1);
+    w.sums = reinterpret_cast<vkop::SumPartial *>(base + l.sums);
+    w.meta = reinterpret_cast<vkop::WaveMeta *>(base + l.meta);
+    w.recs = reinterpret_cast<uint4 *>(base + l.recs);
+    w.seg = c.seg;
+    w.seg_shift = c.seg_shift;
     const uint32_t vec = 16 / sizeof(T);
     const bool aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
     const uint32_t blocks = v.g.outer * c.g;
+#define VKOP_ROWS_LAUNCH(NT, V, AL, SG)                                                                         \
+    vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, AL, SG>                                                          \
+        <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w)
 #define VKOP_ROWS_CASE(NT, V)                                                                                   \
     if (c.nt == NT && c.v == V) {                                                                               \
-        if (aligned)                                                                                            \
-            vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, true>                                                    \
-                <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w);   \
-        else                                                                                                    \
-            vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, false>                                                   \
-                <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w);   \
+        if (aligned && c.g == 1) VKOP_ROWS_LAUNCH(NT, V, true, true);                                           \
+        else if (aligned) VKOP_ROWS_LAUNCH(NT, V, true, false);                                                 \
+        else if (c.g == 1) VKOP_ROWS_LAUNCH(NT, V, false, true);                                                \
+        else VKOP_ROWS_LAUNCH(NT, V, false, false);                                                             \
         launched_one = true;                                                                                    \
     }
     bool launched_one = false;
@@ -207,11 +236,12 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
         VKOP_ROWS_CASE(1024, 8)
     }
 #undef VKOP_ROWS_CASE
+#undef VKOP_ROWS_LAUNCH
     if (!launched_one) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
     if (int rc = launched("rows_chunk_kernel")) return rc;
     if (c.g > 1) {
         vkop::rows_merge_kernel<T, SOFTMAX><<<v.g.outer, vkop::kMergeThreads, 0, st>>>(
-            in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, w);
+            in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g * (static_cast<uint32_t>(c.nt) / 64u), w);
         return launched("rows_merge_kernel");
     }
     return VKOP_HIP_OK;
@@ -223,7 +253,7 @@ int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, in
               size_t ws_bytes, hipStream_t st) {
     const RowsCfg c = largest ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
     if (c.ok) {
-        const RowsLayout l = rows_layout(v, k, c);
+        const RowsLayout l = rows_layout(v, c);
         if (ws == nullptr || ws_bytes < l.total)
             return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, l.total);
         return launch_rows<T, false>(in, values, indices, v, k, c, ws, l, st);
@@ -239,7 +269,7 @@ template <typename T>
 int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, int dtype,
                void *ws, hipStream_t st) {
     const RowsCfg c = choose_rows_cfg(v, k, dtype);
-    const RowsLayout l = rows_layout(v, k, c);
+    const RowsLayout l = rows_layout(v, c);
     if (c.ok && largest && probs == nullptr) return launch_rows<T, true>(in, values, indices, v, k, c, ws, l, st);
     // general path: line statistics (and the softmax tensor when asked for), then
     // an exact select keyed by the probabilities those statistics define
@@ -461,7 +491,7 @@ size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int 
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return 0;
     const RowsCfg c = choose_rows_cfg(v, k, dtype);
-    return c.ok ? rows_layout(v, k, c).total : 0;
+    return c.ok ? rows_layout(v, c).total : 0;
 }
 
 int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape, int ndim,
@@ -485,7 +515,7 @@ int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dt
 size_t vkop_hip_softmax_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return 0;
-    return rows_layout(v, k, choose_rows_cfg(v, k, dtype)).total;
+    return rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
 }
 
 int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int32_t *out_indices, int dtype,
@@ -499,7 +529,7 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
     if (in == nullptr || out_values == nullptr || out_indices == nullptr)
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
-    const size_t need = rows_layout(v, k, choose_rows_cfg(v, k, dtype)).total;
+    const size_t need = rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
     if (workspace == nullptr || workspace_bytes < need)
         return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
