@@ -25,6 +25,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script scaled by the same counters over a copy kernel
+# of known size (profiles/ holds the runs); None = not measured for the workload.
+TRAFFIC = {}
+
 WORKLOADS = {
     # name: (description, generator kwargs, k, axis)
     "C1": ("[1,1000] f32 softmax+topk k=5", dict(kind="cls", rows=1, cols=1000), 5),
@@ -81,6 +86,20 @@ def cpu_baseline(x, k, budget_s=12.0):
     }
 
 
+def copy_calibration(nbytes=256 << 20, launches=20):
+    """A plain copy kernel of known size: reads nbytes and writes nbytes per launch."""
+    import torch
+    src = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda").normal_()
+    others = [torch.empty_like(src).normal_() for _ in range(2)]   # push src out of the Infinity Cache
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for i in range(launches):
+        dst.copy_(src if i % 2 == 0 else others[0])
+    torch.cuda.synchronize()
+    print(json.dumps({"copy_bytes_read_per_launch": nbytes, "copy_bytes_written_per_launch": nbytes,
+                      "launches": launches, "kernel": "__amd_rocclr_copyBuffer, the runtime's device copy kernel behind dst.copy_(src)"}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -91,7 +110,13 @@ def main():
     ap.add_argument("--resident", action="store_true", help="reuse one input buffer (Infinity-Cache resident figure)")
     ap.add_argument("--eager", action="store_true",
                     help="issue every call from the host loop instead of replaying a recording of the K calls")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain device copy of known size (the yardstick for the FETCH_SIZE / "
+                         "WRITE_SIZE counters) and print its size")
     args = ap.parse_args()
+    if args.copy_calibration:
+        copy_calibration()
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU; --gpus %d is not supported "
               "(rows are independent: shard the batch and run one process per GPU)" % args.gpus, file=sys.stderr)
@@ -151,41 +176,57 @@ def main():
             step(first + i)
         return capi.graph_end(stream)
 
-    graphs = []
-    if args.eager:
-        for i in range(args.warmup):
-            step(i)
-    else:
-        if args.warmup > 0:
-            gw = record(args.warmup, 0)
-            graphs.append(gw)
-            capi.graph_launch(gw, stream)
-        gk = record(args.steps, args.warmup)
-        graphs.append(gk)
-    capi.stream_sync(stream)
     e0, e1 = capi.event_create(), capi.event_create()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    capi.event_record(e0, stream)
-    if args.eager:
-        for i in range(args.steps):
-            step(args.warmup + i)
-    else:
-        capi.graph_launch(gk, stream)
-    capi.event_record(e1, stream)
-    capi.event_sync(e1)
-    wall_ms = (time.perf_counter() - t0) * 1e3
-    torch.cuda.synchronize()
-    for g in graphs:
-        capi.graph_destroy(g)
-    dev_ms = capi.event_elapsed_ms(e0, e1)
-    ms_per_step = max(dev_ms, 0.0) / args.steps
-    # the bracketing host clock bounds the figure from above; use the larger of
-    # the two so launch-side stalls are never hidden
-    ms_per_step = max(ms_per_step, 0.0)
-    wall_per_step = wall_ms / args.steps
 
-    achieved = algo_bytes / (ms_per_step * 1e-3) / 1e9
+    def timed(stages):
+        """(device ms, host wall ms) of K steps after W warm-up steps, HIP events on `stream`."""
+        capi.tune("rows.stages", stages)
+        graphs = []
+        if args.eager:
+            for i in range(args.warmup):
+                step(i)
+        else:
+            if args.warmup > 0:
+                gw = record(args.warmup, 0)
+                graphs.append(gw)
+                capi.graph_launch(gw, stream)
+            gk = record(args.steps, args.warmup)
+            graphs.append(gk)
+        capi.stream_sync(stream)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        capi.event_record(e0, stream)
+        if args.eager:
+            for i in range(args.steps):
+                step(args.warmup + i)
+        else:
+            capi.graph_launch(gk, stream)
+        capi.event_record(e1, stream)
+        capi.event_sync(e1)
+        wall = (time.perf_counter() - t0) * 1e3
+        torch.cuda.synchronize()
+        for g in graphs:
+            capi.graph_destroy(g)
+        capi.tune("rows.stages", 3)
+        return max(capi.event_elapsed_ms(e0, e1), 0.0), wall
+
+    # each kernel of the path by itself (same launches, same inputs, the other
+    # kernel left out), then the whole step, which is the figure reported
+    stage_ms = {}
+    plan = capi.rows_plan(capi.F32, shape, -1, k)
+    two_kernels = plan[2] > 1
+    if two_kernels:
+        # the merge-only run reads the workspace the whole-step warm-up left
+        timed(3)
+        stage_ms["rows_chunk_kernel"] = timed(1)[0] / args.steps
+        stage_ms["rows_merge_kernel"] = timed(2)[0] / args.steps
+    dev_ms, wall_ms = timed(3)
+    ms_per_step = dev_ms / args.steps
+    wall_per_step = wall_ms / args.steps
+    dominant = max(stage_ms, key=stage_ms.get) if stage_ms else "whole step (single kernel)"
+    dom_ms = stage_ms.get(dominant, ms_per_step)
+
+    achieved = algo_bytes / (dom_ms * 1e-3) / 1e9
     out = {
         "metric": "softmax+topk rows/s and % HBM roofline at [64,128256] fp32, k=50" if args.workload == "C3"
         else "softmax+topk rows/s, " + desc,
@@ -196,14 +237,20 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": desc, "k": k, "input_buffers_rotated": nbuf,
-                   "input_set_bytes": nbuf * in_bytes, "device": capi.device_info()[0]},
+                   "input_set_bytes": nbuf * in_bytes, "device": capi.device_info()[0],
+                   "launch_shape": {"threads": plan[0], "loads_per_thread": plan[1], "chunks_per_row": plan[2]}},
         "device_ms_per_step": ms_per_step,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get(args.workload),
+                     "kernel": dominant,
                      "algorithmic_bytes_per_launch": algo_bytes,
-                     "launch_us": ms_per_step * 1e3,
-                     "timing": "HIP events on the launch stream around %d back-to-back calls (%s)"
-                               % (args.steps, "host loop" if args.eager else "one recorded submission")},
+                     "launch_us": dom_ms * 1e3,
+                     "per_kernel_launch_us": {n: v * 1e3 for n, v in stage_ms.items()},
+                     "whole_step_us": ms_per_step * 1e3,
+                     "whole_step_frac": algo_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "timing": "HIP events on the launch stream around %d back-to-back launches (%s); "
+                               "includes the gap between launches" % (args.steps, "host loop" if args.eager
+                                                                      else "one recorded submission")},
         "parity": parity,
     }
     if not args.no_cpu:

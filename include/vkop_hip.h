@@ -20,9 +20,9 @@
  *    765-801); `axis` may be negative (ops/Softmax.hpp:111-113).
  *  - dtype VKOP_HIP_F16 means IEEE binary16 bits in uint16_t, the reference's
  *    Tensor<uint16_t> (core/Tensor.hpp:116-198).  Arithmetic is float32 either way.
- *  - a workspace must have been cleared once with vkop_hip_workspace_init()
- *    before its first use; calls leave it ready for the next call.  Two calls
- *    that are in flight at the same time must not share a workspace.
+ *  - a workspace holds per-call scratch only (nothing is carried from one
+ *    call to the next and it needs no clearing); two calls that are in flight
+ *    at the same time must not share a workspace.
  */
 #ifndef VKOP_HIP_H_
 #define VKOP_HIP_H_
@@ -129,6 +129,26 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
  * (example/yolo/main.cpp:60-127; ops/Reduce.hpp covers only 4-D images). */
 int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape,
                         int ndim, int axis, void *stream);
+
+/* ---- Tuning and measurement knobs (process-wide; no counterpart in the
+ * reference, whose shaders fix their workgroup shapes at compile time).
+ *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the
+ *       streaming kernel (threads per workgroup, 128-bit loads per thread,
+ *       workgroups per row); all three must be set, 0 = automatic (default).
+ *   "rows.stages": 3 = both kernels of the streaming path (default), 1 = only
+ *       the chunk kernel, 2 = only the merge kernel.  1 and 2 exist so that a
+ *       benchmark can time each kernel by itself; their results are not valid
+ *       top-k output.
+ * Unknown names return VKOP_HIP_ERR_INVALID. */
+int vkop_hip_tune(const char *name, int value);
+
+/* Launch shape the fused / top-k entry points would use for this tensor:
+ * threads per workgroup, 128-bit loads per thread and workgroups per row of the
+ * streaming kernel (a separate merge kernel runs when chunks > 1); all three are
+ * 0 when the general one-workgroup-per-line kernels would run.  Any out pointer
+ * may be NULL. */
+int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k,
+                       int *threads, int *loads, int *chunks);
 
 #ifdef __cplusplus
 }

@@ -84,6 +84,8 @@ def lib():
         "vkop_hip_softmax_topk_workspace_bytes": (sz, [i, ip, i, i, i]),
         "vkop_hip_softmax_topk": (i, [vp, vp, vp, vp, i, ip, i, i, i, i, vp, sz, vp]),
         "vkop_hip_reduce_max": (i, [vp, vp, i, ip, i, i, vp]),
+        "vkop_hip_tune": (i, [ctypes.c_char_p, i]),
+        "vkop_hip_rows_plan": (i, [i, ip, i, i, i, ip, ip, ip]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -227,3 +229,16 @@ def softmax_topk(inp, probs, values, indices, dtype, shape, axis, k, largest=1, 
 def reduce_max(inp, out, dtype, shape, axis, stream=0):
     arr, nd = _shape(shape)
     check(lib().vkop_hip_reduce_max(inp, out, dtype, arr, nd, axis, stream))
+
+
+def tune(name, value):
+    """Process-wide tuning / measurement knob (see include/vkop_hip.h)."""
+    check(lib().vkop_hip_tune(name.encode(), int(value)))
+
+
+def rows_plan(dtype, shape, axis, k):
+    """(threads, loads, chunks) of the streaming kernel for this tensor; zeros = general kernels."""
+    arr, nd = _shape(shape)
+    t, l, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    check(lib().vkop_hip_rows_plan(dtype, arr, nd, axis, k, ctypes.byref(t), ctypes.byref(l), ctypes.byref(c)))
+    return t.value, l.value, c.value

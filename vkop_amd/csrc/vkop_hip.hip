@@ -4,11 +4,11 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
-#include <cstring>
-
 #include <cstdlib>
+#include <cstring>
 
 #include "kernels_general.hpp"
 #include "kernels_rows.hpp"
@@ -80,6 +80,9 @@ int launched(const char *what) {
     return VKOP_HIP_OK;
 }
 
+// vkop_hip_tune state
+std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3};
+
 constexpr int kLineThreads = 256;
 constexpr size_t kAlign = 256;
 inline size_t align_up(size_t b) { return (b + kAlign - 1) / kAlign * kAlign; }
@@ -123,13 +126,11 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     if (v.g.inner != 1 || k > vkop::kFastMaxK || v.g.n == 0 || v.g.outer == 0) return c;
     const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
     const uint32_t n = v.g.n, rows = v.g.outer;
-    static const int shapes_f32[][2] = {{256, 1}, {256, 2}, {256, 4}, {1024, 2}, {1024, 4}, {1024, 8}};
-    static const int shapes_f16[][2] = {{256, 1}, {256, 2}, {256, 4}, {1024, 2}, {1024, 4}, {1024, 4}};
+    static const int shapes_f32[][2] = {{256, 1}, {256, 2}, {256, 4}, {256, 8}, {512, 8}, {1024, 8}};
+    static const int shapes_f16[][2] = {{256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}, {1024, 4}};
     const auto *shapes = dtype == VKOP_HIP_F32 ? shapes_f32 : shapes_f16;
-    int forced_nt = 0, forced_v = 0, forced_g = 0;
-    if (const char *env = std::getenv("VKOP_HIP_ROWS_CFG")) {  // tuning aid: "NT,V,G"
-        if (std::sscanf(env, "%d,%d,%d", &forced_nt, &forced_v, &forced_g) != 3) forced_nt = 0;
-    }
+    int forced_nt = g_rows_threads.load(), forced_v = g_rows_loads.load(), forced_g = g_rows_chunks.load();
+    if (forced_nt <= 0 || forced_v <= 0 || forced_g <= 0) forced_nt = 0;
     const uint32_t nvec = (n + vec - 1) / vec;
     auto fits = [&](int nt, int vv, uint32_t g) {
         const uint32_t nw = static_cast<uint32_t>(nt) / 64u;
@@ -221,7 +222,9 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
         else VKOP_ROWS_LAUNCH(NT, V, false, false);                                                             \
         launched_one = true;                                                                                    \
     }
-    bool launched_one = false;
+    const int stages = c.g > 1 ? g_rows_stages.load() : 3;
+    bool launched_one = (stages & 1) == 0;
+    if (stages & 1) {
     VKOP_ROWS_CASE(256, 1)
     VKOP_ROWS_CASE(256, 2)
     VKOP_ROWS_CASE(256, 4)
@@ -235,11 +238,12 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
         VKOP_ROWS_CASE(512, 8)
         VKOP_ROWS_CASE(1024, 8)
     }
+    }
 #undef VKOP_ROWS_CASE
 #undef VKOP_ROWS_LAUNCH
     if (!launched_one) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
     if (int rc = launched("rows_chunk_kernel")) return rc;
-    if (c.g > 1) {
+    if (c.g > 1 && (stages & 2)) {
         vkop::rows_merge_kernel<T, SOFTMAX><<<v.g.outer, vkop::kMergeThreads, 0, st>>>(
             in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g * (static_cast<uint32_t>(c.nt) / 64u), w);
         return launched("rows_merge_kernel");
@@ -553,6 +557,30 @@ int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape, 
     if (dtype == VKOP_HIP_F32)
         return reduce_max_impl(static_cast<const float *>(in), static_cast<float *>(out), v, as_stream(stream));
     return reduce_max_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, as_stream(stream));
+}
+
+int vkop_hip_tune(const char *name, int value) {
+    if (name == nullptr) return fail(VKOP_HIP_ERR_INVALID, "name is null");
+    if (std::strcmp(name, "rows.threads") == 0) g_rows_threads = value;
+    else if (std::strcmp(name, "rows.loads") == 0) g_rows_loads = value;
+    else if (std::strcmp(name, "rows.chunks") == 0) g_rows_chunks = value;
+    else if (std::strcmp(name, "rows.stages") == 0) {
+        if (value < 1 || value > 3) return fail(VKOP_HIP_ERR_INVALID, "rows.stages must be 1, 2 or 3");
+        g_rows_stages = value;
+    } else return fail(VKOP_HIP_ERR_INVALID, "unknown tuning name '%s'", name);
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k, int *threads, int *loads,
+                       int *chunks) {
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    const RowsCfg c = k >= 1 ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
+    if (threads != nullptr) *threads = c.ok ? c.nt : 0;
+    if (loads != nullptr) *loads = c.ok ? c.v : 0;
+    if (chunks != nullptr) *chunks = c.ok ? static_cast<int>(c.g) : 0;
+    return VKOP_HIP_OK;
 }
 
 }  // extern "C"
