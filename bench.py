@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by the same counters over a copy kernel
 # of known size (profiles/ holds the runs); None = not measured for the workload.
-TRAFFIC = {}
+TRAFFIC = {"C3": 33856010}   # rows_chunk_kernel: 32980213 B read + 875796 B written
 
 WORKLOADS = {
     # name: (description, generator kwargs, k, axis)
@@ -108,6 +108,10 @@ def main():
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--resident", action="store_true", help="reuse one input buffer (Infinity-Cache resident figure)")
+    ap.add_argument("--inflight", type=int, default=3,
+                    help="independent calls in flight (each on its own stream with its own workspace and outputs)")
+    ap.add_argument("--fused", action="store_true",
+                    help="run the streaming path as one kernel (the last chunk of a row merges it) instead of two")
     ap.add_argument("--eager", action="store_true",
                     help="issue every call from the host loop instead of replaying a recording of the K calls")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -130,6 +134,7 @@ def main():
 
     capi.lib()
     capi.init(0)
+    capi.tune("rows.fused", 1 if args.fused else 0)
     desc, spec, k = WORKLOADS[args.workload]
     rows, cols = spec["rows"], spec["cols"]
     shape = (rows, cols)
@@ -142,66 +147,107 @@ def main():
     bufs = []
     for b in range(nbuf):
         bufs.append(torch.from_numpy(host_inputs[b % len(host_inputs)]).cuda())
-    vals = torch.empty((rows, k), dtype=torch.float32, device="cuda")
-    idx = torch.empty((rows, k), dtype=torch.int32, device="cuda")
+    # One "lane" per call in flight: its own stream, workspace and outputs, like the
+    # reference's kInflight = 2 queues (core/runtime.cpp:408-446).  Step i runs on
+    # lane i % L; steps on one lane are serialized, lanes overlap.
     ws_bytes = capi.softmax_topk_workspace_bytes(capi.F32, shape, -1, k)
-    ws = torch.empty(ws_bytes + 256, dtype=torch.uint8, device="cuda")
-    ws_ptr = ws.data_ptr() + (-ws.data_ptr()) % 256
+    lanes = []
+    for _ in range(max(1, args.inflight)):
+        ws = torch.empty(ws_bytes + 256, dtype=torch.uint8, device="cuda")
+        lanes.append({"vals": torch.empty((rows, k), dtype=torch.float32, device="cuda"),
+                      "idx": torch.empty((rows, k), dtype=torch.int32, device="cuda"),
+                      "ws": ws, "ws_ptr": ws.data_ptr() + (-ws.data_ptr()) % 256,
+                      "stream": capi.stream_create(), "event": capi.event_create()})
+    for ln in lanes:
+        capi.workspace_init(ln["ws_ptr"], ws_bytes, ln["stream"])
+        capi.stream_sync(ln["stream"])
     torch.cuda.synchronize()
-    stream = capi.stream_create()
-    capi.workspace_init(ws_ptr, ws_bytes, stream)
+    main_stream = lanes[0]["stream"]
 
-    def step(i):
-        capi.softmax_topk(bufs[i % nbuf].data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), capi.F32, shape, -1, k, 1,
-                          ws_ptr, ws_bytes, stream)
+    def step(i, nlanes):
+        ln = lanes[i % nlanes]
+        capi.softmax_topk(bufs[i % nbuf].data_ptr(), 0, ln["vals"].data_ptr(), ln["idx"].data_ptr(), capi.F32, shape,
+                          -1, k, 1, ln["ws_ptr"], ws_bytes, ln["stream"])
 
-    # parity of what is about to be timed
-    step(0)
-    capi.stream_sync(stream)
+    # parity of what is about to be timed, on every lane
+    parity = {"indices_exact": True, "max_ulp_vs_oracle": 0}
     ov, oix = oracle.softmax_topk(host_inputs[0], k)
-    gi, gv = idx.cpu().numpy(), vals.cpu().numpy()
-    ulp = int(np.abs(gv.view(np.int32).astype(np.int64) - ov.view(np.int32).astype(np.int64)).max())
-    parity = {"indices_exact": bool(np.array_equal(gi, oix)), "max_ulp_vs_oracle": ulp}
-    if not parity["indices_exact"] or ulp > 2:
+    for j, ln in enumerate(lanes):
+        capi.softmax_topk(bufs[0].data_ptr(), 0, ln["vals"].data_ptr(), ln["idx"].data_ptr(), capi.F32, shape, -1, k, 1,
+                          ln["ws_ptr"], ws_bytes, ln["stream"])
+        capi.stream_sync(ln["stream"])
+        gi, gv = ln["idx"].cpu().numpy(), ln["vals"].cpu().numpy()
+        ulp = int(np.abs(gv.view(np.int32).astype(np.int64) - ov.view(np.int32).astype(np.int64)).max())
+        parity["indices_exact"] = parity["indices_exact"] and bool(np.array_equal(gi, oix))
+        parity["max_ulp_vs_oracle"] = max(parity["max_ulp_vs_oracle"], ulp)
+    if not parity["indices_exact"] or parity["max_ulp_vs_oracle"] > 2:
         print("bench.py: parity check failed: %s" % parity, file=sys.stderr)
         sys.exit(1)
 
-    # The K calls are recorded once and the recording is submitted, the way the
-    # reference records each operator into a command buffer and Runtime::Run
-    # submits them (core/runtime.cpp:404-458); a host loop of ~10 us Python calls
-    # could not keep a ~10 us kernel fed.
-    def record(count, first):
-        capi.graph_begin(stream)
-        for i in range(count):
-            step(first + i)
-        return capi.graph_end(stream)
+    def fork(nlanes):
+        """The other lanes' streams start after everything already on the main stream."""
+        if nlanes > 1:
+            capi.event_record(lanes[0]["event"], main_stream)
+            for ln in lanes[1:nlanes]:
+                capi.stream_wait_event(ln["stream"], lanes[0]["event"])
+
+    def join(nlanes):
+        """The main stream continues after everything on the other lanes' streams."""
+        for ln in lanes[1:nlanes]:
+            capi.event_record(ln["event"], ln["stream"])
+            capi.stream_wait_event(main_stream, ln["event"])
+
+    # Each lane's calls are recorded once and the recordings are submitted side by
+    # side, the way the reference records each operator into a command buffer and
+    # Runtime::Run submits one batch per queue (core/runtime.cpp:404-458); a host
+    # loop of ~10 us Python calls could not keep a ~10 us kernel fed.
+    def record(count, first, nlanes):
+        """One recording per lane: the lane's share of steps first .. first+count-1, in order."""
+        graphs = []
+        for j in range(nlanes):
+            capi.graph_begin(lanes[j]["stream"])
+            for i in range(first, first + count):
+                if i % nlanes == j:
+                    step(i, nlanes)
+            graphs.append(capi.graph_end(lanes[j]["stream"]))
+        return graphs
+
+    def submit(graphs, nlanes):
+        fork(nlanes)
+        for j in range(nlanes):
+            capi.graph_launch(graphs[j], lanes[j]["stream"])
+        join(nlanes)
 
     e0, e1 = capi.event_create(), capi.event_create()
 
-    def timed(stages):
-        """(device ms, host wall ms) of K steps after W warm-up steps, HIP events on `stream`."""
+    def timed(stages, nlanes):
+        """(device ms, host wall ms) of K steps after W warm-up steps, HIP events on the main stream."""
         capi.tune("rows.stages", stages)
         graphs = []
         if args.eager:
+            fork(nlanes)
             for i in range(args.warmup):
-                step(i)
+                step(i, nlanes)
+            join(nlanes)
         else:
             if args.warmup > 0:
-                gw = record(args.warmup, 0)
-                graphs.append(gw)
-                capi.graph_launch(gw, stream)
-            gk = record(args.steps, args.warmup)
-            graphs.append(gk)
-        capi.stream_sync(stream)
+                gw = record(args.warmup, 0, nlanes)
+                graphs += gw
+                submit(gw, nlanes)
+            gk = record(args.steps, args.warmup, nlanes)
+            graphs += gk
+        capi.stream_sync(main_stream)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        capi.event_record(e0, stream)
+        capi.event_record(e0, main_stream)
         if args.eager:
+            fork(nlanes)
             for i in range(args.steps):
-                step(args.warmup + i)
+                step(args.warmup + i, nlanes)
+            join(nlanes)
         else:
-            capi.graph_launch(gk, stream)
-        capi.event_record(e1, stream)
+            submit(gk, nlanes)
+        capi.event_record(e1, main_stream)
         capi.event_sync(e1)
         wall = (time.perf_counter() - t0) * 1e3
         torch.cuda.synchronize()
@@ -213,17 +259,23 @@ def main():
     # each kernel of the path by itself (same launches, same inputs, the other
     # kernel left out), then the whole step, which is the figure reported
     stage_ms = {}
+    stage_overlapped = None
     plan = capi.rows_plan(capi.F32, shape, -1, k)
-    two_kernels = plan[2] > 1
+    two_kernels = plan[2] > 1 and not args.fused
     if two_kernels:
-        # the merge-only run reads the workspace the whole-step warm-up left
-        timed(3)
-        stage_ms["rows_chunk_kernel"] = timed(1)[0] / args.steps
-        stage_ms["rows_merge_kernel"] = timed(2)[0] / args.steps
-    dev_ms, wall_ms = timed(3)
+        # one call in flight; the merge-only run reads the workspace the whole-step run left
+        serial_ms = timed(3, 1)[0] / args.steps
+        stage_ms["rows_chunk_kernel"] = timed(1, 1)[0] / args.steps
+        stage_ms["rows_merge_kernel"] = timed(2, 1)[0] / args.steps
+        if len(lanes) > 1:
+            stage_overlapped = {"rows_chunk_kernel": timed(1, len(lanes))[0] / args.steps * 1e3,
+                                "rows_merge_kernel": timed(2, len(lanes))[0] / args.steps * 1e3}
+    else:
+        serial_ms = timed(3, 1)[0] / args.steps
+    dev_ms, wall_ms = timed(3, len(lanes))
     ms_per_step = dev_ms / args.steps
     wall_per_step = wall_ms / args.steps
-    dominant = max(stage_ms, key=stage_ms.get) if stage_ms else "whole step (single kernel)"
+    dominant = max(stage_ms, key=stage_ms.get) if stage_ms else "rows_chunk_kernel (the step's only kernel)"
     dom_ms = stage_ms.get(dominant, ms_per_step)
 
     achieved = algo_bytes / (dom_ms * 1e-3) / 1e9
@@ -236,7 +288,7 @@ def main():
         "ms_per_step": wall_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": desc, "k": k, "input_buffers_rotated": nbuf,
+        "config": {"workload": desc, "k": k, "calls_in_flight": len(lanes), "kernels_per_call": 2 if two_kernels else 1, "input_buffers_rotated": nbuf,
                    "input_set_bytes": nbuf * in_bytes, "device": capi.device_info()[0],
                    "launch_shape": {"threads": plan[0], "loads_per_thread": plan[1], "chunks_per_row": plan[2]}},
         "device_ms_per_step": ms_per_step,
@@ -246,18 +298,22 @@ def main():
                      "algorithmic_bytes_per_launch": algo_bytes,
                      "launch_us": dom_ms * 1e3,
                      "per_kernel_launch_us": {n: v * 1e3 for n, v in stage_ms.items()},
+                     "per_kernel_us_with_calls_in_flight": stage_overlapped,
                      "whole_step_us": ms_per_step * 1e3,
                      "whole_step_frac": algo_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "timing": "HIP events on the launch stream around %d back-to-back launches (%s); "
-                               "includes the gap between launches" % (args.steps, "host loop" if args.eager
-                                                                      else "one recorded submission")},
+                     "whole_step_us_one_in_flight": serial_ms * 1e3,
+                     "timing": "HIP events on the launch stream around %d back-to-back launches of that kernel alone, one "
+                               "call in flight (%s); includes the gap between launches"
+                               % (args.steps, "host loop" if args.eager else "one recorded submission")},
         "parity": parity,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(host_inputs[0], k)
     capi.event_destroy(e0)
     capi.event_destroy(e1)
-    capi.stream_destroy(stream)
+    for ln in lanes:
+        capi.event_destroy(ln["event"])
+        capi.stream_destroy(ln["stream"])
     print(json.dumps(out))
 
 

@@ -20,9 +20,11 @@
  *    765-801); `axis` may be negative (ops/Softmax.hpp:111-113).
  *  - dtype VKOP_HIP_F16 means IEEE binary16 bits in uint16_t, the reference's
  *    Tensor<uint16_t> (core/Tensor.hpp:116-198).  Arithmetic is float32 either way.
- *  - a workspace holds per-call scratch only (nothing is carried from one
- *    call to the next and it needs no clearing); two calls that are in flight
- *    at the same time must not share a workspace.
+ *  - a workspace must have been cleared once with vkop_hip_workspace_init()
+ *    before its first use (it holds per-row arrival counters that every call
+ *    returns to zero); clear it again after a call failed with
+ *    VKOP_HIP_ERR_DEVICE.  Two calls that are in flight at the same time must
+ *    not share a workspace.
  */
 #ifndef VKOP_HIP_H_
 #define VKOP_HIP_H_
@@ -135,10 +137,14 @@ int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape,
  *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the
  *       streaming kernel (threads per workgroup, 128-bit loads per thread,
  *       workgroups per row); all three must be set, 0 = automatic (default).
- *   "rows.stages": 3 = both kernels of the streaming path (default), 1 = only
- *       the chunk kernel, 2 = only the merge kernel.  1 and 2 exist so that a
- *       benchmark can time each kernel by itself; their results are not valid
- *       top-k output.
+ *   "rows.fused": 0 (default) = rows split over several workgroups are merged
+ *       by a second kernel; 1 = one kernel, whose workgroups merge each row as
+ *       its last chunk completes (measured slower on MI355X: the merge then
+ *       waits behind the streaming loads).  Results are identical.
+ *   "rows.stages": with rows.fused = 0 only: 3 = both kernels (default), 1 =
+ *       only the chunk kernel, 2 = only the merge kernel.  1 and 2 exist so
+ *       that a benchmark can time each kernel by itself; their results are not
+ *       valid top-k output.
  * Unknown names return VKOP_HIP_ERR_INVALID. */
 int vkop_hip_tune(const char *name, int value);
 

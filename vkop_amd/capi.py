@@ -242,3 +242,8 @@ def rows_plan(dtype, shape, axis, k):
     t, l, c = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
     check(lib().vkop_hip_rows_plan(dtype, arr, nd, axis, k, ctypes.byref(t), ctypes.byref(l), ctypes.byref(c)))
     return t.value, l.value, c.value
+
+
+def stream_wait_event(stream, event):
+    """Work enqueued on `stream` after this call waits for `event`."""
+    check(lib().vkop_hip_stream_wait_event(stream, event))

@@ -10,24 +10,25 @@
 //      first vector lets the exponentials overlap the rest of the stream),
 //   3. publishes per-lane maxima to LDS; one wave finds, by a ballot descent over
 //      them, a threshold that at least k+1 elements of the chunk reach,
-//   4. compacts the few 128-bit vectors holding an element above the threshold
-//      (ballot + popcount, no atomics) straight into the wave's own segment of
-//      the workspace: the vector as loaded plus a header (index of its first
-//      element, its maximum as an order key),
-//   5. writes one partial (sum, reference, maximum) and one record count per wave.
-// rows_merge_kernel (one workgroup per row; run inside the chunk kernel when
-// G == 1) combines the partial sums, finds the (k+1)-th largest record header,
-// unpacks the few records above it, ranks their elements exactly (key, then
-// lower index), replaces the summed fast terms of the ranked elements by
-// accurate ones, computes the probabilities of the winners only, orders equal
-// probabilities by index and writes the row's result.
-// There are no atomics or fences between workgroups: the kernel boundary
-// publishes the partial results, and every order of summation is fixed, so
-// results are bit-identical from run to run.
-// Whatever the shortcut cannot prove exact (a segment overflows, a partial sum
-// overflows, a probability tie across the k-th place, NaN/inf rows) is redone
-// by the merging workgroup with the exact radix select of select.hpp, so the
-// result is always top-k (probability, then lower index) of the row's softmax.
+//   4. compacts the elements at or above the threshold: the few vectors holding
+//      one go to a per-wave stage in LDS (ballot + popcount), are unpacked one
+//      element per lane, and the survivors are written as (order key, ~index)
+//      composites into the chunk's candidate list,
+//   5. writes one partial (sum, reference, maximum) per wave and the chunk's
+//      candidate count.
+// The workgroup that finishes a row's last chunk (one counter per row) then
+// merges the row: it combines the partial sums, finds the (k+1)-th largest
+// candidate, ranks the candidates above it exactly (key, then lower index),
+// replaces the summed fast terms of the ranked elements by accurate ones,
+// computes the probabilities of the winners only, orders equal probabilities by
+// index and writes the row's result.  Every order of summation is fixed and the
+// ranking does not depend on the order candidates were stored in, so results
+// are bit-identical from run to run.
+// Whatever the shortcut cannot prove exact (a candidate list overflows, a
+// partial sum overflows, a probability tie across the k-th place, NaN/inf rows,
+// rows with fewer than k+1 elements above -inf) is redone by the merging
+// workgroup with the exact radix select of select.hpp, so the result is always
+// top-k (probability, then lower index) of the row's softmax.
 #pragma once
 
 #include <type_traits>
@@ -40,9 +41,10 @@ namespace vkop {
 
 constexpr int kFastCap = 1024;       // LDS slots for elements above the merge threshold
 constexpr int kFastMaxK = 255;       // k + 1 <= 256 ranks are kept in LDS
-constexpr int kMergeThreads = 256;   // rows_merge_kernel workgroup
-constexpr int kMergeRecsMax = 4096;  // record slots per row the merge takes in registers
-constexpr int kMergeWavesMax = 256;  // chunk-kernel waves per row the merge can combine
+constexpr int kMergeThreads = 256;    // rows_merge_kernel workgroup
+constexpr int kMergeRecsMax = 4096;   // candidate slots per row the merge takes in registers
+constexpr int kMergeWavesMax = 256;   // chunk-kernel waves per row the merge can combine
+constexpr int kMergeChunksMax = 64;   // chunks per row
 
 // ---- wave-level helpers (all 64 lanes must be active) -----------------------
 
@@ -135,38 +137,58 @@ __device__ __forceinline__ uint32_t block_kth_largest_floor(const uint32_t *keys
     return prefix;
 }
 
-// ---- workspace ---------------------------------------------------------------
+// ---- memory shared between workgroups ------------------------------------------
+// Everything one workgroup writes for another to read goes through device-scope
+// atomic stores and loads (relaxed): such a store is written through to memory
+// and such a load never takes a stale line from a cache, whichever XCD either
+// workgroup runs on.  No release fence is used: it would write back the whole L2.
 
-struct SumPartial {  // one per wave of the chunk kernel
+__device__ __forceinline__ void publish(uint64_t *p, uint64_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint64_t fetch(const uint64_t *p) {
+    return __hip_atomic_load(const_cast<uint64_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Returns once every store this thread has issued has been performed (for a
+// published value: is visible device-wide).
+__device__ __forceinline__ void drain_stores() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the compiler keeps earlier stores above this point
+    __builtin_amdgcn_s_waitcnt(0);                          // vmcnt(0) expcnt(0) lgkmcnt(0)
+}
+
+struct RowsWorkspace {
+    uint32_t *tickets;  // [rows]: chunks of the row that have published; 0 between calls
+    uint64_t *chunks;   // [rows][G]: candidates the chunk had (low 32 bits); above cap = it could not store them all
+    uint64_t *sums;     // [rows][G * waves per chunk][2]: the wave's sum of exp(x - ref) as double bits, then
+                        // ref (low half) and the wave's maximum (high half) as float bits
+    uint64_t *cand;     // [rows][G][cap]: composites (order key, ~index) of the elements at or above the chunk threshold
+    uint32_t cap;       // candidate slots per chunk (power of two)
+    uint32_t cap_shift;
+};
+
+struct SumPartial {
     double s;   // sum of exp(x - ref) over the wave's elements
     float ref;  // reference of that sum: the maximum of the wave's first vectors, or 0 if that is -inf
     float m;    // the maximum of the wave's elements
 };
 
-struct WaveMeta {  // one per wave
-    uint32_t count;  // records the wave wanted to write; > segment size means overflow
-    float thr;       // chunk threshold: every element with !(x < thr) is in a record
+template <int NT> struct ChunkShared {  // chunk phase
+    uint32_t lane_key[NT];
+    uint4 stage_v[NT];     // per wave: up to 64 vectors holding an element at or above the threshold ...
+    uint32_t stage_e[NT];  // ... and the index of their first element
+    uint32_t wave_thr[16];
+    uint32_t thr, total, over;
 };
 
-struct RowsWorkspace {
-    SumPartial *sums;    // [rows][G][waves per chunk]
-    WaveMeta *meta;      // [rows][G][waves per chunk]
-    uint4 *recs;         // [rows][G][waves per chunk][seg][2]: a 128-bit vector as loaded, then its
-                         // header (index of its first element, its maximum as an order key, 0, 0)
-    uint32_t seg;        // records per wave (power of two)
-    uint32_t seg_shift;  // log2(seg)
-};
-
-struct RowsShared {
+struct RowsShared {  // merge phase
     uint64_t cand[kFastCap];
-    uint16_t cand_src[kFastCap];  // the chunk-kernel wave the element was summed in
     uint32_t rank[kFastCap];
     float prob[kFastMaxK + 1];
     uint32_t pidx[kFastMaxK + 1];
     double corr[kFastMaxK + 1];
     double scale[kMergeWavesMax];  // exp(ref - M) per wave partial
     float ref[kMergeWavesMax];
-    uint32_t cnt[kMergeWavesMax];  // records per wave
+    uint32_t cnt[kMergeChunksMax];  // live candidates per chunk
     uint32_t lane_key[1024];
     uint32_t thr;
     uint32_t count;
@@ -174,7 +196,8 @@ struct RowsShared {
     double total;
 };
 
-union RowsSharedUnion {
+template <int NT> union RowsSharedUnion {
+    ChunkShared<NT> chunk;
     RowsShared fast;
     SelectShared exact;
     __device__ RowsSharedUnion() {}
@@ -263,72 +286,71 @@ template <> struct Vec128<uint16_t> {
 };
 
 // ---- merge of one row's chunk results (all NT threads of a workgroup) --------
-// waves = chunk-kernel waves of this row (G * waves per chunk, <= NT and
-// <= kMergeWavesMax); EM = record slots each thread takes (EM * NT >= waves * seg).
-template <typename T, int NT, int EM, bool SOFTMAX>
-__device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch, double *dscratch, const T *rowp,
-                                          T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t waves,
-                                          const SumPartial *sums, const WaveMeta *meta, const uint4 *recs,
-                                          uint32_t seg, uint32_t seg_shift) {
+// G chunks of `per` elements, each summed and scanned by a workgroup of src_nt
+// threads; G << cap_shift <= kMergeRecsMax, G <= kMergeChunksMax,
+// G * src_nt / 64 <= kMergeWavesMax (the host checks all three).
+template <typename T, int NT, bool SOFTMAX>
+__device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, float *fscratch, double *dscratch,
+                                          const T *rowp, T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
+                                          uint32_t per, uint32_t src_nt, const uint64_t *chunks, const uint64_t *sums,
+                                          const uint64_t *cand, uint32_t cap_shift) {
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
-    RowsShared &sh = smem.fast;
+    constexpr int ES = kMergeRecsMax / NT;  // candidate slots per thread
+    static_assert(NT >= kMergeWavesMax && NT >= kMergeChunksMax, "one thread per wave partial and per chunk");
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t want = k + 1;
     const uint32_t kk = min(k, n);
-    const uint32_t slots = waves << seg_shift;
-    const bool fits = slots <= static_cast<uint32_t>(EM) * NT && waves <= static_cast<uint32_t>(NT) &&
-                      waves <= static_cast<uint32_t>(kMergeWavesMax);
+    const uint32_t cap = 1u << cap_shift;
+    const uint32_t slots = G << cap_shift;
+    const uint32_t src_nw = src_nt / kWave;
+    const uint32_t waves = G * src_nw;
 
-    // ---- A. per-wave metadata and the row's sum from the partials -----------------
-    bool bad = !fits;
-    SumPartial p0{0.0, 0.f, -INFINITY};
-    if (fits && tid < waves) {
-        const WaveMeta mt = meta[tid];
-        p0 = sums[tid];
-        sh.cnt[tid] = min(mt.count, seg);
-        sh.ref[tid] = p0.ref;
-        bad = mt.count > seg;
+    // ---- A. everything the merge reads, in one round trip ---------------------------
+    // (never a branch around a load: out-of-range threads re-read entry 0)
+    const uint32_t wq = tid < waves ? tid : 0u;
+    const uint64_t s_bits = fetch(sums + 2 * wq);
+    const uint64_t rm_bits = fetch(sums + 2 * wq + 1);
+    const uint64_t cm = fetch(chunks + (tid < G ? tid : 0u));
+    uint64_t cv[ES];
+#pragma unroll
+    for (int e = 0; e < ES; e++) {
+        const uint32_t s = static_cast<uint32_t>(e) * NT + tid;
+        cv[e] = fetch(cand + (s < slots ? s : 0u));
     }
-    const float M = block_max<NT>(p0.m, fscratch);  // (barrier: sh.cnt is published)
+
+    // ---- B. the row's maximum and sum from the wave partials --------------------------
+    bool bad = false;
+    SumPartial p0{0.0, 0.f, -INFINITY};
+    if (tid < waves) {
+        p0.s = __longlong_as_double(static_cast<long long>(s_bits));
+        p0.ref = __uint_as_float(static_cast<uint32_t>(rm_bits));
+        p0.m = __uint_as_float(static_cast<uint32_t>(rm_bits >> 32));
+        sh.ref[tid] = p0.ref;
+    }
+    if (tid < G) {
+        const uint32_t c = static_cast<uint32_t>(cm);
+        sh.cnt[tid] = min(c, cap);
+        bad = c > cap;
+    }
+    const float M = block_max<NT>(p0.m, fscratch);  // (barrier: sh.cnt and sh.ref are published)
     double acc = 0.0;
-    if (fits && tid < waves) {
+    if (tid < waves) {
         const double sc = exp(static_cast<double>(p0.ref) - static_cast<double>(M));
         sh.scale[tid] = sc;
         if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
     }
     const double s_base = block_sum<NT>(acc, dscratch);  // (barrier: sh.scale is published)
 
-    // ---- B. record headers: the maximum of every live record ------------------------
-    // Thread t takes the slots q = e * NT + t of the list ordered by (position in
-    // segment, wave): the live records, which sit at the low positions of every
-    // segment, are then spread evenly over the threads.
-    uint32_t rkey[EM], ridx[EM], rslot[EM];
+    // ---- C. threshold: the (k+1)-th largest per-thread maximum -------------------------
     uint32_t lmk = 0;
-    {
-        const uint32_t wv = fits ? waves : 1u;
-        const uint32_t dj = NT / wv, dw = NT - dj * wv;  // one step of e in (j, w)
-        uint32_t j = tid / wv, w = tid - j * wv;
 #pragma unroll
-        for (int e = 0; e < EM; e++) {
-            // never a branch around a load: dead slots read slot 0 and are masked
-            const bool live = fits && j < sh.cnt[w];
-            const uint32_t t = live ? ((w << seg_shift) + j) : 0u;
-            const uint4 hdr = recs[2 * t + 1];
-            rkey[e] = live ? hdr.y : 0u;
-            ridx[e] = hdr.x;
-            rslot[e] = t;
-            lmk = max(lmk, rkey[e]);
-            j += dj;
-            w += dw;
-            if (w >= wv) {
-                w -= wv;
-                j++;
-            }
-        }
+    for (int e = 0; e < ES; e++) {
+        const uint32_t s = static_cast<uint32_t>(e) * NT + tid;
+        const bool live = s < slots && (s & (cap - 1)) < sh.cnt[s < slots ? (s >> cap_shift) : 0u];
+        if (!live) cv[e] = 0;
+        lmk = max(lmk, static_cast<uint32_t>(cv[e] >> 32));
     }
-
-    // ---- C. threshold: the (k+1)-th largest lane maximum --------------------------
     sh.lane_key[tid] = lmk;
     if (tid == 0) {
         sh.count = 0;
@@ -338,7 +360,7 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
     if (bad) sh.flag = 1;  // every writer stores the same value
     if (wave == 0) {
         const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
-        if (lane == 0) sh.thr = max(t, 1u);  // key 0 is "no element"
+        if (lane == 0) sh.thr = t > 1u ? t : 1u;  // key 0 is "no element"
     }
     __syncthreads();
     const uint32_t thr = sh.thr;
@@ -347,45 +369,39 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
     if (SOFTMAX && !(M > -INFINITY && M < INFINITY)) slow = true;
 
     if (!slow) {
-        // ---- D. unpack the few records reaching the threshold ------------------------
-        // (a thread rarely holds more than one: the loop is a round trip or two)
+        // ---- D. the candidates reaching the threshold go to LDS ------------------------
 #pragma unroll
-        for (int e = 0; e < EM; e++) {
-            if (rkey[e] < thr) continue;
-            const uint32_t t = rslot[e];
-            const uint32_t idx0 = ridx[e];
-            Vec128<T> q;
-            q.v = recs[2 * t];
-#pragma unroll
-            for (int c = 0; c < VEC; c++) {
-                const uint32_t key = idx0 + c < n ? order_key(q.get(c)) : 0u;
-                if (key >= thr) {
-                    const uint32_t pos = atomicAdd(&sh.count, 1u);
-                    if (pos < kFastCap) {
-                        sh.cand[pos] = composite(key, idx0 + c);
-                        sh.cand_src[pos] = static_cast<uint16_t>(t >> seg_shift);
-                    }
-                }
+        for (int e = 0; e < ES; e++) {
+            if (static_cast<uint32_t>(cv[e] >> 32) >= thr) {
+                const uint32_t pos = atomicAdd(&sh.count, 1u);
+                if (pos < kFastCap) sh.cand[pos] = cv[e];
             }
         }
         __syncthreads();
         const uint32_t C2 = sh.count;
-        if (C2 > kFastCap) {
+        // fewer than k+1 candidates prove nothing about the elements left out
+        if (C2 > kFastCap || C2 < min(want, n)) {
             slow = true;
         } else {
             // ---- E. exact ranks; accurate terms for the ranked elements ----------------
             block_rank<NT>(sh, C2);
-            const uint32_t ranked = min(C2, static_cast<uint32_t>(kFastMaxK + 1));
+            // only the k+1 largest are used from here on: which other candidates
+            // passed the threshold depends on the order the chunks stored theirs in,
+            // and nothing that reaches the output may
+            const uint32_t ranked = min(C2, want);
             for (uint32_t t = tid; t < C2; t += NT) {
                 const uint32_t r = sh.rank[t];
                 if (r < ranked) {
                     const uint64_t cmp = sh.cand[t];
                     const uint32_t key = static_cast<uint32_t>(cmp >> 32);
-                    sh.pidx[r] = composite_index(cmp);
+                    const uint32_t idx = composite_index(cmp);
+                    sh.pidx[r] = idx;
                     sh.prob[r] = ordered_to_float(key);  // the logit, for now
                     double cr = 0.0;
                     if (SOFTMAX && key != 0xFFFFFFFFu) {
-                        const uint32_t sp = sh.cand_src[t];
+                        // the chunk-kernel wave that summed this element
+                        const uint32_t b = idx / per, off = idx - b * per;
+                        const uint32_t sp = b * src_nw + ((off / VEC) % src_nt) / kWave;
                         const float xv = ordered_to_float(key);
                         // what the element should contribute, exp(fl(x - M)), minus what
                         // its wave added for it, exp2(fl(fl(x - ref) * log2 e)) * exp(ref - M)
@@ -439,22 +455,22 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
     }
 
     // ---- exact path: radix select over the whole row ----------------------------
-    __syncthreads();  // smem changes owner
+    __syncthreads();  // LDS changes owner
     if constexpr (SOFTMAX) {
         // redo the statistics the way the general kernels define them
         const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch);
-        select_topk_line<NT>(smem.exact, n, kk, [&](uint32_t j) {
+        select_topk_line<NT>(exact, n, kk, [&](uint32_t j) {
             return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
         });
         for (uint32_t r = tid; r < kk; r += NT) {
-            const uint32_t idx = composite_index(smem.exact.sel[r]);
+            const uint32_t idx = composite_index(exact.sel[r]);
             store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
             oi[r] = static_cast<int32_t>(idx);
         }
     } else {
-        select_topk_line<NT>(smem.exact, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
+        select_topk_line<NT>(exact, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
         for (uint32_t r = tid; r < kk; r += NT) {
-            const uint32_t idx = composite_index(smem.exact.sel[r]);
+            const uint32_t idx = composite_index(exact.sel[r]);
             ov[r] = rowp[idx];
             oi[r] = static_cast<int32_t>(idx);
         }
@@ -465,33 +481,27 @@ __device__ __forceinline__ void merge_row(RowsSharedUnion &smem, float *fscratch
 // SOFTMAX = false: plain top-k, largest first (values are copies of the input)
 // ALIGNED: every row start is 16-byte aligned and n is a multiple of the vector
 // width, so chunks are read with 128-bit loads.
+// FUSED: the workgroup that publishes a row's last chunk (found with one
+// counter per row) merges the row before it exits; otherwise rows_merge_kernel
+// must follow on the same stream.
 // Launch: rows * G workgroups of NT threads; per = elements per chunk
 // (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
-// SINGLE: G == 1 and the workgroup also merges (no second kernel); otherwise the
-// kernel needs only a few KB of LDS.
-struct ChunkShared {
-    uint32_t lane_key[1024];
-    uint32_t thr;
-};
-
-template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, bool SINGLE>
+template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, bool FUSED>
 __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                         int32_t *__restrict__ indices, uint32_t n, uint32_t k,
                                                         uint32_t G, uint32_t per, RowsWorkspace ws) {
     constexpr int VEC = Vec128<T>::N;
     constexpr int NW = NT / kWave;
-    __shared__ std::conditional_t<SINGLE, RowsSharedUnion, ChunkShared> smem;
-    __shared__ float fscratch[SINGLE ? NW : 1];
-    __shared__ double dscratch[SINGLE ? NW : 1];
-    uint32_t *lane_keys;
-    uint32_t *thr_slot;
-    if constexpr (SINGLE) {
-        lane_keys = smem.fast.lane_key;
-        thr_slot = &smem.fast.thr;
-    } else {
-        lane_keys = smem.lane_key;
-        thr_slot = &smem.thr;
-    }
+    constexpr int VPP = kWave / VEC;    // staged vectors a wave unpacks per pass (one element per lane)
+    constexpr int PASSES = kWave / VPP;  // passes over a full stage of 64 vectors
+    __shared__ std::conditional_t<FUSED, RowsSharedUnion<NT>, ChunkShared<NT>> smem;
+    __shared__ float fscratch[FUSED ? NW : 1];
+    __shared__ double dscratch[FUSED ? NW : 1];
+    __shared__ uint32_t s_last;
+    ChunkShared<NT> *csp;
+    if constexpr (FUSED) csp = &smem.chunk;
+    else csp = &smem;
+    ChunkShared<NT> &cs = *csp;
 
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
@@ -500,6 +510,10 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
     const uint32_t want = k + 1;  // one extra: the merge needs the (k+1)-th to prove the cut
     const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
     const uint32_t went = (row * G + chunk) * NW + wave;  // this wave's slot in the row-major wave list
+    if (tid == 0) {
+        cs.total = 0;
+        cs.over = 0;
+    }
 
     // ---- 1. all loads in flight -----------------------------------------------------
     Vec128<T> q[V];
@@ -518,8 +532,8 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
         }
     }
 
-    // The rest of the kernel exists twice: for a chunk that fills every lane of
-    // every vector (no masking anywhere) and for a ragged one.
+    // The rest of the chunk phase exists twice: for a chunk that fills every lane
+    // of every vector (no masking anywhere) and for a ragged one.
     auto body = [&](auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;
         auto in_range = [&](uint32_t e) { return FULL || e < c1; };
@@ -563,61 +577,168 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
             }
         }
         if constexpr (SOFTMAX) lkey = in_range(e_first) ? order_key(lmax) : 0u;
+        uint32_t thr_block;
 
-        // ---- 3. lane maxima -> LDS; one wave finds the chunk threshold ---------------------
-        lane_keys[tid] = lkey;
-        __syncthreads();
-        if (wave == blockIdx.x % NW) {  // not always wave 0: spreads this serial step over the SIMDs
-            const uint32_t t = block_kth_largest_floor<NW>(lane_keys, want, 16);
-            if (lane == 0) *thr_slot = t;
-        }
+        // ---- 3. the chunk threshold: at least k+1 elements of the chunk reach it -----------
         const float wm = wave_max_f32_uniform(lmax);
         double wsum = 0.0;
         if constexpr (SOFTMAX) wsum = wave_sum_f64_uniform(acc);
-        __syncthreads();
-        const uint32_t thr = *thr_slot;
-        const float thr_f = key_threshold_to_float(thr);
+        if constexpr (FULL) {
+            // Every wave finds the q-th largest of its own 64 lane maxima, q = its share
+            // of k+1.  The (k+1)-th largest lane maximum of the whole workgroup lies
+            // between the smallest and the largest of these, so every wave then
+            // settles the few bits in which the two differ over all lane maxima
+            // (all waves compute the same value: no broadcast).
+            const uint32_t quota = (want + NW - 1) / NW;
+            uint32_t mine_q = 0;
+            if (quota <= static_cast<uint32_t>(kWave)) {
+                for (int bit = 31; bit > 15; bit--) {
+                    const uint32_t trial = mine_q | (1u << bit);
+                    if (static_cast<uint32_t>(__popcll(__ballot(lkey >= trial))) >= quota) mine_q = trial;
+                }
+            }
+            cs.lane_key[tid] = lkey;
+            if (lane == 0) cs.wave_thr[wave] = mine_q;
+            __syncthreads();
+            uint32_t lo = cs.wave_thr[0], hi = lo;
+#pragma unroll
+            for (int w = 1; w < NW; w++) {
+                lo = min(lo, cs.wave_thr[w]);
+                hi = max(hi, cs.wave_thr[w]);
+            }
+            uint32_t t = lo;
+            if (lo != hi) {
+                uint32_t kv[NW];
+#pragma unroll
+                for (int w = 0; w < NW; w++) kv[w] = cs.lane_key[w * kWave + lane];
+                const int d = 31 - __clz(static_cast<int>(lo ^ hi));  // highest bit in which they differ
+                t = hi & ~((2u << d) - 1u);                            // their common prefix
+                for (int bit = d; bit > 15; bit--) {
+                    const uint32_t trial = t | (1u << bit);
+                    uint32_t cnt = 0;
+#pragma unroll
+                    for (int w = 0; w < NW; w++) cnt += static_cast<uint32_t>(__popcll(__ballot(kv[w] >= trial)));
+                    if (cnt >= want) t = trial;
+                }
+            }
+            thr_block = t;
+        } else {
+            // ragged chunk: some waves may hold few elements or none, so one wave takes
+            // the (k+1)-th largest of all lane maxima
+            cs.lane_key[tid] = lkey;
+            __syncthreads();
+            if (wave == blockIdx.x % NW) {
+                const uint32_t t = block_kth_largest_floor<NW>(cs.lane_key, want, 16);
+                if (lane == 0) cs.thr = t;
+            }
+            __syncthreads();
+            thr_block = cs.thr;
+        }
+        // -inf never becomes a candidate: a row with k+1 larger elements does not
+        // need it, and any other row is left to the exact path
+        const uint32_t thr = max(thr_block, kKeyNegInf + 1u);
+        const float thr_f = ordered_to_float(thr);
 
-        // ---- 4. compaction of the vectors reaching the threshold ----------------------------
-        uint4 *rec_out = ws.recs + (static_cast<size_t>(went) << (ws.seg_shift + 1));
-        const uint32_t last_slot = ws.seg - 1;
-        uint32_t wcount = 0;  // wave-uniform
+        // ---- 4a. the wave's vectors holding an element at or above the threshold -> LDS ------
+        uint4 *stv = cs.stage_v + wave * kWave;
+        uint32_t *ste = cs.stage_e + wave * kWave;
+        uint32_t nv = 0;  // wave-uniform
 #pragma unroll
         for (int i = 0; i < V; i++) {
             const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
             bool hit;
             if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
-            else hit = (vkey[i] >= (thr > 1u ? thr : 1u)) && in_range(e0);
+            else hit = vkey[i] >= thr && in_range(e0);
             const uint64_t mask = __ballot(hit);
             if (mask != 0ull) {
                 if (hit) {
-                    // past the end of the segment everything lands in the last slot;
-                    // the count then exceeds the segment and the row takes the exact path
-                    const uint32_t pos = min(wcount + lanes_below(mask), last_slot);
-                    rec_out[2 * pos] = q[i].v;
-                    rec_out[2 * pos + 1] = make_uint4(e0, SOFTMAX ? order_key(vmax[i]) : vkey[i], 0u, 0u);
+                    const uint32_t pos = nv + lanes_below(mask);
+                    if (pos < kWave) {
+                        stv[pos] = q[i].v;
+                        ste[pos] = e0;
+                    }
+                }
+                nv += static_cast<uint32_t>(__popcll(mask));
+            }
+        }
+        const bool over = nv > kWave;
+        nv = min(nv, static_cast<uint32_t>(kWave));
+        __builtin_amdgcn_wave_barrier();  // the stage is read by other lanes of the same wave
+
+        // ---- 4b. one element per lane: keep those at or above the threshold ------------------
+        uint64_t mine[PASSES];
+        uint32_t mpos[PASSES];
+        uint32_t wcount = 0;  // wave-uniform
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            mine[p] = 0;  // 0 = nothing to write
+            mpos[p] = 0;
+            if (static_cast<uint32_t>(p) * VPP < nv) {
+                const uint32_t sv = static_cast<uint32_t>(p) * VPP + lane / VEC;
+                const bool live = sv < nv;
+                Vec128<T> r;
+                r.v = stv[live ? sv : 0u];
+                const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
+                const float x = r.get(static_cast<int>(lane % VEC));
+                const uint32_t key = order_key(x);
+                const bool pass = live && idx < c1 && key >= thr;
+                const uint64_t mask = __ballot(pass);
+                if (pass) {
+                    mine[p] = composite(key, idx);
+                    mpos[p] = wcount + lanes_below(mask);
                 }
                 wcount += static_cast<uint32_t>(__popcll(mask));
             }
         }
-
-        // ---- 5. partials ---------------------------------------------------------------------
+        // room in the chunk's candidate list, reserved once per wave
+        uint32_t base = 0;
         if (lane == 0) {
-            ws.sums[went] = SumPartial{wsum, ref, wm};
-            ws.meta[went] = WaveMeta{wcount, thr_f};
+            base = atomicAdd(&cs.total, wcount);
+            if (over) cs.over = 1;
+        }
+        base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
+        uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            const uint32_t pos = base + mpos[p];
+            if (mine[p] != 0 && pos < ws.cap) publish(cand_out + pos, mine[p]);
+        }
+
+        // ---- 5. the wave's partial sum -----------------------------------------------------------
+        if (lane == 0) {
+            publish(ws.sums + 2 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
+            publish(ws.sums + 2 * static_cast<size_t>(went) + 1,
+                    (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
         }
     };
     if (c1 - c0 == static_cast<uint32_t>(NT) * V * VEC) body(std::true_type{});
     else body(std::false_type{});
 
-    if constexpr (SINGLE) {
-        // ---- single-chunk rows: merge right here ----------------------------------
-        __syncthreads();  // this workgroup's own global writes
-        constexpr int EM1 = (kFastCap / VEC + NT - 1) / NT;
-        const size_t w0 = static_cast<size_t>(row) * NW;
-        merge_row<T, NT, EM1, SOFTMAX>(smem, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
-                                       indices + static_cast<size_t>(row) * k, n, k, NW, ws.sums + w0, ws.meta + w0,
-                                       ws.recs + (w0 << (ws.seg_shift + 1)), ws.seg, ws.seg_shift);
+    // ---- 6. the chunk's candidate count; the row's last chunk merges -------------------------
+    if constexpr (FUSED) drain_stores();  // (a following kernel sees everything anyway)
+    __syncthreads();  // fused: every thread's published values are visible device-wide
+    if (tid == 0) {
+        publish(ws.chunks + (row * G + chunk), cs.over ? 0xFFFFFFFFull : static_cast<uint64_t>(cs.total));
+        uint32_t last = 1;
+        if constexpr (FUSED) {
+            drain_stores();
+            if (G > 1) {
+                const uint32_t done = __hip_atomic_fetch_add(ws.tickets + row, 1u, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT);
+                last = (done == G - 1) ? 1u : 0u;
+                // ready for the next call (nobody else touches this row's counter any more)
+                if (last) __hip_atomic_store(ws.tickets + row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        s_last = last;
+    }
+    if constexpr (FUSED) {
+        __syncthreads();
+        if (s_last == 0u) return;
+        merge_row<T, NT, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
+                                  indices + static_cast<size_t>(row) * k, n, k, G, per, NT,
+                                  ws.chunks + static_cast<size_t>(row) * G, ws.sums + 2 * static_cast<size_t>(row) * G * NW,
+                                  ws.cand + (static_cast<size_t>(row) * G << ws.cap_shift), ws.cap_shift);
     } else {
         (void)values;
         (void)indices;
@@ -626,20 +747,27 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
     }
 }
 
-// One workgroup of kMergeThreads per row; waves = G * (waves per chunk workgroup).
+union MergeShared {
+    RowsShared fast;
+    SelectShared exact;
+    __device__ MergeShared() {}
+};
+
+// Second kernel of the unfused variant: one workgroup of kMergeThreads per row.
 template <typename T, bool SOFTMAX>
 __global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                                    int32_t *__restrict__ indices, uint32_t n,
-                                                                   uint32_t k, uint32_t waves, RowsWorkspace ws) {
-    __shared__ RowsSharedUnion smem;
+                                                                   uint32_t k, uint32_t G, uint32_t per,
+                                                                   uint32_t src_nt, RowsWorkspace ws) {
+    __shared__ MergeShared smem;
     __shared__ float fscratch[kMergeThreads / kWave];
     __shared__ double dscratch[kMergeThreads / kWave];
     const uint32_t row = blockIdx.x;
-    const size_t w0 = static_cast<size_t>(row) * waves;
-    merge_row<T, kMergeThreads, kMergeRecsMax / kMergeThreads, SOFTMAX>(
-        smem, fscratch, dscratch, in + static_cast<size_t>(row) * n, values + static_cast<size_t>(row) * k,
-        indices + static_cast<size_t>(row) * k, n, k, waves, ws.sums + w0, ws.meta + w0,
-        ws.recs + (w0 << (ws.seg_shift + 1)), ws.seg, ws.seg_shift);
+    merge_row<T, kMergeThreads, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, in + static_cast<size_t>(row) * n,
+                                         values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k,
+                                         n, k, G, per, src_nt, ws.chunks + static_cast<size_t>(row) * G,
+                                         ws.sums + 2 * static_cast<size_t>(row) * G * (src_nt / kWave),
+                                         ws.cand + (static_cast<size_t>(row) * G << ws.cap_shift), ws.cap_shift);
 }
 
 }  // namespace vkop

@@ -81,7 +81,7 @@ int launched(const char *what) {
 }
 
 // vkop_hip_tune state
-std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3};
+std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0};
 
 constexpr int kLineThreads = 256;
 constexpr size_t kAlign = 256;
@@ -102,23 +102,23 @@ int softmax_impl(const T *in, T *out, const View &v, int nan_where, float nan_va
 }
 
 // ------------------------------------------------- streaming rows kernel ----
-// Launch shape of rows_topk_kernel: NT threads, V 128-bit loads per thread,
-// G chunks per row of `per` elements each.
+// Launch shape of rows_chunk_kernel: NT threads, V 128-bit loads per thread,
+// G chunks per row of `per` elements each, `cap` candidate slots per chunk.
 struct RowsCfg {
     bool ok = false;
     int nt = 0, v = 0;
     uint32_t g = 0, per = 0;
-    uint32_t seg = 0, seg_shift = 0;  // candidate slots per wave of a chunk workgroup
+    uint32_t cap = 0, cap_shift = 0;
 };
 
-// Slots per wave: four times the wave's quota of the k+1 wanted elements (about
-// 1.5 quotas are used on identically distributed data), at least 32, power of two.
-uint32_t rows_seg(int nt, int k) {
-    const uint32_t nw = static_cast<uint32_t>(nt) / 64u;
-    const uint32_t quota = (static_cast<uint32_t>(k) + 1u + nw - 1u) / nw;
-    uint32_t seg = 32;
-    while (seg < 4u * quota) seg <<= 1;
-    return seg;
+// Candidate slots per chunk: 2.5 times the k+1 wanted elements (a chunk of
+// identically distributed data has about 1.2 times k+1 at or above its
+// threshold), at least 64, power of two.
+uint32_t rows_cap(int k) {
+    const uint32_t want = static_cast<uint32_t>(k) + 1u;
+    uint32_t cap = 64;
+    while (2u * cap < 5u * want) cap <<= 1;
+    return cap;
 }
 
 RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
@@ -132,17 +132,14 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     int forced_nt = g_rows_threads.load(), forced_v = g_rows_loads.load(), forced_g = g_rows_chunks.load();
     if (forced_nt <= 0 || forced_v <= 0 || forced_g <= 0) forced_nt = 0;
     const uint32_t nvec = (n + vec - 1) / vec;
+    const uint32_t cap = rows_cap(k);
     auto fits = [&](int nt, int vv, uint32_t g) {
         const uint32_t nw = static_cast<uint32_t>(nt) / 64u;
-        const uint64_t slots = static_cast<uint64_t>(g) * nw * rows_seg(nt, k);
-        if (g < 1 || g > 64) return false;
-        if (g > 1 && static_cast<uint64_t>(g) * nw > static_cast<uint64_t>(vkop::kMergeWavesMax)) return false;
-        if (g > 1 && slots > vkop::kMergeRecsMax) return false;
-        // a single-chunk row is merged by its own workgroup: (1024 / vec) records per nt threads, rounded up
-        const uint64_t own = (static_cast<uint64_t>(vkop::kFastCap) / vec + nt - 1) / nt * nt;
-        if (g == 1 && slots > own) return false;
-        const uint64_t cap = static_cast<uint64_t>(nt) * vv * vec;
-        return cap * g >= n && static_cast<uint64_t>(rows) * g < (1ull << 31);
+        if (g < 1 || g > static_cast<uint32_t>(vkop::kMergeChunksMax)) return false;
+        if (static_cast<uint64_t>(g) * nw > static_cast<uint64_t>(vkop::kMergeWavesMax)) return false;
+        if (static_cast<uint64_t>(g) * cap > static_cast<uint64_t>(vkop::kMergeRecsMax)) return false;
+        const uint64_t span = static_cast<uint64_t>(nt) * vv * vec;
+        return span * g >= n && static_cast<uint64_t>(rows) * g < (1ull << 31);
     };
     if (forced_nt) {
         if (!fits(forced_nt, forced_v, static_cast<uint32_t>(forced_g))) return c;
@@ -152,47 +149,56 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
         // tensor is too small for that, the smallest shape that covers a row
         int pick = -1;
         for (int i = 0; i < 6; i++) {
-            const uint32_t cap = static_cast<uint32_t>(shapes[i][0]) * shapes[i][1] * vec;
-            const uint32_t g = (n + cap - 1) / cap;
+            const uint32_t span = static_cast<uint32_t>(shapes[i][0]) * shapes[i][1] * vec;
+            const uint32_t g = (n + span - 1) / span;
             if (!fits(shapes[i][0], shapes[i][1], g)) continue;
             if (pick < 0) pick = i;
             if (static_cast<uint64_t>(rows) * g >= 1024) pick = i;
         }
         if (pick < 0) return c;
         c.nt = shapes[pick][0], c.v = shapes[pick][1];
-        const uint32_t cap = static_cast<uint32_t>(c.nt) * c.v * vec;
-        c.g = (n + cap - 1) / cap;
+        const uint32_t span = static_cast<uint32_t>(c.nt) * c.v * vec;
+        c.g = (n + span - 1) / span;
     }
     // chunks are whole multiples of the workgroup's capacity wherever the row allows
     // it, so that all but the last chunk of a row run the unmasked code
     c.per = static_cast<uint32_t>(c.nt) * c.v * vec;
     if (static_cast<uint64_t>(c.per) * (c.g - 1) >= n) c.per = (nvec + c.g - 1) / c.g * vec;
-    c.seg = rows_seg(c.nt, k);
-    while ((1u << c.seg_shift) < c.seg) c.seg_shift++;
+    c.cap = cap;
+    while ((1u << c.cap_shift) < c.cap) c.cap_shift++;
     c.ok = true;
     return c;
 }
 
 struct RowsLayout {
-    size_t sums = 0, meta = 0, recs = 0, stats = 0, total = 0;
+    size_t tickets = 0, chunks = 0, sums = 0, cand = 0, stats = 0, total = 0;
 };
 
 // One layout serves the streaming kernel and the general two-kernel path, so
 // the size does not depend on which of them a call ends up taking.
+//
+// The per-row arrival counters sit at a fixed place, the first kTicketRows words
+// of every workspace, whatever the tensor: each call leaves them at zero, so a
+// workspace cleared once can serve calls of different shapes in turn.  Nothing
+// else is ever stored there.
+constexpr size_t kTicketRows = 16384;
+
 RowsLayout rows_layout(const View &v, const RowsCfg &c) {
     RowsLayout l;
     const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
     size_t off = 0;
+    l.tickets = off;
+    off += align_up(kTicketRows * sizeof(uint32_t));
     l.stats = off;
     off += align_up(lines * sizeof(vkop::LineStats));
     if (c.ok) {
-        const size_t entries = lines * c.g * (static_cast<size_t>(c.nt) / 64);
+        const size_t chunks = lines * c.g;
+        l.chunks = off;
+        off += align_up(chunks * sizeof(uint64_t));
         l.sums = off;
-        off += align_up(entries * sizeof(vkop::SumPartial));
-        l.meta = off;
-        off += align_up(entries * sizeof(vkop::WaveMeta));
-        l.recs = off;
-        off += align_up(entries * c.seg * 32);
+        off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * 2 * sizeof(uint64_t));
+        l.cand = off;
+        off += align_up(chunks * c.cap * sizeof(uint64_t));
     }
     l.total = off;
     return l;
@@ -203,49 +209,49 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
                 const RowsLayout &l, hipStream_t st) {
     vkop::RowsWorkspace w;
     auto *base = static_cast<unsigned char *>(ws);
-    w.sums = reinterpret_cast<vkop::SumPartial *>(base + l.sums);
-    w.meta = reinterpret_cast<vkop::WaveMeta *>(base + l.meta);
-    w.recs = reinterpret_cast<uint4 *>(base + l.recs);
-    w.seg = c.seg;
-    w.seg_shift = c.seg_shift;
+    w.tickets = reinterpret_cast<uint32_t *>(base + l.tickets);
+    w.chunks = reinterpret_cast<uint64_t *>(base + l.chunks);
+    w.sums = reinterpret_cast<uint64_t *>(base + l.sums);
+    w.cand = reinterpret_cast<uint64_t *>(base + l.cand);
+    w.cap = c.cap;
+    w.cap_shift = c.cap_shift;
     const uint32_t vec = 16 / sizeof(T);
     const bool aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
     const uint32_t blocks = v.g.outer * c.g;
-#define VKOP_ROWS_LAUNCH(NT, V, AL, SG)                                                                         \
-    vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, AL, SG>                                                          \
+    // more rows than arrival counters: the merge runs as a kernel of its own
+    const bool fused = c.g == 1 || (g_rows_fused.load() != 0 && v.g.outer <= kTicketRows);
+    const int stages = fused ? 1 : g_rows_stages.load();
+#define VKOP_ROWS_LAUNCH(NT, V, AL, FU)                                                                         \
+    vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, AL, FU>                                                          \
         <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w)
 #define VKOP_ROWS_CASE(NT, V)                                                                                   \
     if (c.nt == NT && c.v == V) {                                                                               \
-        if (aligned && c.g == 1) VKOP_ROWS_LAUNCH(NT, V, true, true);                                           \
+        if (aligned && fused) VKOP_ROWS_LAUNCH(NT, V, true, true);                                              \
         else if (aligned) VKOP_ROWS_LAUNCH(NT, V, true, false);                                                 \
-        else if (c.g == 1) VKOP_ROWS_LAUNCH(NT, V, false, true);                                                \
+        else if (fused) VKOP_ROWS_LAUNCH(NT, V, false, true);                                                   \
         else VKOP_ROWS_LAUNCH(NT, V, false, false);                                                             \
         launched_one = true;                                                                                    \
     }
-    const int stages = c.g > 1 ? g_rows_stages.load() : 3;
     bool launched_one = (stages & 1) == 0;
     if (stages & 1) {
-    VKOP_ROWS_CASE(256, 1)
-    VKOP_ROWS_CASE(256, 2)
-    VKOP_ROWS_CASE(256, 4)
-    VKOP_ROWS_CASE(512, 2)
-    VKOP_ROWS_CASE(512, 4)
-    VKOP_ROWS_CASE(1024, 1)
-    VKOP_ROWS_CASE(1024, 2)
-    VKOP_ROWS_CASE(1024, 4)
-    if constexpr (sizeof(T) == 4) {
-        VKOP_ROWS_CASE(256, 8)
-        VKOP_ROWS_CASE(512, 8)
-        VKOP_ROWS_CASE(1024, 8)
-    }
+        VKOP_ROWS_CASE(256, 1)
+        VKOP_ROWS_CASE(256, 2)
+        VKOP_ROWS_CASE(256, 4)
+        VKOP_ROWS_CASE(512, 4)
+        VKOP_ROWS_CASE(1024, 4)
+        if constexpr (sizeof(T) == 4) {
+            VKOP_ROWS_CASE(256, 8)
+            VKOP_ROWS_CASE(512, 8)
+            VKOP_ROWS_CASE(1024, 8)
+        }
     }
 #undef VKOP_ROWS_CASE
 #undef VKOP_ROWS_LAUNCH
     if (!launched_one) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
     if (int rc = launched("rows_chunk_kernel")) return rc;
-    if (c.g > 1 && (stages & 2)) {
+    if (!fused && (stages & 2)) {
         vkop::rows_merge_kernel<T, SOFTMAX><<<v.g.outer, vkop::kMergeThreads, 0, st>>>(
-            in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g * (static_cast<uint32_t>(c.nt) / 64u), w);
+            in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, static_cast<uint32_t>(c.nt), w);
         return launched("rows_merge_kernel");
     }
     return VKOP_HIP_OK;
@@ -564,6 +570,7 @@ int vkop_hip_tune(const char *name, int value) {
     if (std::strcmp(name, "rows.threads") == 0) g_rows_threads = value;
     else if (std::strcmp(name, "rows.loads") == 0) g_rows_loads = value;
     else if (std::strcmp(name, "rows.chunks") == 0) g_rows_chunks = value;
+    else if (std::strcmp(name, "rows.fused") == 0) g_rows_fused = value != 0;
     else if (std::strcmp(name, "rows.stages") == 0) {
         if (value < 1 || value > 3) return fail(VKOP_HIP_ERR_INVALID, "rows.stages must be 1, 2 or 3");
         g_rows_stages = value;
