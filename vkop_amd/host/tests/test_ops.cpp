@@ -1,0 +1,410 @@
+// Tests of the C++ operator interface, in the shape of the reference's own:
+// tests/setup.hpp:107-294 (TestCase::run_test), tests/SoftmaxTest.cpp:100-230 and
+// tests/TopkTest.cpp:40-127 -- same case lists, same seeds, expectations from
+// libtorch's CPU softmax / topk computed at test time, same comparison rules
+// (exact for integers, the three-band float tolerance), plus a stricter ulp bound
+// and cases for the fused operator.  No test framework: each check prints a line
+// and the process exits non-zero if any failed.
+//
+//   test_ops            all tests (needs an MI355X)
+//   test_ops --no-gpu   host-side logic only
+#include <torch/torch.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+
+#include "ops/OperatorFactory.hpp"
+
+using vkop::core::ITensor;
+using vkop::core::Tensor;
+namespace ops = vkop::ops;
+
+static int g_failed = 0, g_checked = 0;
+#define EXPECT(cond)                                                         \
+    do {                                                                     \
+        g_checked++;                                                         \
+        if (!(cond)) {                                                       \
+            g_failed++;                                                      \
+            std::printf("FAIL %s:%d: %s\n", __FILE__, __LINE__, #cond);     \
+        }                                                                    \
+    } while (0)
+
+static int64_t ulp_distance(float a, float b) {
+    int32_t ia, ib;
+    std::memcpy(&ia, &a, 4);
+    std::memcpy(&ib, &b, 4);
+    if (ia < 0) ia = static_cast<int32_t>(0x80000000u) - ia;
+    if (ib < 0) ib = static_cast<int32_t>(0x80000000u) - ib;
+    return std::llabs(static_cast<int64_t>(ia) - static_cast<int64_t>(ib));
+}
+
+struct TestEnv {
+    static std::shared_ptr<vkop::VulkanDevice> dev;
+    static std::shared_ptr<vkop::VulkanCommandPool> pool;
+    static void initialize() {
+        if (dev) return;
+        dev = std::make_shared<vkop::VulkanDevice>(0);
+        pool = std::make_shared<vkop::VulkanCommandPool>(dev);
+        std::printf("device: %s, %d CUs\n", dev->getDeviceName().c_str(), dev->getComputeUnits());
+    }
+};
+std::shared_ptr<vkop::VulkanDevice> TestEnv::dev;
+std::shared_ptr<vkop::VulkanCommandPool> TestEnv::pool;
+
+// float <-> kFloat32, uint16_t <-> kFloat16 bit copy, int <-> kInt (tests/setup.hpp:107-127)
+template <typename TT> void fill_from_torch(std::shared_ptr<Tensor<TT>> &tensor, const torch::Tensor &t) {
+    auto cpu = t.cpu().contiguous().flatten();
+    std::vector<TT> data(static_cast<size_t>(cpu.numel()));
+    if constexpr (std::is_same_v<TT, uint16_t>) std::memcpy(data.data(), cpu.data_ptr<at::Half>(), data.size() * 2);
+    else std::memcpy(data.data(), cpu.data_ptr<TT>(), data.size() * sizeof(TT));
+    tensor->fillToCPU(data);
+}
+
+template <typename T> struct TestCase {
+    std::string name;
+    int64_t max_ulp = 0;  // worst float distance seen (float outputs only)
+    explicit TestCase(std::string n) : name(std::move(n)) { TestEnv::initialize(); }
+    torch::TensorOptions conf() const {
+        return torch::TensorOptions().dtype(std::is_same_v<T, float> ? torch::kFloat32 : torch::kFloat16);
+    }
+
+    // create -> set device -> attributes -> upload -> record -> submit -> wait ->
+    // read back -> compare (tests/setup.hpp:129-294)
+    bool run_test(const std::vector<std::shared_ptr<ITensor>> &inputs,
+                  const std::vector<std::shared_ptr<ITensor>> &expect_outputs,
+                  const std::function<void(std::unique_ptr<ops::Operator> &)> &attribute_func = nullptr,
+                  std::unique_ptr<ops::Operator> op = nullptr) {
+        auto dev = TestEnv::dev;
+        auto pool = TestEnv::pool;
+        if (!op)
+            op = ops::create_from_type(ops::convert_opstring_to_enum(name), inputs[0]->num_dims() <= 2,
+                                       typeid(T) == typeid(uint16_t) ? 1 : 0, dev->is_support_nv_tensor_core());
+        if (!op) return false;
+        op->set_runtime_device(dev, pool);
+        if (attribute_func) attribute_func(op);
+        std::vector<std::shared_ptr<ITensor>> outputs;
+        for (const auto &e : expect_outputs) {
+            if (e->dtype() == typeid(float)) {
+                auto o = std::make_shared<Tensor<float>>(true);
+                o->resize(e->getShape());
+                outputs.push_back(o);
+            } else if (e->dtype() == typeid(uint16_t)) {
+                auto o = std::make_shared<Tensor<uint16_t>>(true);
+                o->resize(e->getShape());
+                outputs.push_back(o);
+            } else if (e->dtype() == typeid(int)) {
+                auto o = std::make_shared<Tensor<int>>(true);
+                o->resize(e->getShape());
+                outputs.push_back(o);
+            } else {
+                return false;
+            }
+        }
+        for (const auto &in : inputs) {
+            auto t = vkop::core::as_tensor<T>(in);
+            t->as_storage_buffer(dev);
+            t->copyToGPU(pool);
+        }
+        op->onExecute(inputs, outputs, 0);
+        auto cmd = op->get_record();
+        vkop::VulkanCommandBuffer::submit(dev->getComputeQueue(), {cmd->buildSubmitInfo()});
+        cmd->wait();
+        dev->wait_all_done();
+
+        auto check = [&](size_t idx, auto tag) -> bool {
+            using TT = decltype(tag);
+            auto out = vkop::core::as_tensor<TT>(outputs[idx]);
+            out->copyToCPU(pool);
+            auto exp = vkop::core::as_tensor<TT>(expect_outputs[idx]);
+            if (out->num_elements() != exp->num_elements()) return false;
+            for (int i = 0; i < out->num_elements(); i++) {
+                if constexpr (std::is_same_v<TT, int>) {
+                    if ((*out)[i] != (*exp)[i]) {
+                        std::printf("  index mismatch at %d: %d vs %d\n", i, (*out)[i], (*exp)[i]);
+                        return false;
+                    }
+                } else {
+                    const bool half = std::is_same_v<TT, uint16_t>;
+                    float o, e;
+                    if constexpr (std::is_same_v<TT, uint16_t>) {
+                        o = ITensor::fp16_to_fp32((*out)[i]);
+                        e = ITensor::fp16_to_fp32((*exp)[i]);
+                    } else {
+                        o = (*out)[i];
+                        e = (*exp)[i];
+                    }
+                    if (std::isnan(e) || std::isnan(o)) return false;
+                    const float a = std::fabs(e);
+                    float thr;  // the reference's bands (tests/setup.hpp:219-262)
+                    if (half) thr = a > 1.0f ? a * 0.02f : 0.02f;
+                    else thr = a > 1.0f ? a * 0.01f : (a > 0.001f ? std::max(0.003f, a * 0.02f) : 0.002f);
+                    if (std::fabs(o - e) > thr) {
+                        std::printf("  value mismatch at %d: %g vs %g\n", i, o, e);
+                        return false;
+                    }
+                    if (!half) max_ulp = std::max(max_ulp, ulp_distance(o, e));
+                    else if ((*out)[i] != (*exp)[i]) max_ulp = std::max<int64_t>(max_ulp, std::abs(int((*out)[i]) - int((*exp)[i])));
+                }
+            }
+            return true;
+        };
+        for (size_t idx = 0; idx < outputs.size(); idx++) {
+            bool ok = false;
+            if (outputs[idx]->dtype() == typeid(float)) ok = check(idx, float{});
+            else if (outputs[idx]->dtype() == typeid(uint16_t)) ok = check(idx, uint16_t{});
+            else if (outputs[idx]->dtype() == typeid(int)) ok = check(idx, int{});
+            if (!ok) return false;
+        }
+        return true;
+    }
+};
+
+static torch::Tensor randn_shape(const std::vector<int> &s, const torch::TensorOptions &o) {
+    std::vector<int64_t> dims(s.begin(), s.end());
+    return torch::randn(dims, o);
+}
+static std::vector<int> shape_of(const torch::Tensor &t) {
+    std::vector<int> s;
+    for (int64_t i = 0; i < t.dim(); i++) s.push_back(static_cast<int>(t.size(i)));
+    return s;
+}
+
+// tests/SoftmaxTest.cpp:100-230: seed 42, randn, torch::softmax along `dim`
+template <typename T> void softmax_case(const std::vector<int> &shape, int axis) {
+    TestCase<T> tc("Softmax");
+    torch::manual_seed(42);
+    auto x = randn_shape(shape, tc.conf());
+    auto y = torch::softmax(x, axis < 0 ? axis + x.dim() : axis);
+    auto input = std::make_shared<Tensor<T>>(shape);
+    fill_from_torch(input, x);
+    auto expect = std::make_shared<Tensor<T>>(shape_of(y));
+    fill_from_torch(expect, y);
+    const std::unordered_map<std::string, std::string> dim = {{"dim", std::to_string(axis)}};
+    const bool ok = tc.run_test({input}, {expect}, [&](std::unique_ptr<ops::Operator> &op) {
+        auto *sm = dynamic_cast<ops::Softmax *>(op.get());
+        EXPECT(sm != nullptr);
+        if (sm) sm->setAttribute(dim);
+    });
+    std::printf("Softmax %s shape [", std::is_same_v<T, float> ? "fp32" : "fp16");
+    for (int d : shape) std::printf("%d,", d);
+    std::printf("] axis %d: %s, worst distance %lld %s\n", axis, ok ? "ok" : "FAILED", static_cast<long long>(tc.max_ulp),
+                std::is_same_v<T, float> ? "ulp vs libtorch" : "half steps vs libtorch");
+    EXPECT(ok);
+    // libtorch itself is a few ulp from the correctly rounded value on these lines
+    EXPECT(tc.max_ulp <= (std::is_same_v<T, float> ? 4 : 1));
+}
+
+// tests/TopkTest.cpp:40-127: seed 56, randn [r,c], torch::topk(k, axis, largest, sorted)
+template <typename T> void topk_case(const std::vector<int> &shape, int k, int axis) {
+    TestCase<T> tc("TopK");
+    torch::manual_seed(56);
+    auto x = randn_shape(shape, tc.conf());
+    auto [v, i64] = torch::topk(x, k, axis, true, true);
+    auto i32 = i64.to(torch::kInt);
+    auto input = std::make_shared<Tensor<T>>(shape);
+    fill_from_torch(input, x);
+    auto out_shape = shape_of(v);
+    auto ev = std::make_shared<Tensor<T>>(out_shape);
+    fill_from_torch(ev, v);
+    auto ei = std::make_shared<Tensor<int>>(out_shape);
+    fill_from_torch(ei, i32);
+    const std::unordered_map<std::string, std::string> attrs = {
+        {"k", std::to_string(k)}, {"axis", std::to_string(axis)}, {"largest", "1"}, {"sorted", "1"}};
+    // Half inputs can hold equal values, where libtorch's choice of index is its
+    // own.  With a tie among the first k+1 the expected indices come from a
+    // stable descending sort instead (equal values: lower index first); the
+    // values are the same either way.
+    auto sorted = torch::sort(x.to(torch::kFloat32), /*stable=*/true, /*dim=*/-1, /*descending=*/true);
+    const auto &sv = std::get<0>(sorted);
+    const bool ties = (sv.slice(-1, 0, k) == sv.slice(-1, 1, k + 1)).any().template item<bool>();
+    if (ties) fill_from_torch(ei, std::get<1>(sorted).slice(-1, 0, k).to(torch::kInt));
+    const bool ok = tc.run_test({input}, {ev, ei}, [&](std::unique_ptr<ops::Operator> &op) {
+        auto *tk = dynamic_cast<ops::Topk *>(op.get());
+        EXPECT(tk != nullptr);
+        if (tk) tk->setAttribute(attrs);
+    });
+    std::printf("TopK %s shape [%d,%d] k %d axis %d: %s%s\n", std::is_same_v<T, float> ? "fp32" : "fp16", shape[0], shape[1],
+                k, axis, ok ? "ok" : "FAILED", ties ? " (equal values among the first k+1: indices from a stable sort)" : "");
+    EXPECT(ok);
+    EXPECT(tc.max_ulp == 0);  // values are copies of input elements
+}
+
+// The fused operator against top-k of libtorch's softmax evaluated in float64 and
+// rounded once to the tensor type (libtorch's float32 softmax accumulates in
+// float32 and is itself tens of ulp off on 128K-long rows).  Equal probabilities:
+// lower index first, which a stable descending sort gives.
+template <typename T> void fused_case(const std::vector<int> &shape, int k) {
+    TestCase<T> tc("TopK");
+    torch::manual_seed(7);
+    auto x = randn_shape(shape, tc.conf()) * 3;
+    auto p = torch::softmax(x.to(torch::kFloat64), -1).to(tc.conf().dtype());
+    auto sorted = torch::sort(p.to(torch::kFloat32), /*stable=*/true, /*dim=*/-1, /*descending=*/true);
+    auto v = std::get<0>(sorted).slice(-1, 0, k).to(tc.conf().dtype());
+    auto i64 = std::get<1>(sorted).slice(-1, 0, k);
+    auto input = std::make_shared<Tensor<T>>(shape);
+    fill_from_torch(input, x);
+    auto ev = std::make_shared<Tensor<T>>(shape_of(v));
+    fill_from_torch(ev, v);
+    auto ei = std::make_shared<Tensor<int>>(shape_of(v));
+    fill_from_torch(ei, i64.to(torch::kInt));
+    const std::unordered_map<std::string, std::string> attrs = {{"k", std::to_string(k)}, {"axis", "-1"}};
+    const bool ok = tc.run_test({input}, {ev, ei}, [&](std::unique_ptr<ops::Operator> &op) { op->setAttribute(attrs); },
+                                std::make_unique<ops::SoftmaxTopk>(std::is_same_v<T, uint16_t> ? 1 : 0));
+    std::printf("Softmax+TopK %s shape [%d,%d] k %d: %s, worst distance %lld\n", std::is_same_v<T, float> ? "fp32" : "fp16",
+                shape[0], shape[1], k, ok ? "ok" : "FAILED", static_cast<long long>(tc.max_ulp));
+    EXPECT(ok);
+    EXPECT(tc.max_ulp <= 2);
+}
+
+static void host_logic_tests() {
+    // names and numbering (ops/Ops.hpp)
+    EXPECT(static_cast<int>(ops::OpType::SOFTMAX) == 26);
+    EXPECT(static_cast<int>(ops::OpType::TOPK) == 30);
+    EXPECT(static_cast<int>(ops::OpType::WHERE) == 40);
+    EXPECT(ops::convert_optype_to_string(ops::OpType::SOFTMAX) == "Softmax");
+    EXPECT(ops::convert_optype_to_string(ops::OpType::TOPK) == "TopK");
+    EXPECT(ops::convert_optype_to_string(ops::OpType::TOTAL_NUM) == "Unknown");
+    EXPECT(ops::convert_opstring_to_enum("Softmax") == ops::OpType::SOFTMAX);
+    EXPECT(ops::convert_opstring_to_enum("TopK") == ops::OpType::TOPK);
+    EXPECT(ops::convert_opstring_to_enum("Conv") == ops::OpType::CONV2D);
+    EXPECT(ops::convert_opstring_to_enum("BatchNormalization") == ops::OpType::BATCHNORM);
+    EXPECT(ops::convert_opstring_to_enum("topk") == ops::OpType::UNKNOWN);
+    EXPECT(ops::convert_opstring_to_enum("Unknown") == ops::OpType::UNKNOWN);
+    for (int t = 1; t < static_cast<int>(ops::OpType::TOTAL_NUM); t++) {
+        const auto ty = static_cast<ops::OpType>(t);
+        EXPECT(ops::convert_opstring_to_enum(ops::convert_optype_to_string(ty)) == ty);
+    }
+    // factory (ops/OperatorFactory.hpp:56-143)
+    const int before = ops::Operator::instance_count_.load();
+    {
+        auto sm = ops::create_from_type(ops::OpType::SOFTMAX, true);
+        auto tk = ops::create_from_type(ops::OpType::TOPK, false, 1);
+        EXPECT(sm && sm->get_type() == ops::OpType::SOFTMAX && dynamic_cast<ops::Softmax *>(sm.get()));
+        EXPECT(tk && tk->get_type() == ops::OpType::TOPK && dynamic_cast<ops::Topk *>(tk.get()));
+        EXPECT(ops::create_from_type(ops::OpType::CONV2D) == nullptr);
+        EXPECT(ops::create_from_type(ops::OpType::UNKNOWN) == nullptr);
+        EXPECT(ops::Operator::instance_count_.load() == before + 2);
+        sm->set_name("prob");
+        EXPECT(sm->get_name() == "prob");
+        EXPECT(sm->get_record() == nullptr);
+        EXPECT((sm->parse_attr_list<int>("[1,2,3]") == std::vector<int>{1, 2, 3}));
+        EXPECT(sm->parse_attr_list<float>("1,2").empty());
+        bool threw = false;
+        try {
+            sm->parse_attr_list<int>("[1,x]");
+        } catch (const std::runtime_error &) {
+            threw = true;
+        }
+        EXPECT(threw);
+        threw = false;
+        try {
+            sm->onExecute({}, {}, 0);  // no device yet
+        } catch (const std::runtime_error &) {
+            threw = true;
+        }
+        EXPECT(threw);
+    }
+    EXPECT(ops::Operator::instance_count_.load() == before);
+    // tensors (core/Tensor.hpp)
+    Tensor<float> t(std::vector<int>{3, 5});
+    EXPECT(t.num_dims() == 2 && t.size() == 60 && t.num_elements() == 15 && t.dtype() == typeid(float));
+    EXPECT((t.getShape() == std::vector<int>{3, 5}));
+    EXPECT(!t.is_on_GPU());
+    Tensor<uint16_t> h(true);
+    EXPECT(h.size() == 0 && h.is_on_GPU() && h.dtype() == typeid(uint16_t));
+    h.resize(std::vector<int>{2, 3, 4});
+    EXPECT(h.size() == 48 && h.num_dims() == 3);
+    std::shared_ptr<ITensor> it = std::make_shared<Tensor<int>>(std::vector<int>{7});
+    EXPECT(vkop::core::as_tensor<int>(it) != nullptr && vkop::core::as_tensor<float>(it) == nullptr);
+    // binary16 conversions against libtorch's, over every half and a float sweep
+    int bad = 0;
+    for (uint32_t b = 0; b < 65536; b++) {
+        const at::Half hh(static_cast<uint16_t>(b), at::Half::from_bits());
+        const float f = static_cast<float>(hh);
+        const float g = ITensor::fp16_to_fp32(static_cast<uint16_t>(b));
+        if (std::isnan(f) ? !std::isnan(g) : std::memcmp(&f, &g, 4) != 0) bad++;
+        if (!std::isnan(f) && ITensor::fp32_to_fp16(f) != b) bad++;
+    }
+    EXPECT(bad == 0);
+    bad = 0;
+    uint32_t s = 12345;
+    for (int i = 0; i < 2000000; i++) {
+        s = s * 1664525u + 1013904223u;
+        uint32_t bits = s;
+        if (i & 1) bits = (bits & 0x807FFFFFu) | ((100u + (s >> 27)) << 23);  // exponents around the half range
+        float f;
+        std::memcpy(&f, &bits, 4);
+        if (std::isnan(f)) continue;
+        if (ITensor::fp32_to_fp16(f) != at::Half(f).x) bad++;
+    }
+    EXPECT(bad == 0);
+}
+
+int main(int argc, char **argv) {
+    const bool no_gpu = argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0;
+    host_logic_tests();
+    if (!no_gpu) {
+        const std::vector<std::pair<std::vector<int>, int>> softmax_cases = {
+            {{1, 10, 7, 7}, 1}, {{1, 6, 8, 8}, 3}, {{2, 4, 10, 10}, 2}, {{1, 8, 6, 6}, 2}, {{1, 16, 5, 5}, 1}, {{4, 1000}, 1},
+        };
+        for (const auto &[shape, axis] : softmax_cases) {
+            softmax_case<float>(shape, axis);
+            softmax_case<uint16_t>(shape, axis);
+        }
+        softmax_case<float>({1000}, 0);   // a vector is one row
+        softmax_case<float>({4, 1000}, -1);
+        const std::vector<std::tuple<std::vector<int>, int, int>> topk_cases = {
+            {{1, 200}, 7, -1}, {{1, 400}, 8, -1}, {{1, 600}, 7, -1}, {{3, 2000}, 7, -1}, {{1, 2000}, 6, -1},
+        };
+        for (const auto &[shape, k, axis] : topk_cases) {
+            topk_case<float>(shape, k, axis);
+            topk_case<uint16_t>(shape, k, axis);
+        }
+        fused_case<float>({1, 1000}, 5);
+        fused_case<float>({256, 1000}, 5);
+        fused_case<float>({4, 128256}, 50);
+        fused_case<uint16_t>({64, 1000}, 5);
+        // the benchmark's arrangement: full-size outputs, the first k read back
+        {
+            TestEnv::initialize();
+            auto dev = TestEnv::dev;
+            auto pool = TestEnv::pool;
+            torch::manual_seed(3);
+            auto x = torch::randn({1, 1000}) * 3;
+            auto [v, i64] = torch::topk(torch::softmax(x, -1), 5, -1, true, true);
+            auto in = std::make_shared<Tensor<float>>(std::vector<int>{1, 1000});
+            fill_from_torch(in, x);
+            in->as_storage_buffer(dev);
+            in->copyToGPU(pool);
+            auto sf = std::make_shared<Tensor<float>>(true);
+            auto values = std::make_shared<Tensor<float>>(std::vector<int>{1, 1000}, true);
+            auto indexs = std::make_shared<Tensor<int>>(std::vector<int>{1, 1000}, true);
+            auto sm = ops::create_from_type(ops::OpType::SOFTMAX, true);
+            auto tk = ops::create_from_type(ops::OpType::TOPK, true, 0);
+            sm->set_runtime_device(dev, pool);
+            tk->set_runtime_device(dev, pool);
+            sm->setAttribute({{"axis", "-1"}});
+            tk->setAttribute({{"k", "5"}});
+            sm->onExecute({in}, {sf}, 0);
+            tk->onExecute({sf}, {values, indexs}, 0);
+            vkop::VulkanCommandBuffer::submit(dev->getComputeQueue(0),
+                                              {sm->get_record()->buildSubmitInfo(), tk->get_record()->buildSubmitInfo()});
+            tk->get_record()->wait();
+            values->copyToCPU(pool);
+            indexs->copyToCPU(pool);
+            bool ok = true;
+            auto i32 = i64.to(torch::kInt).contiguous();
+            for (int j = 0; j < 5; j++) {
+                ok = ok && (*indexs)[j] == i32.data_ptr<int>()[j];
+                ok = ok && ulp_distance((*values)[j], v.contiguous().data_ptr<float>()[j]) <= 4;
+            }
+            std::printf("Softmax then TopK into full-size outputs (benchmark arrangement): %s\n", ok ? "ok" : "FAILED");
+            EXPECT(ok);
+        }
+    }
+    std::printf("%d checks, %d failed\n", g_checked, g_failed);
+    return g_failed == 0 ? 0 : 1;
+}
