@@ -12,6 +12,7 @@
 
 #include "kernels_general.hpp"
 #include "kernels_rows.hpp"
+#include "kernels_softmax.hpp"
 
 namespace {
 
@@ -83,22 +84,140 @@ int launched(const char *what) {
 // vkop_hip_tune state
 std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0};
 
+// The per-row arrival counters of the one-kernel top-k variant sit at a fixed
+// place, the first kTicketRows words of every workspace, whatever the operator
+// and tensor: each call leaves them at zero, so a workspace cleared once can
+// serve calls of different kinds and shapes in turn.  Nothing else is ever
+// stored there.
+constexpr size_t kTicketRows = 16384;
+constexpr size_t kTicketBytes = kTicketRows * sizeof(uint32_t);  // a multiple of the workspace alignment
+
 constexpr int kLineThreads = 256;
 constexpr size_t kAlign = 256;
 inline size_t align_up(size_t b) { return (b + kAlign - 1) / kAlign * kAlign; }
 
 // ---------------------------------------------------------------- softmax ----
+// Launch shapes shared by the row kernels: threads per workgroup and 128-bit
+// loads per thread, smallest first.
+struct RowShape {
+    int nt, v;
+};
+const RowShape kShapesF32[] = {{256, 1}, {256, 2}, {256, 4}, {256, 8}, {512, 8}, {1024, 8}};
+const RowShape kShapesF16[] = {{256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}, {1024, 4}};
+
+struct SoftmaxPlan {
+    enum Kind { kGeneralLines, kGeneralStrided, kRow, kChunked, kStridedLds } kind = kGeneralLines;
+    RowShape shape{0, 0};
+    uint32_t g = 1, per = 0;
+    size_t workspace = 0;
+};
+
+SoftmaxPlan plan_softmax(const View &v, int dtype) {
+    SoftmaxPlan p;
+    const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
+    const RowShape *shapes = dtype == VKOP_HIP_F32 ? kShapesF32 : kShapesF16;
+    const uint32_t n = v.g.n, rows = v.g.outer;
+    if (v.g.inner != 1) {
+        if (n <= static_cast<uint32_t>(vkop::kStridedMaxN)) p.kind = SoftmaxPlan::kStridedLds;
+        else p.kind = n >= 2048 ? SoftmaxPlan::kGeneralLines : SoftmaxPlan::kGeneralStrided;
+        return p;
+    }
+    const uint32_t biggest = static_cast<uint32_t>(shapes[5].nt) * shapes[5].v * vec;
+    // a whole row per workgroup when rows are short or there are enough of them
+    if (n <= 8192 || (n <= biggest && rows >= 512)) {
+        for (int i = 0; i < 6; i++) {
+            if (static_cast<uint32_t>(shapes[i].nt) * shapes[i].v * vec >= n) {
+                p.kind = SoftmaxPlan::kRow;
+                p.shape = shapes[i];
+                return p;
+            }
+        }
+    }
+    // chunked: the largest chunk that still leaves >= 1024 workgroups, else the smallest
+    int pick = -1;
+    for (int i = 0; i < 6; i++) {
+        const uint32_t span = static_cast<uint32_t>(shapes[i].nt) * shapes[i].v * vec;
+        const uint32_t g = (n + span - 1) / span;
+        if (g > static_cast<uint32_t>(shapes[i].nt) || static_cast<uint64_t>(rows) * g >= (1ull << 31)) continue;
+        if (pick < 0) pick = i;
+        if (static_cast<uint64_t>(rows) * g >= 1024) pick = i;
+    }
+    if (pick < 0) return p;  // (rows of more than 2^25 elements: the general kernel)
+    p.kind = SoftmaxPlan::kChunked;
+    p.shape = shapes[pick];
+    p.per = static_cast<uint32_t>(p.shape.nt) * p.shape.v * vec;
+    p.g = (n + p.per - 1) / p.per;
+    p.workspace = kTicketBytes + align_up(static_cast<size_t>(rows) * p.g * sizeof(vkop::ChunkStat));
+    return p;
+}
+
+#define VKOP_FOR_EACH_ROW_SHAPE(X, T) \
+    X(256, 1) X(256, 2) X(256, 4) X(512, 4) X(1024, 4)                          \
+    if constexpr (sizeof(T) == 4) { X(256, 8) X(512, 8) X(1024, 8) }
+
 template <typename T>
-int softmax_impl(const T *in, T *out, const View &v, int nan_where, float nan_value, hipStream_t st) {
+int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, float nan_value, void *ws,
+                 size_t ws_bytes, hipStream_t st) {
+    const SoftmaxPlan p = plan_softmax(v, dtype);
     const uint32_t lines = v.g.outer * v.g.inner;
-    if (v.g.inner == 1 || v.g.n >= 2048) {
+    const uint32_t vec = 16 / sizeof(T);
+    const bool aligned = reinterpret_cast<uintptr_t>(in) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                         v.g.n % vec == 0;
+    switch (p.kind) {
+    case SoftmaxPlan::kRow: {
+        bool done = false;
+#define VKOP_ROW(NT, V)                                                                                        \
+    if (!done && p.shape.nt == NT && p.shape.v == V) {                                                         \
+        if (aligned) vkop::softmax_row_kernel<T, NT, V, true><<<lines, NT, 0, st>>>(in, out, v.g.n, nan_where, nan_value); \
+        else vkop::softmax_row_kernel<T, NT, V, false><<<lines, NT, 0, st>>>(in, out, v.g.n, nan_where, nan_value);        \
+        done = true;                                                                                           \
+    }
+        VKOP_FOR_EACH_ROW_SHAPE(VKOP_ROW, T)
+#undef VKOP_ROW
+        if (!done) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no softmax_row_kernel for %d x %d", p.shape.nt, p.shape.v);
+        return launched("softmax_row_kernel");
+    }
+    case SoftmaxPlan::kChunked: {
+        if (ws == nullptr || ws_bytes < p.workspace)
+            return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, p.workspace);
+        auto *stats = reinterpret_cast<vkop::ChunkStat *>(static_cast<unsigned char *>(ws) + kTicketBytes);
+        const uint32_t blocks = v.g.outer * p.g;
+        bool done = false;
+#define VKOP_CHUNKED(NT, V)                                                                                    \
+    if (!done && p.shape.nt == NT && p.shape.v == V) {                                                         \
+        if (aligned) {                                                                                         \
+            vkop::softmax_stats_kernel<T, NT, V, true><<<blocks, NT, 0, st>>>(in, stats, v.g.n, p.g, p.per);   \
+            vkop::softmax_scale_kernel<T, NT, V, true>                                                         \
+                <<<blocks, NT, 0, st>>>(in, out, stats, v.g.n, p.g, p.per, nan_where, nan_value);              \
+        } else {                                                                                               \
+            vkop::softmax_stats_kernel<T, NT, V, false><<<blocks, NT, 0, st>>>(in, stats, v.g.n, p.g, p.per);  \
+            vkop::softmax_scale_kernel<T, NT, V, false>                                                        \
+                <<<blocks, NT, 0, st>>>(in, out, stats, v.g.n, p.g, p.per, nan_where, nan_value);              \
+        }                                                                                                      \
+        done = true;                                                                                           \
+    }
+        VKOP_FOR_EACH_ROW_SHAPE(VKOP_CHUNKED, T)
+#undef VKOP_CHUNKED
+        if (!done) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no chunked softmax for %d x %d", p.shape.nt, p.shape.v);
+        return launched("softmax_stats_kernel / softmax_scale_kernel");
+    }
+    case SoftmaxPlan::kStridedLds: {
+        const uint32_t blocks = (lines + vkop::kStridedThreads - 1) / vkop::kStridedThreads;
+        const size_t lds = static_cast<size_t>(v.g.n) * vkop::kStridedThreads * sizeof(float);
+        vkop::softmax_strided_lds_kernel<T><<<blocks, vkop::kStridedThreads, lds, st>>>(in, out, v.g, nan_where, nan_value);
+        return launched("softmax_strided_lds_kernel");
+    }
+    case SoftmaxPlan::kGeneralLines:
         vkop::softmax_lines_kernel<T, kLineThreads>
             <<<lines, kLineThreads, 0, st>>>(in, out, v.g, nan_where, nan_value, nullptr);
         return launched("softmax_lines_kernel");
+    case SoftmaxPlan::kGeneralStrided:
+    default: {
+        const uint32_t blocks = (lines + kLineThreads - 1) / kLineThreads;
+        vkop::softmax_strided_kernel<T, kLineThreads><<<blocks, kLineThreads, 0, st>>>(in, out, v.g, nan_where, nan_value);
+        return launched("softmax_strided_kernel");
     }
-    const uint32_t blocks = (lines + kLineThreads - 1) / kLineThreads;
-    vkop::softmax_strided_kernel<T, kLineThreads><<<blocks, kLineThreads, 0, st>>>(in, out, v.g, nan_where, nan_value);
-    return launched("softmax_strided_kernel");
+    }
 }
 
 // ------------------------------------------------- streaming rows kernel ----
@@ -176,19 +295,14 @@ struct RowsLayout {
 
 // One layout serves the streaming kernel and the general two-kernel path, so
 // the size does not depend on which of them a call ends up taking.
-//
-// The per-row arrival counters sit at a fixed place, the first kTicketRows words
-// of every workspace, whatever the tensor: each call leaves them at zero, so a
-// workspace cleared once can serve calls of different shapes in turn.  Nothing
-// else is ever stored there.
-constexpr size_t kTicketRows = 16384;
+// (the arrival counters come first, see kTicketRows)
 
 RowsLayout rows_layout(const View &v, const RowsCfg &c) {
     RowsLayout l;
     const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
     size_t off = 0;
     l.tickets = off;
-    off += align_up(kTicketRows * sizeof(uint32_t));
+    off += kTicketBytes;
     l.stats = off;
     off += align_up(lines * sizeof(vkop::LineStats));
     if (c.ok) {
@@ -478,23 +592,21 @@ int vkop_hip_workspace_init(void *workspace, size_t bytes, void *stream) {
 size_t vkop_hip_softmax_workspace_bytes(int dtype, const int *shape, int ndim, int axis) {
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
-    return 0;
+    return plan_softmax(v, dtype).workspace;
 }
 
 int vkop_hip_softmax(const void *in, void *out, int dtype, const int *shape, int ndim, int axis, int nan_where,
                      float nan_value, void *workspace, size_t workspace_bytes, void *stream) {
-    (void)workspace;
-    (void)workspace_bytes;
     View v;
     if (int rc = check_dtype(dtype)) return rc;
     if (int rc = make_view(shape, ndim, axis, &v)) return rc;
     if (v.elems == 0) return VKOP_HIP_OK;
     if (in == nullptr || out == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
     if (dtype == VKOP_HIP_F32)
-        return softmax_impl(static_cast<const float *>(in), static_cast<float *>(out), v, nan_where, nan_value,
-                            as_stream(stream));
-    return softmax_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, nan_where, nan_value,
-                        as_stream(stream));
+        return softmax_impl(static_cast<const float *>(in), static_cast<float *>(out), v, dtype, nan_where, nan_value,
+                            workspace, workspace_bytes, as_stream(stream));
+    return softmax_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, dtype, nan_where,
+                        nan_value, workspace, workspace_bytes, as_stream(stream));
 }
 
 size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {

@@ -78,9 +78,12 @@ class Softmax : public Operator {
         const int dtype = para_.fp16 ? VKOP_HIP_F16 : VKOP_HIP_F32;
         const int nan_where = para_.nanwhere;
         const float nan_value = para_.nanvalue;
+        const size_t ws_bytes = vkop_hip_softmax_workspace_bytes(dtype, view.data(), static_cast<int>(view.size()), axis);
+        void *ws = workspace(ws_bytes);
+        const size_t ws_size = workspace_size();
         m_cmd_->record([=](void *stream) {
             return vkop_hip_softmax(in_ptr, out_ptr, dtype, view.data(), static_cast<int>(view.size()), axis, nan_where,
-                                    nan_value, nullptr, 0, stream);
+                                    nan_value, ws, ws_size, stream);
         });
     }
 
