@@ -204,6 +204,32 @@ def test_topk_workloads(ops, golden):
     assert np.array_equal(v.view(np.uint32), golden["c4_val"].view(np.uint32))
 
 
+@pytest.mark.parametrize("rows,n,k,largest,dtype", [
+    (3, 20000, 300, True, np.float32), (3, 20000, 300, False, np.float32), (2, 16385, 2048, True, np.float32),
+    (5, 40001, 256, True, np.float32), (2, 65536, 1000, True, np.float16), (3, 30003, 257, False, np.float16),
+    (1, 262144, 1, False, np.float32)])
+def test_topk_long_rows_large_k(ops, rows, n, k, largest, dtype):
+    """Rows the multi-workgroup radix select takes: k above 255 or smallest-first,
+    odd lengths (unaligned rows), half precision with its many equal values."""
+    rng = np.random.default_rng(n + k)
+    x = rng.standard_normal((rows, n)).astype(np.float32)
+    x[0, ::7] = x[0, 3]            # a run of equal values across chunks
+    x[-1, n // 2:] = np.round(x[-1, n // 2:] * 4) / 4   # a coarse grid: ties at the cut
+    x = x.astype(dtype)
+    v, ix = assert_topk_exact(ops, x, k, -1, largest)
+    check_topk_invariants(x, v, ix, k, largest=largest)
+
+
+def test_topk_long_rows_nan_inf(ops):
+    x = np.random.default_rng(5).standard_normal((2, 50000)).astype(np.float32)
+    x[0, [7, 40000]] = np.nan
+    x[0, 123] = np.inf
+    x[1, 10:20000] = -np.inf
+    x[1, 49999] = -0.0
+    assert_topk_exact(ops, x, 400)
+    assert_topk_exact(ops, x, 400, -1, False)
+
+
 # -------------------------------------------------------------------- fused --
 
 def assert_fused(ops, x, k, axis=-1, largest=True):
@@ -295,6 +321,15 @@ def test_fused_probability_collisions(ops):
     y[:, 17] = 200.0
     assert_fused(ops, y, 10)
     assert_fused(ops, y.astype(np.float16) , 10)
+
+
+@pytest.mark.parametrize("rows,n,k,dtype", [(2, 20000, 300, np.float32), (3, 70001, 1024, np.float32),
+                                             (2, 32768, 500, np.float16)])
+def test_fused_long_rows_large_k(ops, rows, n, k, dtype):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal((rows, n)) * 2).astype(np.float32)
+    x[0, 100:9000] = np.round(x[0, 100:9000])   # equal logits -> equal probabilities
+    assert_fused(ops, x.astype(dtype), k)
 
 
 def test_fused_nan_rows(ops):

@@ -25,6 +25,27 @@ struct SelectShared {
     uint32_t bucket;      // population of the chosen bucket
 };
 
+// Bitonic sort of sel[0..p2) (p2 a power of two) into descending order by all
+// NT threads of the workgroup; sel lives in LDS.  Ends with a barrier.
+template <int NT> __device__ __forceinline__ void bitonic_sort_desc(uint64_t *sel, uint32_t p2) {
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t size = 2; size <= p2; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for (uint32_t t = tid; t < (p2 >> 1); t += NT) {
+                const uint32_t i = ((t & ~(stride - 1)) << 1) | (t & (stride - 1));
+                const uint32_t j = i | stride;
+                const uint64_t a = sel[i], b = sel[j];
+                const bool desc = ((i & size) == 0);
+                if (desc ? (a < b) : (a > b)) {
+                    sel[i] = b;
+                    sel[j] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // KeyFn: uint32_t operator()(uint32_t j) -> order key of element j of the line.
 // On return sh.sel[0..k) holds the k largest composites in descending order
 // (rank order) and all threads have passed a barrier.
@@ -96,22 +117,7 @@ __device__ __forceinline__ void select_topk_line(SelectShared &sh, uint32_t n, u
     for (uint32_t t = k + tid; t < p2; t += NT) sh.sel[t] = 0;  // below every real composite
     __syncthreads();
 
-    // Bitonic sort, descending.
-    for (uint32_t size = 2; size <= p2; size <<= 1) {
-        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
-            for (uint32_t t = tid; t < (p2 >> 1); t += NT) {
-                const uint32_t i = ((t & ~(stride - 1)) << 1) | (t & (stride - 1));
-                const uint32_t j = i | stride;
-                const uint64_t a = sh.sel[i], b = sh.sel[j];
-                const bool desc = ((i & size) == 0);
-                if (desc ? (a < b) : (a > b)) {
-                    sh.sel[i] = b;
-                    sh.sel[j] = a;
-                }
-            }
-            __syncthreads();
-        }
-    }
+    bitonic_sort_desc<NT>(sh.sel, p2);
 }
 
 }  // namespace vkop

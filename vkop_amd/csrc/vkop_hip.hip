@@ -13,6 +13,7 @@
 #include "kernels_general.hpp"
 #include "kernels_rows.hpp"
 #include "kernels_softmax.hpp"
+#include "kernels_bigk.hpp"
 
 namespace {
 
@@ -291,13 +292,34 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
 
 struct RowsLayout {
     size_t tickets = 0, chunks = 0, sums = 0, cand = 0, stats = 0, total = 0;
+    // multi-workgroup radix select (kernels_bigk.hpp)
+    size_t hist = 0, hist_bytes = 0, state = 0, counts = 0, sel = 0, chunkstats = 0;
 };
+
+// Launch shape of the multi-workgroup radix select: chunks of 8192 elements.
+struct BigKCfg {
+    bool ok = false;
+    int v = 0;
+    uint32_t g = 0, per = 0, kpad = 0;
+};
+
+BigKCfg choose_bigk_cfg(const View &v, int k, int dtype) {
+    BigKCfg c;
+    if (v.g.inner != 1 || v.g.n < 16384 || k < 1 || k > vkop::kMaxK || v.g.outer == 0) return c;
+    c.v = dtype == VKOP_HIP_F32 ? 8 : 4;
+    c.per = static_cast<uint32_t>(vkop::kBigThreads) * c.v * (dtype == VKOP_HIP_F32 ? 4u : 8u);
+    c.g = (v.g.n + c.per - 1) / c.per;
+    if (c.g > static_cast<uint32_t>(vkop::kBigThreads) || static_cast<uint64_t>(v.g.outer) * c.g >= (1ull << 31)) return c;
+    c.kpad = (static_cast<uint32_t>(k) + 31u) / 32u * 32u;
+    c.ok = true;
+    return c;
+}
 
 // One layout serves the streaming kernel and the general two-kernel path, so
 // the size does not depend on which of them a call ends up taking.
 // (the arrival counters come first, see kTicketRows)
 
-RowsLayout rows_layout(const View &v, const RowsCfg &c) {
+RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKCfg{}) {
     RowsLayout l;
     const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
     size_t off = 0;
@@ -313,9 +335,62 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c) {
         off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * 2 * sizeof(uint64_t));
         l.cand = off;
         off += align_up(chunks * c.cap * sizeof(uint64_t));
+    } else if (b.ok) {
+        const size_t chunks = lines * b.g;
+        l.hist = off;
+        l.hist_bytes = align_up(3 * lines * vkop::kBigBins * sizeof(uint32_t));
+        off += l.hist_bytes;
+        l.state = off;
+        off += align_up(lines * 8 * sizeof(uint32_t));
+        l.counts = off;
+        off += align_up(chunks * 2 * sizeof(uint32_t));
+        l.sel = off;
+        off += align_up(lines * b.kpad * sizeof(uint64_t));
+        l.chunkstats = off;
+        off += align_up(chunks * sizeof(vkop::ChunkStat));
     }
     l.total = off;
     return l;
+}
+
+template <typename T, bool SOFTMAX>
+int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, const BigKCfg &c, void *ws,
+                const RowsLayout &l, hipStream_t st) {
+    auto *base = static_cast<unsigned char *>(ws);
+    vkop::BigKWorkspace w;
+    w.hist = reinterpret_cast<uint32_t *>(base + l.hist);
+    w.state = reinterpret_cast<uint32_t *>(base + l.state);
+    w.counts = reinterpret_cast<uint32_t *>(base + l.counts);
+    w.sel = reinterpret_cast<uint64_t *>(base + l.sel);
+    auto *stats = reinterpret_cast<vkop::LineStats *>(base + l.stats);
+    w.stats = stats;
+    w.kpad = c.kpad;
+    const uint32_t rows = v.g.outer, n = v.g.n, blocks = rows * c.g;
+    const uint32_t flip = largest ? 0u : 0xFFFFFFFFu;
+    const uint32_t uk = static_cast<uint32_t>(k);
+    const uint32_t vec = 16 / sizeof(T);
+    const bool aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (n % vec == 0);
+    constexpr int V = sizeof(T) == 4 ? 8 : 4;
+    constexpr int NT = vkop::kBigThreads;
+    const size_t words = l.hist_bytes / 4;
+    vkop::fill_zero_kernel<<<static_cast<unsigned>((words + 255) / 256), 256, 0, st>>>(w.hist, words);
+    auto run = [&](auto al) {
+        constexpr bool AL = decltype(al)::value;
+        if constexpr (SOFTMAX) {
+            auto *cs = reinterpret_cast<vkop::ChunkStat *>(base + l.chunkstats);
+            vkop::softmax_stats_kernel<T, NT, V, AL><<<blocks, NT, 0, st>>>(in, cs, n, c.g, c.per);
+            vkop::bigk_row_stats_kernel<<<(rows + 63) / 64, 64, 0, st>>>(cs, stats, rows, c.g);
+        }
+        vkop::bigk_hist_kernel<T, V, SOFTMAX, AL, 0><<<blocks, NT, 0, st>>>(in, n, uk, c.g, c.per, flip, w);
+        vkop::bigk_hist_kernel<T, V, SOFTMAX, AL, 1><<<blocks, NT, 0, st>>>(in, n, uk, c.g, c.per, flip, w);
+        vkop::bigk_hist_kernel<T, V, SOFTMAX, AL, 2><<<blocks, NT, 0, st>>>(in, n, uk, c.g, c.per, flip, w);
+        vkop::bigk_count_kernel<T, V, SOFTMAX, AL><<<blocks, NT, 0, st>>>(in, n, c.g, c.per, flip, w);
+        vkop::bigk_gather_kernel<T, V, SOFTMAX, AL><<<blocks, NT, 0, st>>>(in, n, uk, c.g, c.per, flip, w);
+    };
+    if (aligned) run(std::true_type{});
+    else run(std::false_type{});
+    vkop::bigk_sort_kernel<T, SOFTMAX><<<rows, vkop::kBigSortThreads, 0, st>>>(in, values, indices, n, uk, w);
+    return launched("multi-workgroup radix select");
 }
 
 template <typename T, bool SOFTMAX>
@@ -376,11 +451,15 @@ template <typename T>
 int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int dtype, void *ws,
               size_t ws_bytes, hipStream_t st) {
     const RowsCfg c = largest ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
-    if (c.ok) {
-        const RowsLayout l = rows_layout(v, c);
+    const BigKCfg b = c.ok ? BigKCfg{} : choose_bigk_cfg(v, k, dtype);
+    if (c.ok || b.ok) {
+        const RowsLayout l = rows_layout(v, c, b);
         if (ws == nullptr || ws_bytes < l.total)
             return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, l.total);
-        return launch_rows<T, false>(in, values, indices, v, k, c, ws, l, st);
+        if ((reinterpret_cast<uintptr_t>(ws) & (kAlign - 1)) != 0)
+            return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
+        if (c.ok) return launch_rows<T, false>(in, values, indices, v, k, c, ws, l, st);
+        return launch_bigk<T, false>(in, values, indices, v, k, largest, b, ws, l, st);
     }
     const uint32_t lines = v.g.outer * v.g.inner;
     vkop::topk_lines_kernel<T, kLineThreads>
@@ -389,12 +468,26 @@ int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, in
 }
 
 // ------------------------------------------------------------------ fused ----
+// Which route a fused call takes; the workspace size follows from it.
+struct FusedPlan {
+    RowsCfg rows;
+    BigKCfg big;
+};
+FusedPlan plan_fused(const View &v, int k, int dtype, int largest, bool want_probs) {
+    FusedPlan p;
+    if (want_probs) return p;  // the softmax tensor is written by the general kernels
+    if (largest) p.rows = choose_rows_cfg(v, k, dtype);
+    if (!p.rows.ok) p.big = choose_bigk_cfg(v, k, dtype);
+    return p;
+}
+
 template <typename T>
 int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, int dtype,
                void *ws, hipStream_t st) {
-    const RowsCfg c = choose_rows_cfg(v, k, dtype);
-    const RowsLayout l = rows_layout(v, c);
-    if (c.ok && largest && probs == nullptr) return launch_rows<T, true>(in, values, indices, v, k, c, ws, l, st);
+    const FusedPlan p = plan_fused(v, k, dtype, largest, probs != nullptr);
+    const RowsLayout l = rows_layout(v, p.rows, p.big);
+    if (p.rows.ok) return launch_rows<T, true>(in, values, indices, v, k, p.rows, ws, l, st);
+    if (p.big.ok) return launch_bigk<T, true>(in, values, indices, v, k, largest, p.big, ws, l, st);
     // general path: line statistics (and the softmax tensor when asked for), then
     // an exact select keyed by the probabilities those statistics define
     const uint32_t lines = v.g.outer * v.g.inner;
@@ -404,6 +497,14 @@ int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v
     vkop::softmax_topk_lines_kernel<T, kLineThreads>
         <<<lines, kLineThreads, 0, st>>>(in, stats, values, indices, v.g, static_cast<uint32_t>(k), largest);
     return launched("softmax_topk_lines_kernel");
+}
+
+// Workspace that serves whichever route a top-k or fused call on this tensor can
+// take (largest or smallest, with or without the softmax tensor).
+size_t selection_workspace(const View &v, int k, int dtype) {
+    const size_t a = rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
+    const size_t b = rows_layout(v, RowsCfg{}, choose_bigk_cfg(v, k, dtype)).total;
+    return a > b ? a : b;
 }
 
 template <typename T> int reduce_max_impl(const T *in, T *out, const View &v, hipStream_t st) {
@@ -612,8 +713,7 @@ int vkop_hip_softmax(const void *in, void *out, int dtype, const int *shape, int
 size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return 0;
-    const RowsCfg c = choose_rows_cfg(v, k, dtype);
-    return c.ok ? rows_layout(v, c).total : 0;
+    return selection_workspace(v, k, dtype);
 }
 
 int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape, int ndim,
@@ -637,7 +737,7 @@ int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dt
 size_t vkop_hip_softmax_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return 0;
-    return rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
+    return selection_workspace(v, k, dtype);
 }
 
 int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int32_t *out_indices, int dtype,
@@ -651,7 +751,8 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
     if (in == nullptr || out_values == nullptr || out_indices == nullptr)
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
-    const size_t need = rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
+    const FusedPlan plan = plan_fused(v, k, dtype, largest, out_probs != nullptr);
+    const size_t need = rows_layout(v, plan.rows, plan.big).total;
     if (workspace == nullptr || workspace_bytes < need)
         return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
