@@ -38,5 +38,6 @@ def test_reference_case_lists_through_operator_interface():
     assert r.returncode == 0
     assert " 0 failed" in r.stdout
     for needle in ("Softmax fp32 shape [4,1000,] axis 1: ok", "TopK fp16 shape [3,2000] k 7 axis -1: ok",
-                   "Softmax+TopK fp32 shape [4,128256] k 50: ok"):
+                   "Softmax+TopK fp32 shape [4,128256] k 50: ok", "Runtime post-proc [64,128256] k 50, fused: ok",
+                   "(not fusable): ok"):
         assert needle in r.stdout

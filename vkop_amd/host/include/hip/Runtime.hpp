@@ -129,11 +129,20 @@ class HipCommandBuffer {
     void *stream() const { return pool_->getDevice()->getComputeQueue(id_); }
     int queue_id() const { return id_; }
 
+    // This recording starts only after `other`'s latest submission has finished
+    // (the reference's addWait on a timeline semaphore, core/runtime.cpp:422-426).
+    void addWait(const std::shared_ptr<HipCommandBuffer> &other) {
+        if (other && other.get() != this) waits_.push_back(other);
+    }
+    void clearWaits() { waits_.clear(); }
+
     HipSubmitInfo buildSubmitInfo() { return HipSubmitInfo{this}; }
     // Enqueues every recording on `queue` in order (VulkanCommandBuffer::submit,
     // as used by core/runtime.cpp:435-441 and tests/setup.hpp:197-199).
     static void submit(void *queue, const std::vector<HipSubmitInfo> &infos) {
         for (const auto &info : infos) {
+            for (const auto &w : info.cmd->waits_)
+                if (w->submitted_) hip_check(vkop_hip_stream_wait_event(queue, w->done_), "vkop_hip_stream_wait_event");
             for (const auto &launch : info.cmd->launches_) hip_check(launch(queue), "recorded launch");
             hip_check(vkop_hip_event_record(info.cmd->done_, queue), "vkop_hip_event_record");
             info.cmd->submitted_ = true;
@@ -151,6 +160,7 @@ class HipCommandBuffer {
     bool submitted_ = false;
     void *done_ = nullptr;
     std::vector<Launch> launches_;
+    std::vector<std::shared_ptr<HipCommandBuffer>> waits_;
 };
 
 // The reference's names, so that caller code written against it still compiles.

@@ -16,6 +16,7 @@
 #include <functional>
 #include <string>
 
+#include "core/Runtime.hpp"
 #include "ops/OperatorFactory.hpp"
 
 using vkop::core::ITensor;
@@ -343,6 +344,94 @@ static void host_logic_tests() {
     EXPECT(bad == 0);
 }
 
+// The benchmark's registration sequence (benchmark/main.cpp:85-137) on synthetic
+// logits: SOFTMAX then TOPK, run repeatedly, results read back once.
+static void runtime_postprocess_tests() {
+    TestEnv::initialize();
+    auto dev = TestEnv::dev;
+    auto pool = TestEnv::pool;
+    struct Case {
+        std::vector<int> shape;
+        int k;
+    };
+    for (const Case &c : {Case{{1, 1000}, 10}, Case{{64, 128256}, 50}}) {
+        torch::manual_seed(11);
+        auto x = torch::randn({c.shape[0], c.shape[1]}) * 2.5;
+        auto p = torch::softmax(x.to(torch::kFloat64), -1).to(torch::kFloat32);
+        auto sorted = torch::sort(p, /*stable=*/true, -1, /*descending=*/true);
+        auto ev = std::get<0>(sorted).slice(-1, 0, c.k).contiguous();
+        auto ei = std::get<1>(sorted).slice(-1, 0, c.k).to(torch::kInt).contiguous();
+        std::vector<std::vector<float>> got_v(2);
+        std::vector<std::vector<int>> got_i(2);
+        for (int fuse = 0; fuse < 2; fuse++) {
+            auto rt = std::make_shared<vkop::core::Runtime>(pool, "", 0);
+            rt->set_postprocess_fusion(fuse == 1);
+            auto cls = std::make_shared<Tensor<float>>(c.shape);
+            fill_from_torch(cls, x);
+            cls->as_storage_buffer(dev);
+            cls->copyToGPU(pool);
+            rt->SetOutput(cls);
+            auto shape = vkop::core::as_tensor<float>(rt->GetOutput())->getShape();
+            auto sf = std::make_shared<Tensor<float>>(shape, true);
+            rt->RegisterPostProcess(ops::OpType::SOFTMAX, {{"axis", "-1"}}, {cls}, {sf});
+            auto indexs = std::make_shared<Tensor<int>>(shape, true);      // full-size outputs, as the benchmark passes
+            auto values = std::make_shared<Tensor<float>>(shape, true);
+            rt->RegisterPostProcess(ops::OpType::TOPK, {{"k", std::to_string(c.k)}}, {sf}, {values, indexs});
+            EXPECT(rt->num_nodes() == (fuse ? 1u : 2u));
+            EXPECT(rt->GetRealOutputs().size() == 2 && rt->GetRealOutputs().count("post_TopK0") == 1);
+            double ms = 0;
+            for (int i = 0; i < 5; i++) ms = rt->Run();
+            EXPECT(ms > 0.0);
+            rt->ReadResult();
+            const int rows = c.shape[0];
+            bool ok = true;
+            int64_t worst = 0;
+            for (int r = 0; r < rows; r++) {
+                for (int j = 0; j < c.k; j++) {
+                    const size_t o = static_cast<size_t>(r) * c.k + j;
+                    got_v[fuse].push_back((*values)[o]);
+                    got_i[fuse].push_back((*indexs)[o]);
+                    ok = ok && (*indexs)[o] == ei.data_ptr<int>()[o];
+                    worst = std::max(worst, ulp_distance((*values)[o], ev.data_ptr<float>()[o]));
+                }
+            }
+            std::printf("Runtime post-proc [%d,%d] k %d, %s: %s, worst distance %lld ulp, last Run() %.3f ms (%s)\n", c.shape[0],
+                        c.shape[1], c.k, fuse ? "fused" : "two operators", ok ? "ok" : "FAILED", static_cast<long long>(worst), ms,
+                        rt->node_name(rt->num_nodes() - 1).c_str());
+            EXPECT(ok);
+            EXPECT(worst <= 2);
+        }
+        EXPECT(got_i[0] == got_i[1]);
+        int64_t between = 0;
+        for (size_t i = 0; i < got_v[0].size(); i++) between = std::max(between, ulp_distance(got_v[0][i], got_v[1][i]));
+        EXPECT(between <= 1);
+    }
+    // no fusion when the axes differ or the TOPK reads another tensor
+    {
+        auto rt = std::make_shared<vkop::core::Runtime>(pool, "", 0);
+        auto a = std::make_shared<Tensor<float>>(std::vector<int>{8, 64});
+        torch::manual_seed(21);
+        fill_from_torch(a, torch::randn({8, 64}));
+        a->as_storage_buffer(dev);
+        a->copyToGPU(pool);
+        auto sf = std::make_shared<Tensor<float>>(std::vector<int>{8, 64}, true);
+        rt->RegisterPostProcess(ops::OpType::SOFTMAX, {{"axis", "0"}}, {a}, {sf});
+        auto v = std::make_shared<Tensor<float>>(true);
+        auto ix = std::make_shared<Tensor<int>>(true);
+        rt->RegisterPostProcess(ops::OpType::TOPK, {{"k", "3"}, {"axis", "1"}}, {sf}, {v, ix});
+        EXPECT(rt->num_nodes() == 2);
+        rt->Run();
+        rt->ReadResult();
+        EXPECT((v->getShape() == std::vector<int>{8, 3}));
+        auto want = torch::topk(torch::softmax(torch::from_blob(a->data(), {8, 64}).to(torch::kFloat64), 0).to(torch::kFloat32), 3, 1);
+        bool ok = true;
+        auto wi = std::get<1>(want).to(torch::kInt).contiguous();
+        for (int i = 0; i < 24; i++) ok = ok && (*ix)[i] == wi.data_ptr<int>()[i];
+        std::printf("Runtime post-proc softmax axis 0 then top-k axis 1 (not fusable): %s\n", ok ? "ok" : "FAILED");
+        EXPECT(ok);
+    }
+}
+
 int main(int argc, char **argv) {
     const bool no_gpu = argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0;
     host_logic_tests();
@@ -405,6 +494,7 @@ int main(int argc, char **argv) {
             EXPECT(ok);
         }
     }
+    if (!no_gpu) runtime_postprocess_tests();
     std::printf("%d checks, %d failed\n", g_checked, g_failed);
     return g_failed == 0 ? 0 : 1;
 }
