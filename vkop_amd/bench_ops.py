@@ -1,0 +1,149 @@
+#!/usr/bin/env python3
+"""Times every operator of the library on the five reference workloads.
+
+  python -m vkop_amd.bench_ops [--steps K] [--warmup W] [--only NAME_SUBSTRING]
+
+bench.py at the repository root measures the headline (fused softmax -> top-k on
+[64,128256]); this script covers the rest: plain softmax, plain top-k, the fused
+operator and the detection-style chain on all five workloads, one call in flight,
+K calls recorded once and replayed, HIP events around the replay.  Inputs rotate
+over enough device buffers (> 288 MB) that the Infinity Cache cannot serve them.
+Prints one JSON line per case: microseconds per call and the algorithmic rate
+(compulsory reads + final writes over time).
+"""
+import argparse
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--only", default="")
+    args = ap.parse_args()
+
+    import numpy as np
+    import torch
+
+    from vkop_amd import capi, synth
+
+    capi.init(0)
+    stream = capi.stream_create()
+    e0, e1 = capi.event_create(), capi.event_create()
+    F32, F16 = capi.F32, capi.F16
+
+    def buffers(x):
+        nbuf = min(64, max(2, -(-(288 << 20) // x.nbytes)))
+        return [torch.from_numpy(x).cuda() for _ in range(nbuf)]
+
+    def workspace(nbytes):
+        ws = torch.empty(nbytes + 256, dtype=torch.uint8, device="cuda")
+        ptr = ws.data_ptr() + (-ws.data_ptr()) % 256
+        capi.workspace_init(ptr, nbytes // 4 * 4, stream)
+        capi.stream_sync(stream)
+        return ws, ptr
+
+    def timed(call, nbuf):
+        def record(count, first):
+            capi.graph_begin(stream)
+            for i in range(first, first + count):
+                call(i % nbuf)
+            return capi.graph_end(stream)
+        gw = record(args.warmup, 0)
+        capi.graph_launch(gw, stream)
+        gk = record(args.steps, args.warmup)
+        capi.stream_sync(stream)
+        capi.event_record(e0, stream)
+        capi.graph_launch(gk, stream)
+        capi.event_record(e1, stream)
+        capi.event_sync(e1)
+        ms = capi.event_elapsed_ms(e0, e1)
+        capi.graph_destroy(gw)
+        capi.graph_destroy(gk)
+        return ms / args.steps * 1e3
+
+    def report(name, us, algo_bytes):
+        print(json.dumps({"case": name, "us_per_call": round(us, 2), "algorithmic_bytes": algo_bytes,
+                          "algorithmic_GBps": round(algo_bytes / us / 1e3, 1),
+                          "frac_of_8TBps": round(algo_bytes / us / 1e3 / 8000.0, 4)}), flush=True)
+
+    def softmax_case(name, x, axis):
+        if args.only not in name:
+            return
+        dt = F16 if x.dtype == np.float16 else F32
+        bufs = buffers(x.view(np.uint16) if dt == F16 else x)
+        out = torch.empty_like(bufs[0])
+        nb = capi.softmax_workspace_bytes(dt, x.shape, axis)
+        ws, ptr = workspace(nb + 256)
+        us = timed(lambda b: capi.softmax(bufs[b].data_ptr(), out.data_ptr(), dt, x.shape, axis, 0, 0.0, ptr, nb + 256,
+                                          stream), len(bufs))
+        report(name, us, 2 * x.nbytes)
+
+    def select_case(name, x, k, fused):
+        if args.only not in name:
+            return
+        dt = F16 if x.dtype == np.float16 else F32
+        bufs = buffers(x.view(np.uint16) if dt == F16 else x)
+        rows = int(np.prod(x.shape[:-1]))
+        vals = torch.empty((rows, k), dtype=bufs[0].dtype, device="cuda")
+        idx = torch.empty((rows, k), dtype=torch.int32, device="cuda")
+        nb = (capi.softmax_topk_workspace_bytes if fused else capi.topk_workspace_bytes)(dt, x.shape, -1, k)
+        ws, ptr = workspace(nb + 256)
+        if fused:
+            call = lambda b: capi.softmax_topk(bufs[b].data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), dt, x.shape, -1, k,
+                                               1, ptr, nb + 256, stream)
+        else:
+            call = lambda b: capi.topk(bufs[b].data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, x.shape, -1, k, 1, 1,
+                                       ptr, nb + 256, stream)
+        us = timed(call, len(bufs))
+        report(name, us, x.nbytes + rows * k * (x.itemsize + 4))
+
+    c1 = synth.classifier_logits(1, 1000, synth.SEEDS["C1"])
+    c2 = synth.classifier_logits(256, 1000, synth.SEEDS["C2"])
+    c2h = c2.astype(np.float16)
+    c3 = synth.llm_logits(64, 128256, synth.SEEDS["C3"])
+    c4 = synth.grid_values(8, 262144, synth.SEEDS["C4"])
+    c5 = synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"])
+
+    softmax_case("C1 softmax [1,1000] f32", c1, -1)
+    select_case("C1 topk k=5 [1,1000] f32", c1, 5, False)
+    select_case("C1 softmax+topk k=5 [1,1000] f32", c1, 5, True)
+    softmax_case("C2 softmax [256,1000] f32", c2, -1)
+    softmax_case("C2 softmax [256,1000] f16", c2h, -1)
+    select_case("C2 topk k=5 [256,1000] f32", c2, 5, False)
+    select_case("C2 softmax+topk k=5 [256,1000] f32", c2, 5, True)
+    select_case("C2 softmax+topk k=5 [256,1000] f16", c2h, 5, True)
+    softmax_case("C3 softmax [64,128256] f32", c3, -1)
+    select_case("C3 topk k=50 [64,128256] f32", c3, 50, False)
+    select_case("C3 softmax+topk k=50 [64,128256] f32", c3, 50, True)
+    softmax_case("C4 softmax [8,262144] f32", c4, -1)
+    select_case("C4 topk k=1024 [8,262144] f32 (ties)", c4, 1024, False)
+    select_case("C4 softmax+topk k=1024 [8,262144] f32", c4, 1024, True)
+    softmax_case("C5 softmax axis 1 [16,80,8400] f32", c5, 1)
+    if args.only in "C5 chain softmax axis 1 -> max -> topk k=300":
+        # the detection-style chain: softmax over classes, per-anchor class maximum, top-k anchors
+        bufs = buffers(c5)
+        p = torch.empty_like(bufs[0])
+        m = torch.empty((16, 8400), dtype=torch.float32, device="cuda")
+        vals = torch.empty((16, 300), dtype=torch.float32, device="cuda")
+        idx = torch.empty((16, 300), dtype=torch.int32, device="cuda")
+        nb = max(capi.softmax_workspace_bytes(F32, c5.shape, 1), capi.topk_workspace_bytes(F32, (16, 8400), -1, 300))
+        ws, ptr = workspace(nb + 256)
+
+        def chain(b):
+            capi.softmax(bufs[b].data_ptr(), p.data_ptr(), F32, c5.shape, 1, 0, 0.0, ptr, nb + 256, stream)
+            capi.reduce_max(p.data_ptr(), m.data_ptr(), F32, c5.shape, 1, stream)
+            capi.topk(m.data_ptr(), vals.data_ptr(), idx.data_ptr(), F32, (16, 8400), -1, 300, 1, 1, ptr, nb + 256, stream)
+        report("C5 chain softmax axis 1 -> max -> topk k=300", timed(chain, len(bufs)), c5.nbytes + 16 * 300 * 8)
+    capi.event_destroy(e0)
+    capi.event_destroy(e1)
+    capi.stream_destroy(stream)
+
+
+if __name__ == "__main__":
+    main()

@@ -333,43 +333,68 @@ __global__ __launch_bounds__(kBigThreads) void bigk_gather_kernel(const T *__res
     }
 }
 
-// One workgroup per row: sorts the k composites and writes the result.
+// Orders the k composites of a row and writes the result.  The composites are
+// distinct, so an element's place is the number of larger ones.  A workgroup
+// takes a slice of kBigSortSlice elements of one row; four threads share an
+// element, each counting over a quarter of the row's list held in LDS (all lanes
+// read the same word at a time, a broadcast).  No sorting network, no barrier
+// stages.  Launch: rows * ceil(k / kBigSortSlice) workgroups of kBigSortThreads.
+constexpr int kBigSortSlice = kBigSortThreads / 4;
+
 template <typename T, bool SOFTMAX>
 __global__ __launch_bounds__(kBigSortThreads) void bigk_sort_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                                     int32_t *__restrict__ indices, uint32_t n,
-                                                                    uint32_t k, BigKWorkspace ws) {
+                                                                    uint32_t k, uint32_t slices, BigKWorkspace ws) {
     __shared__ uint64_t sel[kMaxK];
-    const uint32_t tid = threadIdx.x, row = blockIdx.x;
+    __shared__ uint32_t rank[kBigSortSlice];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t row = blockIdx.x / slices, slice = blockIdx.x - row * slices;
     const uint64_t *src = ws.sel + static_cast<size_t>(row) * ws.kpad;
-    uint32_t p2 = 1;
-    while (p2 < k) p2 <<= 1;
-    for (uint32_t t = tid; t < p2; t += kBigSortThreads) sel[t] = t < k ? src[t] : 0ull;  // 0: below every composite
+    const uint32_t k16 = (k + 15u) & ~15u;  // four quarters of whole groups of four
+    for (uint32_t t = tid; t < k16; t += kBigSortThreads) sel[t] = t < k ? src[t] : 0ull;  // 0: below every composite
+    if (tid < kBigSortSlice) rank[tid] = 0;
     __syncthreads();
-    bitonic_sort_desc<kBigSortThreads>(sel, p2);
-    const T *rowp = in + static_cast<size_t>(row) * n;
-    LineStats st{0.f, 0.f, 0.0};
-    if constexpr (SOFTMAX) st = ws.stats[row];
-    for (uint32_t r = tid; r < k; r += kBigSortThreads) {
-        const uint32_t idx = composite_index(sel[r]);
-        if constexpr (SOFTMAX) store_elem(values, static_cast<size_t>(row) * k + r, softmax_prob(load_elem(rowp, idx), st));
-        else values[static_cast<size_t>(row) * k + r] = rowp[idx];  // bit copy
+    const uint32_t local = tid % kBigSortSlice, quarter = tid / kBigSortSlice;
+    const uint32_t t = slice * kBigSortSlice + local;
+    if (t < k) {
+        const uint64_t mine = sel[t];
+        const uint32_t q4 = k16 / 4, j0 = quarter * q4;
+        uint32_t r = 0;
+        for (uint32_t j = j0; j < j0 + q4; j += 4) {
+            const uint64_t a = sel[j], b = sel[j + 1], c = sel[j + 2], d = sel[j + 3];
+            r += (a > mine ? 1u : 0u) + (b > mine ? 1u : 0u) + (c > mine ? 1u : 0u) + (d > mine ? 1u : 0u);
+        }
+        if (r) atomicAdd(&rank[local], r);
+    }
+    __syncthreads();
+    if (quarter == 0 && t < k) {
+        const uint32_t r = rank[local];
+        const uint32_t idx = composite_index(sel[t]);
+        const T *rowp = in + static_cast<size_t>(row) * n;
+        if constexpr (SOFTMAX) {
+            const LineStats st = ws.stats[row];
+            store_elem(values, static_cast<size_t>(row) * k + r, softmax_prob(load_elem(rowp, idx), st));
+        } else {
+            values[static_cast<size_t>(row) * k + r] = rowp[idx];  // bit copy
+        }
         indices[static_cast<size_t>(row) * k + r] = static_cast<int32_t>(idx);
     }
 }
 
 // Per-row softmax statistics from the chunk statistics softmax_stats_kernel
-// leaves: one thread per row, chunks combined in index order.
-__global__ void bigk_row_stats_kernel(const ChunkStat *__restrict__ chunks, LineStats *__restrict__ stats, uint32_t rows,
-                                      uint32_t G) {
-    const uint32_t row = blockIdx.x * blockDim.x + threadIdx.x;
-    if (row >= rows) return;
+// leaves: one wave per row, fixed combination order.  Launch: rows workgroups of 64.
+__global__ __launch_bounds__(kWave) void bigk_row_stats_kernel(const ChunkStat *__restrict__ chunks,
+                                                               LineStats *__restrict__ stats, uint32_t G) {
+    const uint32_t row = blockIdx.x, lane = threadIdx.x;
     const ChunkStat *c = chunks + static_cast<size_t>(row) * G;
     float m = -INFINITY;
-    for (uint32_t g = 0; g < G; g++) m = fmaxf(m, c[g].m);
+    for (uint32_t g = lane; g < G; g += kWave) m = fmaxf(m, c[g].m);
+    m = wave_max(m);
     double s = 0.0;
-    for (uint32_t g = 0; g < G; g++)
+    for (uint32_t g = lane; g < G; g += kWave)
         if (c[g].s != 0.0) s += c[g].s * exp(static_cast<double>(c[g].ref) - static_cast<double>(m));
-    stats[row] = LineStats{m, 0.f, 1.0 / s};
+    s = wave_sum(s);
+    if (lane == 0) stats[row] = LineStats{m, 0.f, 1.0 / s};
 }
 
 }  // namespace vkop

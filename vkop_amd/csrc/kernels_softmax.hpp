@@ -221,17 +221,17 @@ __global__ __launch_bounds__(kStridedThreads) void softmax_strided_lds_kernel(co
     const uint32_t line = blockIdx.x * NT + tid;
     const bool live = line < g.outer * g.inner;
     const size_t base = live ? g.base(line) : 0;
-    // loads in batches of eight, all in flight before the first use
+    // loads in batches of sixteen, all in flight before the first use
     float m = -INFINITY;
-    for (uint32_t j0 = 0; j0 < g.n; j0 += 8) {
-        float x[8];
+    for (uint32_t j0 = 0; j0 < g.n; j0 += 16) {
+        float x[16];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < 16; u++) {
             const uint32_t j = j0 + u < g.n ? j0 + u : 0u;
             x[u] = load_elem(in, base + static_cast<size_t>(j) * g.inner);
         }
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
+        for (int u = 0; u < 16; u++) {
             if (j0 + u < g.n) {
                 stage[(j0 + u) * NT + tid] = x[u];
                 m = fmaxf(m, x[u]);

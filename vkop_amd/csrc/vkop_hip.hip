@@ -379,7 +379,7 @@ int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, 
         if constexpr (SOFTMAX) {
             auto *cs = reinterpret_cast<vkop::ChunkStat *>(base + l.chunkstats);
             vkop::softmax_stats_kernel<T, NT, V, AL><<<blocks, NT, 0, st>>>(in, cs, n, c.g, c.per);
-            vkop::bigk_row_stats_kernel<<<(rows + 63) / 64, 64, 0, st>>>(cs, stats, rows, c.g);
+            vkop::bigk_row_stats_kernel<<<rows, vkop::kWave, 0, st>>>(cs, stats, c.g);
         }
         vkop::bigk_hist_kernel<T, V, SOFTMAX, AL, 0><<<blocks, NT, 0, st>>>(in, n, uk, c.g, c.per, flip, w);
         vkop::bigk_hist_kernel<T, V, SOFTMAX, AL, 1><<<blocks, NT, 0, st>>>(in, n, uk, c.g, c.per, flip, w);
@@ -389,7 +389,9 @@ int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, 
     };
     if (aligned) run(std::true_type{});
     else run(std::false_type{});
-    vkop::bigk_sort_kernel<T, SOFTMAX><<<rows, vkop::kBigSortThreads, 0, st>>>(in, values, indices, n, uk, w);
+    const uint32_t slices = (uk + vkop::kBigSortSlice - 1) / vkop::kBigSortSlice;
+    vkop::bigk_sort_kernel<T, SOFTMAX>
+        <<<rows * slices, vkop::kBigSortThreads, 0, st>>>(in, values, indices, n, uk, slices, w);
     return launched("multi-workgroup radix select");
 }
 
