@@ -137,6 +137,57 @@ __device__ __forceinline__ uint32_t block_kth_largest_floor(const uint32_t *keys
     return prefix;
 }
 
+// Block-wide max / sum with the wave step done by DPP moves (no trips through
+// LDS inside a wave: the merge is a chain of dependent steps, and each of those
+// trips is one of them).  Same contract as block_max / block_sum.
+template <int NT> __device__ __forceinline__ float block_max_fast(float v, float *scratch) {
+    constexpr int NW = NT / kWave;
+    v = wave_max_f32_uniform(v);
+    if constexpr (NW == 1) return v;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) r = fmaxf(r, scratch[w]);
+    return r;
+}
+template <int NT> __device__ __forceinline__ double block_sum_fast(double v, double *scratch) {
+    constexpr int NW = NT / kWave;
+    v = wave_sum_f64_uniform(v);
+    if constexpr (NW == 1) return v;
+    __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) scratch[threadIdx.x / kWave] = v;
+    __syncthreads();
+    double r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) r += scratch[w];  // fixed order: run-to-run stable
+    return r;
+}
+
+// exp(x) in double to a relative error below 1e-13, for rescaling partial sums
+// (x = a reference minus the row maximum, so x <= 0 in practice).
+__device__ __forceinline__ double exp_rescale(double x) {
+    if (!(x == x)) return x;
+    if (x < -745.0) return 0.0;
+    if (x > 709.0) return static_cast<double>(INFINITY);
+    const double n = rint(x * 1.4426950408889634074);
+    const double r = fma(-n, 1.9082149292705877000e-10, fma(-n, 0.693147180369123816490, x));  // ln 2 in two parts
+    double p = 1.0 / 39916800.0;
+    p = fma(p, r, 1.0 / 3628800.0);
+    p = fma(p, r, 1.0 / 362880.0);
+    p = fma(p, r, 1.0 / 40320.0);
+    p = fma(p, r, 1.0 / 5040.0);
+    p = fma(p, r, 1.0 / 720.0);
+    p = fma(p, r, 1.0 / 120.0);
+    p = fma(p, r, 1.0 / 24.0);
+    p = fma(p, r, 1.0 / 6.0);
+    p = fma(p, r, 0.5);
+    p = fma(p, r, 1.0);
+    p = fma(p, r, 1.0);
+    return ldexp(p, static_cast<int>(n));
+}
+
 // ---- memory shared between workgroups ------------------------------------------
 // Everything one workgroup writes for another to read goes through device-scope
 // atomic stores and loads (relaxed): such a store is written through to memory
@@ -333,14 +384,14 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         sh.cnt[tid] = min(c, cap);
         bad = c > cap;
     }
-    const float M = block_max<NT>(p0.m, fscratch);  // (barrier: sh.cnt and sh.ref are published)
+    const float M = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.cnt and sh.ref are published)
     double acc = 0.0;
     if (tid < waves) {
-        const double sc = exp(static_cast<double>(p0.ref) - static_cast<double>(M));
+        const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(M));
         sh.scale[tid] = sc;
         if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
     }
-    const double s_base = block_sum<NT>(acc, dscratch);  // (barrier: sh.scale is published)
+    const double s_base = block_sum_fast<NT>(acc, dscratch);  // (barrier: sh.scale is published)
 
     // ---- C. threshold: the (k+1)-th largest per-thread maximum -------------------------
     uint32_t lmk = 0;
@@ -396,8 +447,8 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                     const uint32_t key = static_cast<uint32_t>(cmp >> 32);
                     const uint32_t idx = composite_index(cmp);
                     sh.pidx[r] = idx;
-                    sh.prob[r] = ordered_to_float(key);  // the logit, for now
                     double cr = 0.0;
+                    float term = 0.f;  // the element's softmax term, exp(fl(x - M))
                     if (SOFTMAX && key != 0xFFFFFFFFu) {
                         // the chunk-kernel wave that summed this element
                         const uint32_t b = idx / per, off = idx - b * per;
@@ -405,9 +456,10 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                         const float xv = ordered_to_float(key);
                         // what the element should contribute, exp(fl(x - M)), minus what
                         // its wave added for it, exp2(fl(fl(x - ref) * log2 e)) * exp(ref - M)
-                        cr = static_cast<double>(exp_accurate(xv - M)) -
-                             static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
+                        term = softmax_term(xv, M);
+                        cr = static_cast<double>(term) - static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
                     }
+                    sh.prob[r] = term;  // scaled to a probability below
                     sh.corr[r] = cr;
                 }
             }
@@ -420,8 +472,10 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
             }
             __syncthreads();
             if constexpr (SOFTMAX) {
-                const LineStats st{M, 0.f, 1.0 / sh.total};
-                if (tid <= kk && tid < ranked) sh.prob[tid] = round_to_storage<T>(softmax_prob(sh.prob[tid], st));
+                // the formula of softmax_prob(): the float term scaled in double, rounded once
+                const double rinv = 1.0 / sh.total;
+                if (tid <= kk && tid < ranked)
+                    sh.prob[tid] = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[tid]) * rinv));
                 __syncthreads();
                 // Probabilities are non-increasing along the rank order, so equal
                 // ones are neighbours.  A tie that reaches past the k-th place
