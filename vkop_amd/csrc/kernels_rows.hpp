@@ -263,7 +263,8 @@ __device__ __forceinline__ float fast_term(float x, float m) {
 }
 
 // Exact ranking of sh.cand[0..C): sh.rank[i] = number of larger composites.
-// All NT threads call with the same C; ends with a barrier.
+// All NT threads call with the same C; sh.rank[0..C) must be zero on entry (and a
+// barrier must lie between that zeroing and the call); ends with a barrier.
 template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uint32_t C) {
     const uint32_t tid = threadIdx.x;
     if (C == 0) return;
@@ -271,10 +272,6 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
         const uint32_t parts = NT / C;                  // >= 1
         const uint32_t span = (C + parts - 1) / parts;  // entries per part
         const uint32_t part = tid / C, i = tid - part * C;
-        if (parts > 1) {
-            for (uint32_t t = tid; t < C; t += NT) sh.rank[t] = 0;
-            __syncthreads();
-        }
         if (part < parts) {
             const uint64_t mine = sh.cand[i];
             const uint32_t j0 = part * span, j1 = min(j0 + span, C);
@@ -371,6 +368,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     }
 
     // ---- B. the row's maximum and sum from the wave partials --------------------------
+    for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;  // for block_rank, barriers away
     bool bad = false;
     SumPartial p0{0.0, 0.f, -INFINITY};
     if (tid < waves) {
@@ -464,16 +462,14 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                 }
             }
             __syncthreads();
-            if (wave == 0) {
-                double c = 0.0;
-                for (uint32_t r = lane; r < ranked; r += kWave) c += sh.corr[r];
-                c = wave_sum_f64_uniform(c);  // same tree every time: run-to-run stable
-                if (lane == 0) sh.total = s_base + c;
-            }
-            __syncthreads();
+            // every wave adds up the corrections itself (same values, same tree, same
+            // result, run after run), which saves a trip through LDS and a barrier
+            double csum = 0.0;
+            for (uint32_t r = lane; r < ranked; r += kWave) csum += sh.corr[r];
+            const double total = s_base + wave_sum_f64_uniform(csum);
             if constexpr (SOFTMAX) {
                 // the formula of softmax_prob(): the float term scaled in double, rounded once
-                const double rinv = 1.0 / sh.total;
+                const double rinv = 1.0 / total;
                 if (tid <= kk && tid < ranked)
                     sh.prob[tid] = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[tid]) * rinv));
                 __syncthreads();
