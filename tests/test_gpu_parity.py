@@ -379,3 +379,106 @@ def test_workspace_too_small_is_an_error(ops):
     with pytest.raises(capi.VkopHipError) as e:
         capi.softmax_topk(x.data_ptr(), 0, v.data_ptr(), ix.data_ptr(), capi.F32, (4, 1000), -1, 5, 1, 0, 0, 0)
     assert e.value.code == capi.ERR_WORKSPACE
+
+
+# ------------------------------------------- recordings, streams, variants --
+
+def _aligned_workspace(capi, nbytes, stream):
+    buf = torch.empty(nbytes + 256, dtype=torch.uint8, device="cuda")
+    ptr = buf.data_ptr() + (-buf.data_ptr()) % 256
+    capi.workspace_init(ptr, nbytes // 4 * 4, stream)
+    capi.stream_sync(stream)
+    return buf, ptr
+
+
+def test_recording_replayed_with_new_inputs(ops):
+    """A recorded fused call is replayed several times; between replays the input
+    buffer is rewritten by ordinary eager work.  Every replay must equal the
+    eager result for the data then in the buffer."""
+    from vkop_amd import capi
+    rows, n, k = 16, 128256, 50
+    shape = (rows, n)
+    stream = capi.stream_create()
+    x = torch.empty(shape, dtype=torch.float32, device="cuda")
+    vals = torch.empty((rows, k), dtype=torch.float32, device="cuda")
+    idx = torch.empty((rows, k), dtype=torch.int32, device="cuda")
+    nb = capi.softmax_topk_workspace_bytes(capi.F32, shape, -1, k)
+    ws, ptr = _aligned_workspace(capi, nb, stream)
+    x.copy_(dev(synth.llm_logits(rows, n, 100)))
+    torch.cuda.synchronize()
+    capi.graph_begin(stream)
+    capi.softmax_topk(x.data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), capi.F32, shape, -1, k, 1, ptr, nb, stream)
+    graph = capi.graph_end(stream)
+    try:
+        for rep in range(4):
+            h = synth.llm_logits(rows, n, 100 + rep)
+            x.copy_(dev(h))          # eager work between replays
+            torch.cuda.synchronize()
+            capi.graph_launch(graph, stream)
+            capi.stream_sync(stream)
+            ev, eix = ops.softmax_topk(x, k)   # eager call, its own workspace
+            torch.cuda.synchronize()
+            assert np.array_equal(host(idx), host(eix)), rep
+            assert np.array_equal(host(vals).view(np.uint32), host(ev).view(np.uint32)), rep
+            ov, oix = oracle.softmax_topk(h, k)
+            assert np.array_equal(host(idx), oix) and ulp_diff(host(vals), ov).max() <= 2
+    finally:
+        capi.graph_destroy(graph)
+        capi.stream_destroy(stream)
+
+
+def test_calls_in_flight_on_separate_streams():
+    """Four independent calls, each on its own stream with its own workspace and
+    outputs, submitted without waiting in between (what bench.py times)."""
+    from vkop_amd import capi
+    rows, n, k = 64, 128256, 50
+    shape = (rows, n)
+    lanes = []
+    for j in range(4):
+        s = capi.stream_create()
+        h = synth.llm_logits(rows, n, 200 + j)
+        nb = capi.softmax_topk_workspace_bytes(capi.F32, shape, -1, k)
+        ws, ptr = _aligned_workspace(capi, nb, s)
+        lanes.append(dict(s=s, h=h, x=dev(h), ws=ws, ptr=ptr, nb=nb,
+                          v=torch.empty((rows, k), dtype=torch.float32, device="cuda"),
+                          i=torch.empty((rows, k), dtype=torch.int32, device="cuda")))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for ln in lanes:
+            capi.softmax_topk(ln["x"].data_ptr(), 0, ln["v"].data_ptr(), ln["i"].data_ptr(), capi.F32, shape, -1, k, 1,
+                              ln["ptr"], ln["nb"], ln["s"])
+    for ln in lanes:
+        capi.stream_sync(ln["s"])
+    for ln in lanes:
+        ov, oix = oracle.softmax_topk(ln["h"], k)
+        assert np.array_equal(host(ln["i"]), oix)
+        assert ulp_diff(host(ln["v"]), ov).max() <= 2
+        capi.stream_destroy(ln["s"])
+
+
+@pytest.mark.parametrize("shape_knobs", [(1024, 4, 8), (512, 8, 8), (256, 4, 32)])
+def test_streaming_variants_agree(ops, shape_knobs):
+    """The one-kernel variant (arrival counters) and other launch shapes give the
+    bits the default gives; the same workspace serves them in turn."""
+    from vkop_amd import capi
+    x = synth.llm_logits(64, 128256, synth.SEEDS["C3"])
+    xd = dev(x)
+    v0, i0 = ops.softmax_topk(xd, 50)
+    t0, j0 = ops.topk(xd, 50)
+    v0, i0, t0, j0 = host(v0), host(i0), host(t0), host(j0)
+    try:
+        for fused in (1, 0):
+            capi.tune("rows.fused", fused)
+            for knobs in (None, shape_knobs):
+                for name, val in zip(("rows.threads", "rows.loads", "rows.chunks"), knobs or (0, 0, 0)):
+                    capi.tune(name, val)
+                for rep in range(2):
+                    v, i = ops.softmax_topk(xd, 50)
+                    assert np.array_equal(host(i), i0), (fused, knobs, rep)
+                    assert ulp_diff(host(v), v0).max() <= 1   # another chunking sums in another order
+                    t, j = ops.topk(xd, 50)
+                    assert np.array_equal(host(j), j0) and np.array_equal(host(t).view(np.uint32), t0.view(np.uint32))
+    finally:
+        capi.tune("rows.fused", 0)
+        for name in ("rows.threads", "rows.loads", "rows.chunks"):
+            capi.tune(name, 0)
