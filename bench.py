@@ -113,6 +113,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-host", action="store_true", help="skip the host-buffer (PCIe) round-trip leg")
     ap.add_argument("--resident", action="store_true", help="reuse one input buffer (Infinity-Cache resident figure)")
     ap.add_argument("--hw-queues", type=int, default=DEFAULT_HW_QUEUES,
                     help="hardware queues this process may use (GPU_MAX_HW_QUEUES); 0 = leave the environment as it is")
@@ -324,6 +325,8 @@ def main():
     # memory, the fused call, results back to pinned memory, one call at a time on
     # one stream.  Reported beside the headline, never as it.
     try:
+        if args.no_host:
+            raise RuntimeError("skipped (--no-host)")
         ln = lanes[0]
         ts = torch.cuda.ExternalStream(ln["stream"])
         pin_in = torch.from_numpy(host_inputs[0]).pin_memory()
