@@ -247,3 +247,13 @@ def rows_plan(dtype, shape, axis, k):
 def stream_wait_event(stream, event):
     """Work enqueued on `stream` after this call waits for `event`."""
     check(lib().vkop_hip_stream_wait_event(stream, event))
+
+
+def memcpy_h2d(dst_device, src_host, nbytes, stream=0):
+    """Blocking host -> device copy ordered on `stream`."""
+    check(lib().vkop_hip_memcpy_h2d(dst_device, src_host, int(nbytes), stream))
+
+
+def memcpy_d2h(dst_host, src_device, nbytes, stream=0):
+    """Blocking device -> host copy ordered on `stream`."""
+    check(lib().vkop_hip_memcpy_d2h(dst_host, src_device, int(nbytes), stream))
