@@ -209,9 +209,9 @@ __device__ __forceinline__ void drain_stores() {
 
 struct RowsWorkspace {
     uint32_t *tickets;  // [rows]: chunks of the row that have published; 0 between calls
-    uint64_t *chunks;   // [rows][G]: candidates the chunk had (low 32 bits); above cap = it could not store them all
-    uint64_t *sums;     // [rows][G * waves per chunk][2]: the wave's sum of exp(x - ref) as double bits, then
-                        // ref (low half) and the wave's maximum (high half) as float bits
+    uint64_t *sums;     // [rows][G * waves per chunk][3]: the wave's sum of exp(x - ref) as double bits; ref (low
+                        // half) and the wave's maximum (high half) as float bits; the candidates the wave
+                        // contributed to its chunk's list (all ones: it could not stage them all)
     uint64_t *cand;     // [rows][G][cap]: composites (order key, ~index) of the elements at or above the chunk threshold
     uint32_t cap;       // candidate slots per chunk (power of two)
     uint32_t cap_shift;
@@ -228,7 +228,7 @@ template <int NT> struct ChunkShared {  // chunk phase
     uint4 stage_v[NT];     // per wave: up to 64 vectors holding an element at or above the threshold ...
     uint32_t stage_e[NT];  // ... and the index of their first element
     uint32_t wave_thr[16];
-    uint32_t thr, total, over;
+    uint32_t thr, total;
 };
 
 struct RowsShared {  // merge phase
@@ -340,7 +340,7 @@ template <> struct Vec128<uint16_t> {
 template <typename T, int NT, bool SOFTMAX>
 __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, float *fscratch, double *dscratch,
                                           const T *rowp, T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
-                                          uint32_t per, uint32_t src_nt, const uint64_t *chunks, const uint64_t *sums,
+                                          uint32_t per, uint32_t src_nt, const uint64_t *sums,
                                           const uint64_t *cand, uint32_t cap_shift) {
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
@@ -357,9 +357,18 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     // ---- A. everything the merge reads, in one round trip ---------------------------
     // (never a branch around a load: out-of-range threads re-read entry 0)
     const uint32_t wq = tid < waves ? tid : 0u;
-    const uint64_t s_bits = fetch(sums + 2 * wq);
-    const uint64_t rm_bits = fetch(sums + 2 * wq + 1);
-    const uint64_t cm = fetch(chunks + (tid < G ? tid : 0u));
+    const uint64_t s_bits = fetch(sums + 3 * wq);
+    const uint64_t rm_bits = fetch(sums + 3 * wq + 1);
+    // thread b < G adds up the candidate counts of chunk b's waves
+    // (four loads in flight at a time; a chunk workgroup has 4, 8 or 16 waves)
+    uint64_t cm = 0;
+    for (uint32_t w0 = 0; w0 < src_nw; w0 += 4) {
+        uint64_t c[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) c[u] = fetch(sums + 3 * ((tid < G ? tid : 0u) * src_nw + w0 + u) + 2);
+#pragma unroll
+        for (int u = 0; u < 4; u++) cm = (c[u] == ~0ull || cm == ~0ull) ? ~0ull : cm + c[u];
+    }
     uint64_t cv[ES];
 #pragma unroll
     for (int e = 0; e < ES; e++) {
@@ -378,9 +387,8 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         sh.ref[tid] = p0.ref;
     }
     if (tid < G) {
-        const uint32_t c = static_cast<uint32_t>(cm);
-        sh.cnt[tid] = min(c, cap);
-        bad = c > cap;
+        sh.cnt[tid] = static_cast<uint32_t>(cm < cap ? cm : cap);
+        bad = cm > cap;
     }
     const float M = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.cnt and sh.ref are published)
     double acc = 0.0;
@@ -560,10 +568,7 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
     const uint32_t want = k + 1;  // one extra: the merge needs the (k+1)-th to prove the cut
     const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
     const uint32_t went = (row * G + chunk) * NW + wave;  // this wave's slot in the row-major wave list
-    if (tid == 0) {
-        cs.total = 0;
-        cs.over = 0;
-    }
+    if (tid == 0) cs.total = 0;
 
     // ---- 1. all loads in flight -----------------------------------------------------
     Vec128<T> q[V];
@@ -742,10 +747,7 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
         }
         // room in the chunk's candidate list, reserved once per wave
         uint32_t base = 0;
-        if (lane == 0) {
-            base = atomicAdd(&cs.total, wcount);
-            if (over) cs.over = 1;
-        }
+        if (lane == 0) base = atomicAdd(&cs.total, wcount);
         base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
         uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
 #pragma unroll
@@ -756,22 +758,22 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
 
         // ---- 5. the wave's partial sum -----------------------------------------------------------
         if (lane == 0) {
-            publish(ws.sums + 2 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
-            publish(ws.sums + 2 * static_cast<size_t>(went) + 1,
+            publish(ws.sums + 3 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
+            publish(ws.sums + 3 * static_cast<size_t>(went) + 1,
                     (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
+            publish(ws.sums + 3 * static_cast<size_t>(went) + 2, over ? ~0ull : static_cast<uint64_t>(wcount));
         }
     };
     if (c1 - c0 == static_cast<uint32_t>(NT) * V * VEC) body(std::true_type{});
     else body(std::false_type{});
 
-    // ---- 6. the chunk's candidate count; the row's last chunk merges -------------------------
-    if constexpr (FUSED) drain_stores();  // (a following kernel sees everything anyway)
-    __syncthreads();  // fused: every thread's published values are visible device-wide
-    if (tid == 0) {
-        publish(ws.chunks + (row * G + chunk), cs.over ? 0xFFFFFFFFull : static_cast<uint64_t>(cs.total));
-        uint32_t last = 1;
-        if constexpr (FUSED) {
-            drain_stores();
+    // ---- 6. one-kernel variant: the row's last chunk merges ------------------------------------
+    // (otherwise the workgroup is done: the merge kernel adds up the waves' counts itself)
+    if constexpr (FUSED) {
+        drain_stores();
+        __syncthreads();  // every thread's published values are visible device-wide
+        if (tid == 0) {
+            uint32_t last = 1;
             if (G > 1) {
                 const uint32_t done = __hip_atomic_fetch_add(ws.tickets + row, 1u, __ATOMIC_RELAXED,
                                                              __HIP_MEMORY_SCOPE_AGENT);
@@ -779,15 +781,15 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
                 // ready for the next call (nobody else touches this row's counter any more)
                 if (last) __hip_atomic_store(ws.tickets + row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
+            s_last = last;
         }
-        s_last = last;
     }
     if constexpr (FUSED) {
         __syncthreads();
         if (s_last == 0u) return;
         merge_row<T, NT, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
                                   indices + static_cast<size_t>(row) * k, n, k, G, per, NT,
-                                  ws.chunks + static_cast<size_t>(row) * G, ws.sums + 2 * static_cast<size_t>(row) * G * NW,
+                                  ws.sums + 3 * static_cast<size_t>(row) * G * NW,
                                   ws.cand + (static_cast<size_t>(row) * G << ws.cap_shift), ws.cap_shift);
     } else {
         (void)values;
@@ -815,8 +817,8 @@ __global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__re
     const uint32_t row = blockIdx.x;
     merge_row<T, kMergeThreads, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, in + static_cast<size_t>(row) * n,
                                          values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k,
-                                         n, k, G, per, src_nt, ws.chunks + static_cast<size_t>(row) * G,
-                                         ws.sums + 2 * static_cast<size_t>(row) * G * (src_nt / kWave),
+                                         n, k, G, per, src_nt,
+                                         ws.sums + 3 * static_cast<size_t>(row) * G * (src_nt / kWave),
                                          ws.cand + (static_cast<size_t>(row) * G << ws.cap_shift), ws.cap_shift);
 }
 

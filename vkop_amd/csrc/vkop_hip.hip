@@ -291,7 +291,7 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
 }
 
 struct RowsLayout {
-    size_t tickets = 0, chunks = 0, sums = 0, cand = 0, stats = 0, total = 0;
+    size_t tickets = 0, sums = 0, cand = 0, stats = 0, total = 0;
     // multi-workgroup radix select (kernels_bigk.hpp)
     size_t hist = 0, hist_bytes = 0, state = 0, counts = 0, sel = 0, chunkstats = 0;
 };
@@ -329,10 +329,8 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
     off += align_up(lines * sizeof(vkop::LineStats));
     if (c.ok) {
         const size_t chunks = lines * c.g;
-        l.chunks = off;
-        off += align_up(chunks * sizeof(uint64_t));
         l.sums = off;
-        off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * 2 * sizeof(uint64_t));
+        off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * 3 * sizeof(uint64_t));
         l.cand = off;
         off += align_up(chunks * c.cap * sizeof(uint64_t));
     } else if (b.ok) {
@@ -401,7 +399,6 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
     vkop::RowsWorkspace w;
     auto *base = static_cast<unsigned char *>(ws);
     w.tickets = reinterpret_cast<uint32_t *>(base + l.tickets);
-    w.chunks = reinterpret_cast<uint64_t *>(base + l.chunks);
     w.sums = reinterpret_cast<uint64_t *>(base + l.sums);
     w.cand = reinterpret_cast<uint64_t *>(base + l.cand);
     w.cap = c.cap;
