@@ -132,6 +132,15 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
 int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape,
                         int ndim, int axis, void *stream);
 
+/* ---- Softmax along `axis` followed by the max over the same axis, without the
+ * softmax tensor: the first two steps of the detection-style post-proc
+ * (per-anchor class max of the class probabilities, example/yolo/main.cpp:60-127)
+ * in one read of the input.  out has the shape of in without `axis` and is bit
+ * for bit what vkop_hip_softmax + vkop_hip_reduce_max give. */
+size_t vkop_hip_softmax_reduce_max_workspace_bytes(int dtype, const int *shape, int ndim, int axis);
+int vkop_hip_softmax_reduce_max(const void *in, void *out, int dtype, const int *shape,
+                                int ndim, int axis, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- Tuning and measurement knobs (process-wide; no counterpart in the
  * reference, whose shaders fix their workgroup shapes at compile time).
  *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the

@@ -371,6 +371,32 @@ def test_detection_style_chain(ops, golden):
     assert reference_float_tolerance_ok(host(ops.reduce_max(ops.softmax(dev(golden["c5_in"]), 1), 1)), golden["c5_max"])
 
 
+@pytest.mark.parametrize("shape,axis,dtype", [((16, 80, 8400), 1, np.float32), ((3, 80, 1000), 1, np.float16),
+                                              ((5, 7, 9), 0, np.float32), ((4, 300), 1, np.float32),
+                                              ((2, 200, 33), 1, np.float32), ((6, 5000), -1, np.float32)])
+def test_softmax_then_max_in_one_pass(ops, shape, axis, dtype):
+    """The per-line maximum of the softmax equals, bit for bit, the max operator
+    applied to the softmax operator's output; NaN and -inf lines included."""
+    x = (np.random.default_rng(sum(shape)).standard_normal(shape) * 2 - 3).astype(np.float32)
+    xm = np.moveaxis(x, axis, -1)
+    xm[..., :] = xm  # (view)
+    flat = xm.reshape(-1, xm.shape[-1])
+    flat[0, 1] = np.nan
+    flat[1, :] = -np.inf
+    flat[2, 0] = np.inf
+    x = x.astype(dtype)
+    fused = host(ops.softmax_reduce_max(dev(x), axis))
+    chain = host(ops.reduce_max(ops.softmax(dev(x), axis), axis))
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    assert fused.shape == chain.shape
+    assert np.array_equal(np.isnan(fused), np.isnan(chain))
+    ok = ~np.isnan(chain)
+    assert np.array_equal(fused.view(bits)[ok], chain.view(bits)[ok])
+    if dtype == np.float32:
+        want = oracle.reduce_max(oracle.softmax(x, axis), axis)
+        assert ulp_diff(fused[ok], want[ok]).max() <= 2
+
+
 def test_workspace_too_small_is_an_error(ops):
     from vkop_amd import capi
     x = dev(synth.classifier_logits(4, 1000, 1))

@@ -140,6 +140,11 @@ def main():
             capi.reduce_max(p.data_ptr(), m.data_ptr(), F32, c5.shape, 1, stream)
             capi.topk(m.data_ptr(), vals.data_ptr(), idx.data_ptr(), F32, (16, 8400), -1, 300, 1, 1, ptr, nb + 256, stream)
         report("C5 chain softmax axis 1 -> max -> topk k=300", timed(chain, len(bufs)), c5.nbytes + 16 * 300 * 8)
+
+        def chain_one_pass(b):   # softmax and class maximum in one read, then the same top-k
+            capi.softmax_reduce_max(bufs[b].data_ptr(), m.data_ptr(), F32, c5.shape, 1, ptr, nb + 256, stream)
+            capi.topk(m.data_ptr(), vals.data_ptr(), idx.data_ptr(), F32, (16, 8400), -1, 300, 1, 1, ptr, nb + 256, stream)
+        report("C5 chain (softmax+max in one pass) -> topk k=300", timed(chain_one_pass, len(bufs)), c5.nbytes + 16 * 300 * 8)
     capi.event_destroy(e0)
     capi.event_destroy(e1)
     capi.stream_destroy(stream)

@@ -84,6 +84,8 @@ def lib():
         "vkop_hip_softmax_topk_workspace_bytes": (sz, [i, ip, i, i, i]),
         "vkop_hip_softmax_topk": (i, [vp, vp, vp, vp, i, ip, i, i, i, i, vp, sz, vp]),
         "vkop_hip_reduce_max": (i, [vp, vp, i, ip, i, i, vp]),
+        "vkop_hip_softmax_reduce_max_workspace_bytes": (sz, [i, ip, i, i]),
+        "vkop_hip_softmax_reduce_max": (i, [vp, vp, i, ip, i, i, vp, sz, vp]),
         "vkop_hip_tune": (i, [ctypes.c_char_p, i]),
         "vkop_hip_rows_plan": (i, [i, ip, i, i, i, ip, ip, ip]),
     }
@@ -257,3 +259,13 @@ def memcpy_h2d(dst_device, src_host, nbytes, stream=0):
 def memcpy_d2h(dst_host, src_device, nbytes, stream=0):
     """Blocking device -> host copy ordered on `stream`."""
     check(lib().vkop_hip_memcpy_d2h(dst_host, src_device, int(nbytes), stream))
+
+
+def softmax_reduce_max_workspace_bytes(dtype, shape, axis):
+    arr, nd = _shape(shape)
+    return lib().vkop_hip_softmax_reduce_max_workspace_bytes(dtype, arr, nd, axis)
+
+
+def softmax_reduce_max(inp, out, dtype, shape, axis, workspace=0, workspace_bytes=0, stream=0):
+    arr, nd = _shape(shape)
+    check(lib().vkop_hip_softmax_reduce_max(inp, out, dtype, arr, nd, axis, workspace, workspace_bytes, stream))

@@ -177,6 +177,17 @@ __global__ __launch_bounds__(NT) void softmax_topk_lines_kernel(const T *__restr
     }
 }
 
+// ---- largest softmax entry of a line from its statistics ---------------------------------
+// The line's maximum has the term exp_accurate(0) = 1, so its probability is
+// (float)(1 / S); NaN statistics (NaN or +inf in the line) give NaN, as the
+// softmax tensor itself would.
+template <typename T> __global__ void stats_to_max_kernel(const LineStats *__restrict__ stats, T *out, uint32_t lines) {
+    const uint32_t line = blockIdx.x * blockDim.x + threadIdx.x;
+    if (line >= lines) return;
+    const LineStats st = stats[line];
+    store_elem(out, line, softmax_prob(st.m, st));
+}
+
 // ---- workspace clear ---------------------------------------------------------
 __global__ void fill_zero_kernel(uint32_t *p, size_t words) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;

@@ -212,7 +212,10 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
 constexpr int kStridedThreads = 128;
 constexpr int kStridedMaxN = 128;
 
-template <typename T>
+// MAX_ONLY: instead of the softmax tensor write, per line, its largest entry --
+// the probability of the line's maximum, (float)(exp_accurate(0) / S) -- to
+// out[line]: softmax followed by a max over the same axis, in one read.
+template <typename T, bool MAX_ONLY>
 __global__ __launch_bounds__(kStridedThreads) void softmax_strided_lds_kernel(const T *in, T *out, LineGeom g,
                                                                               int nan_where, float nan_value) {
     constexpr int NT = kStridedThreads;
@@ -238,14 +241,40 @@ __global__ __launch_bounds__(kStridedThreads) void softmax_strided_lds_kernel(co
             }
         }
     }
+    // four independent exponentials in flight per thread (few waves fit beside
+    // this much LDS, so the instruction-level parallelism has to come from here);
+    // the sum itself stays in index order
     double s = 0.0;
-    for (uint32_t j = 0; j < g.n; j++) {
+    uint32_t j4 = 0;
+    for (; j4 + 4 <= g.n; j4 += 4) {
+        float e[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) e[u] = softmax_term(stage[(j4 + u) * NT + tid], m);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            stage[(j4 + u) * NT + tid] = e[u];
+            s += static_cast<double>(e[u]);
+        }
+    }
+    for (uint32_t j = j4; j < g.n; j++) {
         const float e = softmax_term(stage[j * NT + tid], m);
         stage[j * NT + tid] = e;
         s += static_cast<double>(e);
     }
     const double rinv = 1.0 / s;
     if (!live) return;
+    if constexpr (MAX_ONLY) {
+        // the largest term is exp_accurate(0) = 1 unless the line holds no finite maximum
+        float top = 0.f;
+        for (uint32_t j = 0; j < g.n; j++) {
+            const float e = stage[j * NT + tid];
+            top = (e != e) ? e : ((top != top) ? top : fmaxf(top, e));  // NaN propagates
+        }
+        float p = round_to_storage<T>(static_cast<float>(static_cast<double>(top) * rinv));
+        if (nan_where && p != p) p = nan_value;
+        store_elem(out, line, p);
+        return;
+    }
     for (uint32_t j = 0; j < g.n; j++) {
         float p = round_to_storage<T>(static_cast<float>(static_cast<double>(stage[j * NT + tid]) * rinv));
         if (nan_where && p != p) p = nan_value;

@@ -205,7 +205,7 @@ int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, f
     case SoftmaxPlan::kStridedLds: {
         const uint32_t blocks = (lines + vkop::kStridedThreads - 1) / vkop::kStridedThreads;
         const size_t lds = static_cast<size_t>(v.g.n) * vkop::kStridedThreads * sizeof(float);
-        vkop::softmax_strided_lds_kernel<T><<<blocks, vkop::kStridedThreads, lds, st>>>(in, out, v.g, nan_where, nan_value);
+        vkop::softmax_strided_lds_kernel<T, false><<<blocks, vkop::kStridedThreads, lds, st>>>(in, out, v.g, nan_where, nan_value);
         return launched("softmax_strided_lds_kernel");
     }
     case SoftmaxPlan::kGeneralLines:
@@ -461,8 +461,12 @@ int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, in
         return launch_bigk<T, false>(in, values, indices, v, k, largest, b, ws, l, st);
     }
     const uint32_t lines = v.g.outer * v.g.inner;
-    vkop::topk_lines_kernel<T, kLineThreads>
-        <<<lines, kLineThreads, 0, st>>>(in, values, indices, v.g, static_cast<uint32_t>(k), largest);
+    // one workgroup per line: a big one when the line is long and lines are few
+    if (v.g.n >= 4096 && lines <= 1024)
+        vkop::topk_lines_kernel<T, 1024><<<lines, 1024, 0, st>>>(in, values, indices, v.g, static_cast<uint32_t>(k), largest);
+    else
+        vkop::topk_lines_kernel<T, kLineThreads>
+            <<<lines, kLineThreads, 0, st>>>(in, values, indices, v.g, static_cast<uint32_t>(k), largest);
     return launched("topk_lines_kernel");
 }
 
@@ -504,6 +508,27 @@ size_t selection_workspace(const View &v, int k, int dtype) {
     const size_t a = rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
     const size_t b = rows_layout(v, RowsCfg{}, choose_bigk_cfg(v, k, dtype)).total;
     return a > b ? a : b;
+}
+
+// max over `axis` of the softmax along `axis`, without the softmax tensor
+template <typename T>
+int softmax_reduce_max_impl(const T *in, T *out, const View &v, void *ws, size_t ws_bytes, hipStream_t st) {
+    const uint32_t lines = v.g.outer * v.g.inner;
+    if (v.g.n <= static_cast<uint32_t>(vkop::kStridedMaxN)) {
+        const uint32_t blocks = (lines + vkop::kStridedThreads - 1) / vkop::kStridedThreads;
+        const size_t lds = static_cast<size_t>(v.g.n) * vkop::kStridedThreads * sizeof(float);
+        vkop::softmax_strided_lds_kernel<T, true><<<blocks, vkop::kStridedThreads, lds, st>>>(in, out, v.g, 0, 0.f);
+        return launched("softmax_strided_lds_kernel");
+    }
+    // longer lines: the line statistics, then exp_accurate(0) / S per line
+    const size_t need = kTicketBytes + align_up(static_cast<size_t>(lines) * sizeof(vkop::LineStats));
+    if (ws == nullptr || ws_bytes < need)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    auto *stats = reinterpret_cast<vkop::LineStats *>(static_cast<unsigned char *>(ws) + kTicketBytes);
+    vkop::softmax_lines_kernel<T, kLineThreads>
+        <<<lines, kLineThreads, 0, st>>>(in, static_cast<T *>(nullptr), v.g, 0, 0.f, stats);
+    vkop::stats_to_max_kernel<T><<<(lines + 255) / 256, 256, 0, st>>>(stats, out, lines);
+    return launched("softmax_lines_kernel / stats_to_max_kernel");
 }
 
 template <typename T> int reduce_max_impl(const T *in, T *out, const View &v, hipStream_t st) {
@@ -800,6 +825,28 @@ int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k, i
     if (loads != nullptr) *loads = c.ok ? c.v : 0;
     if (chunks != nullptr) *chunks = c.ok ? static_cast<int>(c.g) : 0;
     return VKOP_HIP_OK;
+}
+
+size_t vkop_hip_softmax_reduce_max_workspace_bytes(int dtype, const int *shape, int ndim, int axis) {
+    View v;
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
+    if (v.g.n <= static_cast<uint32_t>(vkop::kStridedMaxN)) return 0;
+    return kTicketBytes + align_up(static_cast<size_t>(v.g.outer) * v.g.inner * sizeof(vkop::LineStats));
+}
+
+int vkop_hip_softmax_reduce_max(const void *in, void *out, int dtype, const int *shape, int ndim, int axis,
+                                void *workspace, size_t workspace_bytes, void *stream) {
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
+    if (v.g.n == 0) return fail(VKOP_HIP_ERR_INVALID, "max over an empty axis");
+    if (in == nullptr || out == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    if (dtype == VKOP_HIP_F32)
+        return softmax_reduce_max_impl(static_cast<const float *>(in), static_cast<float *>(out), v, workspace,
+                                       workspace_bytes, as_stream(stream));
+    return softmax_reduce_max_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, workspace,
+                                   workspace_bytes, as_stream(stream));
 }
 
 }  // extern "C"

@@ -96,6 +96,18 @@ def softmax_topk(x, k, axis=-1, largest=True, return_probs=False, workspace=None
     return (values, indices, probs) if return_probs else (values, indices)
 
 
+def softmax_reduce_max(x, axis, workspace=None):
+    """max over `axis` of softmax along `axis`, in one read (bit-equal to reduce_max(softmax(x, axis), axis))."""
+    x, dt = _prep(x)
+    shape = list(x.shape)
+    del shape[axis if axis >= 0 else axis + x.dim()]
+    out = torch.empty(shape, dtype=x.dtype, device=x.device)
+    ws = workspace or _default_ws
+    ptr, size = ws.get(capi.softmax_reduce_max_workspace_bytes(dt, x.shape, axis))
+    capi.softmax_reduce_max(x.data_ptr(), out.data_ptr(), dt, x.shape, axis, ptr, size, _stream())
+    return out
+
+
 def reduce_max(x, axis):
     x, dt = _prep(x)
     shape = list(x.shape)
