@@ -508,3 +508,19 @@ def test_streaming_variants_agree(ops, shape_knobs):
         capi.tune("rows.fused", 0)
         for name in ("rows.threads", "rows.loads", "rows.chunks"):
             capi.tune(name, 0)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_fused_quantised_logits_tie_at_the_cut(ops, dtype):
+    """Logits that went through bfloat16 (8 mantissa bits) repeat a lot: equal
+    logits, hence equal probabilities, straddle the k-th place in most rows."""
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal((32, 128256)) * 1.25).astype(np.float32)
+    x = (x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)   # truncate to bfloat16 precision
+    x = np.ascontiguousarray(x.astype(dtype))
+    k = 50
+    sx = np.sort(x.astype(np.float32), axis=-1)[:, ::-1]
+    assert (sx[:, k - 1] == sx[:, k]).mean() > 0.3      # the case is really there
+    assert_fused(ops, x, k)
+    # and a short-row shape, where one workgroup owns the row
+    assert_fused(ops, np.ascontiguousarray(x[:, :1000]), 5)

@@ -211,7 +211,8 @@ struct RowsWorkspace {
     uint32_t *tickets;  // [rows]: chunks of the row that have published; 0 between calls
     uint64_t *sums;     // [rows][G * waves per chunk][3]: the wave's sum of exp(x - ref) as double bits; ref (low
                         // half) and the wave's maximum (high half) as float bits; the candidates the wave
-                        // contributed to its chunk's list (all ones: it could not stage them all)
+                        // contributed to its chunk's list (low half; all ones: it could not stage them all)
+                        // and the chunk's threshold as an order key (high half)
     uint64_t *cand;     // [rows][G][cap]: composites (order key, ~index) of the elements at or above the chunk threshold
     uint32_t cap;       // candidate slots per chunk (power of two)
     uint32_t cap_shift;
@@ -239,7 +240,10 @@ struct RowsShared {  // merge phase
     double corr[kFastMaxK + 1];
     double scale[kMergeWavesMax];  // exp(ref - M) per wave partial
     float ref[kMergeWavesMax];
-    uint32_t cnt[kMergeChunksMax];  // live candidates per chunk
+    uint32_t cnt[kMergeChunksMax];   // live candidates per chunk
+    uint32_t cthr[kMergeChunksMax];  // threshold per chunk: the chunk's elements at or above it are candidates
+    uint32_t pkey[kFastMaxK + 1];    // order key of the logit, by rank
+    uint32_t g0, xlo;                // tie at the cut: first rank of the tied group, smallest key in it
     uint32_t lane_key[1024];
     uint32_t thr;
     uint32_t count;
@@ -333,6 +337,94 @@ template <> struct Vec128<uint16_t> {
     }
 };
 
+// A probability tie across the k-th place.  Probability is monotone in the logit,
+// so the tied group is an interval of logits [x_lo, x_hi]: x_hi is the logit at
+// the group's first rank g0, x_lo is found by a 64-way search over order keys (six
+// rounds of one exponential per lane).  Elements of that interval that are not
+// among the candidates yet (below the merge threshold or their chunk's) are
+// fetched from the row, then the k - g0 members with the lowest indices take the
+// places g0 .. k-1.  Writes those places; returns g0, or all ones if the group
+// does not fit the candidate array.  All NT threads call.
+template <typename T, int NT, int ES>
+__device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&cv)[ES], const T *rowp, T *ov, int32_t *oi,
+                                               uint32_t n, uint32_t kk, uint32_t per, uint32_t G, uint32_t thr, float p_cut,
+                                               float M, double rinv) {
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    auto prob_of_key = [&](uint32_t key) {
+        return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(key), M)) * rinv));
+    };
+    if (tid < kk && sh.prob[tid] == p_cut && (tid == 0 || sh.prob[tid - 1] != p_cut)) sh.g0 = tid;
+    if (wave == 0) {
+        // invariant: probability(b) == p_cut, probability(a) < p_cut (a = 0 stands for "below everything")
+        uint64_t a = 0, b = sh.pkey[kk];
+        while (b - a > 1) {
+            const uint64_t step = (b - a + 63) / 64;
+            uint64_t probe = a + step * (lane + 1);
+            probe = probe < b ? probe : b;
+            const bool in = prob_of_key(static_cast<uint32_t>(probe)) >= p_cut;  // false ... false true ... true
+            const int f = __ffsll(static_cast<long long>(__ballot(in))) - 1;      // lane 63 probes b: f >= 0
+            const uint32_t blo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f));
+            const uint32_t alo = f > 0 ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f > 0 ? f - 1 : 0))
+                                       : static_cast<uint32_t>(a);
+            b = blo;
+            a = alo;
+        }
+        if (lane == 0) sh.xlo = static_cast<uint32_t>(b);
+    }
+    __syncthreads();
+    const uint32_t g0 = sh.g0, xlo = sh.xlo, xhi = sh.pkey[g0];
+    // Members of the group that are not in the candidate array yet: candidates this
+    // workgroup loaded but left below the merge threshold (still in registers), and
+    // elements their chunk never listed (below the chunk's threshold: those chunks
+    // are read again, which a chunk threshold far below the k-th place never needs).
+    bool added = false;
+    if (xlo < thr) {
+#pragma unroll
+        for (int e = 0; e < ES; e++) {
+            const uint32_t key = static_cast<uint32_t>(cv[e] >> 32);
+            if (key >= xlo && key < thr) {
+                const uint32_t pos = atomicAdd(&sh.count, 1u);
+                if (pos < kFastCap) sh.cand[pos] = cv[e];
+            }
+        }
+        added = true;
+    }
+    for (uint32_t b = 0; b < G; b++) {
+        const uint32_t ct = sh.cthr[b];
+        if (ct <= xlo) continue;  // (same for every thread)
+        const uint32_t c0 = min(b * per, n), c1 = min(c0 + per, n);
+        for (uint32_t j = c0 + tid; j < c1; j += NT) {
+            const uint32_t key = order_key(load_elem(rowp, j));
+            if (key >= xlo && key < ct) {
+                const uint32_t pos = atomicAdd(&sh.count, 1u);
+                if (pos < kFastCap) sh.cand[pos] = composite(key, j);
+            }
+        }
+        added = true;
+    }
+    if (added) __syncthreads();
+    const uint32_t C3 = sh.count;
+    if (C3 > kFastCap) return 0xFFFFFFFFu;
+    const uint32_t places = kk - g0;
+    for (uint32_t t = tid; t < C3; t += NT) {
+        const uint64_t mine = sh.cand[t];
+        const uint32_t key = static_cast<uint32_t>(mine >> 32);
+        if (key < xlo || key > xhi) continue;
+        const uint32_t idx = composite_index(mine);
+        uint32_t before = 0;  // members of the group with a lower index
+        for (uint32_t u = 0; u < C3; u++) {
+            const uint64_t other = sh.cand[u];
+            const uint32_t okey = static_cast<uint32_t>(other >> 32);
+            before += (okey >= xlo && okey <= xhi && composite_index(other) < idx) ? 1u : 0u;
+        }
+        if (before < places) {
+            store_elem(ov, g0 + before, p_cut);
+            oi[g0 + before] = static_cast<int32_t>(idx);
+        }
+    }
+    return g0;
+}
+
 // ---- merge of one row's chunk results (all NT threads of a workgroup) --------
 // G chunks of `per` elements, each summed and scanned by a workgroup of src_nt
 // threads; G << cap_shift <= kMergeRecsMax, G <= kMergeChunksMax,
@@ -361,13 +453,18 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     const uint64_t rm_bits = fetch(sums + 3 * wq + 1);
     // thread b < G adds up the candidate counts of chunk b's waves
     // (four loads in flight at a time; a chunk workgroup has 4, 8 or 16 waves)
-    uint64_t cm = 0;
+    uint64_t cm = 0;       // the chunk's candidates, all ones if any of its waves overflowed
+    uint32_t cthr = 0;     // the chunk's threshold
     for (uint32_t w0 = 0; w0 < src_nw; w0 += 4) {
         uint64_t c[4];
 #pragma unroll
         for (int u = 0; u < 4; u++) c[u] = fetch(sums + 3 * ((tid < G ? tid : 0u) * src_nw + w0 + u) + 2);
 #pragma unroll
-        for (int u = 0; u < 4; u++) cm = (c[u] == ~0ull || cm == ~0ull) ? ~0ull : cm + c[u];
+        for (int u = 0; u < 4; u++) {
+            const uint32_t cnt = static_cast<uint32_t>(c[u]);
+            cm = (cnt == 0xFFFFFFFFu || cm == ~0ull) ? ~0ull : cm + cnt;
+            cthr = static_cast<uint32_t>(c[u] >> 32);
+        }
     }
     uint64_t cv[ES];
 #pragma unroll
@@ -388,6 +485,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     }
     if (tid < G) {
         sh.cnt[tid] = static_cast<uint32_t>(cm < cap ? cm : cap);
+        sh.cthr[tid] = cthr;
         bad = cm > cap;
     }
     const float M = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.cnt and sh.ref are published)
@@ -422,6 +520,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     __syncthreads();
     const uint32_t thr = sh.thr;
     bool slow = sh.flag != 0u;
+    uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a probability tie across the k-th place, if there is one
     if (SOFTMAX && !(s_base > 0.0 && s_base < 1e300)) slow = true;  // NaN / inf rows, overflowed partials
     if (SOFTMAX && !(M > -INFINITY && M < INFINITY)) slow = true;
 
@@ -453,6 +552,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                     const uint32_t key = static_cast<uint32_t>(cmp >> 32);
                     const uint32_t idx = composite_index(cmp);
                     sh.pidx[r] = idx;
+                    sh.pkey[r] = key;
                     double cr = 0.0;
                     float term = 0.f;  // the element's softmax term, exp(fl(x - M))
                     if (SOFTMAX && key != 0xFFFFFFFFu) {
@@ -482,22 +582,32 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                     sh.prob[tid] = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[tid]) * rinv));
                 __syncthreads();
                 // Probabilities are non-increasing along the rank order, so equal
-                // ones are neighbours.  A tie that reaches past the k-th place
-                // cannot be settled from the candidates.
-                if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) slow = true;
+                // ones are neighbours.  A tie that reaches past the k-th place is
+                // settled by index over every element of the row with that
+                // probability, candidates or not.
+                if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
+                    const float p_cut = sh.prob[kk];
+                    if (!(p_cut > 0.f)) {
+                        slow = true;  // a tie at 0 (or NaN) takes in the underflowed tail of the row
+                    } else {
+                        tie_g0 = settle_tie<T, NT, ES>(sh, cv, rowp, ov, oi, n, kk, per, G, thr, p_cut, M, rinv);
+                        if (tie_g0 == 0xFFFFFFFFu) slow = true;  // the tied group does not fit
+                    }
+                }
             }
         }
     }
 
     if (!slow) {
-        for (uint32_t r = tid; r < kk; r += NT) {
+        const uint32_t plain = min(kk, tie_g0);  // ranks at or after tie_g0 were written by settle_tie
+        for (uint32_t r = tid; r < plain; r += NT) {
             const uint32_t idx = sh.pidx[r];
             if constexpr (SOFTMAX) {
                 const float p = sh.prob[r];
                 // final place inside a run of equal probabilities: by index
                 uint32_t lo = r, hi = r, pos = r;
                 while (lo > 0 && sh.prob[lo - 1] == p) lo--;
-                while (hi + 1 < kk && sh.prob[hi + 1] == p) hi++;
+                while (hi + 1 < plain && sh.prob[hi + 1] == p) hi++;
                 if (hi > lo) {
                     pos = lo;
                     for (uint32_t q = lo; q <= hi; q++) pos += (sh.pidx[q] < idx) ? 1u : 0u;
@@ -761,7 +871,8 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
             publish(ws.sums + 3 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
             publish(ws.sums + 3 * static_cast<size_t>(went) + 1,
                     (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
-            publish(ws.sums + 3 * static_cast<size_t>(went) + 2, over ? ~0ull : static_cast<uint64_t>(wcount));
+            publish(ws.sums + 3 * static_cast<size_t>(went) + 2,
+                    (static_cast<uint64_t>(thr) << 32) | (over ? 0xFFFFFFFFull : static_cast<uint64_t>(wcount)));
         }
     };
     if (c1 - c0 == static_cast<uint32_t>(NT) * V * VEC) body(std::true_type{});
