@@ -524,3 +524,31 @@ def test_fused_quantised_logits_tie_at_the_cut(ops, dtype):
     assert_fused(ops, x, k)
     # and a short-row shape, where one workgroup owns the row
     assert_fused(ops, np.ascontiguousarray(x[:, :1000]), 5)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_fused_ordered_and_clustered_rows(ops, dtype):
+    """Rows whose large values sit side by side (sorted rows, one hot region):
+    the lanes that hold them are few, so a bound taken from lane maxima lets far
+    too many elements through and the chunk has to find its exact threshold."""
+    rng = np.random.default_rng(123)
+    n, k = 128256, 50
+    base = (rng.standard_normal((6, n)) * 2).astype(np.float32)
+    x = base.copy()
+    x[0] = np.sort(base[0])                 # ascending: the top sits in the last chunk
+    x[1] = np.sort(base[1])[::-1]           # descending
+    x[2, 40000:43000] += 9.0                # a hot region inside one chunk
+    x[3, 8000:8200] += 12.0                 # a narrow one: more than k, fewer than a list holds
+    x[4] = np.sort(base[4])
+    x[4, ::2] = x[4, ::2][::-1]             # interleaved ascending / descending
+    x[5, 100000:100064] = 30.0              # equal values at the top, more than k of them
+    x = np.ascontiguousarray(x.astype(dtype))
+    assert_fused(ops, x, k)
+    for largest in (True, False):
+        v, ix = ops.topk(dev(x), k, -1, largest)
+        ev, eix = oracle.topk(x, k, -1, largest)
+        bits = np.uint16 if dtype == np.float16 else np.uint32
+        assert np.array_equal(host(ix), eix) and np.array_equal(host(v).view(bits), ev.view(bits))
+    # ragged chunks (row length not a multiple of the vector width) take the other code path
+    y = np.ascontiguousarray(np.sort(base[:2, :70001], axis=-1).astype(dtype))
+    assert_fused(ops, y, 64)

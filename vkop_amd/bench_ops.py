@@ -124,6 +124,8 @@ def main():
     # the same logits after a round trip through bfloat16: equal values straddle the k-th place in most rows
     c3q = np.ascontiguousarray((c3.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32))
     select_case("C3 bf16-valued softmax+topk k=50 [64,128256] f32", c3q, 50, True)
+    # every row sorted: the top of a row sits in neighbouring lanes of one chunk
+    select_case("C3 sorted-rows softmax+topk k=50 [64,128256] f32", np.ascontiguousarray(np.sort(c3, axis=-1)), 50, True)
     softmax_case("C4 softmax [8,262144] f32", c4, -1)
     select_case("C4 topk k=1024 [8,262144] f32 (ties)", c4, 1024, False)
     select_case("C4 softmax+topk k=1024 [8,262144] f32", c4, 1024, True)

@@ -229,7 +229,8 @@ template <int NT> struct ChunkShared {  // chunk phase
     uint4 stage_v[NT];     // per wave: up to 64 vectors holding an element at or above the threshold ...
     uint32_t stage_e[NT];  // ... and the index of their first element
     uint32_t wave_thr[16];
-    uint32_t thr, total;
+    uint32_t refine[32];  // element counts per bit of the exact threshold search
+    uint32_t thr, total, over;
 };
 
 struct RowsShared {  // merge phase
@@ -261,10 +262,25 @@ template <int NT> union RowsSharedUnion {
 // Fast term for the running sum: exp2((x - m) * log2 e) on the hardware
 // exponential unit.  Only ever summed; every probability that is output uses
 // exp_accurate, and the merge replaces the fast terms of the row's largest
-// elements (the ones it ranks) by accurate ones.
+// elements (the ones it ranks) by accurate ones.  Its relative error grows with
+// |x - m| (the float argument of exp2 carries an absolute rounding error of
+// about |x - m| * 2^-24), which is harmless below m, where the term shrinks
+// faster than the error grows, and not above it.
 __device__ __forceinline__ float fast_term(float x, float m) {
     return __builtin_amdgcn_exp2f((x - m) * 1.44269504088896341f);
 }
+
+// A wave sums its terms against a reference taken from the first vectors it
+// receives, so that the exponentials overlap the loads still in flight: kRefLift
+// above the maximum of those vectors.  Should a later element lie more than
+// kTermSwitch above that reference (rare on any data with a spread of a few
+// units), the wave sums again against its true maximum once everything has
+// arrived.  Either way no element is far above the reference its term was taken
+// against, the record the wave publishes names that reference, and
+// fast_term(x, reference) is what the wave added for x: the merge calls it to
+// take back the fast terms of the elements it ranks.
+constexpr float kRefLift = 2.0f;
+constexpr float kTermSwitch = 1.0f;
 
 // Exact ranking of sh.cand[0..C): sh.rank[i] = number of larger composites.
 // All NT threads call with the same C; sh.rank[0..C) must be zero on entry (and a
@@ -561,7 +577,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                         const uint32_t sp = b * src_nw + ((off / VEC) % src_nt) / kWave;
                         const float xv = ordered_to_float(key);
                         // what the element should contribute, exp(fl(x - M)), minus what
-                        // its wave added for it, exp2(fl(fl(x - ref) * log2 e)) * exp(ref - M)
+                        // its wave added for it, fast_term(x, ref) * exp(ref - M)
                         term = softmax_term(xv, M);
                         cr = static_cast<double>(term) - static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
                     }
@@ -678,7 +694,10 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
     const uint32_t want = k + 1;  // one extra: the merge needs the (k+1)-th to prove the cut
     const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
     const uint32_t went = (row * G + chunk) * NW + wave;  // this wave's slot in the row-major wave list
-    if (tid == 0) cs.total = 0;
+    if (tid == 0) {
+        cs.total = 0;
+        cs.over = 0;
+    }
 
     // ---- 1. all loads in flight -----------------------------------------------------
     Vec128<T> q[V];
@@ -735,7 +754,7 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
                     // vectors; 0 if they hold no finite element (terms are then 0, or
                     // NaN, which must survive -- never -inf - -inf)
                     const float wm0 = wave_max_f32_uniform(vm);
-                    ref = (wm0 > -INFINITY) ? wm0 : 0.f;
+                    ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
                 }
 #pragma unroll
                 for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(xv[c], ref));
@@ -801,78 +820,175 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
         }
         // -inf never becomes a candidate: a row with k+1 larger elements does not
         // need it, and any other row is left to the exact path
-        const uint32_t thr = max(thr_block, kKeyNegInf + 1u);
-        const float thr_f = ordered_to_float(thr);
+        uint32_t thr = max(thr_block, kKeyNegInf + 1u);
 
-        // ---- 4a. the wave's vectors holding an element at or above the threshold -> LDS ------
-        uint4 *stv = cs.stage_v + wave * kWave;
-        uint32_t *ste = cs.stage_e + wave * kWave;
-        uint32_t nv = 0;  // wave-uniform
+        // ---- 4. the elements at or above the threshold go to the chunk's candidate list --------
+        // Returns the wave's count, or all ones if the wave had more than 64 vectors to stage.
+        auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors) -> uint32_t {
+            const float thr_f = ordered_to_float(thr_key);
+            // 4a. the wave's vectors holding such an element -> LDS
+            uint4 *stv = cs.stage_v + wave * kWave;
+            uint32_t *ste = cs.stage_e + wave * kWave;
+            uint32_t nv = 0;  // wave-uniform
 #pragma unroll
-        for (int i = 0; i < V; i++) {
-            const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-            bool hit;
-            if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
-            else hit = vkey[i] >= thr && in_range(e0);
-            const uint64_t mask = __ballot(hit);
-            if (mask != 0ull) {
-                if (hit) {
-                    const uint32_t pos = nv + lanes_below(mask);
-                    if (pos < kWave) {
-                        stv[pos] = q[i].v;
-                        ste[pos] = e0;
+            for (int i = 0; i < V; i++) {
+                const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+                bool hit;
+                if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
+                else hit = vkey[i] >= thr_key && in_range(e0);
+                const uint64_t mask = __ballot(hit);
+                if (mask != 0ull) {
+                    if (hit) {
+                        const uint32_t pos = nv + lanes_below(mask);
+                        if (pos < kWave) {
+                            stv[pos] = q[i].v;
+                            ste[pos] = e0;
+                        }
                     }
+                    nv += static_cast<uint32_t>(__popcll(mask));
                 }
-                nv += static_cast<uint32_t>(__popcll(mask));
             }
-        }
-        const bool over = nv > kWave;
-        nv = min(nv, static_cast<uint32_t>(kWave));
-        __builtin_amdgcn_wave_barrier();  // the stage is read by other lanes of the same wave
+            const bool over = nv > kWave;
+            nv = min(nv, static_cast<uint32_t>(kWave));
+            staged_vectors = nv;
+            __builtin_amdgcn_wave_barrier();  // the stage is read by other lanes of the same wave
 
-        // ---- 4b. one element per lane: keep those at or above the threshold ------------------
-        uint64_t mine[PASSES];
-        uint32_t mpos[PASSES];
-        uint32_t wcount = 0;  // wave-uniform
+            // 4b. one element per lane: keep those at or above the threshold
+            uint64_t mine[PASSES];
+            uint32_t mpos[PASSES];
+            uint32_t wcount = 0;  // wave-uniform
 #pragma unroll
-        for (int p = 0; p < PASSES; p++) {
-            mine[p] = 0;  // 0 = nothing to write
-            mpos[p] = 0;
-            if (static_cast<uint32_t>(p) * VPP < nv) {
-                const uint32_t sv = static_cast<uint32_t>(p) * VPP + lane / VEC;
-                const bool live = sv < nv;
-                Vec128<T> r;
-                r.v = stv[live ? sv : 0u];
-                const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
-                const float x = r.get(static_cast<int>(lane % VEC));
-                const uint32_t key = order_key(x);
-                const bool pass = live && idx < c1 && key >= thr;
-                const uint64_t mask = __ballot(pass);
-                if (pass) {
-                    mine[p] = composite(key, idx);
-                    mpos[p] = wcount + lanes_below(mask);
+            for (int p = 0; p < PASSES; p++) {
+                mine[p] = 0;  // 0 = nothing to write
+                mpos[p] = 0;
+                if (static_cast<uint32_t>(p) * VPP < nv) {
+                    const uint32_t sv = static_cast<uint32_t>(p) * VPP + lane / VEC;
+                    const bool live = sv < nv;
+                    Vec128<T> r;
+                    r.v = stv[live ? sv : 0u];
+                    const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
+                    const float x = r.get(static_cast<int>(lane % VEC));
+                    const uint32_t key = order_key(x);
+                    const bool pass = live && idx < c1 && key >= thr_key;
+                    const uint64_t mask = __ballot(pass);
+                    if (pass) {
+                        mine[p] = composite(key, idx);
+                        mpos[p] = wcount + lanes_below(mask);
+                    }
+                    wcount += static_cast<uint32_t>(__popcll(mask));
                 }
-                wcount += static_cast<uint32_t>(__popcll(mask));
             }
-        }
-        // room in the chunk's candidate list, reserved once per wave
-        uint32_t base = 0;
-        if (lane == 0) base = atomicAdd(&cs.total, wcount);
-        base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
-        uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
+            // room in the chunk's candidate list, reserved once per wave
+            uint32_t base = 0;
+            if (lane == 0) {
+                base = atomicAdd(&cs.total, wcount);
+                if (over) cs.over = 1;
+            }
+            base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
+            uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
 #pragma unroll
-        for (int p = 0; p < PASSES; p++) {
-            const uint32_t pos = base + mpos[p];
-            if (mine[p] != 0 && pos < ws.cap) publish(cand_out + pos, mine[p]);
+            for (int p = 0; p < PASSES; p++) {
+                const uint32_t pos = base + mpos[p];
+                if (mine[p] != 0 && pos < ws.cap) publish(cand_out + pos, mine[p]);
+            }
+            return over ? 0xFFFFFFFFu : wcount;
+        };
+        uint32_t staged = 0;
+        uint32_t wave_candidates = compact(thr, staged);
+        __syncthreads();
+        if (cs.total > ws.cap || cs.over != 0u) {
+            // Too many: the lane maxima gave a loose bound (values in order or in
+            // clusters put many large elements into few lanes).  Take the exact
+            // (k+1)-th largest element of the chunk instead and list again; only
+            // equal values beyond the list's size can still overflow it.  The value
+            // lies between the bound just used and the chunk's maximum: a descent
+            // over the bits in which the two differ, counting over the staged
+            // elements (everything at or above the old bound is among them) or, if
+            // a wave's stage was too small, over every element held in registers.
+            const bool from_stage = cs.over == 0u;
+            const uint32_t wk = wave_max_u32(lkey);
+            if (lane == 0) cs.wave_thr[wave] = wk;
+            if (tid < 32) cs.refine[tid] = 0;
+            __syncthreads();
+            uint32_t hi = cs.wave_thr[0];
+#pragma unroll
+            for (int w = 1; w < NW; w++) hi = max(hi, cs.wave_thr[w]);
+            auto exact_threshold = [&](const uint32_t *keys, auto count_tag) -> uint32_t {
+                constexpr int NK = decltype(count_tag)::value;
+                if (thr >= hi) return thr;
+                const int d = 31 - __clz(static_cast<int>(thr ^ hi));  // highest bit in which they differ
+                uint32_t t = hi & ~((2u << d) - 1u);                    // their common prefix
+                for (int bit = d; bit >= 0; bit--) {
+                    const uint32_t trial = t | (1u << bit);
+                    uint32_t c = 0;  // wave-uniform
+#pragma unroll
+                    for (int e = 0; e < NK; e++) c += static_cast<uint32_t>(__popcll(__ballot(keys[e] >= trial)));
+                    if (lane == 0 && c) atomicAdd(&cs.refine[bit], c);
+                    __syncthreads();
+                    if (cs.refine[bit] >= want) t = trial;
+                }
+                return max(t, thr);
+            };
+            if (from_stage) {
+                const uint4 *stv = cs.stage_v + wave * kWave;
+                const uint32_t *ste = cs.stage_e + wave * kWave;
+                uint32_t keys[PASSES];
+#pragma unroll
+                for (int p = 0; p < PASSES; p++) {
+                    const uint32_t sv = static_cast<uint32_t>(p) * VPP + lane / VEC;
+                    const bool live = sv < staged;
+                    Vec128<T> r;
+                    r.v = stv[live ? sv : 0u];
+                    const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
+                    keys[p] = (live && idx < c1) ? order_key(r.get(static_cast<int>(lane % VEC))) : 0u;
+                }
+                thr = exact_threshold(keys, std::integral_constant<int, PASSES>{});
+            } else {
+                uint32_t keys[V * VEC];
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++)
+                        keys[i * VEC + c] = in_range(ALIGNED ? e0 : e0 + c) ? order_key(q[i].get(c)) : 0u;
+                }
+                thr = exact_threshold(keys, std::integral_constant<int, V * VEC>{});
+            }
+            drain_stores();  // the first attempt's stores have landed before the same slots are written again
+            __syncthreads();  // (and every wave is done with its stage)
+            if (tid == 0) {
+                cs.total = 0;
+                cs.over = 0;
+            }
+            __syncthreads();
+            wave_candidates = compact(thr, staged);
         }
 
         // ---- 5. the wave's partial sum -----------------------------------------------------------
+        if constexpr (SOFTMAX) {
+            if (wm - ref > kTermSwitch) {  // wave-uniform
+                // an element well above the reference: its fast term is poor (or has
+                // overflowed); everything is in registers, so sum again against the maximum
+                ref = (wm < INFINITY) ? wm : ref;
+                acc = 0.0;
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        const float x = in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY;
+                        acc += static_cast<double>(fast_term(x, ref));
+                    }
+                }
+                wsum = wave_sum_f64_uniform(acc);
+            }
+        }
         if (lane == 0) {
             publish(ws.sums + 3 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
             publish(ws.sums + 3 * static_cast<size_t>(went) + 1,
                     (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
             publish(ws.sums + 3 * static_cast<size_t>(went) + 2,
-                    (static_cast<uint64_t>(thr) << 32) | (over ? 0xFFFFFFFFull : static_cast<uint64_t>(wcount)));
+                    (static_cast<uint64_t>(thr) << 32) | static_cast<uint64_t>(wave_candidates));
         }
     };
     if (c1 - c0 == static_cast<uint32_t>(NT) * V * VEC) body(std::true_type{});
