@@ -22,14 +22,20 @@ def ulp_diff(a, b):
 
 
 def half_ulp_diff(a, b):
-    """Distance in binary16 ulps between two float16 (or uint16-bit) arrays."""
-    def oi(h):
+    """Distance in binary16 ulps between two float16 (or uint16-bit) arrays;
+    NaN vs NaN counts as 0, NaN vs number as a huge distance."""
+    def bits(h):
         h = np.asarray(h)
-        if h.dtype == np.float16:
-            h = h.view(np.uint16)
-        s = h.astype(np.int64)
+        return h.view(np.uint16) if h.dtype == np.float16 else h
+    def oi(h):
+        s = bits(h).astype(np.int64)
         return np.where(s & 0x8000, -(s & 0x7FFF), s)
-    return np.abs(oi(a) - oi(b))
+    def nan(h):
+        return (bits(h) & 0x7FFF) > 0x7C00
+    d = np.abs(oi(a) - oi(b))
+    an, bn = nan(a), nan(b)
+    d = np.where(an & bn, 0, d)
+    return np.where(an ^ bn, 1 << 40, d)
 
 
 def topk_brute(x, k, axis=-1, largest=True):

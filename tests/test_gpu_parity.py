@@ -552,3 +552,50 @@ def test_fused_ordered_and_clustered_rows(ops, dtype):
     # ragged chunks (row length not a multiple of the vector width) take the other code path
     y = np.ascontiguousarray(np.sort(base[:2, :70001], axis=-1).astype(dtype))
     assert_fused(ops, y, 64)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_masked_and_underflowed_rows(ops, dtype):
+    """Rows where the k-th place falls among probabilities that are exactly 0
+    (masked logits at -inf, a tail that underflows) or among -inf elements: the
+    places behind the positive probabilities go to the lowest indices."""
+    rng = np.random.default_rng(321)
+    n, k = 128256, 50
+    x = (rng.standard_normal((8, n)) * 2).astype(np.float32)
+    allowed = rng.choice(n, 20, replace=False)
+    x[0] = -np.inf
+    x[0, allowed] = rng.standard_normal(20).astype(np.float32)       # 20 allowed tokens, k = 50
+    x[1] = -np.inf
+    x[1, 77777] = 1.5                                                # a single allowed token
+    x[2, 5000] = 150.0 if dtype == np.float32 else 60.0              # everything else underflows (or nearly)
+    x[3, :] = -np.inf
+    x[3, 100:100 + k] = 0.25                                         # exactly k finite elements, all equal
+    x[4, ::3] = -np.inf                                              # a third masked: plenty left
+    x[5] = -np.inf                                                   # nothing left: NaN row
+    x[6, 1000] = np.inf                                              # NaN row
+    x[7, 64000:64100] = 120.0 if dtype == np.float32 else 50.0      # a plateau far above a tail that underflows
+    x = np.ascontiguousarray(x.astype(dtype))
+    v, ix = ops.softmax_topk(dev(x), k)
+    v, ix = host(v), host(ix)
+    ov, oix = oracle.softmax_topk(x, k)
+    assert np.array_equal(ix, oix)
+    if dtype == np.float16:
+        assert half_ulp_diff(v, ov).max() <= 1
+    else:
+        assert ulp_diff(v, ov).max() <= 2
+    # the same through the softmax tensor route
+    assert_fused(ops, x[[0, 1, 2, 3, 4, 7]], k)
+    # plain top-k: -inf elements tie by index behind the finite ones
+    for largest in (True, False):
+        y = x if largest else -x
+        y = np.ascontiguousarray(y[[0, 1, 3, 4, 5]])
+        t, j = ops.topk(dev(y), k, -1, largest)
+        et, ej = oracle.topk(y, k, -1, largest)
+        bits = np.uint16 if dtype == np.float16 else np.uint32
+        assert np.array_equal(host(j), ej) and np.array_equal(host(t).view(bits), et.view(bits))
+    # short rows, one workgroup per row
+    short = np.ascontiguousarray(x[:5, :1000])
+    short[0, allowed[:3] % 1000] = np.array([0.5, -1.0, 2.0], dtype)   # 3 allowed tokens, k = 5
+    short[1, 777] = 1.5
+    short[2, 500] = 150.0 if dtype == np.float32 else 60.0
+    assert_fused(ops, short, 5)

@@ -126,6 +126,10 @@ def main():
     select_case("C3 bf16-valued softmax+topk k=50 [64,128256] f32", c3q, 50, True)
     # every row sorted: the top of a row sits in neighbouring lanes of one chunk
     select_case("C3 sorted-rows softmax+topk k=50 [64,128256] f32", np.ascontiguousarray(np.sort(c3, axis=-1)), 50, True)
+    # constrained decoding: all but 20 logits of every row masked with -inf, fewer than k are left
+    c3m = np.full_like(c3, -np.inf)
+    c3m[:, 1000:128000:6350] = c3[:, 1000:128000:6350]
+    select_case("C3 masked-rows softmax+topk k=50 [64,128256] f32", c3m, 50, True)
     softmax_case("C4 softmax [8,262144] f32", c4, -1)
     select_case("C4 topk k=1024 [8,262144] f32 (ties)", c4, 1024, False)
     select_case("C4 softmax+topk k=1024 [8,262144] f32", c4, 1024, True)

@@ -245,6 +245,7 @@ struct RowsShared {  // merge phase
     uint32_t cthr[kMergeChunksMax];  // threshold per chunk: the chunk's elements at or above it are candidates
     uint32_t pkey[kFastMaxK + 1];    // order key of the logit, by rank
     uint32_t g0, xlo;                // tie at the cut: first rank of the tied group, smallest key in it
+    uint32_t scan_counts[2 * 16];    // fill_group_by_scan: members per wave, double-buffered
     uint32_t lane_key[1024];
     uint32_t thr;
     uint32_t count;
@@ -353,14 +354,70 @@ template <> struct Vec128<uint16_t> {
     }
 };
 
+// Places g0 .. kk-1 of a row's result go to the lowest-index elements whose order
+// key lies in [xlo, xhi] (a group of equal rank too large to collect): the row is
+// read from its start, NT * 4 elements at a time, until enough members are found
+// -- soon, for a group that large.  SOFTMAX: every member's value is tie_value (the
+// group's probability); otherwise the element itself.  counts: 2 * NT / 64 words
+// of LDS.  All NT threads call.
+template <typename T, int NT, bool SOFTMAX>
+__device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *rowp, T *ov, int32_t *oi, uint32_t n,
+                                                   uint32_t g0, uint32_t kk, uint32_t xlo, uint32_t xhi, float tie_value) {
+    constexpr int NW = NT / kWave;
+    constexpr int U = 4;
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t places = kk - g0;
+    uint32_t found = 0;  // the same in every thread
+    uint32_t round = 0;
+    for (uint32_t base = 0; base < n && found < places; base += NT * U, round++) {
+        const uint32_t j0 = base + tid * U;
+        bool member[U];
+        uint32_t below = 0, in_wave = 0;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t j = j0 + u;
+            const uint32_t key = order_key(load_elem(rowp, j < n ? j : 0u));
+            member[u] = j < n && key >= xlo && key <= xhi;
+            const uint64_t mask = __ballot(member[u]);
+            below += lanes_below(mask);
+            in_wave += static_cast<uint32_t>(__popcll(mask));
+        }
+        uint32_t *wc = counts + (round & 1u) * NW;
+        if (lane == 0) wc[wave] = in_wave;
+        __syncthreads();
+        // index order inside the tile: thread, then u
+        uint32_t pos = found + below, in_tile = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const uint32_t c = wc[w];
+            pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
+            in_tile += c;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (member[u]) {
+                if (pos < places) {
+                    if constexpr (SOFTMAX) store_elem(ov, g0 + pos, tie_value);
+                    else ov[g0 + pos] = rowp[j0 + u];
+                    oi[g0 + pos] = static_cast<int32_t>(j0 + u);
+                }
+                pos++;
+            }
+        }
+        found += in_tile;
+    }
+}
+
 // A probability tie across the k-th place.  Probability is monotone in the logit,
 // so the tied group is an interval of logits [x_lo, x_hi]: x_hi is the logit at
 // the group's first rank g0, x_lo is found by a 64-way search over order keys (six
 // rounds of one exponential per lane).  Elements of that interval that are not
 // among the candidates yet (below the merge threshold or their chunk's) are
 // fetched from the row, then the k - g0 members with the lowest indices take the
-// places g0 .. k-1.  Writes those places; returns g0, or all ones if the group
-// does not fit the candidate array.  All NT threads call.
+// places g0 .. k-1.  A group that does not fit the candidate array, and the
+// group of probability 0 (the underflowed tail of the row and its -inf
+// elements), is filled by fill_group_by_scan instead.  Writes those places and
+// returns g0.  All NT threads call.
 template <typename T, int NT, int ES>
 __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&cv)[ES], const T *rowp, T *ov, int32_t *oi,
                                                uint32_t n, uint32_t kk, uint32_t per, uint32_t G, uint32_t thr, float p_cut,
@@ -370,6 +427,13 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
         return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(key), M)) * rinv));
     };
     if (tid < kk && sh.prob[tid] == p_cut && (tid == 0 || sh.prob[tid - 1] != p_cut)) sh.g0 = tid;
+    if (!(p_cut > 0.f)) {
+        // probability 0: every element from the group's largest logit down
+        __syncthreads();
+        const uint32_t g0 = sh.g0;
+        fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, 0u, sh.pkey[g0], p_cut);
+        return g0;
+    }
     if (wave == 0) {
         // invariant: probability(b) == p_cut, probability(a) < p_cut (a = 0 stands for "below everything")
         uint64_t a = 0, b = sh.pkey[kk];
@@ -420,7 +484,10 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
     }
     if (added) __syncthreads();
     const uint32_t C3 = sh.count;
-    if (C3 > kFastCap) return 0xFFFFFFFFu;
+    if (C3 > kFastCap) {
+        fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, xlo, xhi, p_cut);
+        return g0;
+    }
     const uint32_t places = kk - g0;
     for (uint32_t t = tid; t < C3; t += NT) {
         const uint64_t mine = sh.cand[t];
@@ -536,9 +603,18 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     __syncthreads();
     const uint32_t thr = sh.thr;
     bool slow = sh.flag != 0u;
-    uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a probability tie across the k-th place, if there is one
-    if (SOFTMAX && !(s_base > 0.0 && s_base < 1e300)) slow = true;  // NaN / inf rows, overflowed partials
-    if (SOFTMAX && !(M > -INFINITY && M < INFINITY)) slow = true;
+    uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
+    if constexpr (SOFTMAX) {
+        if (!(s_base > 0.0 && s_base < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY)) {
+            // a NaN or +inf element, or nothing above -inf: every probability of the
+            // row is NaN, all of them tie, the lowest indices win
+            for (uint32_t r = tid; r < kk; r += NT) {
+                store_elem(ov, r, __uint_as_float(0x7FC00000u));
+                oi[r] = static_cast<int32_t>(r);
+            }
+            return;
+        }
+    }
 
     if (!slow) {
         // ---- D. the candidates reaching the threshold go to LDS ------------------------
@@ -551,8 +627,10 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         }
         __syncthreads();
         const uint32_t C2 = sh.count;
-        // fewer than k+1 candidates prove nothing about the elements left out
-        if (C2 > kFastCap || C2 < min(want, n)) {
+        // Fewer than k+1 candidates: no chunk had k+1 elements above -inf, so every
+        // chunk listed all it has and the rest of the row is -inf (probability 0).
+        const bool partial = C2 < min(want, n);
+        if (C2 > kFastCap) {
             slow = true;
         } else {
             // ---- E. exact ranks; accurate terms for the ranked elements ----------------
@@ -601,15 +679,23 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                 // ones are neighbours.  A tie that reaches past the k-th place is
                 // settled by index over every element of the row with that
                 // probability, candidates or not.
-                if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
-                    const float p_cut = sh.prob[kk];
-                    if (!(p_cut > 0.f)) {
-                        slow = true;  // a tie at 0 (or NaN) takes in the underflowed tail of the row
-                    } else {
-                        tie_g0 = settle_tie<T, NT, ES>(sh, cv, rowp, ov, oi, n, kk, per, G, thr, p_cut, M, rinv);
-                        if (tie_g0 == 0xFFFFFFFFu) slow = true;  // the tied group does not fit
-                    }
+                if (partial) {
+                    // the candidates of probability 0, if any, and the -inf elements form one
+                    // group behind every positive probability: lowest indices first
+                    if (tid == 0) sh.g0 = C2;
+                    __syncthreads();
+                    if (tid < C2 && sh.prob[tid] == 0.f && (tid == 0 || sh.prob[tid - 1] != 0.f)) sh.g0 = tid;
+                    __syncthreads();
+                    tie_g0 = sh.g0;
+                    fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, tie_g0, kk, 0u,
+                                                    tie_g0 < C2 ? sh.pkey[tie_g0] : kKeyNegInf, 0.f);
+                } else if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
+                    tie_g0 = settle_tie<T, NT, ES>(sh, cv, rowp, ov, oi, n, kk, per, G, thr, sh.prob[kk], M, rinv);
                 }
+            } else if (partial) {
+                // the -inf elements follow the candidates, lowest indices first
+                tie_g0 = C2;
+                fill_group_by_scan<T, NT, false>(sh.scan_counts, rowp, ov, oi, n, C2, kk, kKeyNegInf, kKeyNegInf, 0.f);
             }
         }
     }
