@@ -599,3 +599,26 @@ def test_masked_and_underflowed_rows(ops, dtype):
     short[1, 777] = 1.5
     short[2, 500] = 150.0 if dtype == np.float32 else 60.0
     assert_fused(ops, short, 5)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("levels", [17, 256, 3])
+def test_heavily_quantised_rows(ops, dtype, levels):
+    """Logits on a coarse grid: hundreds or thousands of elements equal the value
+    at the k-th place, in every chunk of the row; the lowest indices win."""
+    rng = np.random.default_rng(levels)
+    n, k = 128256, 50
+    if levels == 256:    # int8-like: a bell shape over 256 levels
+        x = np.clip(np.round(rng.standard_normal((6, n)) * 40), -128, 127).astype(np.float32) * np.float32(0.125)
+    else:
+        x = rng.integers(0, levels, size=(6, n)).astype(np.float32) * np.float32(0.5) - np.float32(2.0)
+    x[1, :20000] = x[1].min()        # the first chunks of the row hold nothing of interest
+    x[2] = np.sort(x[2])             # equal values side by side
+    x = np.ascontiguousarray(x.astype(dtype))
+    assert_fused(ops, x, k)
+    assert_fused(ops, np.ascontiguousarray(x[:, :70001]), 200)
+    for largest in (True, False):
+        t, j = ops.topk(dev(x), k, -1, largest)
+        et, ej = oracle.topk(x, k, -1, largest)
+        bits = np.uint16 if dtype == np.float16 else np.uint32
+        assert np.array_equal(host(j), ej) and np.array_equal(host(t).view(bits), et.view(bits))

@@ -130,6 +130,10 @@ def main():
     c3m = np.full_like(c3, -np.inf)
     c3m[:, 1000:128000:6350] = c3[:, 1000:128000:6350]
     select_case("C3 masked-rows softmax+topk k=50 [64,128256] f32", c3m, 50, True)
+    # int8-like logits: 256 levels, hundreds of elements equal the value at the k-th place
+    c3i = np.ascontiguousarray(np.clip(np.round(c3 * 16), -128, 127).astype(np.float32) * np.float32(0.125))
+    select_case("C3 int8-valued softmax+topk k=50 [64,128256] f32", c3i, 50, True)
+    select_case("C3 int8-valued topk k=50 [64,128256] f32", c3i, 50, False)
     softmax_case("C4 softmax [8,262144] f32", c4, -1)
     select_case("C4 topk k=1024 [8,262144] f32 (ties)", c4, 1024, False)
     select_case("C4 softmax+topk k=1024 [8,262144] f32", c4, 1024, True)

@@ -229,7 +229,7 @@ template <int NT> struct ChunkShared {  // chunk phase
     uint4 stage_v[NT];     // per wave: up to 64 vectors holding an element at or above the threshold ...
     uint32_t stage_e[NT];  // ... and the index of their first element
     uint32_t wave_thr[16];
-    uint32_t refine[32];  // element counts per bit of the exact threshold search
+    uint32_t refine[34];  // element counts per bit of the exact threshold search; reaching / exceeding the result
     uint32_t thr, total, over;
 };
 
@@ -602,6 +602,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     }
     __syncthreads();
     const uint32_t thr = sh.thr;
+    uint32_t merge_thr = thr;  // candidates with keys at or above it are in sh.cand (of equal keys maybe only the first)
     bool slow = sh.flag != 0u;
     uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
     if constexpr (SOFTMAX) {
@@ -626,7 +627,64 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
             }
         }
         __syncthreads();
-        const uint32_t C2 = sh.count;
+        uint32_t C2 = sh.count;
+        if (C2 > kFastCap) {
+            // Too many reach the threshold (it comes from per-thread maxima and is
+            // rounded down; rows full of equal values).  Take the exact cut over all
+            // candidates instead: the (k+1)-th largest key, then among the
+            // candidates equal to it the ones with the lowest indices -- k+1 of them
+            // for the softmax variant (a tie across the k-th place is settled among
+            // equal probabilities by index), else as many as make k+1 in all.
+            uint32_t round = 0;
+            auto count_if = [&](auto pred) -> uint32_t {  // over every candidate of the row; all threads call
+                uint32_t c = 0;
+#pragma unroll
+                for (int e = 0; e < ES; e++) c += static_cast<uint32_t>(__popcll(__ballot(pred(cv[e]))));
+                uint32_t *wc = sh.scan_counts + (round & 1u) * NW;
+                round++;
+                if (lane == 0) wc[wave] = c;
+                __syncthreads();
+                uint32_t total = 0;
+#pragma unroll
+                for (int w = 0; w < NW; w++) total += wc[w];
+                return total;
+            };
+            // the key lies in [thr, all ones]: those share the leading ones of thr
+            uint32_t cutkey = thr;
+            if (thr != 0xFFFFFFFFu) {
+                const int d = 31 - __clz(static_cast<int>(~thr));  // highest zero bit of thr
+                cutkey = thr & ~((2u << d) - 1u);
+                for (int bit = d; bit >= 0; bit--) {
+                    const uint32_t trial = cutkey | (1u << bit);
+                    if (count_if([&](uint64_t c) { return static_cast<uint32_t>(c >> 32) >= trial; }) >= want) cutkey = trial;
+                }
+                cutkey = max(cutkey, thr);
+            }
+            const uint32_t reach = count_if([&](uint64_t c) { return static_cast<uint32_t>(c >> 32) >= cutkey; });
+            const uint32_t exceed = count_if([&](uint64_t c) { return static_cast<uint32_t>(c >> 32) > cutkey; });
+            const uint32_t keep = SOFTMAX ? exceed + want : want;
+            uint64_t cut = static_cast<uint64_t>(cutkey) << 32;
+            if (reach > keep) {
+                // the keep-th largest composite: descent over the index half
+                for (int bit = 31; bit >= 0; bit--) {
+                    const uint64_t trial = cut | (1ull << bit);
+                    if (count_if([&](uint64_t c) { return c >= trial; }) >= keep) cut = trial;
+                }
+            }
+            __syncthreads();
+            if (tid == 0) sh.count = 0;
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < ES; e++) {
+                if (cv[e] >= cut && cv[e] != 0) {
+                    const uint32_t pos = atomicAdd(&sh.count, 1u);
+                    if (pos < kFastCap) sh.cand[pos] = cv[e];
+                }
+            }
+            __syncthreads();
+            C2 = sh.count;
+            merge_thr = cutkey;
+        }
         // Fewer than k+1 candidates: no chunk had k+1 elements above -inf, so every
         // chunk listed all it has and the rest of the row is -inf (probability 0).
         const bool partial = C2 < min(want, n);
@@ -690,7 +748,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                     fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, tie_g0, kk, 0u,
                                                     tie_g0 < C2 ? sh.pkey[tie_g0] : kKeyNegInf, 0.f);
                 } else if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
-                    tie_g0 = settle_tie<T, NT, ES>(sh, cv, rowp, ov, oi, n, kk, per, G, thr, sh.prob[kk], M, rinv);
+                    tie_g0 = settle_tie<T, NT, ES>(sh, cv, rowp, ov, oi, n, kk, per, G, merge_thr, sh.prob[kk], M, rinv);
                 }
             } else if (partial) {
                 // the -inf elements follow the candidates, lowest indices first
@@ -757,7 +815,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
 // Launch: rows * G workgroups of NT threads; per = elements per chunk
 // (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
 template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, bool FUSED>
-__global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && ALIGNED && NT == 256 ? 5 : 1))) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                         int32_t *__restrict__ indices, uint32_t n, uint32_t k,
                                                         uint32_t G, uint32_t per, RowsWorkspace ws) {
     constexpr int VEC = Vec128<T>::N;
@@ -909,19 +967,37 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
         uint32_t thr = max(thr_block, kKeyNegInf + 1u);
 
         // ---- 4. the elements at or above the threshold go to the chunk's candidate list --------
-        // Returns the wave's count, or all ones if the wave had more than 64 vectors to stage.
-        auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors) -> uint32_t {
+        // Returns the wave's count (all ones if the wave had more than 64 vectors to stage;
+        // staged_vectors = how many it staged).  With the truncation tag, of the elements
+        // equal to the threshold only those up to index idx_limit are listed.
+        uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
+        uint4 *stv = cs.stage_v + wave * kWave;
+        uint32_t *ste = cs.stage_e + wave * kWave;
+        auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors, auto trunc_tag, uint32_t idx_limit) -> uint32_t {
+            constexpr bool TRUNC = decltype(trunc_tag)::value;
             const float thr_f = ordered_to_float(thr_key);
             // 4a. the wave's vectors holding such an element -> LDS
-            uint4 *stv = cs.stage_v + wave * kWave;
-            uint32_t *ste = cs.stage_e + wave * kWave;
             uint32_t nv = 0;  // wave-uniform
 #pragma unroll
             for (int i = 0; i < V; i++) {
                 const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
                 bool hit;
-                if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
-                else hit = vkey[i] >= thr_key && in_range(e0);
+                if constexpr (!TRUNC) {
+                    if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
+                    else hit = vkey[i] >= thr_key && in_range(e0);
+                } else {
+                    // (the vector's largest key again from the vector itself: nothing the
+                    // first pass used stays live for the sake of this one)
+                    uint32_t vk = 0u;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        float x = q[i].get(c);
+                        asm volatile("" : "+v"(x));
+                        const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
+                        vk = max(vk, in_range(ALIGNED ? e0 : e0 + c) ? key : 0u);
+                    }
+                    hit = vk >= thr_key && in_range(e0) && (vk > thr_key || e0 <= idx_limit);
+                }
                 const uint64_t mask = __ballot(hit);
                 if (mask != 0ull) {
                     if (hit) {
@@ -955,7 +1031,8 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
                     const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
                     const float x = r.get(static_cast<int>(lane % VEC));
                     const uint32_t key = order_key(x);
-                    const bool pass = live && idx < c1 && key >= thr_key;
+                    bool pass = live && idx < c1 && key >= thr_key;
+                    if constexpr (TRUNC) pass = pass && (key > thr_key || idx <= idx_limit);
                     const uint64_t mask = __ballot(pass);
                     if (pass) {
                         mine[p] = composite(key, idx);
@@ -971,7 +1048,6 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
                 if (over) cs.over = 1;
             }
             base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
-            uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
 #pragma unroll
             for (int p = 0; p < PASSES; p++) {
                 const uint32_t pos = base + mpos[p];
@@ -980,77 +1056,9 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
             return over ? 0xFFFFFFFFu : wcount;
         };
         uint32_t staged = 0;
-        uint32_t wave_candidates = compact(thr, staged);
-        __syncthreads();
-        if (cs.total > ws.cap || cs.over != 0u) {
-            // Too many: the lane maxima gave a loose bound (values in order or in
-            // clusters put many large elements into few lanes).  Take the exact
-            // (k+1)-th largest element of the chunk instead and list again; only
-            // equal values beyond the list's size can still overflow it.  The value
-            // lies between the bound just used and the chunk's maximum: a descent
-            // over the bits in which the two differ, counting over the staged
-            // elements (everything at or above the old bound is among them) or, if
-            // a wave's stage was too small, over every element held in registers.
-            const bool from_stage = cs.over == 0u;
-            const uint32_t wk = wave_max_u32(lkey);
-            if (lane == 0) cs.wave_thr[wave] = wk;
-            if (tid < 32) cs.refine[tid] = 0;
-            __syncthreads();
-            uint32_t hi = cs.wave_thr[0];
-#pragma unroll
-            for (int w = 1; w < NW; w++) hi = max(hi, cs.wave_thr[w]);
-            auto exact_threshold = [&](const uint32_t *keys, auto count_tag) -> uint32_t {
-                constexpr int NK = decltype(count_tag)::value;
-                if (thr >= hi) return thr;
-                const int d = 31 - __clz(static_cast<int>(thr ^ hi));  // highest bit in which they differ
-                uint32_t t = hi & ~((2u << d) - 1u);                    // their common prefix
-                for (int bit = d; bit >= 0; bit--) {
-                    const uint32_t trial = t | (1u << bit);
-                    uint32_t c = 0;  // wave-uniform
-#pragma unroll
-                    for (int e = 0; e < NK; e++) c += static_cast<uint32_t>(__popcll(__ballot(keys[e] >= trial)));
-                    if (lane == 0 && c) atomicAdd(&cs.refine[bit], c);
-                    __syncthreads();
-                    if (cs.refine[bit] >= want) t = trial;
-                }
-                return max(t, thr);
-            };
-            if (from_stage) {
-                const uint4 *stv = cs.stage_v + wave * kWave;
-                const uint32_t *ste = cs.stage_e + wave * kWave;
-                uint32_t keys[PASSES];
-#pragma unroll
-                for (int p = 0; p < PASSES; p++) {
-                    const uint32_t sv = static_cast<uint32_t>(p) * VPP + lane / VEC;
-                    const bool live = sv < staged;
-                    Vec128<T> r;
-                    r.v = stv[live ? sv : 0u];
-                    const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
-                    keys[p] = (live && idx < c1) ? order_key(r.get(static_cast<int>(lane % VEC))) : 0u;
-                }
-                thr = exact_threshold(keys, std::integral_constant<int, PASSES>{});
-            } else {
-                uint32_t keys[V * VEC];
-#pragma unroll
-                for (int i = 0; i < V; i++) {
-                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-#pragma unroll
-                    for (int c = 0; c < VEC; c++)
-                        keys[i * VEC + c] = in_range(ALIGNED ? e0 : e0 + c) ? order_key(q[i].get(c)) : 0u;
-                }
-                thr = exact_threshold(keys, std::integral_constant<int, V * VEC>{});
-            }
-            drain_stores();  // the first attempt's stores have landed before the same slots are written again
-            __syncthreads();  // (and every wave is done with its stage)
-            if (tid == 0) {
-                cs.total = 0;
-                cs.over = 0;
-            }
-            __syncthreads();
-            wave_candidates = compact(thr, staged);
-        }
+        uint32_t wave_candidates = compact(thr, staged, std::false_type{}, 0u);
 
-        // ---- 5. the wave's partial sum -----------------------------------------------------------
+        // ---- the wave's partial sum (here, so that none of it is live across what follows) ------
         if constexpr (SOFTMAX) {
             if (wm - ref > kTermSwitch) {  // wave-uniform
                 // an element well above the reference: its fast term is poor (or has
@@ -1073,6 +1081,133 @@ __global__ __launch_bounds__(NT) void rows_chunk_kernel(const T *__restrict__ in
             publish(ws.sums + 3 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
             publish(ws.sums + 3 * static_cast<size_t>(went) + 1,
                     (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
+        }
+        __syncthreads();
+        if (__builtin_expect(cs.total > ws.cap || cs.over != 0u, 0)) {
+            // Too many.  The lane maxima give a loose bound when values in order or in
+            // clusters put many large elements into few lanes, or when many are equal.
+            // The list is made once more, with the exact (k+1)-th largest element of
+            // the chunk as the threshold.  It lies between the bound just used and the
+            // chunk's maximum: a descent over the bits in which the two differ, counting
+            // over the staged elements (everything at or above the old bound is among
+            // them) or, if a wave's stage was too small, over every element held in
+            // registers.  Of the elements equal to that value only the first k+1 (by
+            // index) are listed, so that no number of equal values overflows the list:
+            // the others cannot reach the row's result, k+1 elements of this chunk come
+            // before each.
+            // (Keys are derived from the loaded vectors at every use: the empty asm keeps
+            // the compiler from holding them all in registers, which would cost the whole
+            // kernel waves per SIMD for the sake of this path.)
+            auto key_of = [&](int i, int c) {
+                const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+                float x = q[i].get(c);
+                asm volatile("" : "+v"(x));
+                return in_range(ALIGNED ? e0 : e0 + c) ? order_key(x) : 0u;
+            };
+            const bool from_stage = cs.over == 0u;
+            uint32_t wk = 0;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) wk = max(wk, key_of(i, c));
+            }
+            wk = wave_max_u32(wk);
+            if (lane == 0) cs.wave_thr[wave] = wk;
+            if (tid < 32) cs.refine[tid] = 0;
+            __syncthreads();
+            uint32_t hi = cs.wave_thr[0];
+#pragma unroll
+            for (int w = 1; w < NW; w++) hi = max(hi, cs.wave_thr[w]);
+            // count(trial): elements of this wave at or above trial (wave-uniform)
+            auto exact_threshold = [&](auto count) -> uint32_t {
+                if (thr >= hi) return thr;
+                const int d = 31 - __clz(static_cast<int>(thr ^ hi));  // highest bit in which they differ
+                uint32_t t = hi & ~((2u << d) - 1u);                    // their common prefix
+                for (int bit = d; bit >= 0; bit--) {
+                    const uint32_t trial = t | (1u << bit);
+                    const uint32_t c = count(trial);
+                    if (lane == 0 && c) atomicAdd(&cs.refine[bit], c);
+                    __syncthreads();
+                    if (cs.refine[bit] >= want) t = trial;
+                }
+                return max(t, thr);
+            };
+            if (from_stage) {
+                uint32_t keys[PASSES];
+#pragma unroll
+                for (int p = 0; p < PASSES; p++) {
+                    const uint32_t sv = static_cast<uint32_t>(p) * VPP + lane / VEC;
+                    const bool live = sv < staged;
+                    Vec128<T> r;
+                    r.v = stv[live ? sv : 0u];
+                    const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
+                    keys[p] = (live && idx < c1) ? order_key(r.get(static_cast<int>(lane % VEC))) : 0u;
+                }
+                thr = exact_threshold([&](uint32_t trial) {
+                    uint32_t c = 0;
+#pragma unroll
+                    for (int p = 0; p < PASSES; p++) c += static_cast<uint32_t>(__popcll(__ballot(keys[p] >= trial)));
+                    return c;
+                });
+            } else {
+                thr = exact_threshold([&](uint32_t trial) {
+                    uint32_t c = 0;
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+#pragma unroll
+                        for (int cc = 0; cc < VEC; cc++) c += static_cast<uint32_t>(__popcll(__ballot(key_of(i, cc) >= trial)));
+                    }
+                    return c;
+                });
+            }
+            // Index of the last equal element to list: elements are in index order by
+            // (vector, wave, lane, position in the vector).
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                uint32_t ties = 0;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) ties += static_cast<uint32_t>(__popcll(__ballot(key_of(i, c) == thr)));
+                if (lane == 0) cs.lane_key[i * NW + wave] = ties;
+            }
+            drain_stores();  // the first attempt's stores have landed before the same slots are written again
+            __syncthreads();  // (and every wave is done with its stage)
+            // exclusive prefix over the (vector, wave) table, one entry per thread
+            uint32_t mine_before = 0;
+            if (tid < static_cast<uint32_t>(V * NW)) {
+#pragma unroll 1
+                for (uint32_t j = 0; j < tid; j++) mine_before += cs.lane_key[j];
+            }
+            __syncthreads();
+            if (tid < static_cast<uint32_t>(V * NW)) cs.lane_key[tid] = mine_before;
+            if (tid == 0) {
+                cs.total = 0;
+                cs.over = 0;
+                cs.thr = 0xFFFFFFFFu;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                uint32_t pos = cs.lane_key[i * NW + wave];  // equal elements before this wave's vector i
+                bool tie[VEC];
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    tie[c] = key_of(i, c) == thr;
+                    pos += lanes_below(__ballot(tie[c]));
+                }
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    if (tie[c]) {
+                        if (pos == want - 1u) cs.thr = e_first + static_cast<uint32_t>(i) * NT * VEC + c;
+                        pos++;
+                    }
+                }
+            }
+            __syncthreads();
+            wave_candidates = compact(thr, staged, std::true_type{}, cs.thr);
+        }
+
+        // ---- 5. the chunk's threshold and the wave's candidate count -------------------------------
+        if (lane == 0) {
             publish(ws.sums + 3 * static_cast<size_t>(went) + 2,
                     (static_cast<uint64_t>(thr) << 32) | static_cast<uint64_t>(wave_candidates));
         }
