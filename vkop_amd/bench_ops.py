@@ -121,6 +121,9 @@ def main():
     softmax_case("C3 softmax [64,128256] f32", c3, -1)
     select_case("C3 topk k=50 [64,128256] f32", c3, 50, False)
     select_case("C3 softmax+topk k=50 [64,128256] f32", c3, 50, True)
+    c3h = c3.astype(np.float16)
+    select_case("C3 softmax+topk k=50 [64,128256] f16", c3h, 50, True)
+    select_case("C3 topk k=50 [64,128256] f16", c3h, 50, False)
     # the same logits after a round trip through bfloat16: equal values straddle the k-th place in most rows
     c3q = np.ascontiguousarray((c3.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32))
     select_case("C3 bf16-valued softmax+topk k=50 [64,128256] f32", c3q, 50, True)

@@ -5,30 +5,38 @@
 // Each workgroup
 //   1. issues all of its 128-bit loads (V per thread) at once,
 //   2. consumes the vectors in the order they arrive: per vector its maximum and
-//      the sum of exp(x - ref), where ref is the maximum of the wave's FIRST
-//      vector (any reference is valid for a partial sum; taking it from the
-//      first vector lets the exponentials overlap the rest of the stream),
-//   3. publishes per-lane maxima to LDS; one wave finds, by a ballot descent over
+//      the sum of exp(x - ref), where ref is taken from the wave's FIRST vector
+//      (any reference is valid for a partial sum; taking it from the first
+//      vector lets the exponentials overlap the rest of the stream; a wave that
+//      later meets an element well above it sums again against its maximum),
+//   3. publishes per-lane maxima to LDS; the waves find, by ballot descents over
 //      them, a threshold that at least k+1 elements of the chunk reach,
 //   4. compacts the elements at or above the threshold: the few vectors holding
 //      one go to a per-wave stage in LDS (ballot + popcount), are unpacked one
 //      element per lane, and the survivors are written as (order key, ~index)
-//      composites into the chunk's candidate list,
-//   5. writes one partial (sum, reference, maximum) per wave and the chunk's
-//      candidate count.
-// The workgroup that finishes a row's last chunk (one counter per row) then
-// merges the row: it combines the partial sums, finds the (k+1)-th largest
-// candidate, ranks the candidates above it exactly (key, then lower index),
-// replaces the summed fast terms of the ranked elements by accurate ones,
-// computes the probabilities of the winners only, orders equal probabilities by
-// index and writes the row's result.  Every order of summation is fixed and the
-// ranking does not depend on the order candidates were stored in, so results
-// are bit-identical from run to run.
-// Whatever the shortcut cannot prove exact (a candidate list overflows, a
-// partial sum overflows, a probability tie across the k-th place, NaN/inf rows,
-// rows with fewer than k+1 elements above -inf) is redone by the merging
-// workgroup with the exact radix select of select.hpp, so the result is always
-// top-k (probability, then lower index) of the row's softmax.
+//      composites into the chunk's candidate list; a list that overflows (values
+//      in order or in clusters, many equal values) is made again with the
+//      chunk's exact (k+1)-th largest element as the threshold and only the
+//      first k+1 elements equal to it,
+//   5. writes one record per wave: partial sum, reference, maximum, threshold
+//      and the candidates it contributed.
+// The merge (rows_merge_kernel, or in the one-kernel variant the workgroup that
+// finishes a row's last chunk, found with one counter per row) combines the
+// partial sums, finds the (k+1)-th largest candidate, ranks the candidates
+// above it exactly (key, then lower index), replaces the summed fast terms of
+// the ranked elements by accurate ones, computes the probabilities of the
+// winners only, orders equal probabilities by index and writes the row's
+// result.  Every order of summation is fixed and the ranking does not depend on
+// the order candidates were stored in, so results are bit-identical from run to
+// run.  The merge also settles by itself: a probability tie across the k-th
+// place (the tied logit interval is searched, its members fetched or, if they
+// are many, taken from the start of the row), rows of NaN, rows with fewer than
+// k+1 elements above -inf, ties at probability 0, and more candidates than its
+// LDS array holds (exact cut over the candidates in registers).  What is left
+// for the exact radix select of select.hpp over the whole row -- a candidate
+// list that overflows even after the second attempt -- needs an adversarial
+// layout of equal values; the result is always top-k (probability, then lower
+// index) of the row's softmax.
 #pragma once
 
 #include <type_traits>
