@@ -42,6 +42,9 @@ WORKLOADS = {
     "C2": ("[256,1000] f32 softmax+topk k=5", dict(kind="cls", rows=256, cols=1000), 5),
     "C3": ("[64,128256] f32 softmax+topk k=50", dict(kind="llm", rows=64, cols=128256), 50),
     "C4": ("[8,262144] f32 softmax+topk k=1024", dict(kind="grid", rows=8, cols=262144), 1024),
+    # not a BASELINE config: C3's logits truncated to bfloat16 precision (what a bf16 LM head hands over);
+    # equal logits then straddle the k-th place in most rows and the merge settles a tie per row
+    "C3bf16": ("[64,128256] f32 softmax+topk k=50, bf16-valued logits", dict(kind="llm_bf16", rows=64, cols=128256), 50),
 }
 
 
@@ -51,6 +54,10 @@ def make_input(spec, seed):
         return synth.classifier_logits(spec["rows"], spec["cols"], seed)
     if spec["kind"] == "llm":
         return synth.llm_logits(spec["rows"], spec["cols"], seed)
+    if spec["kind"] == "llm_bf16":
+        import numpy as np
+        x = synth.llm_logits(spec["rows"], spec["cols"], seed)
+        return np.ascontiguousarray((x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32))
     return synth.grid_values(spec["rows"], spec["cols"], seed)
 
 
@@ -156,7 +163,7 @@ def main():
     algo_bytes = in_bytes + rows * k * 8
     nbuf = 1 if args.resident else max(2, -(-(288 << 20) // in_bytes))
     nbuf = min(nbuf, 64)
-    seed0 = synth.SEEDS.get(args.workload, 1)
+    seed0 = synth.SEEDS.get(args.workload[:2], 1)
     host_inputs = [make_input(spec, seed0 + 7919 * b) for b in range(min(nbuf, 3))]
     bufs = []
     for b in range(nbuf):

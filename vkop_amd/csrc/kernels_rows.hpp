@@ -253,6 +253,7 @@ struct RowsShared {  // merge phase
     uint32_t cthr[kMergeChunksMax];  // threshold per chunk: the chunk's elements at or above it are candidates
     uint32_t pkey[kFastMaxK + 1];    // order key of the logit, by rank
     uint32_t g0, xlo;                // tie at the cut: first rank of the tied group, smallest key in it
+    uint32_t members;                // ... and how many of its members are in lane_key[] (their indices)
     uint32_t scan_counts[2 * 16];    // fill_group_by_scan: members per wave, double-buffered
     uint32_t lane_key[1024];
     uint32_t thr;
@@ -442,9 +443,20 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
         fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, 0u, sh.pkey[g0], p_cut);
         return g0;
     }
+    if (tid == 0) sh.members = 0;
     if (wave == 0) {
         // invariant: probability(b) == p_cut, probability(a) < p_cut (a = 0 stands for "below everything")
         uint64_t a = 0, b = sh.pkey[kk];
+        {
+            // First the keys b - 1, b - 2, b - 4, ...: the interval is usually a few keys
+            // wide (one, for float logits away from 0), and this finds its size class at once.
+            const uint32_t off = lane < 32 ? (1u << lane) : 0xFFFFFFFFu;
+            const uint64_t probe = b > off ? b - off : 0;
+            const bool in = probe != 0 && prob_of_key(static_cast<uint32_t>(probe)) >= p_cut;  // true ... true false ... false
+            const int f = __ffsll(static_cast<long long>(~__ballot(in))) - 1;                   // lanes 32.. are false: f >= 0
+            a = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f));
+            if (f > 0) b = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f > 0 ? f - 1 : 0));
+        }
         while (b - a > 1) {
             const uint64_t step = (b - a + 63) / 64;
             uint64_t probe = a + step * (lane + 1);
@@ -496,18 +508,19 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
         fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, xlo, xhi, p_cut);
         return g0;
     }
+    // the group's members (their indices) side by side, then each counts the members before it
     const uint32_t places = kk - g0;
     for (uint32_t t = tid; t < C3; t += NT) {
         const uint64_t mine = sh.cand[t];
         const uint32_t key = static_cast<uint32_t>(mine >> 32);
-        if (key < xlo || key > xhi) continue;
-        const uint32_t idx = composite_index(mine);
+        if (key >= xlo && key <= xhi) sh.lane_key[atomicAdd(&sh.members, 1u)] = composite_index(mine);
+    }
+    __syncthreads();
+    const uint32_t members = sh.members;
+    for (uint32_t t = tid; t < members; t += NT) {
+        const uint32_t idx = sh.lane_key[t];
         uint32_t before = 0;  // members of the group with a lower index
-        for (uint32_t u = 0; u < C3; u++) {
-            const uint64_t other = sh.cand[u];
-            const uint32_t okey = static_cast<uint32_t>(other >> 32);
-            before += (okey >= xlo && okey <= xhi && composite_index(other) < idx) ? 1u : 0u;
-        }
+        for (uint32_t u = 0; u < members; u++) before += (sh.lane_key[u] < idx) ? 1u : 0u;
         if (before < places) {
             store_elem(ov, g0 + before, p_cut);
             oi[g0 + before] = static_cast<int32_t>(idx);
