@@ -188,10 +188,4 @@ template <typename T> __global__ void stats_to_max_kernel(const LineStats *__res
     store_elem(out, line, softmax_prob(st.m, st));
 }
 
-// ---- workspace clear ---------------------------------------------------------
-__global__ void fill_zero_kernel(uint32_t *p, size_t words) {
-    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < words) p[i] = 0u;
-}
-
 }  // namespace vkop

@@ -53,6 +53,7 @@ constexpr int kMergeThreads = 256;    // rows_merge_kernel workgroup
 constexpr int kMergeRecsMax = 4096;   // candidate slots per row the merge takes in registers
 constexpr int kMergeWavesMax = 256;   // chunk-kernel waves per row the merge can combine
 constexpr int kMergeChunksMax = 64;   // chunks per row
+constexpr int kLocalCap = 1024;       // candidate slots of the LDS-resident list of a one-workgroup row (cap for k = 255)
 
 // ---- wave-level helpers (all 64 lanes must be active) -----------------------
 
@@ -533,15 +534,18 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
 // G chunks of `per` elements, each summed and scanned by a workgroup of src_nt
 // threads; G << cap_shift <= kMergeRecsMax, G <= kMergeChunksMax,
 // G * src_nt / 64 <= kMergeWavesMax (the host checks all three).
-template <typename T, int NT, bool SOFTMAX>
+// RECS: candidate slots the merge can take in (a multiple of NT).
+template <typename T, int NT, bool SOFTMAX, int RECS = kMergeRecsMax>
 __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, float *fscratch, double *dscratch,
                                           const T *rowp, T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
                                           uint32_t per, uint32_t src_nt, const uint64_t *sums,
                                           const uint64_t *cand, uint32_t cap_shift) {
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
-    constexpr int ES = kMergeRecsMax / NT;  // candidate slots per thread
-    static_assert(NT >= kMergeWavesMax && NT >= kMergeChunksMax, "one thread per wave partial and per chunk");
+    constexpr int ES = RECS / NT;  // candidate slots per thread
+    // one thread per wave partial and per chunk (a workgroup that merges only its own
+    // row, RECS = kLocalCap, has one chunk and NT / 64 waves)
+    static_assert(RECS == kLocalCap || (NT >= kMergeWavesMax && NT >= kMergeChunksMax), "merge workgroup too small");
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t want = k + 1;
     const uint32_t kk = min(k, n);
@@ -562,10 +566,11 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     for (uint32_t w0 = 0; w0 < src_nw; w0 += 4) {
         uint64_t c[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) c[u] = fetch(sums + 3 * ((tid < G ? tid : 0u) * src_nw + w0 + u) + 2);
+        for (int u = 0; u < 4; u++)  // (a one-wave workgroup has a single record: it is read four times, counted once)
+            c[u] = fetch(sums + 3 * ((tid < G ? tid : 0u) * src_nw + (w0 + u < src_nw ? w0 + u : 0u)) + 2);
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            const uint32_t cnt = static_cast<uint32_t>(c[u]);
+            const uint32_t cnt = w0 + u < src_nw ? static_cast<uint32_t>(c[u]) : 0u;
             cm = (cnt == 0xFFFFFFFFu || cm == ~0ull) ? ~0ull : cm + cnt;
             cthr = static_cast<uint32_t>(c[u] >> 32);
         }
@@ -617,12 +622,13 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     }
     __syncthreads();
     if (bad) sh.flag = 1;  // every writer stores the same value
-    if (wave == 0) {
+    // (a single chunk's list is already cut at that chunk's threshold: everything in it is taken)
+    if (G > 1 && wave == 0) {
         const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
         if (lane == 0) sh.thr = t > 1u ? t : 1u;  // key 0 is "no element"
     }
-    __syncthreads();
-    const uint32_t thr = sh.thr;
+    __syncthreads();  // (sh.flag as well)
+    const uint32_t thr = G > 1 ? sh.thr : 1u;
     uint32_t merge_thr = thr;  // candidates with keys at or above it are in sh.cand (of equal keys maybe only the first)
     bool slow = sh.flag != 0u;
     uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
@@ -830,22 +836,30 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
 // SOFTMAX = false: plain top-k, largest first (values are copies of the input)
 // ALIGNED: every row start is 16-byte aligned and n is a multiple of the vector
 // width, so chunks are read with 128-bit loads.
-// FUSED: the workgroup that publishes a row's last chunk (found with one
-// counter per row) merges the row before it exits; otherwise rows_merge_kernel
-// must follow on the same stream.
+// MERGE: kMergeSplit    -- rows_merge_kernel must follow on the same stream;
+//        kMergeByTicket -- the workgroup that publishes a row's last chunk (found
+//                          with one counter per row) merges the row before it exits;
+//        kMergeLocal    -- one workgroup holds the whole row (G = 1): what the chunk
+//                          phase hands to the merge stays in LDS instead of making
+//                          the trip through memory.
 // Launch: rows * G workgroups of NT threads; per = elements per chunk
 // (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
-template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, bool FUSED>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && ALIGNED && NT == 256 ? 5 : 1))) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
+constexpr int kMergeSplit = 0, kMergeByTicket = 1, kMergeLocal = 2;
+
+template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, int MERGE>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && ALIGNED && NT == 256 && MERGE == kMergeSplit ? 5 : 1))) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                         int32_t *__restrict__ indices, uint32_t n, uint32_t k,
                                                         uint32_t G, uint32_t per, RowsWorkspace ws) {
     constexpr int VEC = Vec128<T>::N;
     constexpr int NW = NT / kWave;
     constexpr int VPP = kWave / VEC;    // staged vectors a wave unpacks per pass (one element per lane)
     constexpr int PASSES = kWave / VPP;  // passes over a full stage of 64 vectors
+    constexpr bool FUSED = MERGE != kMergeSplit;
+    constexpr bool LOCAL = MERGE == kMergeLocal;
     __shared__ std::conditional_t<FUSED, RowsSharedUnion<NT>, ChunkShared<NT>> smem;
     __shared__ float fscratch[FUSED ? NW : 1];
     __shared__ double dscratch[FUSED ? NW : 1];
+    __shared__ uint64_t local_ws[LOCAL ? kLocalCap + 3 * NW : 1];  // candidate list, then the wave records
     __shared__ uint32_t s_last;
     ChunkShared<NT> *csp;
     if constexpr (FUSED) csp = &smem.chunk;
@@ -991,7 +1005,12 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         // Returns the wave's count (all ones if the wave had more than 64 vectors to stage;
         // staged_vectors = how many it staged).  With the truncation tag, of the elements
         // equal to the threshold only those up to index idx_limit are listed.
-        uint64_t *cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
+        uint64_t *cand_out;
+        if constexpr (LOCAL) cand_out = local_ws;
+        else cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
+        uint64_t *record;  // this wave's
+        if constexpr (LOCAL) record = local_ws + kLocalCap + 3 * wave;
+        else record = ws.sums + 3 * static_cast<size_t>(went);
         uint4 *stv = cs.stage_v + wave * kWave;
         uint32_t *ste = cs.stage_e + wave * kWave;
         auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors, auto trunc_tag, uint32_t idx_limit) -> uint32_t {
@@ -1099,9 +1118,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             }
         }
         if (lane == 0) {
-            publish(ws.sums + 3 * static_cast<size_t>(went), static_cast<uint64_t>(__double_as_longlong(wsum)));
-            publish(ws.sums + 3 * static_cast<size_t>(went) + 1,
-                    (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
+            publish(record, static_cast<uint64_t>(__double_as_longlong(wsum)));
+            publish(record + 1, (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
         }
         __syncthreads();
         if (__builtin_expect(cs.total > ws.cap || cs.over != 0u, 0)) {
@@ -1229,8 +1247,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
 
         // ---- 5. the chunk's threshold and the wave's candidate count -------------------------------
         if (lane == 0) {
-            publish(ws.sums + 3 * static_cast<size_t>(went) + 2,
-                    (static_cast<uint64_t>(thr) << 32) | static_cast<uint64_t>(wave_candidates));
+            publish(record + 2, (static_cast<uint64_t>(thr) << 32) | static_cast<uint64_t>(wave_candidates));
         }
     };
     if (c1 - c0 == static_cast<uint32_t>(NT) * V * VEC) body(std::true_type{});
@@ -1238,7 +1255,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
 
     // ---- 6. one-kernel variant: the row's last chunk merges ------------------------------------
     // (otherwise the workgroup is done: the merge kernel adds up the waves' counts itself)
-    if constexpr (FUSED) {
+    if constexpr (MERGE == kMergeByTicket) {
         drain_stores();
         __syncthreads();  // every thread's published values are visible device-wide
         if (tid == 0) {
@@ -1253,7 +1270,13 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             s_last = last;
         }
     }
-    if constexpr (FUSED) {
+    if constexpr (LOCAL) {
+        __syncthreads();  // the list and the records are in LDS; so is what the merge builds, in other arrays
+        merge_row<T, NT, SOFTMAX, kLocalCap>(smem.fast, smem.exact, fscratch, dscratch, rowp,
+                                             values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k, n, k,
+                                             1u, per, NT, local_ws + kLocalCap, local_ws, ws.cap_shift);
+        (void)s_last;
+    } else if constexpr (FUSED) {
         __syncthreads();
         if (s_last == 0u) return;
         merge_row<T, NT, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,

@@ -1,0 +1,65 @@
+// One (element type, variant) slice of the streaming row kernels:
+//   hipcc -DVKOP_ROWS_T=float|uint16_t -DVKOP_ROWS_SOFTMAX=true|false -c rows_inst.hip
+#include "rows_launch.hpp"
+
+#ifndef VKOP_ROWS_T
+#error "define VKOP_ROWS_T (float or uint16_t) and VKOP_ROWS_SOFTMAX (true or false)"
+#endif
+
+namespace vkop {
+
+template <typename T, bool SOFTMAX> bool launch_rows_chunk(const RowsLaunch &a) {
+    const T *in = static_cast<const T *>(a.in);
+    T *values = static_cast<T *>(a.values);
+    const uint32_t blocks = a.rows * a.g;
+#define VKOP_ROWS_LAUNCH(NT, V, AL, MERGE)                       \
+    rows_chunk_kernel<T, NT, V, SOFTMAX, AL, MERGE>              \
+        <<<blocks, NT, 0, a.stream>>>(in, values, a.indices, a.n, a.k, a.g, a.per, a.ws)
+#define VKOP_ROWS_CASE(NT, V)                                                                  \
+    if (a.nt == NT && a.v == V) {                                                              \
+        if (a.aligned && a.merge == kMergeLocal) VKOP_ROWS_LAUNCH(NT, V, true, kMergeLocal);   \
+        else if (a.aligned && a.merge == kMergeByTicket) VKOP_ROWS_LAUNCH(NT, V, true, kMergeByTicket); \
+        else if (a.aligned) VKOP_ROWS_LAUNCH(NT, V, true, kMergeSplit);                        \
+        else if (a.merge == kMergeLocal) VKOP_ROWS_LAUNCH(NT, V, false, kMergeLocal);          \
+        else if (a.merge == kMergeByTicket) VKOP_ROWS_LAUNCH(NT, V, false, kMergeByTicket);    \
+        else VKOP_ROWS_LAUNCH(NT, V, false, kMergeSplit);                                      \
+        return true;                                                                           \
+    }
+    // one wave per row (short rows, small k): no barrier costs anything, nothing leaves the wave
+#define VKOP_ROWS_CASE_WAVE(V)                                                 \
+    if (a.nt == 64 && a.v == V && a.merge == kMergeLocal) {                    \
+        if (a.aligned) VKOP_ROWS_LAUNCH(64, V, true, kMergeLocal);             \
+        else VKOP_ROWS_LAUNCH(64, V, false, kMergeLocal);                      \
+        return true;                                                           \
+    }
+    VKOP_ROWS_CASE_WAVE(1)
+    VKOP_ROWS_CASE_WAVE(2)
+    VKOP_ROWS_CASE_WAVE(4)
+    if constexpr (sizeof(T) == 4) {
+        VKOP_ROWS_CASE_WAVE(8)
+    }
+#undef VKOP_ROWS_CASE_WAVE
+    VKOP_ROWS_CASE(256, 1)
+    VKOP_ROWS_CASE(256, 2)
+    VKOP_ROWS_CASE(256, 4)
+    VKOP_ROWS_CASE(512, 4)
+    VKOP_ROWS_CASE(1024, 4)
+    if constexpr (sizeof(T) == 4) {
+        VKOP_ROWS_CASE(256, 8)
+        VKOP_ROWS_CASE(512, 8)
+        VKOP_ROWS_CASE(1024, 8)
+    }
+#undef VKOP_ROWS_CASE
+#undef VKOP_ROWS_LAUNCH
+    return false;
+}
+
+template <typename T, bool SOFTMAX> void launch_rows_merge(const RowsLaunch &a) {
+    rows_merge_kernel<T, SOFTMAX><<<a.rows, kMergeThreads, 0, a.stream>>>(
+        static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, a.per, a.nt, a.ws);
+}
+
+template bool launch_rows_chunk<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
+template void launch_rows_merge<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
+
+}  // namespace vkop

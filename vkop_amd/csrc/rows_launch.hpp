@@ -1,0 +1,41 @@
+// Host-side launch of the streaming row kernels (kernels_rows.hpp).  Their many
+// instantiations (threads x loads x aligned x merge mode) are compiled one
+// translation unit per (element type, softmax or plain top-k), rows_inst.hip
+// built four times, so that the library builds in parallel; the C ABI source
+// only sees these declarations.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "kernels_rows.hpp"
+
+namespace vkop {
+
+struct RowsLaunch {
+    const void *in;
+    void *values;
+    int32_t *indices;
+    uint32_t rows, n, k;
+    uint32_t nt, v;    // threads per workgroup, 128-bit loads per thread
+    uint32_t g, per;   // chunks per row, elements per chunk
+    bool aligned;      // rows start on 16 bytes and n is a multiple of the vector width
+    int merge;         // kMergeSplit / kMergeByTicket / kMergeLocal
+    RowsWorkspace ws;
+    hipStream_t stream;
+};
+
+// Enqueues rows_chunk_kernel; false if no kernel is built for (nt, v).
+template <typename T, bool SOFTMAX> bool launch_rows_chunk(const RowsLaunch &a);
+// Enqueues rows_merge_kernel (after a chunk kernel launched with kMergeSplit).
+template <typename T, bool SOFTMAX> void launch_rows_merge(const RowsLaunch &a);
+
+extern template bool launch_rows_chunk<float, true>(const RowsLaunch &);
+extern template bool launch_rows_chunk<float, false>(const RowsLaunch &);
+extern template bool launch_rows_chunk<uint16_t, true>(const RowsLaunch &);
+extern template bool launch_rows_chunk<uint16_t, false>(const RowsLaunch &);
+extern template void launch_rows_merge<float, true>(const RowsLaunch &);
+extern template void launch_rows_merge<float, false>(const RowsLaunch &);
+extern template void launch_rows_merge<uint16_t, true>(const RowsLaunch &);
+extern template void launch_rows_merge<uint16_t, false>(const RowsLaunch &);
+
+}  // namespace vkop

@@ -1,5 +1,5 @@
 // C ABI of the softmax / top-k library (declared in include/vkop_hip.h):
-// argument checking, kernel selection and launches.  No kernel code lives here.
+// argument checking, kernel selection and launches (the only kernel here clears a workspace).
 #include "../../include/vkop_hip.h"
 
 #include <hip/hip_runtime.h>
@@ -12,8 +12,19 @@
 
 #include "kernels_general.hpp"
 #include "kernels_rows.hpp"
+#include "rows_launch.hpp"
 #include "kernels_softmax.hpp"
 #include "kernels_bigk.hpp"
+
+namespace vkop {
+
+// workspace clear (a kernel, not a memset: safe inside a captured graph)
+__global__ void fill_zero_kernel(uint32_t *p, size_t words) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < words) p[i] = 0u;
+}
+
+}  // namespace vkop
 
 namespace {
 
@@ -241,6 +252,8 @@ uint32_t rows_cap(int k) {
     return cap;
 }
 
+constexpr int kWaveRowMaxK = 32;  // largest k served by the one-wave-per-row launch
+
 RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     RowsCfg c;
     if (v.g.inner != 1 || k > vkop::kFastMaxK || v.g.n == 0 || v.g.outer == 0) return c;
@@ -261,9 +274,14 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
         const uint64_t span = static_cast<uint64_t>(nt) * vv * vec;
         return span * g >= n && static_cast<uint64_t>(rows) * g < (1ull << 31);
     };
+    // short rows and a small k: one wave per row (64 threads, up to 8 loads each)
+    const uint32_t wave_loads = (nvec + 63) / 64;
     if (forced_nt) {
         if (!fits(forced_nt, forced_v, static_cast<uint32_t>(forced_g))) return c;
         c.nt = forced_nt, c.v = forced_v, c.g = static_cast<uint32_t>(forced_g);
+    } else if (k <= kWaveRowMaxK && wave_loads <= (dtype == VKOP_HIP_F32 ? 8u : 4u)) {
+        c.nt = 64, c.g = 1;
+        c.v = wave_loads <= 1 ? 1 : wave_loads <= 2 ? 2 : wave_loads <= 4 ? 4 : 8;
     } else {
         // largest per-workgroup chunk that still leaves >= 1024 workgroups; if the
         // tensor is too small for that, the smallest shape that covers a row
@@ -404,42 +422,34 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
     w.cap = c.cap;
     w.cap_shift = c.cap_shift;
     const uint32_t vec = 16 / sizeof(T);
-    const bool aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
-    const uint32_t blocks = v.g.outer * c.g;
     // more rows than arrival counters: the merge runs as a kernel of its own
-    const bool fused = c.g == 1 || (g_rows_fused.load() != 0 && v.g.outer <= kTicketRows);
-    const int stages = fused ? 1 : g_rows_stages.load();
-#define VKOP_ROWS_LAUNCH(NT, V, AL, FU)                                                                         \
-    vkop::rows_chunk_kernel<T, NT, V, SOFTMAX, AL, FU>                                                          \
-        <<<blocks, NT, 0, st>>>(in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, w)
-#define VKOP_ROWS_CASE(NT, V)                                                                                   \
-    if (c.nt == NT && c.v == V) {                                                                               \
-        if (aligned && fused) VKOP_ROWS_LAUNCH(NT, V, true, true);                                              \
-        else if (aligned) VKOP_ROWS_LAUNCH(NT, V, true, false);                                                 \
-        else if (fused) VKOP_ROWS_LAUNCH(NT, V, false, true);                                                   \
-        else VKOP_ROWS_LAUNCH(NT, V, false, false);                                                             \
-        launched_one = true;                                                                                    \
-    }
-    bool launched_one = (stages & 1) == 0;
+    const bool by_ticket = g_rows_fused.load() != 0 && v.g.outer <= kTicketRows;
+    vkop::RowsLaunch a;
+    a.in = in;
+    a.values = values;
+    a.indices = indices;
+    a.rows = v.g.outer;
+    a.n = v.g.n;
+    a.k = static_cast<uint32_t>(k);
+    a.nt = static_cast<uint32_t>(c.nt);
+    a.v = static_cast<uint32_t>(c.v);
+    a.g = c.g;
+    a.per = c.per;
+    a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
+    // a row that one workgroup holds never leaves it: list and records stay in LDS
+    a.merge = (c.g == 1 && c.cap <= static_cast<uint32_t>(vkop::kLocalCap)) ? vkop::kMergeLocal
+              : (c.g == 1 || by_ticket)                                         ? vkop::kMergeByTicket
+                                                                                : vkop::kMergeSplit;
+    a.ws = w;
+    a.stream = st;
+    const int stages = a.merge != vkop::kMergeSplit ? 1 : g_rows_stages.load();
     if (stages & 1) {
-        VKOP_ROWS_CASE(256, 1)
-        VKOP_ROWS_CASE(256, 2)
-        VKOP_ROWS_CASE(256, 4)
-        VKOP_ROWS_CASE(512, 4)
-        VKOP_ROWS_CASE(1024, 4)
-        if constexpr (sizeof(T) == 4) {
-            VKOP_ROWS_CASE(256, 8)
-            VKOP_ROWS_CASE(512, 8)
-            VKOP_ROWS_CASE(1024, 8)
-        }
+        if (!vkop::launch_rows_chunk<T, SOFTMAX>(a))
+            return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
+        if (int rc = launched("rows_chunk_kernel")) return rc;
     }
-#undef VKOP_ROWS_CASE
-#undef VKOP_ROWS_LAUNCH
-    if (!launched_one) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
-    if (int rc = launched("rows_chunk_kernel")) return rc;
-    if (!fused && (stages & 2)) {
-        vkop::rows_merge_kernel<T, SOFTMAX><<<v.g.outer, vkop::kMergeThreads, 0, st>>>(
-            in, values, indices, v.g.n, static_cast<uint32_t>(k), c.g, c.per, static_cast<uint32_t>(c.nt), w);
+    if (a.merge == vkop::kMergeSplit && (stages & 2)) {
+        vkop::launch_rows_merge<T, SOFTMAX>(a);
         return launched("rows_merge_kernel");
     }
     return VKOP_HIP_OK;
