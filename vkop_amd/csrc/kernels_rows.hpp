@@ -256,6 +256,7 @@ struct RowsShared {  // merge phase
     uint32_t g0, xlo;                // tie at the cut: first rank of the tied group, smallest key in it
     uint32_t members;                // ... and how many of its members are in lane_key[] (their indices)
     uint32_t scan_counts[2 * 16];    // fill_group_by_scan: members per wave, double-buffered
+    uint32_t wave_thr[16];           // merge threshold: each wave's bound
     uint32_t lane_key[1024];
     uint32_t thr;
     uint32_t count;
@@ -575,15 +576,26 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
             cthr = static_cast<uint32_t>(c[u] >> 32);
         }
     }
+    // Slot s of the row's lists = entry (s mod cap) + 37 * chunk (mod cap) of chunk s / cap.
+    // A chunk fills its list from entry 0, so without the rotation the threads with a
+    // small (s mod cap) would hold every live candidate and the others none; with
+    // it each thread's slots spread over the positions, every thread holds a few
+    // live candidates, and the per-thread maxima below bound the row's (k+1)-th
+    // largest much more tightly (fewer candidates left to rank).
+    auto slot_pos = [&](uint32_t s) { return ((s & (cap - 1)) + 37u * (s >> cap_shift)) & (cap - 1); };
     uint64_t cv[ES];
 #pragma unroll
     for (int e = 0; e < ES; e++) {
         const uint32_t s = static_cast<uint32_t>(e) * NT + tid;
-        cv[e] = fetch(cand + (s < slots ? s : 0u));
+        cv[e] = fetch(cand + (s < slots ? (s & ~(cap - 1)) + slot_pos(s) : 0u));
     }
 
     // ---- B. the row's maximum and sum from the wave partials --------------------------
     for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;  // for block_rank, barriers away
+    if (tid == 0) {
+        sh.count = 0;
+        sh.flag = 0;
+    }
     bool bad = false;
     SumPartial p0{0.0, 0.f, -INFINITY};
     if (tid < waves) {
@@ -611,24 +623,41 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
 #pragma unroll
     for (int e = 0; e < ES; e++) {
         const uint32_t s = static_cast<uint32_t>(e) * NT + tid;
-        const bool live = s < slots && (s & (cap - 1)) < sh.cnt[s < slots ? (s >> cap_shift) : 0u];
+        const bool live = s < slots && slot_pos(s) < sh.cnt[s < slots ? (s >> cap_shift) : 0u];
         if (!live) cv[e] = 0;
         lmk = max(lmk, static_cast<uint32_t>(cv[e] >> 32));
     }
+    // Every wave takes, by a ballot descent over its own 64 thread maxima (18 bits),
+    // the largest value that its share of k+1 of them reach: the smallest of
+    // these bounds is reached by k+1 thread maxima in all, hence by k+1
+    // candidates.  (The rotation above keeps the waves alike, so little is lost
+    // against the exact (k+1)-th largest.)  A share of more than half a wave, or a
+    // wave without enough live threads, leaves it to one wave and all the maxima.
+    const uint32_t quota = (want + NW - 1) / NW;
+    uint32_t mine_q = 0;
+    if (G > 1 && quota <= 32u) {
+        for (int bit = 31; bit > 13; bit--) {
+            const uint32_t trial = mine_q | (1u << bit);
+            if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= quota) mine_q = trial;
+        }
+    }
     sh.lane_key[tid] = lmk;
-    if (tid == 0) {
-        sh.count = 0;
-        sh.flag = 0;
-    }
+    if (lane == 0) sh.wave_thr[wave] = mine_q;
+    if (bad) sh.flag = 1;  // every writer stores the same value (cleared before the barriers of B)
     __syncthreads();
-    if (bad) sh.flag = 1;  // every writer stores the same value
+    uint32_t thr = sh.wave_thr[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) thr = min(thr, sh.wave_thr[w]);
     // (a single chunk's list is already cut at that chunk's threshold: everything in it is taken)
-    if (G > 1 && wave == 0) {
-        const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
-        if (lane == 0) sh.thr = t > 1u ? t : 1u;  // key 0 is "no element"
+    if (G > 1 && thr <= 1u) {  // (the same for every thread)
+        if (wave == 0) {
+            const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
+            if (lane == 0) sh.thr = t > 1u ? t : 1u;  // key 0 is "no element"
+        }
+        __syncthreads();
+        thr = sh.thr;
     }
-    __syncthreads();  // (sh.flag as well)
-    const uint32_t thr = G > 1 ? sh.thr : 1u;
+    if (G == 1) thr = 1u;
     uint32_t merge_thr = thr;  // candidates with keys at or above it are in sh.cand (of equal keys maybe only the first)
     bool slow = sh.flag != 0u;
     uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
