@@ -678,3 +678,24 @@ def test_awkward_rows_against_the_oracle(ops, n, k):
             et, ej = oracle.topk(x, k, -1, largest)
             bits = np.uint16 if dtype == np.float16 else np.uint32
             assert np.array_equal(host(j), ej) and np.array_equal(host(t).view(bits), et.view(bits)), (n, k, largest)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("n,k", [(8400, 300), (8400, 255), (8400, 256), (8400, 408), (8400, 409), (32768, 400), (1200, 100),
+                                 (300, 299)])
+def test_large_k_on_rows_one_workgroup_holds(ops, dtype, n, k):
+    """k beyond the merge kernel's 255 ranks (and large k in general) on rows short
+    enough for one workgroup: [16,8400] k = 300 is the detection workload's select."""
+    rng = np.random.default_rng(n * 7 + k)
+    x = rng.random((16, n)).astype(np.float32)
+    x[1] = np.round(x[1] * 50) / 50            # heavy ties
+    x[2] = np.sort(x[2])
+    x[3, : n // 2] = -np.inf
+    x[4] = 0.5
+    x = np.ascontiguousarray(x.astype(dtype))
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    for largest in (True, False):
+        t, j = ops.topk(dev(x), k, -1, largest)
+        et, ej = oracle.topk(x, k, -1, largest)
+        assert np.array_equal(host(j), ej) and np.array_equal(host(t).view(bits), et.view(bits)), (n, k, largest)
+    assert_fused(ops, x * 8, k)

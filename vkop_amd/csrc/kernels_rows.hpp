@@ -48,7 +48,8 @@
 namespace vkop {
 
 constexpr int kFastCap = 1024;       // LDS slots for elements above the merge threshold
-constexpr int kFastMaxK = 255;       // k + 1 <= 256 ranks are kept in LDS
+constexpr int kFastMaxK = 511;       // k + 1 <= 512 ranks are kept in LDS (the merging workgroup has a thread per rank:
+                                     // k <= 255 for rows_merge_kernel, more only where one larger workgroup holds the row)
 constexpr int kMergeThreads = 256;    // rows_merge_kernel workgroup
 constexpr int kMergeRecsMax = 4096;   // candidate slots per row the merge takes in registers
 constexpr int kMergeWavesMax = 256;   // chunk-kernel waves per row the merge can combine

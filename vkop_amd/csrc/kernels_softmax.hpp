@@ -11,10 +11,9 @@
 //                           read of the input comes from the Infinity Cache for
 //                           tensors that fit it.
 // Strided lines (another axis, short lines):
-//   softmax_strided_lds_kernel  one thread per line, threads along the
-//                           contiguous inner axis; the line's elements are staged
-//                           in LDS ([element][thread], conflict free), so the
-//                           input is read once and the loops stay loops.
+//   softmax_strided_reg_kernel  one thread per line, threads along the
+//                           contiguous inner axis; the line's elements stay in
+//                           registers, so the input is read once.
 // All of them produce what kernels_general.hpp defines: terms exp_accurate(x - M),
 // the sum in double, one rounding of term * (1 / sum).  The chunked variant sums
 // hardware-exp terms (argument scaled with a two-part log2 e, so the scaling adds
@@ -207,78 +206,89 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
     }
 }
 
-// ---- short strided lines, staged in LDS --------------------------------------------------
-// One thread per line; n <= kStridedMaxN.  Dynamic LDS: n * NT floats.
+// ---- short strided lines held in registers -------------------------------------------------
+// Lines along a non-last axis with n <= kStridedMaxN elements (scores laid out
+// [batch, classes, anchors]: softmax over the classes).  Lanes run along the
+// contiguous inner axis, so every load is a coalesced piece of a row of the slab.
+// P lanes of a wave share a line (lane l and l + 64/P, ...: element j belongs to
+// part j mod P), each keeps its part in registers: one read of the input, no LDS,
+// and enough waves to hide the loads and the exponentials even when the lines
+// are few (one thread per line left two waves per SIMD on [16,80,8400]; staging
+// the lines in LDS, the first version, no more).  NMAX: compile-time bound of n,
+// a multiple of 16 and of P (the loops are unrolled over NMAX / P and masked).
 constexpr int kStridedThreads = 128;
 constexpr int kStridedMaxN = 128;
 
 // MAX_ONLY: instead of the softmax tensor write, per line, its largest entry --
 // the probability of the line's maximum, (float)(exp_accurate(0) / S) -- to
 // out[line]: softmax followed by a max over the same axis, in one read.
-template <typename T, bool MAX_ONLY>
-__global__ __launch_bounds__(kStridedThreads) void softmax_strided_lds_kernel(const T *in, T *out, LineGeom g,
+template <typename T, int NMAX, int P, bool MAX_ONLY>
+__global__ __launch_bounds__(kStridedThreads) void softmax_strided_reg_kernel(const T *in, T *out, LineGeom g,
                                                                               int nan_where, float nan_value) {
-    constexpr int NT = kStridedThreads;
-    extern __shared__ float stage[];  // [n][NT]
-    const uint32_t tid = threadIdx.x;
-    const uint32_t line = blockIdx.x * NT + tid;
-    const bool live = line < g.outer * g.inner;
-    const size_t base = live ? g.base(line) : 0;
-    // loads in batches of sixteen, all in flight before the first use
+    constexpr int LPW = kWave / P;  // lines per wave
+    constexpr int NPER = NMAX / P;  // elements per lane
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t part = lane / LPW;
+    const uint32_t wave_id = (blockIdx.x * kStridedThreads + threadIdx.x) / kWave;
+    const uint32_t lines = g.outer * g.inner;
+    const uint32_t line_raw = wave_id * LPW + (lane % LPW);
+    const bool live = line_raw < lines;
+    const uint32_t line = live ? line_raw : 0u;  // (idle lanes shadow line 0 and store nothing)
+    const size_t base = g.base(line);
+    const uint32_t n = g.n;
+    float x[NPER];
+    // every load in flight before the first use (slots past the line re-read element 0)
+#pragma unroll
+    for (int i = 0; i < NPER; i++) {
+        const uint32_t j = static_cast<uint32_t>(i) * P + part;
+        x[i] = load_elem(in, base + static_cast<size_t>(j < n ? j : 0u) * g.inner);
+    }
     float m = -INFINITY;
-    for (uint32_t j0 = 0; j0 < g.n; j0 += 16) {
-        float x[16];
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
-            const uint32_t j = j0 + u < g.n ? j0 + u : 0u;
-            x[u] = load_elem(in, base + static_cast<size_t>(j) * g.inner);
-        }
+    for (int i = 0; i < NPER; i++)
+        if (static_cast<uint32_t>(i) * P + part < n) m = fmaxf(m, x[i]);
 #pragma unroll
-        for (int u = 0; u < 16; u++) {
-            if (j0 + u < g.n) {
-                stage[(j0 + u) * NT + tid] = x[u];
-                m = fmaxf(m, x[u]);
-            }
-        }
-    }
-    // four independent exponentials in flight per thread (few waves fit beside
-    // this much LDS, so the instruction-level parallelism has to come from here);
-    // the sum itself stays in index order
+    for (int o = LPW; o < kWave; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, kWave));
+    // terms replace the elements; the parts' sums are added in a fixed order
     double s = 0.0;
-    uint32_t j4 = 0;
-    for (; j4 + 4 <= g.n; j4 += 4) {
-        float e[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) e[u] = softmax_term(stage[(j4 + u) * NT + tid], m);
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            stage[(j4 + u) * NT + tid] = e[u];
-            s += static_cast<double>(e[u]);
+    for (int i = 0; i < NPER; i++) {
+        if (static_cast<uint32_t>(i) * P + part < n) {
+            x[i] = softmax_term(x[i], m);
+            s += static_cast<double>(x[i]);
         }
     }
-    for (uint32_t j = j4; j < g.n; j++) {
-        const float e = softmax_term(stage[j * NT + tid], m);
-        stage[j * NT + tid] = e;
-        s += static_cast<double>(e);
-    }
+#pragma unroll
+    for (int o = LPW; o < kWave; o <<= 1) s += __shfl_xor(s, o, kWave);
     const double rinv = 1.0 / s;
-    if (!live) return;
     if constexpr (MAX_ONLY) {
         // the largest term is exp_accurate(0) = 1 unless the line holds no finite maximum
         float top = 0.f;
-        for (uint32_t j = 0; j < g.n; j++) {
-            const float e = stage[j * NT + tid];
-            top = (e != e) ? e : ((top != top) ? top : fmaxf(top, e));  // NaN propagates
+#pragma unroll
+        for (int i = 0; i < NPER; i++) {
+            if (static_cast<uint32_t>(i) * P + part < n) {
+                const float e = x[i];
+                top = (e != e) ? e : ((top != top) ? top : fmaxf(top, e));  // NaN propagates
+            }
+        }
+#pragma unroll
+        for (int o = LPW; o < kWave; o <<= 1) {
+            const float other = __shfl_xor(top, o, kWave);
+            top = (other != other) ? other : ((top != top) ? top : fmaxf(top, other));
         }
         float p = round_to_storage<T>(static_cast<float>(static_cast<double>(top) * rinv));
         if (nan_where && p != p) p = nan_value;
-        store_elem(out, line, p);
+        if (live && part == 0) store_elem(out, line, p);
         return;
     }
-    for (uint32_t j = 0; j < g.n; j++) {
-        float p = round_to_storage<T>(static_cast<float>(static_cast<double>(stage[j * NT + tid]) * rinv));
-        if (nan_where && p != p) p = nan_value;
-        store_elem(out, base + static_cast<size_t>(j) * g.inner, p);
+#pragma unroll
+    for (int i = 0; i < NPER; i++) {
+        const uint32_t j = static_cast<uint32_t>(i) * P + part;
+        if (live && j < n) {
+            float p = round_to_storage<T>(static_cast<float>(static_cast<double>(x[i]) * rinv));
+            if (nan_where && p != p) p = nan_value;
+            store_elem(out, base + static_cast<size_t>(j) * g.inner, p);
+        }
     }
 }
 

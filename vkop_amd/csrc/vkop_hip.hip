@@ -118,11 +118,34 @@ const RowShape kShapesF32[] = {{256, 1}, {256, 2}, {256, 4}, {256, 8}, {512, 8},
 const RowShape kShapesF16[] = {{256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}, {1024, 4}};
 
 struct SoftmaxPlan {
-    enum Kind { kGeneralLines, kGeneralStrided, kRow, kChunked, kStridedLds } kind = kGeneralLines;
+    enum Kind { kGeneralLines, kGeneralStrided, kRow, kChunked, kStridedRegs } kind = kGeneralLines;
     RowShape shape{0, 0};
     uint32_t g = 1, per = 0;
     size_t workspace = 0;
 };
+
+// Lines of up to kStridedMaxN elements along a non-last axis, held in registers: the
+// kernel is compiled for a few bounds of n and the smallest that fits is launched;
+// longer lines are shared by two or four lanes.
+template <typename T, bool MAX_ONLY>
+void launch_strided_reg(const T *in, T *out, const View &v, int nan_where, float nan_value, hipStream_t st) {
+    const uint32_t lines = v.g.outer * v.g.inner;
+#define VKOP_STRIDED_CASE(NMAX, P)                                                          \
+    if (v.g.n <= NMAX) {                                                                    \
+        const uint32_t per_block = vkop::kStridedThreads / P;                               \
+        vkop::softmax_strided_reg_kernel<T, NMAX, P, MAX_ONLY>                              \
+            <<<(lines + per_block - 1) / per_block, vkop::kStridedThreads, 0, st>>>(in, out, v.g, nan_where, nan_value); \
+        return;                                                                             \
+    }
+    VKOP_STRIDED_CASE(16, 1)
+    VKOP_STRIDED_CASE(32, 2)
+    VKOP_STRIDED_CASE(48, 4)
+    VKOP_STRIDED_CASE(64, 4)
+    VKOP_STRIDED_CASE(80, 4)
+    VKOP_STRIDED_CASE(96, 4)
+    VKOP_STRIDED_CASE(128, 4)
+#undef VKOP_STRIDED_CASE
+}
 
 SoftmaxPlan plan_softmax(const View &v, int dtype) {
     SoftmaxPlan p;
@@ -130,7 +153,7 @@ SoftmaxPlan plan_softmax(const View &v, int dtype) {
     const RowShape *shapes = dtype == VKOP_HIP_F32 ? kShapesF32 : kShapesF16;
     const uint32_t n = v.g.n, rows = v.g.outer;
     if (v.g.inner != 1) {
-        if (n <= static_cast<uint32_t>(vkop::kStridedMaxN)) p.kind = SoftmaxPlan::kStridedLds;
+        if (n <= static_cast<uint32_t>(vkop::kStridedMaxN)) p.kind = SoftmaxPlan::kStridedRegs;
         else p.kind = n >= 2048 ? SoftmaxPlan::kGeneralLines : SoftmaxPlan::kGeneralStrided;
         return p;
     }
@@ -213,11 +236,9 @@ int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, f
         if (!done) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no chunked softmax for %d x %d", p.shape.nt, p.shape.v);
         return launched("softmax_stats_kernel / softmax_scale_kernel");
     }
-    case SoftmaxPlan::kStridedLds: {
-        const uint32_t blocks = (lines + vkop::kStridedThreads - 1) / vkop::kStridedThreads;
-        const size_t lds = static_cast<size_t>(v.g.n) * vkop::kStridedThreads * sizeof(float);
-        vkop::softmax_strided_lds_kernel<T, false><<<blocks, vkop::kStridedThreads, lds, st>>>(in, out, v.g, nan_where, nan_value);
-        return launched("softmax_strided_lds_kernel");
+    case SoftmaxPlan::kStridedRegs: {
+        launch_strided_reg<T, false>(in, out, v, nan_where, nan_value, st);
+        return launched("softmax_strided_reg_kernel");
     }
     case SoftmaxPlan::kGeneralLines:
         vkop::softmax_lines_kernel<T, kLineThreads>
@@ -253,6 +274,7 @@ uint32_t rows_cap(int k) {
 }
 
 constexpr int kWaveRowMaxK = 32;  // largest k served by the one-wave-per-row launch
+constexpr int kWideRowMinK = 64;  // above it a row that fits one workgroup is given to one (of enough threads)
 
 RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     RowsCfg c;
@@ -276,7 +298,23 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     };
     // short rows and a small k: one wave per row (64 threads, up to 8 loads each)
     const uint32_t wave_loads = (nvec + 63) / 64;
-    if (forced_nt) {
+    // A large k on a row that one workgroup can hold: that workgroup takes the whole
+    // row, list in LDS, if it has at least 2 (k + 1) threads (its waves share the
+    // staging of the candidates, 64 vectors each, and the ranking; several chunks of
+    // 256 threads would hand a merge of 256 threads more candidates than it ranks
+    // quickly).  Beyond 255 ranks it is the only way: the merge kernel has a thread
+    // per rank.
+    int wide = -1;
+    if (cap <= static_cast<uint32_t>(vkop::kLocalCap)) {
+        for (int i = 0; i < 6 && wide < 0; i++) {
+            const uint64_t span = static_cast<uint64_t>(shapes[i][0]) * shapes[i][1] * vec;
+            if (span >= n && shapes[i][0] >= 2 * (k + 1)) wide = i;
+        }
+    }
+    if (k > vkop::kMergeThreads - 1 && wide < 0) return c;
+    if (wide >= 0 && (k > vkop::kMergeThreads - 1 || (k > kWideRowMinK && !forced_nt))) {
+        c.nt = shapes[wide][0], c.v = shapes[wide][1], c.g = 1;
+    } else if (forced_nt) {
         if (!fits(forced_nt, forced_v, static_cast<uint32_t>(forced_g))) return c;
         c.nt = forced_nt, c.v = forced_v, c.g = static_cast<uint32_t>(forced_g);
     } else if (k <= kWaveRowMaxK && wave_loads <= (dtype == VKOP_HIP_F32 ? 8u : 4u)) {
@@ -525,10 +563,8 @@ template <typename T>
 int softmax_reduce_max_impl(const T *in, T *out, const View &v, void *ws, size_t ws_bytes, hipStream_t st) {
     const uint32_t lines = v.g.outer * v.g.inner;
     if (v.g.n <= static_cast<uint32_t>(vkop::kStridedMaxN)) {
-        const uint32_t blocks = (lines + vkop::kStridedThreads - 1) / vkop::kStridedThreads;
-        const size_t lds = static_cast<size_t>(v.g.n) * vkop::kStridedThreads * sizeof(float);
-        vkop::softmax_strided_lds_kernel<T, true><<<blocks, vkop::kStridedThreads, lds, st>>>(in, out, v.g, 0, 0.f);
-        return launched("softmax_strided_lds_kernel");
+        launch_strided_reg<T, true>(in, out, v, 0, 0.f, st);
+        return launched("softmax_strided_reg_kernel");
     }
     // longer lines: the line statistics, then exp_accurate(0) / S per line
     const size_t need = kTicketBytes + align_up(static_cast<size_t>(lines) * sizeof(vkop::LineStats));
