@@ -96,19 +96,42 @@ __global__ __launch_bounds__(NT) void softmax_strided_kernel(const T *in, T *out
 }
 
 // ---- max along an axis ------------------------------------------------------
+// Strided lines: lanes run along the contiguous inner axis (coalesced rows of the
+// slab); four lanes of a wave share a line (lane l, l + 16, l + 32, l + 48 take
+// every fourth element), eight loads in flight per lane, so that few and short
+// lines still keep the memory system busy.
 template <typename T, int NT>
 __global__ __launch_bounds__(NT) void reduce_max_strided_kernel(const T *__restrict__ in, T *out, LineGeom g) {
-    const uint32_t line = blockIdx.x * NT + threadIdx.x;
-    if (line >= g.outer * g.inner) return;
-    const size_t base = g.base(line);
+    constexpr uint32_t P = 4, LPW = kWave / P, U = 8;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t part = lane / LPW;
+    const uint32_t wave_id = (blockIdx.x * NT + threadIdx.x) / kWave;
+    const uint32_t lines = g.outer * g.inner;
+    const uint32_t line_raw = wave_id * LPW + (lane % LPW);
+    const bool live = line_raw < lines;
+    const size_t base = g.base(live ? line_raw : 0u);
     float m = -INFINITY;
     bool nan = false;
-    for (uint32_t j = 0; j < g.n; j++) {
-        const float v = load_elem(in, base + static_cast<size_t>(j) * g.inner);
-        nan |= (v != v);
-        m = fmaxf(m, v);
+    for (uint32_t j0 = part; j0 < g.n; j0 += P * U) {
+        float v[U];
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) {
+            const uint32_t j = j0 + u * P;
+            v[u] = load_elem(in, base + static_cast<size_t>(j < g.n ? j : part) * g.inner);  // (re-reads one of its own)
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) {
+            nan |= (v[u] != v[u]);
+            m = fmaxf(m, v[u]);
+        }
     }
-    store_elem(out, line, nan ? __uint_as_float(0x7FC00000u) : m);
+    float nanf = nan ? 1.f : 0.f;
+#pragma unroll
+    for (uint32_t o = LPW; o < kWave; o <<= 1) {
+        m = fmaxf(m, __shfl_xor(m, o, kWave));
+        nanf = fmaxf(nanf, __shfl_xor(nanf, o, kWave));
+    }
+    if (live && part == 0) store_elem(out, line_raw, nanf != 0.f ? __uint_as_float(0x7FC00000u) : m);
 }
 
 template <typename T, int NT>

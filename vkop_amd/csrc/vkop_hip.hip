@@ -583,7 +583,8 @@ template <typename T> int reduce_max_impl(const T *in, T *out, const View &v, hi
         vkop::reduce_max_lines_kernel<T, kLineThreads><<<lines, kLineThreads, 0, st>>>(in, out, v.g);
         return launched("reduce_max_lines_kernel");
     }
-    const uint32_t blocks = (lines + kLineThreads - 1) / kLineThreads;
+    const uint32_t per_block = kLineThreads / 4;  // four lanes per line
+    const uint32_t blocks = (lines + per_block - 1) / per_block;
     vkop::reduce_max_strided_kernel<T, kLineThreads><<<blocks, kLineThreads, 0, st>>>(in, out, v.g);
     return launched("reduce_max_strided_kernel");
 }
