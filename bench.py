@@ -42,7 +42,8 @@ WORKLOADS = {
     "C2": ("[256,1000] f32 softmax+topk k=5", dict(kind="cls", rows=256, cols=1000), 5),
     "C3": ("[64,128256] f32 softmax+topk k=50", dict(kind="llm", rows=64, cols=128256), 50),
     "C4": ("[8,262144] f32 softmax+topk k=1024", dict(kind="grid", rows=8, cols=262144), 1024),
-    # not a BASELINE config: C3's logits truncated to bfloat16 precision (what a bf16 LM head hands over);
+    # a variant of C3, not one of the reference's configurations: its logits truncated to bfloat16 precision
+    # (what a bf16 LM head hands over);
     # equal logits then straddle the k-th place in most rows and the merge settles a tie per row
     "C3bf16": ("[64,128256] f32 softmax+topk k=50, bf16-valued logits", dict(kind="llm_bf16", rows=64, cols=128256), 50),
 }
