@@ -256,6 +256,7 @@ struct RowsShared {  // merge phase
     uint32_t pkey[kFastMaxK + 1];    // order key of the logit, by rank
     uint32_t g0, xlo;                // tie at the cut: first rank of the tied group, smallest key in it
     uint32_t members;                // ... and how many of its members are in lane_key[] (their indices)
+    float row_max;                   // the row's maximum; its sum of terms is `total`
     uint32_t scan_counts[2 * 16];    // fill_group_by_scan: members per wave, double-buffered
     uint32_t wave_thr[16];           // merge threshold: each wave's bound
     uint32_t lane_key[1024];
@@ -610,22 +611,46 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         sh.cthr[tid] = cthr;
         bad = cm > cap;
     }
-    const float M = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.cnt and sh.ref are published)
-    double acc = 0.0;
-    if (tid < waves) {
-        const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(M));
-        sh.scale[tid] = sc;
-        if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
+    // With at most 64 wave records (one per lane of wave 0) that wave alone combines
+    // them, by cross-lane steps, while the others go on to the threshold; the
+    // results are published by the barrier there.
+    if (waves <= static_cast<uint32_t>(kWave)) {
+        if (wave == 0) {
+            const float m = wave_max_f32_uniform(p0.m);
+            double acc = 0.0;
+            if (tid < waves) {
+                const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+                sh.scale[tid] = sc;
+                if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
+            }
+            const double total = wave_sum_f64_uniform(acc);
+            if (lane == 0) {
+                sh.row_max = m;
+                sh.total = total;
+            }
+        }
+    } else {
+        const float m = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.ref is published)
+        double acc = 0.0;
+        if (tid < waves) {
+            const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+            sh.scale[tid] = sc;
+            if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
+        }
+        const double total = block_sum_fast<NT>(acc, dscratch);  // (barrier: sh.scale is published)
+        if (tid == 0) {
+            sh.row_max = m;
+            sh.total = total;
+        }
     }
-    const double s_base = block_sum_fast<NT>(acc, dscratch);  // (barrier: sh.scale is published)
 
     // ---- C. threshold: the (k+1)-th largest per-thread maximum -------------------------
     uint32_t lmk = 0;
 #pragma unroll
     for (int e = 0; e < ES; e++) {
-        const uint32_t s = static_cast<uint32_t>(e) * NT + tid;
-        const bool live = s < slots && slot_pos(s) < sh.cnt[s < slots ? (s >> cap_shift) : 0u];
-        if (!live) cv[e] = 0;
+        // (the unused entries of a list are 0, the chunk kernel sees to that; slots past
+        // the row's lists were read from entry 0)
+        if (static_cast<uint32_t>(e) * NT + tid >= slots) cv[e] = 0;
         lmk = max(lmk, static_cast<uint32_t>(cv[e] >> 32));
     }
     // Every wave takes, by a ballot descent over its own 64 thread maxima (18 bits),
@@ -646,6 +671,8 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     if (lane == 0) sh.wave_thr[wave] = mine_q;
     if (bad) sh.flag = 1;  // every writer stores the same value (cleared before the barriers of B)
     __syncthreads();
+    const float M = sh.row_max;
+    const double s_base = sh.total;
     uint32_t thr = sh.wave_thr[0];
 #pragma unroll
     for (int w = 1; w < NW; w++) thr = min(thr, sh.wave_thr[w]);
@@ -1273,7 +1300,11 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             }
             __syncthreads();
             wave_candidates = compact(thr, staged, std::true_type{}, cs.thr);
+            __syncthreads();  // (cs.total is final)
         }
+        // the unused entries of the list read as "no element": the merge tells live
+        // candidates from stale ones by that alone
+        for (uint32_t p = min(cs.total, ws.cap) + tid; p < ws.cap; p += NT) publish(cand_out + p, 0ull);
 
         // ---- 5. the chunk's threshold and the wave's candidate count -------------------------------
         if (lane == 0) {
