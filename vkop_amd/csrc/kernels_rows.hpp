@@ -703,15 +703,33 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
 
     if (!slow) {
         // ---- D. the candidates reaching the threshold go to LDS ------------------------
+        // (counted per wave with ballots first, so that every one has its place
+        // without an atomic and its wait)
+        uint32_t wave_n = 0;  // wave-uniform
+#pragma unroll
+        for (int e = 0; e < ES; e++)
+            wave_n += static_cast<uint32_t>(__popcll(__ballot(static_cast<uint32_t>(cv[e] >> 32) >= thr)));
+        if (lane == 0) sh.scan_counts[wave] = wave_n;
+        __syncthreads();
+        uint32_t C2 = 0, pos = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const uint32_t c = sh.scan_counts[w];
+            pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
+            C2 += c;
+        }
+        if (tid == 0) sh.count = C2;
 #pragma unroll
         for (int e = 0; e < ES; e++) {
-            if (static_cast<uint32_t>(cv[e] >> 32) >= thr) {
-                const uint32_t pos = atomicAdd(&sh.count, 1u);
-                if (pos < kFastCap) sh.cand[pos] = cv[e];
+            const bool pass = static_cast<uint32_t>(cv[e] >> 32) >= thr;
+            const uint64_t mask = __ballot(pass);
+            if (mask != 0ull) {
+                const uint32_t p = pos + lanes_below(mask);
+                if (pass && p < kFastCap) sh.cand[p] = cv[e];
+                pos += static_cast<uint32_t>(__popcll(mask));
             }
         }
         __syncthreads();
-        uint32_t C2 = sh.count;
         if (C2 > kFastCap) {
             // Too many reach the threshold (it comes from per-thread maxima and is
             // rounded down; rows full of equal values).  Take the exact cut over all
