@@ -546,9 +546,9 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
     constexpr int ES = RECS / NT;  // candidate slots per thread
-    // one thread per wave partial and per chunk (a workgroup that merges only its own
-    // row, RECS = kLocalCap, has one chunk and NT / 64 waves)
-    static_assert(RECS == kLocalCap || (NT >= kMergeWavesMax && NT >= kMergeChunksMax), "merge workgroup too small");
+    // (the caller sees to it that there is a thread per wave record and per chunk:
+    // G * src_nt / 64 <= NT and G <= NT)
+    static_assert(RECS % NT == 0, "whole slots per thread");
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t want = k + 1;
     const uint32_t kk = min(k, n);
@@ -1377,7 +1377,9 @@ union MergeShared {
 };
 
 // Second kernel of the unfused variant: one workgroup of kMergeThreads per row.
-template <typename T, bool SOFTMAX>
+// RECS: candidate slots it takes in, at least G * cap (1024, 2048 or kMergeRecsMax:
+// the smallest that holds the row's lists keeps the per-thread loops short).
+template <typename T, bool SOFTMAX, int RECS>
 __global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                                    int32_t *__restrict__ indices, uint32_t n,
                                                                    uint32_t k, uint32_t G, uint32_t per,
@@ -1386,7 +1388,7 @@ __global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__re
     __shared__ float fscratch[kMergeThreads / kWave];
     __shared__ double dscratch[kMergeThreads / kWave];
     const uint32_t row = blockIdx.x;
-    merge_row<T, kMergeThreads, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, in + static_cast<size_t>(row) * n,
+    merge_row<T, kMergeThreads, SOFTMAX, RECS>(smem.fast, smem.exact, fscratch, dscratch, in + static_cast<size_t>(row) * n,
                                          values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k,
                                          n, k, G, per, src_nt,
                                          ws.sums + 3 * static_cast<size_t>(row) * G * (src_nt / kWave),

@@ -55,8 +55,14 @@ template <typename T, bool SOFTMAX> bool launch_rows_chunk(const RowsLaunch &a) 
 }
 
 template <typename T, bool SOFTMAX> void launch_rows_merge(const RowsLaunch &a) {
-    rows_merge_kernel<T, SOFTMAX><<<a.rows, kMergeThreads, 0, a.stream>>>(
-        static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, a.per, a.nt, a.ws);
+    const uint32_t slots = a.g << a.ws.cap_shift;
+#define VKOP_MERGE_LAUNCH(RECS)                                               \
+    rows_merge_kernel<T, SOFTMAX, RECS><<<a.rows, kMergeThreads, 0, a.stream>>>( \
+        static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, a.per, a.nt, a.ws)
+    if (slots <= 1024) VKOP_MERGE_LAUNCH(1024);
+    else if (slots <= 2048) VKOP_MERGE_LAUNCH(2048);
+    else VKOP_MERGE_LAUNCH(kMergeRecsMax);
+#undef VKOP_MERGE_LAUNCH
 }
 
 template bool launch_rows_chunk<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
