@@ -1021,12 +1021,13 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         const float wm = wave_max_f32_uniform(lmax);
         double wsum = 0.0;
         if constexpr (SOFTMAX) wsum = wave_sum_f64_uniform(acc);
-        if constexpr (FULL) {
+        {
             // Every wave finds the q-th largest of its own 64 lane maxima, q = its share
             // of k+1.  The (k+1)-th largest lane maximum of the whole workgroup lies
             // between the smallest and the largest of these, so every wave then
             // settles the few bits in which the two differ over all lane maxima
-            // (all waves compute the same value: no broadcast).
+            // (all waves compute the same value: no broadcast).  A wave short of lane
+            // maxima (a ragged chunk) reports 0, which only widens that search.
             const uint32_t quota = (want + NW - 1) / NW;
             uint32_t mine_q = 0;
             if (quota <= static_cast<uint32_t>(kWave)) {
@@ -1060,17 +1061,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 }
             }
             thr_block = t;
-        } else {
-            // ragged chunk: some waves may hold few elements or none, so one wave takes
-            // the (k+1)-th largest of all lane maxima
-            cs.lane_key[tid] = lkey;
-            __syncthreads();
-            if (wave == blockIdx.x % NW) {
-                const uint32_t t = block_kth_largest_floor<NW>(cs.lane_key, want, 16);
-                if (lane == 0) cs.thr = t;
-            }
-            __syncthreads();
-            thr_block = cs.thr;
         }
         // -inf never becomes a candidate: a row with k+1 larger elements does not
         // need it, and any other row is left to the exact path
