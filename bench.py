@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by the same counters over a copy kernel
 # of known size (profiles/ holds the runs); None = not measured for the workload.
-TRAFFIC = {"C3": 33972605}   # rows_chunk_kernel: 32997814 B read + 974792 B written
+TRAFFIC = {"C3": 34599831}   # rows_chunk_kernel: 33011902 B read + 1587929 B written
 
 WORKLOADS = {
     # name: (description, generator kwargs, k, axis)
