@@ -127,6 +127,8 @@ def main():
                     help="hardware queues this process may use (GPU_MAX_HW_QUEUES); 0 = leave the environment as it is")
     ap.add_argument("--inflight", type=int, default=0,
                     help="independent calls in flight (each on its own stream with its own workspace and outputs)")
+    ap.add_argument("--launch-shape", default="",
+                    help="threads,loads,chunks for the streaming kernel instead of the library's choice (experiments)")
     ap.add_argument("--fused", action="store_true",
                     help="run the streaming path as one kernel (the last chunk of a row merges it) instead of two")
     ap.add_argument("--eager", action="store_true",
@@ -157,6 +159,9 @@ def main():
     capi.lib()
     capi.init(0)
     capi.tune("rows.fused", 1 if args.fused else 0)
+    if args.launch_shape:
+        for name, value in zip(("rows.threads", "rows.loads", "rows.chunks"), args.launch_shape.split(",")):
+            capi.tune(name, int(value))
     desc, spec, k = WORKLOADS[args.workload]
     rows, cols = spec["rows"], spec["cols"]
     shape = (rows, cols)
