@@ -48,6 +48,8 @@ def lib():
         L.vkop_oracle_reduce_max_f32.argtypes = [vp, vp, c_int, c_int, c_int]
         L.vkop_oracle_get_top_k_predictions.restype = c_int
         L.vkop_oracle_get_top_k_predictions.argtypes = [vp, c_int, c_int, vp, vp]
+        L.vkop_oracle_nms_f32.restype = c_int
+        L.vkop_oracle_nms_f32.argtypes = [vp, vp, vp, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int]
         _lib = L
     return _lib
 
@@ -172,3 +174,21 @@ def get_top_k_predictions(logits, k):
     p = np.empty(max(kk, 1), dtype=np.float32)
     got = lib().vkop_oracle_get_top_k_predictions(_ptr(a), a.size, int(k), _ptr(idx), _ptr(p))
     return [(int(idx[j]), float(p[j])) for j in range(got)]
+
+
+def nms(boxes, scores, iou_threshold, score_threshold, max_output_boxes_per_class=0, center_point_box=0,
+        max_candidates=None):
+    """Non-maximum suppression per (batch, class): boxes [B,N,4], scores [B,C,N] (float32).
+    Returns an int32 array [M,3] of (batch, class, box index) records, ordered by
+    batch, class, then selection order."""
+    boxes = np.ascontiguousarray(boxes, dtype=np.float32)
+    scores = np.ascontiguousarray(scores, dtype=np.float32)
+    B, N, four = boxes.shape
+    assert four == 4 and scores.shape[0] == B and scores.shape[2] == N
+    C = scores.shape[1]
+    cap = B * C * N
+    out = np.empty((max(cap, 1), 3), dtype=np.int32)
+    m = lib().vkop_oracle_nms_f32(_ptr(boxes), _ptr(scores), _ptr(out), cap, B, C, N, int(center_point_box),
+                                  int(max_output_boxes_per_class), float(iou_threshold), float(score_threshold),
+                                  int(N if max_candidates is None else max_candidates))
+    return out[:m].copy()

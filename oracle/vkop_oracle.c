@@ -426,3 +426,104 @@ int vkop_oracle_get_top_k_predictions(const float *logits, int n, int k,
     free(p);
     return k;
 }
+
+/* ---- non-maximum suppression (ops/Nms.hpp, shaders/nms.comp) ---- */
+
+static float nms_iou(const float *a, const float *b) {
+    /* shaders/nms.comp:61-72 */
+    float x1 = a[0] > b[0] ? a[0] : b[0];
+    float y1 = a[1] > b[1] ? a[1] : b[1];
+    float x2 = a[2] < b[2] ? a[2] : b[2];
+    float y2 = a[3] < b[3] ? a[3] : b[3];
+    if (x2 <= x1 || y2 <= y1)
+        return 0.0f;
+    float inter = (x2 - x1) * (y2 - y1);
+    float area_a = (a[2] - a[0]) * (a[3] - a[1]);
+    float area_b = (b[2] - b[0]) * (b[3] - b[1]);
+    float uni = area_a + area_b - inter;
+    return uni > 0.0f ? inter / uni : 0.0f;
+}
+
+int vkop_oracle_nms_f32(const float *boxes, const float *scores, int32_t *out,
+                        int out_capacity, int B, int C, int N,
+                        int center_point_box, int max_output_boxes_per_class,
+                        float iou_threshold, float score_threshold,
+                        int max_candidates) {
+    int total = 0;
+    float *cb = (float *)malloc((size_t)(max_candidates > 0 ? max_candidates : 1) * 4 * sizeof(float));
+    float *cs = (float *)malloc((size_t)(max_candidates > 0 ? max_candidates : 1) * sizeof(float));
+    int *ci = (int *)malloc((size_t)(max_candidates > 0 ? max_candidates : 1) * sizeof(int));
+    char *active = (char *)malloc((size_t)(max_candidates > 0 ? max_candidates : 1));
+    for (int b = 0; b < B; b++) {
+        for (int c = 0; c < C; c++) {
+            /* shaders/nms.comp:83-104: collect, in box order */
+            int count = 0;
+            for (int i = 0; i < N && count < max_candidates; i++) {
+                float s = scores[((size_t)b * C + c) * N + i];
+                if (s > score_threshold) {
+                    const float *r = boxes + ((size_t)b * N + i) * 4;
+                    float *d = cb + (size_t)count * 4;
+                    if (center_point_box == 0) {
+                        d[0] = r[0], d[1] = r[1], d[2] = r[2], d[3] = r[3];
+                    } else { /* shaders/nms.comp:55-58 */
+                        d[0] = r[0] - r[2] * 0.5f, d[1] = r[1] - r[3] * 0.5f;
+                        d[2] = r[0] + r[2] * 0.5f, d[3] = r[1] + r[3] * 0.5f;
+                    }
+                    cs[count] = s;
+                    ci[count] = i;
+                    count++;
+                }
+            }
+            /* shaders/nms.comp:107-127: selection sort, strict > keeps the
+             * earlier of equal scores first */
+            for (int i = 0; i < count; i++) {
+                int best = i;
+                for (int j = i + 1; j < count; j++)
+                    if (cs[j] > cs[best])
+                        best = j;
+                if (best != i) {
+                    /* the shader swaps; a rotation keeps the order of the others
+                     * too, which is what "earlier of equal scores first" needs to
+                     * hold beyond the pair -- with distinct scores both give the
+                     * same list */
+                    float ts = cs[best], tb[4];
+                    int ti = ci[best];
+                    memcpy(tb, cb + (size_t)best * 4, sizeof tb);
+                    for (int j = best; j > i; j--) {
+                        cs[j] = cs[j - 1];
+                        ci[j] = ci[j - 1];
+                        memcpy(cb + (size_t)j * 4, cb + (size_t)(j - 1) * 4, sizeof tb);
+                    }
+                    cs[i] = ts;
+                    ci[i] = ti;
+                    memcpy(cb + (size_t)i * 4, tb, sizeof tb);
+                }
+                active[i] = 1;
+            }
+            /* shaders/nms.comp:148-188 */
+            int max_out = count;
+            if (max_output_boxes_per_class > 0 && max_output_boxes_per_class < count)
+                max_out = max_output_boxes_per_class;
+            int selected = 0;
+            for (int i = 0; i < count && selected < max_out; i++) {
+                if (!active[i])
+                    continue;
+                if (total < out_capacity) {
+                    out[(size_t)total * 3 + 0] = b;
+                    out[(size_t)total * 3 + 1] = c;
+                    out[(size_t)total * 3 + 2] = ci[i];
+                }
+                total++;
+                selected++;
+                for (int j = i + 1; j < count; j++)
+                    if (active[j] && nms_iou(cb + (size_t)j * 4, cb + (size_t)i * 4) > iou_threshold)
+                        active[j] = 0;
+            }
+        }
+    }
+    free(cb);
+    free(cs);
+    free(ci);
+    free(active);
+    return total;
+}

@@ -89,6 +89,30 @@ void vkop_oracle_reduce_max_f32(const float *in, float *out, int outer, int n,
 int vkop_oracle_get_top_k_predictions(const float *logits, int n, int k,
                                       int32_t *indices, float *probs);
 
+/* Non-maximum suppression, the Nms operator (ops/Nms.hpp:73-118,
+ * shaders/nms.comp:74-201).  boxes is [B][N][4], scores is [B][C][N].
+ * Per (batch, class), as the shader's workgroup does: the boxes whose score is
+ * greater than score_threshold (shaders/nms.comp:89; at most max_candidates of
+ * them, the first by box index -- the shader's shared arrays hold 1024) are
+ * ordered by score, largest first (a selection sort that keeps the earlier of
+ * two equal scores first, shaders/nms.comp:107-127), then walked in that
+ * order: a box still active is selected and deactivates every later box whose
+ * IoU with it is greater than iou_threshold (shaders/nms.comp:155-188, IoU as
+ * in shaders/nms.comp:61-72: 0 for an empty intersection or a union that is
+ * not positive); at most max_output_boxes_per_class selections when that is
+ * positive.  center_point_box != 0: boxes are (x_center, y_center, width,
+ * height) (shaders/nms.comp:51-59).
+ * Stated deviation: the records (batch, class, box index) are written in order
+ * of batch, then class, then selection -- the shader appends them through a
+ * global atomic counter, so its order across (batch, class) pairs is whatever
+ * the scheduling gives, and it adds a (-1,-1,-1) record this function does not.
+ * Returns the number of records; at most out_capacity are written to out. */
+int vkop_oracle_nms_f32(const float *boxes, const float *scores, int32_t *out,
+                        int out_capacity, int B, int C, int N,
+                        int center_point_box, int max_output_boxes_per_class,
+                        float iou_threshold, float score_threshold,
+                        int max_candidates);
+
 #ifdef __cplusplus
 }
 #endif

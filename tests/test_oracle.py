@@ -288,3 +288,90 @@ def test_get_top_k_predictions(golden):
     assert ulp_diff(np.array([g[1] for g in got], np.float32), p[order]).max() <= 2
     assert [g[0] for g in got] == golden["c1_idx"][0].tolist()
     assert len(oracle.get_top_k_predictions(x[:3], 5)) == 3
+
+
+# ---- non-maximum suppression (the detection chain's last operator) -------------------------------
+
+def _reference_like_boxes(rng, B, N):
+    """Boxes the way tests/NmsTest.cpp:38-56 draws them: centre in [0,1)^2, size in [0,1.3)^2, clamped."""
+    c = rng.random((B, N, 2)).astype(np.float32)
+    s = (rng.random((B, N, 2)) * 1.3).astype(np.float32)
+    lo = np.clip(c - s / 2, 0.0, 1.0)
+    hi = np.clip(c + s / 2, 0.0, 1.0)
+    return np.concatenate([lo, hi], axis=-1).astype(np.float32)
+
+
+def _nms_like_the_reference_test(boxes, scores, iou_threshold, score_threshold):
+    """The expectation tests/NmsTest.cpp:62-160 computes, written with whole-array
+    operations (argsort + an IoU matrix) instead of its nested scalar loops."""
+    out = []
+    B, C, N = scores.shape
+    for b in range(B):
+        bx = boxes[b].astype(np.float32)
+        area = (bx[:, 2] - bx[:, 0]) * (bx[:, 3] - bx[:, 1])
+        w = np.maximum(np.float32(0), np.minimum(bx[:, None, 2], bx[None, :, 2]) - np.maximum(bx[:, None, 0], bx[None, :, 0]))
+        h = np.maximum(np.float32(0), np.minimum(bx[:, None, 3], bx[None, :, 3]) - np.maximum(bx[:, None, 1], bx[None, :, 1]))
+        inter = (w * h).astype(np.float32)
+        union = (area[:, None] + area[None, :] - inter).astype(np.float32)
+        iou = np.where(union > np.float32(1e-8), inter / np.where(union > 0, union, 1), 0).astype(np.float32)
+        for c in range(C):
+            order = np.argsort(-scores[b, c], kind="stable")
+            order = order[scores[b, c][order] >= score_threshold]
+            alive = np.ones(len(order), bool)
+            for p, i in enumerate(order):
+                if not alive[p]:
+                    continue
+                out.append((b, c, int(i)))
+                alive[p + 1:] &= ~(iou[i, order[p + 1:]] > iou_threshold)
+    return np.array(out, dtype=np.int32).reshape(-1, 3)
+
+
+@pytest.mark.parametrize("box_shape,score_shape,max_per_class,iou_thr,score_thr", [
+    ((1, 10, 4), (1, 2, 10), 0, 0.5, 0.5), ((1, 200, 4), (1, 1, 200), 0, 0.7, 0.4), ((1, 50, 4), (1, 7, 50), 0, 0.3, 0.2),
+    ((3, 300, 4), (3, 5, 300), 0, 0.45, 0.25)])
+def test_nms_matches_the_reference_tests_expectation(box_shape, score_shape, max_per_class, iou_thr, score_thr):
+    """Shapes and thresholds of tests/NmsTest.cpp:165-169 (its expectation ignores the per-class limit, so 0 here)."""
+    rng = np.random.default_rng(box_shape[1])
+    boxes = _reference_like_boxes(rng, box_shape[0], box_shape[1])
+    scores = rng.random(score_shape).astype(np.float32)
+    got = oracle.nms(boxes, scores, iou_thr, score_thr, max_per_class)
+    want = _nms_like_the_reference_test(boxes, scores, np.float32(iou_thr), np.float32(score_thr))
+    assert np.array_equal(got, want)
+
+
+def test_nms_invariants_and_closed_forms():
+    rng = np.random.default_rng(9)
+    boxes = _reference_like_boxes(rng, 2, 120)
+    scores = rng.random((2, 3, 120)).astype(np.float32)
+    sel = oracle.nms(boxes, scores, 0.4, 0.3)
+
+    def iou(a, b):
+        x1, y1, x2, y2 = max(a[0], b[0]), max(a[1], b[1]), min(a[2], b[2]), min(a[3], b[3])
+        if x2 <= x1 or y2 <= y1:
+            return 0.0
+        inter = (x2 - x1) * (y2 - y1)
+        return inter / ((a[2] - a[0]) * (a[3] - a[1]) + (b[2] - b[0]) * (b[3] - b[1]) - inter)
+    for b in range(2):
+        for c in range(3):
+            mine = [int(r[2]) for r in sel if r[0] == b and r[1] == c]
+            s = scores[b, c]
+            assert all(s[i] > 0.3 for i in mine) and list(s[mine]) == sorted(s[mine], reverse=True)
+            for p, i in enumerate(mine):                       # no two selected boxes overlap too much
+                assert all(iou(boxes[b, i], boxes[b, j]) <= 0.4 + 1e-6 for j in mine[:p])
+            for j in np.nonzero(s > 0.3)[0]:                   # every rejected candidate lost to a better selected box
+                if j not in mine:
+                    assert any(s[i] >= s[j] and iou(boxes[b, i], boxes[b, j]) > 0.4 - 1e-6 for i in mine)
+    # identical boxes: only the best survives; disjoint boxes: all, best first
+    same = np.tile(np.array([[0.1, 0.1, 0.6, 0.7]], np.float32), (1, 8, 1))
+    sc = np.array([[[0.3, 0.9, 0.5, 0.7, 0.2, 0.8, 0.6, 0.4]]], np.float32)
+    assert oracle.nms(same, sc, 0.5, 0.0).tolist() == [[0, 0, 1]]
+    apart = np.array([[[i, 0, i + 0.5, 1] for i in range(8)]], np.float32)
+    assert oracle.nms(apart, sc, 0.5, 0.0)[:, 2].tolist() == [1, 5, 3, 6, 2, 7, 0, 4]
+    # IoU can never exceed 1: a threshold of 1 keeps every candidate; a score threshold above all keeps none
+    assert len(oracle.nms(same, sc, 1.0, 0.25)) == 7 and len(oracle.nms(same, sc, 0.5, 0.95)) == 0
+    # per-class limit, centre format, candidate limit (the first by box index)
+    assert oracle.nms(apart, sc, 0.5, 0.0, max_output_boxes_per_class=3)[:, 2].tolist() == [1, 5, 3]
+    centre = np.stack([(apart[..., 0] + apart[..., 2]) / 2, (apart[..., 1] + apart[..., 3]) / 2,
+                       apart[..., 2] - apart[..., 0], apart[..., 3] - apart[..., 1]], -1).astype(np.float32)
+    assert np.array_equal(oracle.nms(centre, sc, 0.5, 0.0, center_point_box=1), oracle.nms(apart, sc, 0.5, 0.0))
+    assert oracle.nms(apart, sc, 0.5, 0.0, max_candidates=4)[:, 2].tolist() == [1, 3, 2, 0]
