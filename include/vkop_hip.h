@@ -141,6 +141,28 @@ size_t vkop_hip_softmax_reduce_max_workspace_bytes(int dtype, const int *shape, 
 int vkop_hip_softmax_reduce_max(const void *in, void *out, int dtype, const int *shape,
                                 int ndim, int axis, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- Non-maximum suppression: replaces Nms::execute (ops/Nms.hpp:73-118) and
+ * shaders/nms.comp, the operator that follows the top-k in the detection-style
+ * post-processing.  boxes [B][N][4] and scores [B][C][N] of `dtype`; per (batch,
+ * class) the boxes whose score is greater than score_threshold are walked from
+ * the best score down (equal scores: lower box index first), a box still active
+ * is selected and deactivates every later box whose IoU with it is greater than
+ * iou_threshold; max_output_boxes_per_class > 0 limits the selections per pair;
+ * center_point_box != 0: boxes are (x_center, y_center, width, height).
+ * out receives (batch, class, box index) records, [out_capacity][3] int32, in
+ * order of batch, then class, then selection (the reference appends them through
+ * an atomic counter in scheduling order and adds a (-1,-1,-1) record; neither is
+ * carried over).  out_count: two int32 on the device: the number of records (all
+ * of them, also when out_capacity holds fewer) and 1 if some pair had more than
+ * VKOP_HIP_NMS_MAX_CANDIDATES boxes above the score threshold (the later ones by
+ * box index were left out; the reference's shader keeps 1024). */
+#define VKOP_HIP_NMS_MAX_CANDIDATES 2048
+size_t vkop_hip_nms_workspace_bytes(int B, int C, int N, int max_output_boxes_per_class);
+int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_capacity,
+                 int32_t *out_count, int dtype, int B, int C, int N, int center_point_box,
+                 int max_output_boxes_per_class, float iou_threshold, float score_threshold,
+                 void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---- Tuning and measurement knobs (process-wide; no counterpart in the
  * reference, whose shaders fix their workgroup shapes at compile time).
  *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the

@@ -699,3 +699,40 @@ def test_large_k_on_rows_one_workgroup_holds(ops, dtype, n, k):
         et, ej = oracle.topk(x, k, -1, largest)
         assert np.array_equal(host(j), ej) and np.array_equal(host(t).view(bits), et.view(bits)), (n, k, largest)
     assert_fused(ops, x * 8, k)
+
+
+# ---- non-maximum suppression ------------------------------------------------------------------------
+
+def _nms_boxes(rng, B, N, spread=1.3):
+    c = rng.random((B, N, 2)).astype(np.float32)
+    s = (rng.random((B, N, 2)) * spread).astype(np.float32)
+    return np.concatenate([np.clip(c - s / 2, 0, 1), np.clip(c + s / 2, 0, 1)], axis=-1).astype(np.float32)
+
+
+@pytest.mark.parametrize("B,C,N,max_per_class,iou_thr,score_thr", [
+    (1, 2, 10, 0, 0.5, 0.5), (1, 1, 200, 50, 0.7, 0.4), (1, 7, 50, 0, 0.3, 0.2),      # tests/NmsTest.cpp:165-169
+    (3, 5, 300, 0, 0.45, 0.25), (2, 3, 3000, 100, 0.5, 0.3), (16, 4, 8400, 0, 0.6, 0.9), (1, 1, 1, 0, 0.5, 0.1),
+    (2, 2, 1500, 0, 0.5, -1.0)])
+def test_nms_matches_the_oracle(ops, B, C, N, max_per_class, iou_thr, score_thr):
+    rng = np.random.default_rng(B * 1000 + N)
+    boxes = _nms_boxes(rng, B, N, 1.3 if N <= 300 else 0.2)
+    scores = rng.random((B, C, N)).astype(np.float32)
+    if N >= 300:
+        scores[0, 0, 5:40] = scores[0, 0, 5]              # equal scores: lower box index first
+    got, over = ops.nms(dev(boxes), dev(scores), iou_thr, score_thr, max_per_class)
+    want = oracle.nms(boxes, scores, iou_thr, score_thr, max_per_class, max_candidates=2048)
+    assert np.array_equal(host(got), want)
+    assert over == bool(((scores > score_thr).sum(axis=-1) > 2048).any())
+    # centre format, and half precision inputs (the same numbers after widening)
+    centre = np.stack([(boxes[..., 0] + boxes[..., 2]) / 2, (boxes[..., 1] + boxes[..., 3]) / 2,
+                       boxes[..., 2] - boxes[..., 0], boxes[..., 3] - boxes[..., 1]], -1).astype(np.float32)
+    got_c, _ = ops.nms(dev(centre), dev(scores), iou_thr, score_thr, max_per_class, center_point_box=1)
+    assert np.array_equal(host(got_c), oracle.nms(centre, scores, iou_thr, score_thr, max_per_class, 1, max_candidates=2048))
+    bh, sh = boxes.astype(np.float16), scores.astype(np.float16)
+    got_h, _ = ops.nms(dev(bh), dev(sh), iou_thr, score_thr, max_per_class)
+    want_h = oracle.nms(bh.astype(np.float32), sh.astype(np.float32), iou_thr, score_thr, max_per_class, max_candidates=2048)
+    assert np.array_equal(host(got_h), want_h)
+    # a small output buffer keeps the first records; the count still says how many there are
+    if len(want) > 3:
+        few, _ = ops.nms(dev(boxes), dev(scores), iou_thr, score_thr, max_per_class, out_capacity=3)
+        assert np.array_equal(host(few), want[:3])

@@ -54,6 +54,8 @@ def lib():
     i, f, vp, sz = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
     ip = ctypes.POINTER(ctypes.c_int)
     sig = {
+        "vkop_hip_nms_workspace_bytes": (sz, [i, i, i, i]),
+        "vkop_hip_nms": (i, [vp, vp, vp, i, vp, i, i, i, i, i, i, f, f, vp, sz, vp]),
         "vkop_hip_init": (i, [i]),
         "vkop_hip_shutdown": (i, []),
         "vkop_hip_last_error": (ctypes.c_char_p, []),
@@ -269,3 +271,14 @@ def softmax_reduce_max_workspace_bytes(dtype, shape, axis):
 def softmax_reduce_max(inp, out, dtype, shape, axis, workspace=0, workspace_bytes=0, stream=0):
     arr, nd = _shape(shape)
     check(lib().vkop_hip_softmax_reduce_max(inp, out, dtype, arr, nd, axis, workspace, workspace_bytes, stream))
+
+
+def nms_workspace_bytes(B, C, N, max_output_boxes_per_class=0):
+    return int(lib().vkop_hip_nms_workspace_bytes(int(B), int(C), int(N), int(max_output_boxes_per_class)))
+
+
+def nms(boxes, scores, out, out_capacity, out_count, dtype, B, C, N, center_point_box, max_output_boxes_per_class,
+        iou_threshold, score_threshold, workspace, workspace_bytes, stream=0):
+    check(lib().vkop_hip_nms(boxes, scores, out, int(out_capacity), out_count, int(dtype), int(B), int(C), int(N),
+                             int(center_point_box), int(max_output_boxes_per_class), float(iou_threshold),
+                             float(score_threshold), workspace, int(workspace_bytes), stream))

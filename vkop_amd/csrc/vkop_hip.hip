@@ -15,6 +15,7 @@
 #include "rows_launch.hpp"
 #include "kernels_softmax.hpp"
 #include "kernels_bigk.hpp"
+#include "kernels_nms.hpp"
 
 namespace vkop {
 
@@ -589,6 +590,36 @@ template <typename T> int reduce_max_impl(const T *in, T *out, const View &v, hi
     return launched("reduce_max_strided_kernel");
 }
 
+// ---------------------------------------------------------------- nms ----
+uint32_t nms_max_sel(int N, int max_per_class) {
+    uint32_t m = static_cast<uint32_t>(N) < static_cast<uint32_t>(vkop::kNmsMaxCandidates)
+                     ? static_cast<uint32_t>(N) : static_cast<uint32_t>(vkop::kNmsMaxCandidates);
+    if (max_per_class > 0 && static_cast<uint32_t>(max_per_class) < m) m = static_cast<uint32_t>(max_per_class);
+    return m < 1 ? 1 : m;
+}
+size_t nms_workspace(int B, int C, int N, int max_per_class) {
+    const size_t pairs = static_cast<size_t>(B) * C;
+    return kTicketBytes + align_up(2 * pairs * sizeof(uint32_t)) + align_up(pairs * nms_max_sel(N, max_per_class) * sizeof(int32_t));
+}
+
+template <typename T>
+int nms_impl(const T *boxes, const T *scores, int32_t *out, int out_capacity, int32_t *out_count, int B, int C, int N,
+             int center_point_box, int max_per_class, float iou_threshold, float score_threshold, void *ws, hipStream_t st) {
+    const uint32_t pairs = static_cast<uint32_t>(B) * static_cast<uint32_t>(C);
+    auto *base = static_cast<unsigned char *>(ws) + kTicketBytes;
+    auto *counts = reinterpret_cast<uint32_t *>(base);
+    auto *selected = reinterpret_cast<int32_t *>(base + align_up(2 * static_cast<size_t>(pairs) * sizeof(uint32_t)));
+    const uint32_t max_sel = nms_max_sel(N, max_per_class);
+    vkop::nms_kernel<T><<<pairs, vkop::kNmsThreads, 0, st>>>(boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C),
+                                                             static_cast<uint32_t>(N), center_point_box,
+                                                             max_per_class > 0 ? static_cast<uint32_t>(max_per_class) : 0u,
+                                                             iou_threshold, score_threshold, max_sel);
+    if (int rc = launched("nms_kernel")) return rc;
+    vkop::nms_pack_kernel<<<pairs, 256, 0, st>>>(selected, counts, out, out_count, pairs, static_cast<uint32_t>(C), max_sel,
+                                                 static_cast<uint32_t>(out_capacity));
+    return launched("nms_pack_kernel");
+}
+
 }  // namespace
 
 extern "C" {
@@ -894,6 +925,39 @@ int vkop_hip_softmax_reduce_max(const void *in, void *out, int dtype, const int 
                                        workspace_bytes, as_stream(stream));
     return softmax_reduce_max_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, workspace,
                                    workspace_bytes, as_stream(stream));
+}
+
+size_t vkop_hip_nms_workspace_bytes(int B, int C, int N, int max_output_boxes_per_class) {
+    if (B < 0 || C < 0 || N < 0) return 0;
+    return nms_workspace(B, C, N, max_output_boxes_per_class);
+}
+
+int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_capacity, int32_t *out_count, int dtype, int B,
+                 int C, int N, int center_point_box, int max_output_boxes_per_class, float iou_threshold,
+                 float score_threshold, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int rc = check_dtype(dtype)) return rc;
+    if (B < 0 || C < 0 || N < 0 || out_capacity < 0) return fail(VKOP_HIP_ERR_INVALID, "negative extent");
+    if (static_cast<uint64_t>(B) * static_cast<uint64_t>(C) >= (1ull << 31) || static_cast<uint64_t>(N) >= (1ull << 31) / 4)
+        return fail(VKOP_HIP_ERR_UNSUPPORTED, "too many (batch, class) pairs or boxes");
+    if (out_count == nullptr) return fail(VKOP_HIP_ERR_INVALID, "out_count is null");
+    if (B == 0 || C == 0) {
+        vkop::fill_zero_kernel<<<1, 64, 0, as_stream(stream)>>>(reinterpret_cast<uint32_t *>(out_count), 2);  // (no memset: capture-safe)
+        return launched("fill_zero_kernel");
+    }
+    if (boxes == nullptr || scores == nullptr || (out == nullptr && out_capacity > 0))
+        return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    const size_t need = nms_workspace(B, C, N, max_output_boxes_per_class);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
+    if (dtype == VKOP_HIP_F32)
+        return nms_impl(static_cast<const float *>(boxes), static_cast<const float *>(scores), out, out_capacity, out_count,
+                        B, C, N, center_point_box, max_output_boxes_per_class, iou_threshold, score_threshold, workspace,
+                        as_stream(stream));
+    return nms_impl(static_cast<const uint16_t *>(boxes), static_cast<const uint16_t *>(scores), out, out_capacity, out_count,
+                    B, C, N, center_point_box, max_output_boxes_per_class, iou_threshold, score_threshold, workspace,
+                    as_stream(stream));
 }
 
 }  // extern "C"

@@ -115,3 +115,26 @@ def reduce_max(x, axis):
     out = torch.empty(shape, dtype=x.dtype, device=x.device)
     capi.reduce_max(x.data_ptr(), out.data_ptr(), dt, x.shape, axis, _stream())
     return out
+
+
+def nms(boxes, scores, iou_threshold, score_threshold, max_output_boxes_per_class=0, center_point_box=0,
+        out_capacity=None, workspace=None):
+    """Non-maximum suppression per (batch, class): boxes [B,N,4], scores [B,C,N] (both float32 or both float16).
+    Returns (records, overflow): an int32 tensor [M,3] of (batch, class, box index), ordered by batch, class and
+    selection, and whether some pair had more candidates than the kernel holds."""
+    boxes, dt = _prep(boxes)
+    scores, dt2 = _prep(scores)
+    assert dt == dt2 and boxes.dim() == 3 and scores.dim() == 3 and boxes.shape[2] == 4
+    B, N, _ = boxes.shape
+    C = scores.shape[1]
+    assert scores.shape[0] == B and scores.shape[2] == N
+    per_pair = min(N, 2048) if max_output_boxes_per_class <= 0 else min(N, 2048, max_output_boxes_per_class)
+    cap = B * C * per_pair if out_capacity is None else out_capacity
+    out = torch.empty((max(cap, 1), 3), dtype=torch.int32, device=boxes.device)
+    count = torch.zeros(2, dtype=torch.int32, device=boxes.device)
+    ws = workspace or _default_ws
+    ptr, size = ws.get(capi.nms_workspace_bytes(B, C, N, max_output_boxes_per_class))
+    capi.nms(boxes.data_ptr(), scores.data_ptr(), out.data_ptr(), cap, count.data_ptr(), dt, B, C, N, center_point_box,
+             max_output_boxes_per_class, iou_threshold, score_threshold, ptr, size, _stream())
+    m, over = (int(v) for v in count.cpu().tolist())
+    return out[:min(m, cap)], bool(over)
