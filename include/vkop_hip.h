@@ -151,8 +151,9 @@ int vkop_hip_softmax_reduce_max(const void *in, void *out, int dtype, const int 
  * center_point_box != 0: boxes are (x_center, y_center, width, height).
  * out receives (batch, class, box index) records, [out_capacity][3] int32, in
  * order of batch, then class, then selection (the reference appends them through
- * an atomic counter in scheduling order and adds a (-1,-1,-1) record; neither is
- * carried over).  out_count: two int32 on the device: the number of records (all
+ * an atomic counter in scheduling order, with a (-1,-1,-1) record somewhere among
+ * them; here that record follows the last one, when out_capacity has room for it).
+ * out_count: two int32 on the device: the number of records (all
  * of them, also when out_capacity holds fewer) and 1 if some pair had more than
  * VKOP_HIP_NMS_MAX_CANDIDATES boxes above the score threshold (the later ones by
  * box index were left out; the reference's shader keeps 1024). */

@@ -146,7 +146,8 @@ __global__ __launch_bounds__(kNmsThreads) void nms_kernel(const T *__restrict__ 
 
 // The records of all pairs one after the other.  out: [capacity][3]; out_count[0] =
 // records in all (also when capacity holds fewer), out_count[1] = 1 if some pair
-// had more candidates than kNmsMaxCandidates.  Launch: B * C workgroups of 256.
+// had more candidates than kNmsMaxCandidates; a (-1,-1,-1) record follows the last
+// one when capacity allows.  Launch: B * C workgroups of 256.
 __global__ __launch_bounds__(256) void nms_pack_kernel(const int32_t *__restrict__ selected,
                                                               const uint32_t *__restrict__ counts, int32_t *__restrict__ out,
                                                               int32_t *__restrict__ out_count, uint32_t pairs, uint32_t C,
@@ -179,8 +180,14 @@ __global__ __launch_bounds__(256) void nms_pack_kernel(const int32_t *__restrict
     if (pair == pairs - 1 && tid == 0) {
         uint32_t any = 0;
         for (int w = 0; w < 256 / kWave; w++) any |= scratch[w];
-        out_count[0] = static_cast<int32_t>(offset + n);
+        const uint32_t total = offset + n;
+        out_count[0] = static_cast<int32_t>(total);
         out_count[1] = any ? 1 : 0;
+        if (total < capacity) {  // end of the list for a reader of the tensor alone (the reference writes such a record too)
+            out[static_cast<size_t>(total) * 3 + 0] = -1;
+            out[static_cast<size_t>(total) * 3 + 1] = -1;
+            out[static_cast<size_t>(total) * 3 + 2] = -1;
+        }
     }
 }
 

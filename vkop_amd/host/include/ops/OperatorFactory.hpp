@@ -7,6 +7,7 @@
 #include <memory>
 
 #include "ops/Operator.hpp"
+#include "ops/Nms.hpp"
 #include "ops/Softmax.hpp"
 #include "ops/Topk.hpp"
 
@@ -21,6 +22,8 @@ static inline std::unique_ptr<Operator> create_from_type(OpType type, bool use_s
         return std::make_unique<Topk>(fp16);
     case OpType::SOFTMAX:
         return std::make_unique<Softmax>(use_ssbo);
+    case OpType::NMS:
+        return std::make_unique<Nms>();
     default:
         return nullptr;
     }

@@ -260,6 +260,65 @@ template <typename T> void fused_case(const std::vector<int> &shape, int k) {
     EXPECT(tc.max_ulp <= 2);
 }
 
+// tests/NmsTest.cpp:29-160: boxes from uniform centres and sizes, uniform scores;
+// expectation: per (batch, class) the boxes at or above the score threshold, best
+// first, each kept box removing the later ones whose IoU with it exceeds the
+// threshold.  Written here over an IoU matrix and a sort of the whole score row.
+template <typename T>
+void nms_case(const std::vector<int> &box_shape, const std::vector<int> &score_shape, int per_class, float iou_thr,
+              float score_thr) {
+    TestCase<T> tc("Nms");
+    torch::manual_seed(11);
+    const int64_t B = box_shape[0], N = box_shape[1], C = score_shape[1];
+    auto scores = torch::rand({B, C, N}, tc.conf());
+    auto centre = torch::rand({B, N, 2}, tc.conf()), size = torch::rand({B, N, 2}, tc.conf()) * 1.3F;
+    auto boxes = torch::cat({torch::clamp(centre - size / 2, 0.0F, 1.0F), torch::clamp(centre + size / 2, 0.0F, 1.0F)}, -1);
+    auto bf = boxes.to(torch::kFloat32), sf = scores.to(torch::kFloat32);
+    std::vector<int> records;
+    for (int64_t b = 0; b < B; b++) {
+        auto x1 = bf[b].select(-1, 0), y1 = bf[b].select(-1, 1), x2 = bf[b].select(-1, 2), y2 = bf[b].select(-1, 3);
+        auto area = (x2 - x1) * (y2 - y1);
+        auto w = torch::clamp_min(torch::min(x2.unsqueeze(1), x2.unsqueeze(0)) - torch::max(x1.unsqueeze(1), x1.unsqueeze(0)), 0);
+        auto h = torch::clamp_min(torch::min(y2.unsqueeze(1), y2.unsqueeze(0)) - torch::max(y1.unsqueeze(1), y1.unsqueeze(0)), 0);
+        auto inter = w * h;
+        auto uni = area.unsqueeze(1) + area.unsqueeze(0) - inter;
+        auto iou = torch::where(uni > 1e-8F, inter / uni, torch::zeros_like(inter)).contiguous();
+        const float *m = iou.template data_ptr<float>();
+        for (int64_t c = 0; c < C; c++) {
+            auto order = std::get<1>(torch::sort(sf[b][c], /*stable=*/true, /*dim=*/0, /*descending=*/true)).contiguous();
+            const int64_t *o = order.template data_ptr<int64_t>();
+            std::vector<char> dead(static_cast<size_t>(N), 0);
+            for (int64_t p = 0; p < N; p++) {
+                if (sf[b][c][o[p]].template item<float>() < score_thr) break;
+                if (dead[static_cast<size_t>(p)]) continue;
+                records.insert(records.end(), {static_cast<int>(b), static_cast<int>(c), static_cast<int>(o[p])});
+                for (int64_t q = p + 1; q < N; q++)
+                    if (m[o[p] * N + o[q]] > iou_thr) dead[static_cast<size_t>(q)] = 1;
+            }
+        }
+    }
+    auto in_boxes = std::make_shared<Tensor<T>>(box_shape);
+    fill_from_torch(in_boxes, boxes);
+    auto in_scores = std::make_shared<Tensor<T>>(score_shape);
+    fill_from_torch(in_scores, scores);
+    const int M = static_cast<int>(records.size() / 3);
+    auto expect = std::make_shared<Tensor<int>>(std::vector<int>{M, 3});
+    expect->fillToCPU(records);
+    const std::unordered_map<std::string, std::string> attrs = {{"max_output_boxes_per_class", std::to_string(per_class)},
+                                                                {"iou_threshold", std::to_string(iou_thr)},
+                                                                {"score_threshold", std::to_string(score_thr)}};
+    bool ok = M > 0;
+    if (M > 0)
+        ok = tc.run_test({in_boxes, in_scores}, {expect}, [&](std::unique_ptr<ops::Operator> &op) {
+            auto *nms = dynamic_cast<ops::Nms *>(op.get());
+            EXPECT(nms != nullptr);
+            if (nms) nms->setAttribute(attrs);
+        });
+    std::printf("Nms %s boxes [%d,%d,4] classes %d: %s, %d records\n", std::is_same_v<T, float> ? "fp32" : "fp16", box_shape[0],
+                box_shape[1], score_shape[1], ok ? "ok" : "FAILED", M);
+    EXPECT(ok);
+}
+
 static void host_logic_tests() {
     // names and numbering (ops/Ops.hpp)
     EXPECT(static_cast<int>(ops::OpType::SOFTMAX) == 26);
@@ -286,6 +345,10 @@ static void host_logic_tests() {
         EXPECT(sm && sm->get_type() == ops::OpType::SOFTMAX && dynamic_cast<ops::Softmax *>(sm.get()));
         EXPECT(tk && tk->get_type() == ops::OpType::TOPK && dynamic_cast<ops::Topk *>(tk.get()));
         EXPECT(ops::create_from_type(ops::OpType::CONV2D) == nullptr);
+        {
+            auto nm = ops::create_from_type(ops::OpType::NMS);
+            EXPECT(nm && nm->get_type() == ops::OpType::NMS && dynamic_cast<ops::Nms *>(nm.get()));
+        }
         EXPECT(ops::create_from_type(ops::OpType::UNKNOWN) == nullptr);
         EXPECT(ops::Operator::instance_count_.load() == before + 2);
         sm->set_name("prob");
@@ -456,6 +519,11 @@ int main(int argc, char **argv) {
         fused_case<float>({256, 1000}, 5);
         fused_case<float>({4, 128256}, 50);
         fused_case<uint16_t>({64, 1000}, 5);
+        // tests/NmsTest.cpp:165-169 (its expectation never applies the per-class limit: 0 here)
+        nms_case<float>({1, 10, 4}, {1, 2, 10}, 0, 0.5F, 0.5F);
+        nms_case<float>({1, 200, 4}, {1, 1, 200}, 0, 0.7F, 0.4F);
+        nms_case<float>({1, 50, 4}, {1, 7, 50}, 0, 0.3F, 0.2F);
+        nms_case<uint16_t>({2, 300, 4}, {2, 3, 300}, 0, 0.5F, 0.3F);
         // the benchmark's arrangement: full-size outputs, the first k read back
         {
             TestEnv::initialize();
