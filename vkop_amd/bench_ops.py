@@ -161,6 +161,36 @@ def main():
             capi.softmax_reduce_max(bufs[b].data_ptr(), m.data_ptr(), F32, c5.shape, 1, ptr, nb + 256, stream)
             capi.topk(m.data_ptr(), vals.data_ptr(), idx.data_ptr(), F32, (16, 8400), -1, 300, 1, 1, ptr, nb + 256, stream)
         report("C5 chain (softmax+max in one pass) -> topk k=300", timed(chain_one_pass, len(bufs)), c5.nbytes + 16 * 300 * 8)
+
+    def nms_case(name, boxes, scores, per_class, iou_thr, score_thr):
+        if args.only not in name:
+            return
+        B, C, N = scores.shape
+        bx, sc = torch.from_numpy(boxes).cuda(), torch.from_numpy(scores).cuda()
+        cap = B * C * (min(N, per_class) if per_class > 0 else min(N, 2048))
+        out = torch.empty((cap, 3), dtype=torch.int32, device="cuda")
+        count = torch.zeros(2, dtype=torch.int32, device="cuda")
+        nb = capi.nms_workspace_bytes(B, C, N, per_class)
+        ws, ptr = workspace(nb + 256)
+        us = timed(lambda b: capi.nms(bx.data_ptr(), sc.data_ptr(), out.data_ptr(), cap, count.data_ptr(), F32, B, C, N, 0,
+                                      per_class, iou_thr, score_thr, ptr, nb + 256, stream), 1)
+        m = int(count.cpu()[0])
+        print(json.dumps({"case": name, "us_per_call": round(us, 2), "selected": m,
+                          "algorithmic_bytes": boxes.nbytes + scores.nbytes + 12 * m,
+                          "algorithmic_GBps": round((boxes.nbytes + scores.nbytes + 12 * m) / us / 1e3, 1)}), flush=True)
+
+    # detection head after the chain above: softmax scores [16,80,8400], uniform boxes, the usual thresholds
+    rng = np.random.default_rng(synth.SEEDS["C5"] + 1)
+    ctr, size = rng.random((16, 8400, 2), dtype=np.float32), rng.random((16, 8400, 2), dtype=np.float32) * np.float32(0.2)
+    boxes = np.ascontiguousarray(np.concatenate([ctr - size / 2, ctr + size / 2], axis=-1))
+    e = np.exp(c5 - c5.max(axis=1, keepdims=True))
+    nms_case("C5 nms [16,80,8400] f32 iou 0.45 score 0.25 max 100", boxes, np.ascontiguousarray((e / e.sum(axis=1, keepdims=True))
+             .astype(np.float32)), 100, 0.45, 0.25)
+    # the longest walk one (batch, class) pair can ask for: 2048 candidates, none suppressed early
+    nms_case("nms [1,1,2048] f32 all candidates, iou 0.7", boxes[:1, :2048], rng.random((1, 1, 2048), dtype=np.float32), 0,
+             0.7, 0.0)
+    nms_case("nms [8,80,2048] f32 all candidates, iou 0.5 max 200", boxes[:8, :2048],
+             rng.random((8, 80, 2048), dtype=np.float32), 200, 0.5, 0.0)
     capi.event_destroy(e0)
     capi.event_destroy(e1)
     capi.stream_destroy(stream)
