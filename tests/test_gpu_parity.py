@@ -7,6 +7,8 @@ reported through the reference harness's tolerance, not gated tighter: libtorch
 sums in ISA-dependent float lanes and is itself many ulp from an exact sum on
 long rows.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -736,3 +738,41 @@ def test_nms_matches_the_oracle(ops, B, C, N, max_per_class, iou_thr, score_thr)
     if len(want) > 3:
         few, _ = ops.nms(dev(boxes), dev(scores), iou_thr, score_thr, max_per_class, out_capacity=3)
         assert np.array_equal(host(few), want[:3])
+
+
+# ---- models from .vkopbin files ---------------------------------------------------------------------
+
+GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_model_files_drive_the_operators(ops, dtype):
+    from vkop_amd import runtime, vkopbin
+    # classifier head, fused and not: the same ranking; values to the fused operator's bar
+    head = vkopbin.read_model(os.path.join(GOLDEN_DIR, "classifier_head.vkopbin"))
+    x = np.ascontiguousarray(synth.classifier_logits(8, 1000, 77).astype(dtype))
+    fused = runtime.run_model(head, {"logits": dev(x)})
+    plain = runtime.run_model(head, {"logits": dev(x)}, fuse=False)
+    p = oracle.softmax(x, -1)
+    ev, ei = oracle.topk(p, 5, -1)
+    assert np.array_equal(host(plain["indices"]), ei)
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    close = half_ulp_diff if dtype == np.float16 else ulp_diff
+    assert close(host(plain["values"]), ev).max() <= 2
+    assert close(host(fused["values"]), host(plain["values"])).max() <= 2
+    if not np.array_equal(host(fused["indices"]), ei):       # only equal probabilities may trade places
+        assert np.array_equal(np.take_along_axis(p, host(fused["indices"]).astype(np.int64), -1).view(bits), ev.view(bits))
+    # K from the second input; the probabilities are an output as well
+    shared = vkopbin.read_model(os.path.join(GOLDEN_DIR, "classifier_head_k_input.vkopbin"))
+    out = runtime.run_model(shared, {"logits": dev(x[:4])})
+    assert host(out["values"]).shape == (4, 7)
+    ev7, ei7 = oracle.topk(host(out["probs"]), 7, -1)
+    assert np.array_equal(host(out["indices"]), ei7) and np.array_equal(host(out["values"]).view(bits), ev7.view(bits))
+    # detection tail
+    tail = vkopbin.read_model(os.path.join(GOLDEN_DIR, "detection_tail.vkopbin"))
+    rng = np.random.default_rng(9)
+    boxes = _nms_boxes(rng, 2, 300, 0.3).astype(dtype)
+    scores = rng.random((2, 3, 300)).astype(dtype)
+    got = runtime.run_model(tail, {"boxes": dev(boxes), "scores": dev(scores)})["selected"]
+    want = oracle.nms(boxes.astype(np.float32), scores.astype(np.float32), 0.5, 0.25, 0, max_candidates=2048)
+    assert np.array_equal(host(got), want) and len(want) > 0

@@ -1,15 +1,29 @@
-// The post-processing slice of the reference's Runtime (core/runtime.cpp):
-// RegisterPostProcess (:480-520), Run (:404-458), ReadResult (:460-478).
+// The part of the reference's Runtime (core/runtime.cpp) around the operators
+// of this library: LoadModel (:33-363) for models made of them, GetInput /
+// GetOutput / GetInitializer (:365-402), RegisterPostProcess (:480-520), Run
+// (:404-458), ReadResult (:460-478).
 //
-// The model part of the reference's Runtime (loading a .vkopbin, building the
-// operator graph) is not here; the tensor the model would produce is handed in
-// with SetOutput().  Post-processing operators are appended one level at a
-// time, each depending on the level before it, exactly as the reference does,
-// with one addition: a TOPK registered on the output of the SOFTMAX registered
-// just before it replaces the pair by one fused operator.  That is legal
-// because every registration clears the set of tensors read back
-// (core/runtime.cpp:515-519), so after the TOPK registration the softmax tensor
-// is neither read back nor an input of anything else.
+// LoadModel reads a .vkopbin (model/load.hpp), creates the tensors and builds
+// the plan level by level from the file's concurrent levels and dependencies,
+// as the reference does.  Differences, on purpose:
+//   * a node whose operator this library does not have stops the load with an
+//     error naming it (the reference skips the node and fails later);
+//   * tensors of index outputs (TopK's second, Nms's) are int32 whatever the
+//     precision; every intermediate tensor gets storage of its own;
+//   * model inputs are plain buffers of the runtime's precision (the reference
+//     makes them fp16 images for its convolution front end);
+//   * a TopK node without a K attribute takes K from its second input when
+//     that is an int64 initializer (ONNX keeps K there).
+// Without a model, the tensor a model would produce is handed in with
+// SetOutput().  Post-processing operators are appended one level at a time,
+// each depending on the level before it, exactly as the reference does.
+//
+// One addition in both paths: a TopK that alone reads the output of a Softmax
+// along the same axis replaces the pair by one fused operator.  For registered
+// post-processing that is legal because every registration clears the set of
+// tensors read back (core/runtime.cpp:515-519), so after the TOPK registration
+// the softmax tensor is neither read back nor an input of anything else; for a
+// model the softmax output must have that one consumer and not be a model output.
 #ifndef VKOP_HIP_CORE_RUNTIME_HPP_
 #define VKOP_HIP_CORE_RUNTIME_HPP_
 
@@ -18,8 +32,10 @@
 #include <memory>
 #include <string>
 #include <unordered_map>
+#include <unordered_set>
 #include <vector>
 
+#include "model/load.hpp"
 #include "ops/OperatorFactory.hpp"
 
 namespace vkop {
@@ -33,7 +49,161 @@ class Runtime {
 
     // Stands in for the model: the tensor post-processing starts from.
     void SetOutput(const std::shared_ptr<ITensor> &t) { output_ = t; }
-    std::shared_ptr<ITensor> GetOutput() const { return output_; }
+
+    void setPrecision(int precision) { precision_ = precision; }
+    int getPrecision() const { return precision_; }
+
+    void LoadModel() {
+        const load::VkModel model(model_path_);
+        std::unordered_map<std::string, std::shared_ptr<ITensor>> tensor_map;
+        std::unordered_map<std::string, int> consumers;
+        std::unordered_map<std::string, const load::Node *> node_by_name, producer;
+        std::unordered_map<std::string, size_t> output_slot;
+        for (const auto &n : model.nodes) {
+            node_by_name[n.name] = &n;
+            for (const auto &in : n.inputs) consumers[in.name] += 1;
+            for (size_t i = 0; i < n.outputs.size(); ++i) {
+                producer[n.outputs[i].name] = &n;
+                output_slot[n.outputs[i].name] = i;
+            }
+            if (ops::convert_opstring_to_enum(n.op_type) == ops::OpType::UNKNOWN || !ops::create_from_type(ops::convert_opstring_to_enum(n.op_type)))
+                throw std::runtime_error("LoadModel: node " + n.name + " needs operator " + n.op_type + ", which this library does not have");
+        }
+        auto dev = m_cmdpool_->getVulkanDevice();
+        auto make = [this](const std::vector<uint32_t> &dims, bool index, bool on_device = true) -> std::shared_ptr<ITensor> {
+            if (index) return std::make_shared<Tensor<int>>(dims, on_device);
+            if (precision_ == 1) return std::make_shared<Tensor<uint16_t>>(dims, on_device);
+            return std::make_shared<Tensor<float>>(dims, on_device);
+        };
+        auto holds_indices = [&](const std::string &tensor) {
+            auto it = producer.find(tensor);
+            if (it == producer.end()) return false;
+            const auto type = ops::convert_opstring_to_enum(it->second->op_type);
+            return (type == ops::OpType::TOPK && output_slot[tensor] == 1) || type == ops::OpType::NMS;
+        };
+        for (const auto &i : model.inputs) {
+            auto t = make(i.dims, false, /*on_device=*/false);  // filled on the host, then copyToGPU()
+            t->set_ref_cnt_forever();
+            inputs_[i.name] = t;
+            tensor_map[i.name] = t;
+        }
+        for (const auto &o : model.outputs) {
+            auto t = make(o.dims, holds_indices(o.name));
+            t->set_ref_cnt_forever();
+            outputs_[o.name] = t;
+            tensor_map[o.name] = t;
+            real_outputs_[o.name] = t;
+        }
+        for (const auto &it : model.initializers) {
+            const auto &init = it.second;
+            const uint8_t *src = model.initializer_data(init.name);
+            auto host_only = [&](auto t, const auto *data) {
+                t->set_ref_cnt_forever();
+                t->fillToCPU(data);
+                tensor_map[init.name] = t;
+                initializers_[init.name] = t;
+            };
+            auto on_device = [&](auto t, auto *data) {
+                host_only(t, data);
+                t->as_storage_buffer(dev);
+                t->copyToGPU(m_cmdpool_);
+            };
+            if (init.dtype == "int64") host_only(std::make_shared<Tensor<int64_t>>(init.dims), reinterpret_cast<const int64_t *>(src));
+            else if (init.dtype == "int32") host_only(std::make_shared<Tensor<int>>(init.dims), reinterpret_cast<const int *>(src));
+            else if (init.dtype == "float32") on_device(std::make_shared<Tensor<float>>(init.dims), reinterpret_cast<const float *>(src));
+            else if (init.dtype == "float16") on_device(std::make_shared<Tensor<uint16_t>>(init.dims), reinterpret_cast<const uint16_t *>(src));
+            else throw std::runtime_error("Only float32/float16/int32/int64 initializer is supported for now " + init.dtype);
+        }
+        // a Softmax whose only reader is a TopK along the same axis is left out; the TopK becomes the fused operator
+        std::unordered_map<std::string, const load::Node *> fused_softmax_of;  // TopK node name -> Softmax node
+        if (fuse_) {
+            for (const auto &n : model.nodes) {
+                if (ops::convert_opstring_to_enum(n.op_type) != ops::OpType::TOPK || n.inputs.empty()) continue;
+                auto p = producer.find(n.inputs[0].name);
+                if (p == producer.end() || ops::convert_opstring_to_enum(p->second->op_type) != ops::OpType::SOFTMAX) continue;
+                const auto &sm = *p->second;
+                if (sm.outputs.size() != 1 || sm.inputs.size() != 1 || consumers[sm.outputs[0].name] != 1 || outputs_.count(sm.outputs[0].name)) continue;
+                if (!same_axis(sm.attributes, n.attributes, static_cast<int>(sm.outputs[0].dims.size()))) continue;
+                fused_softmax_of[n.name] = &sm;
+            }
+        }
+        std::unordered_set<std::string> left_out;
+        for (const auto &f : fused_softmax_of) left_out.insert(f.second->name);
+        std::unordered_map<std::string, size_t> index_of_node;
+        for (const auto &level : model.getConcurrentExecutionLevels()) {
+            std::vector<size_t> level_indices;
+            for (const auto &node_name : level) {
+                auto found = node_by_name.find(node_name);
+                if (found == node_by_name.end()) throw std::runtime_error("LoadModel: level names unknown node " + node_name);
+                if (left_out.count(node_name)) continue;
+                const load::Node &n = *found->second;
+                const auto fused = fused_softmax_of.find(n.name);
+                const load::Node &reads = fused == fused_softmax_of.end() ? n : *fused->second;  // whose inputs and dependencies count
+                const auto type = ops::convert_opstring_to_enum(n.op_type);
+
+                std::vector<int> deps;
+                for (const auto &d : reads.dependencies) {
+                    auto at = index_of_node.find(d);
+                    if (at == index_of_node.end()) throw std::runtime_error("LoadModel: node " + n.name + " depends on " + d + ", which does not come before it");
+                    deps.push_back(static_cast<int>(at->second));
+                }
+                std::vector<std::shared_ptr<ITensor>> node_inputs, node_outputs;
+                for (const auto &in : reads.inputs) {
+                    auto t = tensor_map.find(in.name);
+                    if (t != tensor_map.end()) node_inputs.push_back(t->second);
+                    else if (in.dims.empty()) node_inputs.push_back(nullptr);  // optional input left out
+                    else throw std::runtime_error("LoadModel: node " + n.name + " reads " + in.name + ", which nothing produces");
+                }
+                for (size_t i = 0; i < n.outputs.size(); ++i) {
+                    const auto &out = n.outputs[i];
+                    auto t = tensor_map.find(out.name);
+                    if (t == tensor_map.end()) {
+                        auto made = make(out.dims, holds_indices(out.name));
+                        made->set_ref_cnt(static_cast<uint16_t>(consumers[out.name]));
+                        t = tensor_map.emplace(out.name, made).first;
+                    }
+                    node_outputs.push_back(t->second);
+                }
+                auto attributes = n.attributes;
+                if (type == ops::OpType::TOPK && !attributes.count("K") && !attributes.count("k") && n.inputs.size() > 1) {
+                    auto k = initializers_.find(n.inputs[1].name);
+                    if (k != initializers_.end() && k->second->dtype() == typeid(int64_t) && as_tensor<int64_t>(k->second)->num_elements() >= 1)
+                        attributes["K"] = std::to_string((*as_tensor<int64_t>(k->second))[0]);
+                }
+                if (type == ops::OpType::TOPK && node_inputs.size() > 1) node_inputs.resize(1);  // K is an attribute by now
+                std::unique_ptr<ops::Operator> op;
+                if (fused != fused_softmax_of.end()) op = std::make_unique<ops::SoftmaxTopk>(precision_);
+                else op = ops::create_from_type(type, node_outputs[0]->num_dims() <= 2, precision_, dev->is_support_nv_tensor_core());
+                op->set_name(n.name);
+                op->set_runtime_device(dev, m_cmdpool_);
+                op->setAttribute(attributes);
+
+                const size_t idx = node_ops_.size();
+                index_of_node[n.name] = idx;
+                if (fused != fused_softmax_of.end()) index_of_node[fused->second->name] = idx;
+                level_indices.push_back(idx);
+                node_ops_.push_back(std::move(op));
+                node_attrs_.push_back(std::move(attributes));
+                node_input_tensors_.push_back(std::move(node_inputs));
+                node_output_tensors_.push_back(std::move(node_outputs));
+                node_is_post_.push_back(false);
+                node_dependency_indices_.push_back(std::move(deps));
+            }
+            if (!level_indices.empty()) level_node_indices_.push_back(std::move(level_indices));
+        }
+        if (outputs_.size() == 1) output_ = outputs_.begin()->second;
+    }
+
+    // core/runtime.cpp:365-402
+    std::shared_ptr<ITensor> GetInput(const std::string &name = "") const { return pick(inputs_, name, "Input"); }
+    std::shared_ptr<ITensor> GetOutput(const std::string &name = "") const {
+        if (name.empty() && outputs_.empty()) return output_;  // no model: what SetOutput() handed in
+        return pick(outputs_, name, "Output");
+    }
+    std::shared_ptr<ITensor> GetInitializer(const std::string &name) const {
+        auto it = initializers_.find(name);
+        return it == initializers_.end() ? nullptr : it->second;
+    }
 
     // Switches the SOFTMAX + TOPK fusion off (for comparisons); on by default.
     void set_postprocess_fusion(bool on) { fuse_ = on; }
@@ -132,18 +302,27 @@ class Runtime {
 
   private:
     // The softmax must run along the axis the top-k selects on.
-    bool same_axis(size_t softmax_node, const std::unordered_map<std::string, std::string> &topk_attrs,
-                   const std::shared_ptr<ITensor> &t) const {
-        const int rank = t->num_dims();
+    static bool same_axis(const std::unordered_map<std::string, std::string> &s, const std::unordered_map<std::string, std::string> &topk_attrs,
+                          int rank) {
         auto norm = [rank](int a) { return a < 0 ? a + rank : a; };
         int sa = 0;  // Softmax's default (ops/Softmax.hpp: GpuSoftMaxParam starts at 0)
-        const auto &s = node_attrs_[softmax_node];
         if (s.count("axis")) sa = std::stoi(s.at("axis"));
         else if (s.count("dim")) sa = std::stoi(s.at("dim"));
         int ta = -1;  // TopK's default (ops/Topk.hpp:41)
         if (topk_attrs.count("axis")) ta = std::stoi(topk_attrs.at("axis"));
         if (rank == 1) return true;
         return norm(sa) == norm(ta);
+    }
+    bool same_axis(size_t softmax_node, const std::unordered_map<std::string, std::string> &topk_attrs,
+                   const std::shared_ptr<ITensor> &t) const {
+        return same_axis(node_attrs_[softmax_node], topk_attrs, t->num_dims());
+    }
+    static std::shared_ptr<ITensor> pick(const std::map<std::string, std::shared_ptr<ITensor>> &from, const std::string &name,
+                                         const char *what) {
+        if (name.empty() && from.size() > 1) throw std::runtime_error(std::string(what) + " name is empty but there are multiple");
+        if (name.empty() && from.size() == 1) return from.begin()->second;
+        auto it = from.find(name);
+        return it == from.end() ? nullptr : it->second;
     }
     void remove_last_node() {
         node_ops_.pop_back();
@@ -160,6 +339,7 @@ class Runtime {
     int precision_ = 0;
     bool fuse_ = true;
     std::shared_ptr<ITensor> output_;
+    std::map<std::string, std::shared_ptr<ITensor>> inputs_, outputs_, initializers_;
     std::vector<std::unique_ptr<ops::Operator>> node_ops_;
     std::vector<std::unordered_map<std::string, std::string>> node_attrs_;
     std::vector<std::vector<std::shared_ptr<ITensor>>> node_input_tensors_;

@@ -12,8 +12,12 @@
 
 #include <cmath>
 #include <cstdio>
+#include <algorithm>
 #include <cstring>
+#include <filesystem>
+#include <fstream>
 #include <functional>
+#include <iterator>
 #include <string>
 
 #include "core/Runtime.hpp"
@@ -260,20 +264,12 @@ template <typename T> void fused_case(const std::vector<int> &shape, int k) {
     EXPECT(tc.max_ulp <= 2);
 }
 
-// tests/NmsTest.cpp:29-160: boxes from uniform centres and sizes, uniform scores;
-// expectation: per (batch, class) the boxes at or above the score threshold, best
-// first, each kept box removing the later ones whose IoU with it exceeds the
-// threshold.  Written here over an IoU matrix and a sort of the whole score row.
-template <typename T>
-void nms_case(const std::vector<int> &box_shape, const std::vector<int> &score_shape, int per_class, float iou_thr,
-              float score_thr) {
-    TestCase<T> tc("Nms");
-    torch::manual_seed(11);
-    const int64_t B = box_shape[0], N = box_shape[1], C = score_shape[1];
-    auto scores = torch::rand({B, C, N}, tc.conf());
-    auto centre = torch::rand({B, N, 2}, tc.conf()), size = torch::rand({B, N, 2}, tc.conf()) * 1.3F;
-    auto boxes = torch::cat({torch::clamp(centre - size / 2, 0.0F, 1.0F), torch::clamp(centre + size / 2, 0.0F, 1.0F)}, -1);
+// tests/NmsTest.cpp:62-160: per (batch, class) the boxes at or above the score
+// threshold, best first, each kept box removing the later ones whose IoU with it
+// exceeds the threshold.  Written here over an IoU matrix and a sort of the whole score row.
+static std::vector<int> nms_expectation(const torch::Tensor &boxes, const torch::Tensor &scores, float iou_thr, float score_thr) {
     auto bf = boxes.to(torch::kFloat32), sf = scores.to(torch::kFloat32);
+    const int64_t B = bf.size(0), N = bf.size(1), C = sf.size(1);
     std::vector<int> records;
     for (int64_t b = 0; b < B; b++) {
         auto x1 = bf[b].select(-1, 0), y1 = bf[b].select(-1, 1), x2 = bf[b].select(-1, 2), y2 = bf[b].select(-1, 3);
@@ -297,6 +293,23 @@ void nms_case(const std::vector<int> &box_shape, const std::vector<int> &score_s
             }
         }
     }
+    return records;
+}
+
+// tests/NmsTest.cpp:29-160: boxes from uniform centres and sizes, uniform scores;
+// expectation: per (batch, class) the boxes at or above the score threshold, best
+// first, each kept box removing the later ones whose IoU with it exceeds the
+// threshold.  Written here over an IoU matrix and a sort of the whole score row.
+template <typename T>
+void nms_case(const std::vector<int> &box_shape, const std::vector<int> &score_shape, int per_class, float iou_thr,
+              float score_thr) {
+    TestCase<T> tc("Nms");
+    torch::manual_seed(11);
+    const int64_t B = box_shape[0], N = box_shape[1], C = score_shape[1];
+    auto scores = torch::rand({B, C, N}, tc.conf());
+    auto centre = torch::rand({B, N, 2}, tc.conf()), size = torch::rand({B, N, 2}, tc.conf()) * 1.3F;
+    auto boxes = torch::cat({torch::clamp(centre - size / 2, 0.0F, 1.0F), torch::clamp(centre + size / 2, 0.0F, 1.0F)}, -1);
+    std::vector<int> records = nms_expectation(boxes, scores, iou_thr, score_thr);
     auto in_boxes = std::make_shared<Tensor<T>>(box_shape);
     fill_from_torch(in_boxes, boxes);
     auto in_scores = std::make_shared<Tensor<T>>(score_shape);
@@ -495,9 +508,200 @@ static void runtime_postprocess_tests() {
     }
 }
 
+static std::string g_golden;  // directory of the .vkopbin fixtures
+
+static std::vector<uint8_t> file_bytes(const std::string &path) {
+    std::ifstream f(path, std::ios::binary);
+    return std::vector<uint8_t>(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+}
+
+// The model file reader against the reference's own model file and the fixtures
+// written by tests/golden/make_vkopbin.py; no device needed.
+static void model_file_tests() {
+    using vkop::load::VkModel;
+    {
+        // model/add_conv_model.vkopbin as the reference's converter wrote it (Add -> depthwise Conv, int8 weights)
+        const VkModel m(g_golden + "/add_conv_model.vkopbin");
+        EXPECT(m.inputs.size() == 2 && m.inputs[0].name == "input_x1" && m.inputs[1].name == "input_x2");
+        EXPECT((m.inputs[1].dims == std::vector<uint32_t>{1, 16, 8, 8}));
+        EXPECT(m.outputs.size() == 1 && m.outputs[0].name == "output");
+        EXPECT(m.nodes.size() == 2 && m.nodes[0].op_type == "Add" && m.nodes[0].name == "node_add" && m.nodes[0].attributes.empty());
+        EXPECT(m.nodes[0].dependencies.empty() && m.nodes[0].dependents.count("node_conv2d") == 1);
+        const auto &conv = m.nodes[1];
+        EXPECT(conv.op_type == "Conv" && conv.inputs.size() == 4 && conv.inputs[3].name == "conv.weight_scale");
+        EXPECT(conv.attributes.at("group") == "16" && conv.attributes.at("pads") == "[1, 1, 1, 1]" &&
+               conv.attributes.at("auto_pad") == "NOTSET" && conv.attributes.at("strides") == "[1, 1]");
+        EXPECT(conv.dependencies.count("node_add") == 1 && conv.dependents.empty());
+        EXPECT(m.initializers.size() == 3 && m.initializers.at("conv.weight").dtype == "int8");
+        EXPECT((m.initializers.at("conv.weight").dims == std::vector<uint32_t>{16, 1, 3, 3}));
+        const auto *w = reinterpret_cast<const int8_t *>(m.initializer_data("conv.weight"));
+        EXPECT(w[0] == 39 && w[1] == 127 && w[2] == 61 && w[3] == 18);
+        float bias0 = 0;
+        std::memcpy(&bias0, m.initializer_data("conv.bias"), 4);
+        EXPECT(std::fabs(bias0 - 0.03973345F) < 1e-8F);
+        for (const auto &o : m.initializer_offsets) EXPECT(o.second % 64 == 0);
+        EXPECT(m.initializer_bytes.at("conv.weight") == 144 && m.initializer_bytes.at("conv.bias") == 64);
+        EXPECT(m.concurrent_execution_levels.size() == 2 && m.concurrent_execution_levels[1] == std::vector<std::string>{"node_conv2d"});
+        EXPECT(!m.unified && !m.rgba);
+        // a runtime refuses it by the first operator it lacks (the check comes before any device work)
+        bool refused = false;
+        try {
+            vkop::core::Runtime rt(nullptr, g_golden + "/add_conv_model.vkopbin", 0);
+            rt.LoadModel();
+        } catch (const std::runtime_error &e) {
+            refused = std::string(e.what()).find("Add") != std::string::npos;
+        }
+        EXPECT(refused);
+    }
+    {
+        const VkModel m(g_golden + "/detection_tail.vkopbin");  // one attribute of each tagged kind
+        const auto &a = m.nodes.at(0).attributes;
+        EXPECT(m.nodes[0].op_type == "Nms" && a.size() == 7);
+        EXPECT(a.at("center_point_box") == "0" && a.at("iou_threshold") == "0.500000" && a.at("score_threshold") == "0.250000");
+        EXPECT(a.at("note") == "detection tail" && a.at("strides") == "[8, 16, 32]" && a.at("anchors") == "[1.500000, 2.250000]");
+        EXPECT((m.outputs[0].dims == std::vector<uint32_t>{1800, 3}));
+    }
+    {
+        const VkModel m(g_golden + "/classifier_head_k_input.vkopbin");
+        EXPECT(m.initializers.at("k_value").dtype == "int64" && m.initializers.at("k_value").dims == std::vector<uint32_t>{1});
+        int64_t k = 0;
+        std::memcpy(&k, m.initializer_data("k_value"), 8);
+        EXPECT(k == 7);
+        EXPECT(m.nodes[1].attributes.count("K") == 0 && m.nodes[1].inputs.size() == 2);
+    }
+    {
+        // every proper prefix of a file is refused with an exception, and so is a wrong tag, an
+        // oversized count and an oversized string; nothing reads past the bytes given
+        const auto bytes = file_bytes(g_golden + "/classifier_head.vkopbin");
+        EXPECT(bytes.size() > 100);
+        const VkModel whole(bytes.data(), bytes.size());
+        EXPECT(whole.nodes.size() == 2 && whole.nodes[1].attributes.at("K") == "5");
+        size_t refused = 0;
+        for (size_t n = 0; n < bytes.size(); ++n) {
+            std::vector<uint8_t> part(bytes.begin(), bytes.begin() + static_cast<std::ptrdiff_t>(n));  // exact-size heap block
+            try {
+                const VkModel m(part.data(), part.size());
+            } catch (const std::runtime_error &) {
+                refused++;
+            }
+        }
+        EXPECT(refused == bytes.size());
+        auto broken = [&](size_t at, uint8_t value) {
+            auto copy = bytes;
+            copy[at] = value;
+            try {
+                const VkModel m(copy.data(), copy.size());
+            } catch (const std::runtime_error &) {
+                return true;
+            }
+            return false;
+        };
+        EXPECT(broken(3, 0x7F));  // input count of 2 billion
+        EXPECT(broken(7, 0x7F));  // name length of 2 billion
+        const std::string key = "axis";
+        auto it = std::search(bytes.begin(), bytes.end(), key.begin(), key.end());
+        EXPECT(it != bytes.end());
+        if (it != bytes.end()) EXPECT(broken(static_cast<size_t>(it - bytes.begin()) + 4, 9));  // attribute tag 9
+    }
+}
+
+// Models from .vkopbin files through Runtime::LoadModel / Run / ReadResult.
+template <typename T> static void model_head_case(const std::string &file, int rows, int k, bool fuse, size_t want_nodes) {
+    auto pool = TestEnv::pool;
+    const int precision = std::is_same_v<T, uint16_t> ? 1 : 0;
+    vkop::core::Runtime rt(pool, g_golden + "/" + file, precision);
+    rt.set_postprocess_fusion(fuse);
+    rt.LoadModel();
+    EXPECT(rt.num_nodes() == want_nodes);
+    torch::manual_seed(5);
+    auto x = (torch::randn({rows, 1000}) * 3).to(precision ? torch::kFloat16 : torch::kFloat32);
+    auto in = vkop::core::as_tensor<T>(rt.GetInput("logits"));
+    EXPECT(in != nullptr && rt.GetInput() == rt.GetInput("logits") && rt.GetInput("nothing") == nullptr);
+    fill_from_torch(in, x);
+    in->copyToGPU(pool);
+    double ms = 0;
+    for (int i = 0; i < 3; i++) ms = rt.Run();
+    rt.ReadResult();
+    auto p = torch::softmax(x.to(torch::kFloat64), -1).to(precision ? torch::kFloat16 : torch::kFloat32);
+    auto sorted = torch::sort(p, /*stable=*/true, -1, /*descending=*/true);
+    auto ev = std::get<0>(sorted).slice(-1, 0, k).to(torch::kFloat32).contiguous();
+    auto ei = std::get<1>(sorted).slice(-1, 0, k).to(torch::kInt).contiguous();
+    auto values = vkop::core::as_tensor<T>(rt.GetOutput("values"));
+    auto indices = vkop::core::as_tensor<int>(rt.GetOutput("indices"));
+    EXPECT(values != nullptr && indices != nullptr);
+    bool ok = values && indices && values->getShape() == std::vector<int>{rows, k};
+    double worst = 0;
+    for (int i = 0; ok && i < rows * k; i++) {
+        const float got = precision ? ITensor::fp16_to_fp32(static_cast<uint16_t>((*values)[static_cast<size_t>(i)]))
+                                    : static_cast<float>((*values)[static_cast<size_t>(i)]);
+        const float want = ev.data_ptr<float>()[i];
+        worst = std::max(worst, static_cast<double>(std::fabs(got - want)) / std::max(1e-30, static_cast<double>(std::fabs(want))));
+        // equal probabilities (frequent in half precision) may come in either order in the sorted expectation only
+        // when they are equal: compare the index where the value is unique in its row
+        const int r = i / k, j = i % k;
+        const bool tied = (j > 0 && ev.data_ptr<float>()[i - 1] == want) || (j + 1 < k && ev.data_ptr<float>()[i + 1] == want) ||
+                          (j + 1 == k && std::get<0>(sorted)[r][k].item<float>() == want);
+        if (!tied) ok = ok && (*indices)[static_cast<size_t>(i)] == ei.data_ptr<int>()[i];
+    }
+    ok = ok && worst <= (precision ? 2e-3 : 3e-7);
+    if (rt.GetOutput("probs")) {  // the variant that also returns the probabilities
+        auto probs = vkop::core::as_tensor<T>(rt.GetOutput("probs"));
+        double sum = 0;
+        for (int i = 0; i < 1000; i++)
+            sum += precision ? ITensor::fp16_to_fp32(static_cast<uint16_t>((*probs)[static_cast<size_t>(i)])) : static_cast<float>((*probs)[static_cast<size_t>(i)]);
+        ok = ok && std::fabs(sum - 1.0) < (precision ? 2e-2 : 1e-5);
+    }
+    std::printf("Model %s %s [%d,1000] k %d, %zu operator(s) (%s): %s, worst relative difference %.2e, last Run() %.3f ms\n", file.c_str(),
+                precision ? "fp16" : "fp32", rows, k, rt.num_nodes(), rt.node_name(rt.num_nodes() - 1).c_str(), ok ? "ok" : "FAILED", worst, ms);
+    EXPECT(ok);
+}
+
+static void model_run_tests() {
+    TestEnv::initialize();
+    auto pool = TestEnv::pool;
+    model_head_case<float>("classifier_head.vkopbin", 8, 5, true, 1);
+    model_head_case<float>("classifier_head.vkopbin", 8, 5, false, 2);
+    model_head_case<uint16_t>("classifier_head.vkopbin", 8, 5, true, 1);
+    model_head_case<float>("classifier_head_k_input.vkopbin", 4, 7, true, 2);  // probabilities are an output: two operators
+    model_head_case<uint16_t>("classifier_head_k_input.vkopbin", 4, 7, true, 2);
+    {
+        vkop::core::Runtime rt(pool, g_golden + "/detection_tail.vkopbin", 0);
+        rt.LoadModel();
+        EXPECT(rt.num_nodes() == 1);
+        bool threw = false;
+        try {
+            rt.GetInput();
+        } catch (const std::runtime_error &) {
+            threw = true;
+        }
+        EXPECT(threw);  // two inputs: a name is needed (core/runtime.cpp:366-369)
+        torch::manual_seed(11);
+        auto scores = torch::rand({2, 3, 300});
+        auto centre = torch::rand({2, 300, 2}), size = torch::rand({2, 300, 2}) * 0.3F;
+        auto boxes = torch::cat({centre - size / 2, centre + size / 2}, -1);
+        auto tb = vkop::core::as_tensor<float>(rt.GetInput("boxes"));
+        auto ts = vkop::core::as_tensor<float>(rt.GetInput("scores"));
+        fill_from_torch(tb, boxes);
+        fill_from_torch(ts, scores);
+        tb->copyToGPU(pool);
+        ts->copyToGPU(pool);
+        rt.Run();
+        rt.ReadResult();
+        const auto want = nms_expectation(boxes, scores, 0.5F, 0.25F);
+        auto out = vkop::core::as_tensor<int>(rt.GetOutput());
+        bool ok = out && want.size() + 3 <= static_cast<size_t>(out->num_elements());
+        for (size_t i = 0; ok && i < want.size(); i++) ok = (*out)[i] == want[i];
+        for (size_t i = want.size(); ok && i < want.size() + 3; i++) ok = (*out)[i] == -1;  // the end of the list
+        std::printf("Model detection_tail.vkopbin: %s, %zu records\n", ok ? "ok" : "FAILED", want.size() / 3);
+        EXPECT(ok && !want.empty());
+    }
+}
+
 int main(int argc, char **argv) {
     const bool no_gpu = argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0;
+    g_golden = (std::filesystem::path(argv[0]).parent_path() / ".." / ".." / ".." / "tests" / "golden").string();
     host_logic_tests();
+    model_file_tests();
     if (!no_gpu) {
         const std::vector<std::pair<std::vector<int>, int>> softmax_cases = {
             {{1, 10, 7, 7}, 1}, {{1, 6, 8, 8}, 3}, {{2, 4, 10, 10}, 2}, {{1, 8, 6, 6}, 2}, {{1, 16, 5, 5}, 1}, {{4, 1000}, 1},
@@ -524,6 +728,7 @@ int main(int argc, char **argv) {
         nms_case<float>({1, 200, 4}, {1, 1, 200}, 0, 0.7F, 0.4F);
         nms_case<float>({1, 50, 4}, {1, 7, 50}, 0, 0.3F, 0.2F);
         nms_case<uint16_t>({2, 300, 4}, {2, 3, 300}, 0, 0.5F, 0.3F);
+        model_run_tests();
         // the benchmark's arrangement: full-size outputs, the first k read back
         {
             TestEnv::initialize();
