@@ -714,7 +714,8 @@ def _nms_boxes(rng, B, N, spread=1.3):
 @pytest.mark.parametrize("B,C,N,max_per_class,iou_thr,score_thr", [
     (1, 2, 10, 0, 0.5, 0.5), (1, 1, 200, 50, 0.7, 0.4), (1, 7, 50, 0, 0.3, 0.2),      # tests/NmsTest.cpp:165-169
     (3, 5, 300, 0, 0.45, 0.25), (2, 3, 3000, 100, 0.5, 0.3), (16, 4, 8400, 0, 0.6, 0.9), (1, 1, 1, 0, 0.5, 0.1),
-    (2, 2, 1500, 0, 0.5, -1.0)])
+    (2, 2, 1500, 0, 0.5, -1.0),
+    (1, 2, 30000, 0, 0.5, 0.95), (1, 1, 40000, 50, 0.5, 0.9), (2, 1, 12289, 0, 0.4, 0.9)])   # several rounds of the scan
 def test_nms_matches_the_oracle(ops, B, C, N, max_per_class, iou_thr, score_thr):
     rng = np.random.default_rng(B * 1000 + N)
     boxes = _nms_boxes(rng, B, N, 1.3 if N <= 300 else 0.2)
@@ -738,6 +739,26 @@ def test_nms_matches_the_oracle(ops, B, C, N, max_per_class, iou_thr, score_thr)
     if len(want) > 3:
         few, _ = ops.nms(dev(boxes), dev(scores), iou_thr, score_thr, max_per_class, out_capacity=3)
         assert np.array_equal(host(few), want[:3])
+
+
+def test_nms_detection_workload_full_size(ops):
+    """The detection-shaped case of the operator benchmark, and a dense one with a per-class limit, against the oracle."""
+    c5 = synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"])
+    e = np.exp(c5 - c5.max(axis=1, keepdims=True))
+    scores = np.ascontiguousarray((e / e.sum(axis=1, keepdims=True)).astype(np.float32))
+    rng = np.random.default_rng(synth.SEEDS["C5"] + 1)
+    boxes = _nms_boxes(rng, 16, 8400, 0.2)
+    got, over = ops.nms(dev(boxes), dev(scores), 0.45, 0.25, 100)
+    want = oracle.nms(boxes, scores, 0.45, 0.25, 100, max_candidates=2048)
+    assert not over and len(want) > 10000 and np.array_equal(host(got), want)
+    # keeping is idempotent: the kept boxes of a pair suppress nothing among themselves
+    first = want[(want[:, 0] == 3) & (want[:, 1] == 7)][:, 2]
+    again, _ = ops.nms(dev(boxes[3:4, first]), dev(scores[3:4, 7:8, first]), 0.45, 0.25, 100)
+    assert len(host(again)) == len(first)
+    dense_scores = rng.random((4, 20, 2048)).astype(np.float32)
+    got, over = ops.nms(dev(boxes[:4, :2048]), dev(dense_scores), 0.5, 0.0, 200)
+    want = oracle.nms(boxes[:4, :2048], dense_scores, 0.5, 0.0, 200, max_candidates=2048)
+    assert not over and np.array_equal(host(got), want) and len(want) == 4 * 20 * 200
 
 
 # ---- models from .vkopbin files ---------------------------------------------------------------------
