@@ -177,6 +177,9 @@ int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_ca
  *       only the chunk kernel, 2 = only the merge kernel.  1 and 2 exist so
  *       that a benchmark can time each kernel by itself; their results are not
  *       valid top-k output.
+ *   "nms.threads": threads per workgroup of the Nms kernel: 0 (default) = 256
+ *       from 1024 (batch, class) pairs on, else 1024; 256 or 1024 force one.
+ *       Results are identical.
  * Unknown names return VKOP_HIP_ERR_INVALID. */
 int vkop_hip_tune(const char *name, int value);
 

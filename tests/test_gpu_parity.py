@@ -741,6 +741,26 @@ def test_nms_matches_the_oracle(ops, B, C, N, max_per_class, iou_thr, score_thr)
         assert np.array_equal(host(few), want[:3])
 
 
+@pytest.mark.parametrize("threads", [256, 1024])
+def test_nms_either_workgroup_size(ops, threads):
+    """The kernel has a 256-thread and a 1024-thread form, picked by the number of pairs: each on sparse, dense,
+    multi-block and overflowing candidate sets."""
+    from vkop_amd import capi
+    capi.tune("nms.threads", threads)
+    try:
+        for B, C, N, per_class, iou_thr, score_thr in [(1, 3, 50, 0, 0.3, 0.2), (2, 3, 3000, 100, 0.5, 0.3), (1, 2, 2048, 0, 0.6, -1.0),
+                                                       (1, 1, 600, 0, 0.5, 0.1), (1, 2, 30000, 0, 0.5, 0.95), (3, 2, 700, 7, 0.4, 0.5)]:
+            rng = np.random.default_rng(N + threads)
+            boxes = _nms_boxes(rng, B, N, 1.3 if N <= 300 else 0.2)
+            scores = rng.random((B, C, N)).astype(np.float32)
+            got, over = ops.nms(dev(boxes), dev(scores), iou_thr, score_thr, per_class)
+            want = oracle.nms(boxes, scores, iou_thr, score_thr, per_class, max_candidates=2048)
+            assert np.array_equal(host(got), want), (threads, B, C, N)
+            assert over == bool(((scores > score_thr).sum(axis=-1) > 2048).any())
+    finally:
+        capi.tune("nms.threads", 0)
+
+
 def test_nms_detection_workload_full_size(ops):
     """The detection-shaped case of the operator benchmark, and a dense one with a per-class limit, against the oracle."""
     c5 = synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"])

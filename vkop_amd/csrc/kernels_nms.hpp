@@ -5,9 +5,9 @@
 // the whole workgroup instead of its first thread:
 //   1. the boxes whose score is greater than the threshold are collected in box
 //      order (ballot prefix per tile of 1024 boxes), at most kNmsMaxCandidates;
-//   2. they are sorted by (score, then lower box index) with a bitonic network over
-//      64-bit composites in LDS, and their corner coordinates are staged in LDS in
-//      that order;
+//   2. they are sorted by (score, then lower box index) as 64-bit composites in LDS
+//      (counting sort for few, bitonic network for many), and every thread loads the
+//      corner coordinates of its own sorted positions into registers;
 //   3. the sorted list is walked in blocks of 64: all waves compute, for every
 //      candidate of the block, which earlier ones of the block would suppress it
 //      (IoU as in shaders/nms.comp:61-72, every operation rounded on its own so
@@ -29,7 +29,9 @@
 
 namespace vkop {
 
-constexpr int kNmsThreads = 1024;
+constexpr int kNmsThreadsWide = 1024;   // few (batch, class) pairs
+constexpr int kNmsThreadsNarrow = 256;  // many
+constexpr int kNmsNarrowMinPairs = 1024;
 constexpr int kNmsMaxCandidates = 2048;  // per (batch, class); the reference's shader holds 1024
 constexpr int kNmsRankSortMax = 512;     // up to here a counting sort beats the bitonic network's barriers
 
@@ -49,47 +51,57 @@ __device__ __forceinline__ float nms_iou(const float4 &a, const float4 &b) {
 
 // counts[pair] = boxes selected; counts[pairs + pair] = 1 if more than
 // kNmsMaxCandidates boxes passed the score threshold (the later ones were left out).
-// selected: [pairs][max_sel] box indices.  Launch: B * C workgroups of kNmsThreads.
-template <typename T>
-__global__ __launch_bounds__(kNmsThreads) __attribute__((amdgpu_waves_per_eu(8))) void nms_kernel(const T *__restrict__ boxes, const T *__restrict__ scores,
-                                                          int32_t *__restrict__ selected, uint32_t *__restrict__ counts,
-                                                          uint32_t pairs, uint32_t C, uint32_t N, int center_point_box,
-                                                          uint32_t max_out, float iou_threshold, float score_threshold,
-                                                          uint32_t max_sel) {
-    constexpr int NT = kNmsThreads;
+// selected: [pairs][max_sel] box indices.  Launch: B * C workgroups of NT threads:
+// 1024 when there are few pairs (one pair's work spread wide), 256 when there are
+// enough pairs to put many workgroups on a CU, so that one's score loads overlap
+// another's sort and walk.  Each thread keeps the boxes of its own kNmsMaxCandidates / NT
+// sorted candidates in registers; LDS holds the composites and two blocks of 64 boxes.
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nms_kernel(
+    const T *__restrict__ boxes, const T *__restrict__ scores, int32_t *__restrict__ selected, uint32_t *__restrict__ counts,
+    uint32_t pairs, uint32_t C, uint32_t N, int center_point_box, uint32_t max_out, float iou_threshold, float score_threshold,
+    uint32_t max_sel) {
+    static_assert(NT % kWave == 0 && kNmsMaxCandidates % NT == 0 && (kNmsRankSortMax % NT == 0 || NT % kNmsRankSortMax == 0), "workgroup size");
     constexpr int NW = NT / kWave;
-    constexpr int PER = kNmsMaxCandidates / NT;  // sorted candidates per thread
+    constexpr int PER = kNmsMaxCandidates / NT;      // sorted candidates per thread
+    constexpr int SMALL = NT >= kNmsRankSortMax ? 1 : kNmsRankSortMax / NT;  // of them, when the counting sort applies
+    constexpr int JP = kWave / NW;                   // candidates of a block each wave tests the block against
+    constexpr int TILES = NT >= 1024 ? 12 : 36;      // scores per thread and round
     __shared__ uint64_t comp[kNmsMaxCandidates];
-    __shared__ float4 sbox[kNmsMaxCandidates];
+    __shared__ float4 block_box[2][kWave];
     __shared__ unsigned long long active[kNmsMaxCandidates / 64];
     __shared__ unsigned long long block_cols[kWave];
     __shared__ unsigned long long block_keep;
-    constexpr int TILES = 12;  // scores per thread and round
     __shared__ uint32_t wave_n[2][NW];
-    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = uniform_u32(tid) / kWave;  // (scalar)
     const uint32_t pair = blockIdx.x, batch = pair / C;
     const T *srow = scores + static_cast<size_t>(pair) * N;
     const T *brow = boxes + static_cast<size_t>(batch) * N * 4;
+    if (tid < static_cast<uint32_t>(kNmsMaxCandidates / 64)) active[tid] = ~0ull;  // positions at or after K are masked where read
+    if (tid >= NT - kWave) block_cols[lane] = 0;
 
     // ---- 1. candidates, in box order ----------------------------------------------
-    // A round covers NT * TILES boxes, each wave a contiguous run of them, so that all of a thread's scores are
-    // in flight together and the places inside a wave follow from scalar counts; one barrier per round.
+    // A round covers NT * TILES boxes, each wave a contiguous run of them (tiles of 64), so that all of a thread's
+    // scores are in flight together; one barrier per round.  Candidates are rare in a detection head, and every
+    // wave instruction here is paid NT / 64 times per workgroup: per tile the vector unit sees the load, its
+    // address and one comparison per pass; tile bounds, counts and places are scalar, and a tile without a
+    // candidate is left with one scalar branch.
     uint32_t found = 0, round = 0;  // the same in every thread
     for (uint32_t base = 0; base < N; base += NT * TILES, round++) {  // (to the end: the count tells whether boxes were left out)
         const uint32_t tiles = min(static_cast<uint32_t>(TILES), (N - base + NT - 1) / NT);  // per wave, this round
-        const uint32_t first = base + wave * tiles * kWave + lane;
+        const uint32_t wave_first = base + wave * tiles * kWave;
         float s[TILES];
 #pragma unroll
-        for (int u = 0; u < TILES; u++) {
-            const uint32_t i = first + static_cast<uint32_t>(u) * kWave;
-            s[u] = load_elem(srow, (static_cast<uint32_t>(u) < tiles && i < N) ? i : 0u);
-        }
+        for (int u = 0; u < TILES; u++)  // (past the end of the row: its last score again, masked out below)
+            s[u] = load_elem(srow, min(wave_first + static_cast<uint32_t>(u) * kWave + lane, N - 1));
+        auto candidates = [&](int u) -> uint64_t {
+            const uint32_t t0 = wave_first + static_cast<uint32_t>(u) * kWave;
+            const uint64_t valid = (static_cast<uint32_t>(u) >= tiles || t0 >= N) ? 0ull : (N - t0 >= kWave ? ~0ull : (1ull << (N - t0)) - 1ull);
+            return __ballot(s[u] > score_threshold) & valid;
+        };
         uint32_t in_wave = 0;
 #pragma unroll
-        for (int u = 0; u < TILES; u++) {
-            const uint32_t i = first + static_cast<uint32_t>(u) * kWave;
-            in_wave += static_cast<uint32_t>(__popcll(__ballot(static_cast<uint32_t>(u) < tiles && i < N && s[u] > score_threshold)));
-        }
+        for (int u = 0; u < TILES; u++) in_wave += static_cast<uint32_t>(__popcll(candidates(u)));
         if (lane == 0) wave_n[round & 1u][wave] = in_wave;
         __syncthreads();
         uint32_t pos = found;
@@ -99,45 +111,55 @@ __global__ __launch_bounds__(kNmsThreads) __attribute__((amdgpu_waves_per_eu(8))
             pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
             found += c;
         }
+        if (in_wave != 0) {
 #pragma unroll
-        for (int u = 0; u < TILES; u++) {
-            const uint32_t i = first + static_cast<uint32_t>(u) * kWave;
-            const bool pass = static_cast<uint32_t>(u) < tiles && i < N && s[u] > score_threshold;
-            const uint64_t mask = __ballot(pass);  // (again rather than kept: a dozen masks crowd the scalar registers)
-            const uint32_t at = pos + lanes_below(mask);
-            if (pass && at < static_cast<uint32_t>(kNmsMaxCandidates)) comp[at] = composite(order_key(s[u]), i);
-            pos += static_cast<uint32_t>(__popcll(mask));
+            for (int u = 0; u < TILES; u++) {
+                const uint64_t mask = candidates(u);  // (again rather than kept: dozens of masks crowd the scalar registers)
+                if (mask != 0) {
+                    const uint32_t at = pos + lanes_below(mask);
+                    if (((mask >> lane) & 1ull) && at < static_cast<uint32_t>(kNmsMaxCandidates))
+                        comp[at] = composite(order_key(s[u]), wave_first + static_cast<uint32_t>(u) * kWave + lane);
+                    pos += static_cast<uint32_t>(__popcll(mask));
+                }
+            }
         }
     }
     const uint32_t K = min(found, static_cast<uint32_t>(kNmsMaxCandidates));
-    uint32_t p2 = 1;
-    while (p2 < K) p2 <<= 1;
-    __syncthreads();
-    for (uint32_t t = K + tid; t < p2; t += NT) comp[t] = 0;  // below every real composite
-    if (tid >= NT - kWave) block_cols[lane] = 0;
-    if (tid < static_cast<uint32_t>(kNmsMaxCandidates / 64)) {
-        const uint32_t first = tid * 64;
-        active[tid] = first + 64 <= K ? ~0ull : (first < K ? ((1ull << (K - first)) - 1ull) : 0ull);
-    }
     __syncthreads();
 
     // ---- 2. by score, largest first; equal scores: lower box index first --------------
     if (K > static_cast<uint32_t>(kNmsRankSortMax)) {
+        uint32_t p2 = 1;
+        while (p2 < K) p2 <<= 1;
+        for (uint32_t t = K + tid; t < p2; t += NT) comp[t] = 0;  // below every real composite
+        __syncthreads();
         bitonic_sort_desc<NT>(comp, p2);
     } else if (K > 1) {
         // few candidates: each counts the composites above its own (all distinct) and moves there; two barriers
         // instead of one per step of the network
-        const uint64_t c = tid < K ? comp[tid] : 0;
-        uint32_t rank = 0;
+        uint64_t c[SMALL];
+        uint32_t rank[SMALL];
+#pragma unroll
+        for (int e = 0; e < SMALL; e++) {
+            const uint32_t p = static_cast<uint32_t>(e) * NT + tid;
+            c[e] = p < K ? comp[p] : 0;
+            rank[e] = 0;
+        }
         if (tid < K) {
-#pragma unroll 8
-            for (uint32_t q = 0; q < K; q++) rank += comp[q] > c ? 1u : 0u;
+#pragma unroll 16
+            for (uint32_t q = 0; q < K; q++) {
+                const uint64_t other = comp[q];
+#pragma unroll
+                for (int e = 0; e < SMALL; e++) rank[e] += other > c[e] ? 1u : 0u;
+            }
         }
         __syncthreads();
-        if (tid < K) comp[rank] = c;
+#pragma unroll
+        for (int e = 0; e < SMALL; e++)
+            if (static_cast<uint32_t>(e) * NT + tid < K) comp[rank[e]] = c[e];
         __syncthreads();
     }
-    float4 mine[PER];
+    float4 mine[PER];  // corners of this thread's candidates: sorted positions e * NT + tid
 #pragma unroll
     for (int e = 0; e < PER; e++) {
         const uint32_t p = static_cast<uint32_t>(e) * NT + tid;
@@ -150,26 +172,35 @@ __global__ __launch_bounds__(kNmsThreads) __attribute__((amdgpu_waves_per_eu(8))
                 b = make_float4(__fsub_rn(b.x, hw), __fsub_rn(b.y, hh), __fadd_rn(b.x, hw), __fadd_rn(b.y, hh));
             }
             mine[e] = b;
-            sbox[p] = b;
         }
     }
-    __syncthreads();
 
     // ---- 3. walk the list, 64 candidates at a time ------------------------------------
     const uint32_t limit = max_out > 0 ? min(max_out, K) : K;
     uint32_t chosen = 0;
     for (uint32_t base = 0; base < K && chosen < limit; base += kWave) {
+        // the block's boxes go to LDS: its 64 positions belong to the lanes of one wave (two buffers in turn:
+        // the block before may still be read by slower waves in step c)
+        float4(&box)[kWave] = block_box[(base / kWave) & 1u];
+        if (wave == (base % NT) / kWave) {
+            float4 b = mine[0];
+#pragma unroll
+            for (int e = 1; e < PER; e++)
+                if (static_cast<uint32_t>(e) == base / NT) b = mine[e];
+            box[lane] = b;
+        }
+        __syncthreads();
         // a. for candidate i of the block (one per lane, in every wave) the earlier candidates of the block that
-        //    would suppress it: each wave tests four of them and adds its four bits to the lane's word
-        //    (positions at or after K hold nothing: they are never active below)
-        const float4 bi = sbox[base + lane];
+        //    would suppress it: each wave tests JP of them and adds its bits to the lane's word
+        //    (positions at or after K hold zeros: they are never active below)
+        const float4 bi = box[lane];
         uint32_t bits = 0;
 #pragma unroll
-        for (int r = 0; r < kWave / NW; r++) {
-            const uint32_t j = wave * (kWave / NW) + static_cast<uint32_t>(r);
-            if (lane > j && nms_iou(bi, sbox[base + j]) > iou_threshold) bits |= 1u << r;
+        for (int r = 0; r < JP; r++) {
+            const uint32_t j = wave * JP + static_cast<uint32_t>(r);
+            if (lane > j && nms_iou(bi, box[j]) > iou_threshold) bits |= 1u << r;
         }
-        if (bits != 0) atomicOr(&block_cols[lane], static_cast<unsigned long long>(bits) << (wave * (kWave / NW)));
+        if (bits != 0) atomicOr(&block_cols[lane], static_cast<unsigned long long>(bits) << (wave * JP));
         __syncthreads();  // (also: the bits cleared by the block before are in place)
         // b. the first wave resolves the block.  Kept = active and suppressed by nobody kept before it: that set is
         //    the only fixed point of  S -> { i active : no member of S suppresses i },  and iterating from any S
@@ -177,7 +208,7 @@ __global__ __launch_bounds__(kNmsThreads) __attribute__((amdgpu_waves_per_eu(8))
         if (wave == 0) {
             const unsigned long long col = block_cols[lane];
             block_cols[lane] = 0;  // for the next block (its additions come after the next barrier)
-            const bool alive = (active[base / kWave] >> lane) & 1ull;
+            const bool alive = base + lane < K && ((active[base / kWave] >> lane) & 1ull);
             uint64_t keep = __ballot(alive);
             for (int step = 0; step < kWave; step++) {
                 const uint64_t next = __ballot(alive && (col & keep) == 0);
@@ -206,11 +237,11 @@ __global__ __launch_bounds__(kNmsThreads) __attribute__((amdgpu_waves_per_eu(8))
             if (p >= base + kWave && p < K && ((active[p / 64] >> (p % 64)) & 1ull)) {
                 bool dead = false;
                 for (uint64_t kk = keep; kk != 0 && !dead; kk &= kk - 1)
-                    dead = nms_iou(mine[e], sbox[base + static_cast<uint32_t>(__builtin_ctzll(kk))]) > iou_threshold;
+                    dead = nms_iou(mine[e], box[static_cast<uint32_t>(__builtin_ctzll(kk))]) > iou_threshold;
                 if (dead) atomicAnd(&active[p / 64], ~(1ull << (p % 64)));
             }
         }
-        // (no barrier here: a. of the next block touches neither the mask nor block_keep, and its barrier orders the rest)
+        // (no barrier here: the next block writes the other box buffer, and its barriers order the rest)
     }
     if (tid == 0) {
         counts[pair] = min(chosen, max_sel);

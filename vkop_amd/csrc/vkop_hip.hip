@@ -95,7 +95,7 @@ int launched(const char *what) {
 }
 
 // vkop_hip_tune state
-std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0};
+std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0}, g_nms_threads{0};
 
 // The per-row arrival counters of the one-kernel top-k variant sit at a fixed
 // place, the first kTicketRows words of every workspace, whatever the operator
@@ -610,10 +610,17 @@ int nms_impl(const T *boxes, const T *scores, int32_t *out, int out_capacity, in
     auto *counts = reinterpret_cast<uint32_t *>(base);
     auto *selected = reinterpret_cast<int32_t *>(base + align_up(2 * static_cast<size_t>(pairs) * sizeof(uint32_t)));
     const uint32_t max_sel = nms_max_sel(N, max_per_class);
-    vkop::nms_kernel<T><<<pairs, vkop::kNmsThreads, 0, st>>>(boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C),
-                                                             static_cast<uint32_t>(N), center_point_box,
-                                                             max_per_class > 0 ? static_cast<uint32_t>(max_per_class) : 0u,
-                                                             iou_threshold, score_threshold, max_sel);
+    const uint32_t per = max_per_class > 0 ? static_cast<uint32_t>(max_per_class) : 0u;
+    const int knob = g_nms_threads;  // 0: by the number of pairs
+    const bool narrow = knob > 0 ? knob == vkop::kNmsThreadsNarrow : pairs >= static_cast<uint32_t>(vkop::kNmsNarrowMinPairs);
+    if (narrow)
+        vkop::nms_kernel<T, vkop::kNmsThreadsNarrow><<<pairs, vkop::kNmsThreadsNarrow, 0, st>>>(
+            boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C), static_cast<uint32_t>(N), center_point_box, per,
+            iou_threshold, score_threshold, max_sel);
+    else
+        vkop::nms_kernel<T, vkop::kNmsThreadsWide><<<pairs, vkop::kNmsThreadsWide, 0, st>>>(
+            boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C), static_cast<uint32_t>(N), center_point_box, per,
+            iou_threshold, score_threshold, max_sel);
     if (int rc = launched("nms_kernel")) return rc;
     vkop::nms_pack_kernel<<<pairs, 256, 0, st>>>(selected, counts, out, out_count, pairs, static_cast<uint32_t>(C), max_sel,
                                                  static_cast<uint32_t>(out_capacity));
@@ -886,6 +893,11 @@ int vkop_hip_tune(const char *name, int value) {
     else if (std::strcmp(name, "rows.loads") == 0) g_rows_loads = value;
     else if (std::strcmp(name, "rows.chunks") == 0) g_rows_chunks = value;
     else if (std::strcmp(name, "rows.fused") == 0) g_rows_fused = value != 0;
+    else if (std::strcmp(name, "nms.threads") == 0) {
+        if (value != 0 && value != vkop::kNmsThreadsNarrow && value != vkop::kNmsThreadsWide)
+            return fail(VKOP_HIP_ERR_INVALID, "nms.threads must be 0, %d or %d", vkop::kNmsThreadsNarrow, vkop::kNmsThreadsWide);
+        g_nms_threads = value;
+    }
     else if (std::strcmp(name, "rows.stages") == 0) {
         if (value < 1 || value > 3) return fail(VKOP_HIP_ERR_INVALID, "rows.stages must be 1, 2 or 3");
         g_rows_stages = value;
