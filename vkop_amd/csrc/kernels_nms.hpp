@@ -94,11 +94,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nm
 #pragma unroll
         for (int u = 0; u < TILES; u++)  // (past the end of the row: its last score again, masked out below)
             s[u] = load_elem(srow, min(wave_first + static_cast<uint32_t>(u) * kWave + lane, N - 1));
-        auto candidates = [&](int u) -> uint64_t {
-            const uint32_t t0 = wave_first + static_cast<uint32_t>(u) * kWave;
-            const uint64_t valid = (static_cast<uint32_t>(u) >= tiles || t0 >= N) ? 0ull : (N - t0 >= kWave ? ~0ull : (1ull << (N - t0)) - 1ull);
-            return __ballot(s[u] > score_threshold) & valid;
-        };
+        // lane l's score of tile u exists iff u * 64 < reach: inside the row and inside this wave's run
+        const int32_t reach = static_cast<int32_t>(min(N - min(N, wave_first), tiles * kWave)) - static_cast<int32_t>(lane);
+        auto candidates = [&](int u) -> uint64_t { return __ballot(s[u] > score_threshold && reach > u * kWave); };
         uint32_t in_wave = 0;
 #pragma unroll
         for (int u = 0; u < TILES; u++) in_wave += static_cast<uint32_t>(__popcll(candidates(u)));
@@ -114,7 +112,10 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nm
         if (in_wave != 0) {
 #pragma unroll
             for (int u = 0; u < TILES; u++) {
-                const uint64_t mask = candidates(u);  // (again rather than kept: dozens of masks crowd the scalar registers)
+                // (again rather than kept: dozens of masks crowd the scalar registers and get spilled; the empty
+                //  statement keeps the compiler from reusing the first pass's)
+                asm volatile("" : "+v"(s[u]));
+                const uint64_t mask = candidates(u);
                 if (mask != 0) {
                     const uint32_t at = pos + lanes_below(mask);
                     if (((mask >> lane) & 1ull) && at < static_cast<uint32_t>(kNmsMaxCandidates))
