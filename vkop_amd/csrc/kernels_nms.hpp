@@ -117,6 +117,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nm
                 asm volatile("" : "+v"(s[u]));
                 const uint64_t mask = candidates(u);
                 if (mask != 0) {
+                    asm volatile("; a tile with candidates");  // (a real branch: as straight-line code all tiles pay for the few)
                     const uint32_t at = pos + lanes_below(mask);
                     if (((mask >> lane) & 1ull) && at < static_cast<uint32_t>(kNmsMaxCandidates))
                         comp[at] = composite(order_key(s[u]), wave_first + static_cast<uint32_t>(u) * kWave + lane);
