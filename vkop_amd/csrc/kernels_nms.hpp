@@ -39,6 +39,16 @@ __device__ __forceinline__ uint32_t uniform_u32(uint32_t x) {
     return static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(x)));
 }
 
+// Four consecutive scores starting at element i (i a multiple of four, the row 16-byte aligned).
+__device__ __forceinline__ float4 nms_load4(const float *p, uint32_t i) { return *reinterpret_cast<const float4 *>(p + i); }
+__device__ __forceinline__ float4 nms_load4(const uint16_t *p, uint32_t i) {
+    const uint2 w = *reinterpret_cast<const uint2 *>(p + i);
+    return make_float4(__half2float(__ushort_as_half(static_cast<unsigned short>(w.x & 0xFFFFu))),
+                       __half2float(__ushort_as_half(static_cast<unsigned short>(w.x >> 16))),
+                       __half2float(__ushort_as_half(static_cast<unsigned short>(w.y & 0xFFFFu))),
+                       __half2float(__ushort_as_half(static_cast<unsigned short>(w.y >> 16))));
+}
+
 __device__ __forceinline__ float nms_iou(const float4 &a, const float4 &b) {
     const float x1 = fmaxf(a.x, b.x), y1 = fmaxf(a.y, b.y), x2 = fminf(a.z, b.z), y2 = fminf(a.w, b.w);
     if (x2 <= x1 || y2 <= y1) return 0.f;
@@ -56,7 +66,7 @@ __device__ __forceinline__ float nms_iou(const float4 &a, const float4 &b) {
 // enough pairs to put many workgroups on a CU, so that one's score loads overlap
 // another's sort and walk.  Each thread keeps the boxes of its own kNmsMaxCandidates / NT
 // sorted candidates in registers; LDS holds the composites and two blocks of 64 boxes.
-template <typename T, int NT>
+template <typename T, int NT, bool VEC>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nms_kernel(
     const T *__restrict__ boxes, const T *__restrict__ scores, int32_t *__restrict__ selected, uint32_t *__restrict__ counts,
     uint32_t pairs, uint32_t C, uint32_t N, int center_point_box, uint32_t max_out, float iou_threshold, float score_threshold,
@@ -87,6 +97,61 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nm
     // address and one comparison per pass; tile bounds, counts and places are scalar, and a tile without a
     // candidate is left with one scalar branch.
     uint32_t found = 0, round = 0;  // the same in every thread
+    if constexpr (VEC) {
+        // Rows that start on a 16-byte boundary and hold a multiple of four scores: a lane takes four consecutive
+        // scores with one load, a quarter of the loads, addresses and bounds checks of the form below.  Places stay
+        // in box order: lanes below, then the lane's own components below.
+        constexpr int VT = TILES / 4;
+        for (uint32_t base = 0; base < N; base += NT * TILES, round++) {
+            const uint32_t tiles = min(static_cast<uint32_t>(VT), (N - base + NT * 4 - 1) / (NT * 4));  // per wave, this round
+            const uint32_t wave_first = base + wave * tiles * (kWave * 4);
+            float4 s[VT];
+#pragma unroll
+            for (int u = 0; u < VT; u++)  // (past the end of the row: its last four again, masked out below)
+                s[u] = nms_load4(srow, min(wave_first + static_cast<uint32_t>(u) * (kWave * 4) + lane * 4, N - 4));
+            const int32_t reach = static_cast<int32_t>(min(N - min(N, wave_first), tiles * (kWave * 4))) - static_cast<int32_t>(lane * 4);
+            uint32_t in_wave = 0;
+#pragma unroll
+            for (int u = 0; u < VT; u++) {
+                const bool here = reach > u * (kWave * 4);
+                in_wave += static_cast<uint32_t>(__popcll(__ballot(here && s[u].x > score_threshold)) + __popcll(__ballot(here && s[u].y > score_threshold)) +
+                                                 __popcll(__ballot(here && s[u].z > score_threshold)) + __popcll(__ballot(here && s[u].w > score_threshold)));
+            }
+            if (lane == 0) wave_n[round & 1u][wave] = in_wave;
+            __syncthreads();
+            uint32_t pos = found;
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                const uint32_t c = wave_n[round & 1u][w];
+                pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
+                found += c;
+            }
+            if (in_wave != 0) {
+#pragma unroll
+                for (int u = 0; u < VT; u++) {
+                    asm volatile("" : "+v"(s[u].x), "+v"(s[u].y), "+v"(s[u].z), "+v"(s[u].w));  // (masks again, not kept: see below)
+                    const bool here = reach > u * (kWave * 4);
+                    const float v[4] = {s[u].x, s[u].y, s[u].z, s[u].w};
+                    uint64_t mask[4];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) mask[c] = __ballot(here && v[c] > score_threshold);
+                    if ((mask[0] | mask[1] | mask[2] | mask[3]) != 0) {
+                        asm volatile("; four tiles with candidates");  // (a real branch)
+                        uint32_t at = pos + lanes_below(mask[0]) + lanes_below(mask[1]) + lanes_below(mask[2]) + lanes_below(mask[3]);
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            if ((mask[c] >> lane) & 1ull) {
+                                if (at < static_cast<uint32_t>(kNmsMaxCandidates))
+                                    comp[at] = composite(order_key(v[c]), wave_first + static_cast<uint32_t>(u) * (kWave * 4) + lane * 4 + static_cast<uint32_t>(c));
+                                at++;
+                            }
+                            pos += static_cast<uint32_t>(__popcll(mask[c]));
+                        }
+                    }
+                }
+            }
+        }
+    } else
     for (uint32_t base = 0; base < N; base += NT * TILES, round++) {  // (to the end: the count tells whether boxes were left out)
         const uint32_t tiles = min(static_cast<uint32_t>(TILES), (N - base + NT - 1) / NT);  // per wave, this round
         const uint32_t wave_first = base + wave * tiles * kWave;
@@ -151,8 +216,14 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nm
 #pragma unroll 16
             for (uint32_t q = 0; q < K; q++) {
                 const uint64_t other = comp[q];
+                rank[0] += other > c[0] ? 1u : 0u;
+            }
 #pragma unroll
-                for (int e = 0; e < SMALL; e++) rank[e] += other > c[e] ? 1u : 0u;
+            for (int e = 1; e < SMALL; e++) {
+                if (K > static_cast<uint32_t>(e) * NT) {  // (the same for the whole workgroup)
+#pragma unroll 16
+                    for (uint32_t q = 0; q < K; q++) rank[e] += comp[q] > c[e] ? 1u : 0u;
+                }
             }
         }
         __syncthreads();
@@ -200,6 +271,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nm
 #pragma unroll
         for (int r = 0; r < JP; r++) {
             const uint32_t j = wave * JP + static_cast<uint32_t>(r);
+            if (j >= K - base) break;  // (past the block's candidates; the same for the whole wave)
             if (lane > j && nms_iou(bi, box[j]) > iou_threshold) bits |= 1u << r;
         }
         if (bits != 0) atomicOr(&block_cols[lane], static_cast<unsigned long long>(bits) << (wave * JP));

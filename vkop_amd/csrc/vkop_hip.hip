@@ -613,14 +613,17 @@ int nms_impl(const T *boxes, const T *scores, int32_t *out, int out_capacity, in
     const uint32_t per = max_per_class > 0 ? static_cast<uint32_t>(max_per_class) : 0u;
     const int knob = g_nms_threads;  // 0: by the number of pairs
     const bool narrow = knob > 0 ? knob == vkop::kNmsThreadsNarrow : pairs >= static_cast<uint32_t>(vkop::kNmsNarrowMinPairs);
-    if (narrow)
-        vkop::nms_kernel<T, vkop::kNmsThreadsNarrow><<<pairs, vkop::kNmsThreadsNarrow, 0, st>>>(
-            boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C), static_cast<uint32_t>(N), center_point_box, per,
-            iou_threshold, score_threshold, max_sel);
-    else
-        vkop::nms_kernel<T, vkop::kNmsThreadsWide><<<pairs, vkop::kNmsThreadsWide, 0, st>>>(
-            boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C), static_cast<uint32_t>(N), center_point_box, per,
-            iou_threshold, score_threshold, max_sel);
+    // rows that start on 16-byte boundaries and hold a multiple of four scores are read four scores per load
+    const bool vec = N % 4 == 0 && N >= 4 && (reinterpret_cast<uintptr_t>(scores) & 15u) == 0;
+#define VKOP_NMS_LAUNCH(NT, VEC)                                                                                          \
+    vkop::nms_kernel<T, NT, VEC><<<pairs, NT, 0, st>>>(boxes, scores, selected, counts, pairs, static_cast<uint32_t>(C),  \
+                                                       static_cast<uint32_t>(N), center_point_box, per, iou_threshold,   \
+                                                       score_threshold, max_sel)
+    if (narrow && vec) VKOP_NMS_LAUNCH(vkop::kNmsThreadsNarrow, true);
+    else if (narrow) VKOP_NMS_LAUNCH(vkop::kNmsThreadsNarrow, false);
+    else if (vec) VKOP_NMS_LAUNCH(vkop::kNmsThreadsWide, true);
+    else VKOP_NMS_LAUNCH(vkop::kNmsThreadsWide, false);
+#undef VKOP_NMS_LAUNCH
     if (int rc = launched("nms_kernel")) return rc;
     vkop::nms_pack_kernel<<<pairs, 256, 0, st>>>(selected, counts, out, out_count, pairs, static_cast<uint32_t>(C), max_sel,
                                                  static_cast<uint32_t>(out_capacity));
