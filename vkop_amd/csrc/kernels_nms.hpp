@@ -67,7 +67,7 @@ __device__ __forceinline__ float nms_iou(const float4 &a, const float4 &b) {
 // another's sort and walk.  Each thread keeps the boxes of its own kNmsMaxCandidates / NT
 // sorted candidates in registers; LDS holds the composites and two blocks of 64 boxes.
 template <typename T, int NT, bool VEC>
-__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(8))) void nms_kernel(
+__global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT >= 1024 ? 8 : 6))) void nms_kernel(
     const T *__restrict__ boxes, const T *__restrict__ scores, int32_t *__restrict__ selected, uint32_t *__restrict__ counts,
     uint32_t pairs, uint32_t C, uint32_t N, int center_point_box, uint32_t max_out, float iou_threshold, float score_threshold,
     uint32_t max_sel) {
