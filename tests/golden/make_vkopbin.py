@@ -10,6 +10,9 @@
                             Attributes of all five tagged kinds appear (a string and two lists ride
                             along, unused by the operator).
 
+  detection_chain.vkopbin   class scores [2,80,840] -> Softmax(axis 1) -> Reduce(max, axes [1], keepdims 0) ->
+                            TopK(K 30): the detection-style post-processing (example/yolo/main.cpp:60-127).
+
 add_conv_model.vkopbin is not written here: it is the reference's own model file
 (model/add_conv_model.vkopbin, made by its converter), kept as a reading fixture.
 """
@@ -54,6 +57,16 @@ def main():
                          "anchors": [1.5, 2.25]},
           "inputs": [shape("boxes", (2, 300, 4)), shape("scores", (2, 3, 300))], "outputs": [shape("selected", (1800, 3))]}])
     open(os.path.join(HERE, "detection_tail.vkopbin"), "wb").write(tail)
+
+    chain = vkopbin.write_model(
+        [shape("scores", (2, 80, 840))], [shape("values", (2, 30)), shape("anchors", (2, 30))],
+        [{"op_type": "Softmax", "name": "node_softmax", "attributes": {"axis": 1},
+          "inputs": [shape("scores", (2, 80, 840))], "outputs": [shape("probs", (2, 80, 840))]},
+         {"op_type": "Reduce", "name": "node_max", "attributes": {"reduce_op": "max", "axes": [1], "keepdims": 0},
+          "inputs": [shape("probs", (2, 80, 840))], "outputs": [shape("best", (2, 840))]},
+         {"op_type": "TopK", "name": "node_topk", "attributes": {"K": 30, "axis": -1},
+          "inputs": [shape("best", (2, 840))], "outputs": [shape("values", (2, 30)), shape("anchors", (2, 30))]}])
+    open(os.path.join(HERE, "detection_chain.vkopbin"), "wb").write(chain)
 
 
 if __name__ == "__main__":

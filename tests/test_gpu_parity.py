@@ -809,6 +809,15 @@ def test_model_files_drive_the_operators(ops, dtype):
     assert host(out["values"]).shape == (4, 7)
     ev7, ei7 = oracle.topk(host(out["probs"]), 7, -1)
     assert np.array_equal(host(out["indices"]), ei7) and np.array_equal(host(out["values"]).view(bits), ev7.view(bits))
+    # detection chain: softmax over classes, class maximum (one operator when fused), top anchors
+    chain = vkopbin.read_model(os.path.join(GOLDEN_DIR, "detection_chain.vkopbin"))
+    sc = np.ascontiguousarray(synth.detection_scores(2, 80, 840, 5).astype(dtype))
+    probs = oracle.softmax(sc, 1)
+    best = oracle.reduce_max(probs, 1) if dtype == np.float32 else probs.max(axis=1)   # (a maximum has no rounding)
+    bv, bi = oracle.topk(best, 30, -1)
+    for fuse in (True, False):
+        out = runtime.run_model(chain, {"scores": dev(sc)}, fuse=fuse)
+        assert np.array_equal(host(out["anchors"]), bi) and np.array_equal(host(out["values"]).view(bits), bv.view(bits)), fuse
     # detection tail
     tail = vkopbin.read_model(os.path.join(GOLDEN_DIR, "detection_tail.vkopbin"))
     rng = np.random.default_rng(9)

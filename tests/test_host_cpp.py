@@ -42,5 +42,7 @@ def test_reference_case_lists_through_operator_interface():
                    "(not fusable): ok", "Nms fp32 boxes [1,50,4] classes 7: ok", "Nms fp16 boxes [2,300,4] classes 3: ok",
                    "Model classifier_head.vkopbin fp32 [8,1000] k 5, 1 operator(s) (node_topk): ok",
                    "Model classifier_head_k_input.vkopbin fp16 [4,1000] k 7, 2 operator(s) (node_topk): ok",
-                   "Model detection_tail.vkopbin: ok"):
+                   "Model detection_tail.vkopbin: ok", "Reduce max fp32 shape [16,80,8400] axis 1 keepdims 0: ok",
+                   "Reduce max fp16 shape [4,80,1000] axis -2 keepdims 0: ok", "Model detection_chain.vkopbin, 2 operator(s): ok",
+                   "Model detection_chain.vkopbin, 3 operator(s): ok"):
         assert needle in r.stdout

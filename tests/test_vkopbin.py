@@ -61,7 +61,7 @@ def test_damaged_files_are_refused():
 
 
 def test_fixture_generator_reproduces_the_committed_files(tmp_path):
-    names = ["classifier_head.vkopbin", "classifier_head_k_input.vkopbin", "detection_tail.vkopbin"]
+    names = ["classifier_head.vkopbin", "classifier_head_k_input.vkopbin", "detection_tail.vkopbin", "detection_chain.vkopbin"]
     before = {n: open(os.path.join(GOLDEN, n), "rb").read() for n in names}
     src = open(os.path.join(GOLDEN, "make_vkopbin.py")).read().replace("HERE = os.path.dirname(os.path.abspath(__file__))",
                                                                       f"HERE = {str(tmp_path)!r}")
@@ -86,3 +86,23 @@ def test_plan_fuses_only_a_private_softmax_along_the_same_axis():
          {"op_type": "TopK", "name": "t", "attributes": {"K": 2, "axis": 1}, "inputs": [{"name": "p", "shape": [4, 8]}],
           "outputs": [{"name": "v", "shape": [4, 2]}, {"name": "i", "shape": [4, 2]}]}]))
     assert [k for k, _, _ in runtime.plan(other_axis)] == ["softmax", "topk"]
+
+
+def test_plan_fuses_the_class_maximum_with_its_softmax():
+    chain = vkopbin.read_model(os.path.join(GOLDEN, "detection_chain.vkopbin"))
+    assert [(k, n["name"]) for k, n, _ in runtime.plan(chain)] == [("softmax_reduce_max", "node_max"), ("topk", "node_topk")]
+    assert [k for k, _, _ in runtime.plan(chain, fuse=False)] == ["softmax", "reduce_max", "topk"]
+    for attrs in ({"reduce_op": "sum", "axes": [1]}, {"reduce_op": "max", "axes": [0, 1]}):
+        bad = vkopbin.read_model(vkopbin.write_model(
+            [{"name": "x", "shape": [4, 8]}], [{"name": "y", "shape": [4]}],
+            [{"op_type": "Reduce", "name": "r", "attributes": attrs, "inputs": [{"name": "x", "shape": [4, 8]}],
+              "outputs": [{"name": "y", "shape": [4]}]}]))
+        with pytest.raises(NotImplementedError, match="Reduce"):
+            runtime.plan(bad)
+    other_axis = vkopbin.read_model(vkopbin.write_model(
+        [{"name": "x", "shape": [4, 8]}], [{"name": "y", "shape": [4]}],
+        [{"op_type": "Softmax", "name": "s", "attributes": {"axis": 0}, "inputs": [{"name": "x", "shape": [4, 8]}],
+          "outputs": [{"name": "p", "shape": [4, 8]}]},
+         {"op_type": "Reduce", "name": "r", "attributes": {"reduce_op": "max", "axes": [1], "keepdims": 0},
+          "inputs": [{"name": "p", "shape": [4, 8]}], "outputs": [{"name": "y", "shape": [4]}]}]))
+    assert [k for k, _, _ in runtime.plan(other_axis)] == ["softmax", "reduce_max"]

@@ -19,7 +19,8 @@
 // each depending on the level before it, exactly as the reference does.
 //
 // One addition in both paths: a TopK that alone reads the output of a Softmax
-// along the same axis replaces the pair by one fused operator.  For registered
+// along the same axis replaces the pair by one fused operator (in a model also a
+// Reduce "max" over that one axis: the class maximum of class probabilities).  For registered
 // post-processing that is legal because every registration clears the set of
 // tensors read back (core/runtime.cpp:515-519), so after the TOPK registration
 // the softmax tensor is neither read back nor an input of anything else; for a
@@ -127,6 +128,23 @@ class Runtime {
                 fused_softmax_of[n.name] = &sm;
             }
         }
+        // the same for a Reduce "max" over the one axis the Softmax in front of it runs along
+        if (fuse_) {
+            for (const auto &n : model.nodes) {
+                if (ops::convert_opstring_to_enum(n.op_type) != ops::OpType::REDUCE || n.inputs.empty()) continue;
+                auto p = producer.find(n.inputs[0].name);
+                if (p == producer.end() || ops::convert_opstring_to_enum(p->second->op_type) != ops::OpType::SOFTMAX) continue;
+                const auto &sm = *p->second;
+                if (sm.outputs.size() != 1 || sm.inputs.size() != 1 || consumers[sm.outputs[0].name] != 1 || outputs_.count(sm.outputs[0].name)) continue;
+                ops::Reduce probe;
+                probe.setAttribute(n.attributes);
+                const int rank = static_cast<int>(sm.outputs[0].dims.size());
+                if (probe.reduce_op() != static_cast<int>(ops::reduce::ReduceType::MAX) || probe.axes().size() != 1) continue;
+                std::unordered_map<std::string, std::string> as_axis = {{"axis", std::to_string(probe.axes()[0])}};
+                if (rank < 2 || !same_axis(sm.attributes, as_axis, rank)) continue;
+                fused_softmax_of[n.name] = &sm;
+            }
+        }
         std::unordered_set<std::string> left_out;
         for (const auto &f : fused_softmax_of) left_out.insert(f.second->name);
         std::unordered_map<std::string, size_t> index_of_node;
@@ -172,7 +190,8 @@ class Runtime {
                 }
                 if (type == ops::OpType::TOPK && node_inputs.size() > 1) node_inputs.resize(1);  // K is an attribute by now
                 std::unique_ptr<ops::Operator> op;
-                if (fused != fused_softmax_of.end()) op = std::make_unique<ops::SoftmaxTopk>(precision_);
+                if (fused != fused_softmax_of.end() && type == ops::OpType::REDUCE) op = std::make_unique<ops::SoftmaxReduceMax>();
+                else if (fused != fused_softmax_of.end()) op = std::make_unique<ops::SoftmaxTopk>(precision_);
                 else op = ops::create_from_type(type, node_outputs[0]->num_dims() <= 2, precision_, dev->is_support_nv_tensor_core());
                 op->set_name(n.name);
                 op->set_runtime_device(dev, m_cmdpool_);

@@ -8,6 +8,7 @@
 
 #include "ops/Operator.hpp"
 #include "ops/Nms.hpp"
+#include "ops/Reduce.hpp"
 #include "ops/Softmax.hpp"
 #include "ops/Topk.hpp"
 
@@ -24,6 +25,8 @@ static inline std::unique_ptr<Operator> create_from_type(OpType type, bool use_s
         return std::make_unique<Softmax>(use_ssbo);
     case OpType::NMS:
         return std::make_unique<Nms>();
+    case OpType::REDUCE:
+        return std::make_unique<Reduce>();
     default:
         return nullptr;
     }

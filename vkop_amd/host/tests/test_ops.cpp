@@ -359,6 +359,26 @@ static void host_logic_tests() {
         EXPECT(tk && tk->get_type() == ops::OpType::TOPK && dynamic_cast<ops::Topk *>(tk.get()));
         EXPECT(ops::create_from_type(ops::OpType::CONV2D) == nullptr);
         {
+            using ops::Reduce;
+            EXPECT((Reduce::calculateOutputShape({16, 80, 8400}, {1}, false) == std::vector<int>{16, 8400}));
+            EXPECT((Reduce::calculateOutputShape({16, 80, 8400}, {-2}, true) == std::vector<int>{16, 1, 8400}));
+            EXPECT((Reduce::calculateOutputShape({2, 3, 4, 5}, {0, -1, 9}, false) == std::vector<int>{3, 4}));
+            EXPECT((Reduce::calculateOutputShape({7}, {0}, false).empty()));
+            auto rd = ops::create_from_type(ops::OpType::REDUCE);
+            auto *r = dynamic_cast<Reduce *>(rd.get());
+            EXPECT(r != nullptr && r->get_type() == ops::OpType::REDUCE);
+            if (r) {
+                EXPECT(r->reduce_op() == 0 && r->keepdims() == 1 && r->axes().empty());  // ops/Reduce.hpp:150-152
+                r->setAttribute({{"reduce_op", "max"}, {"axes", "[1, -1]"}, {"keepdims", "0"}});
+                EXPECT(r->reduce_op() == static_cast<int>(ops::reduce::ReduceType::MAX) && r->keepdims() == 0);
+                EXPECT((r->axes() == std::vector<int>{1, -1}));
+                r->setAttribute({{"reduce_op", "sum_square"}});
+                EXPECT(r->reduce_op() == 9 && r->keepdims() == 0);
+                r->setAttribute({{"reduce_op", "no such"}});
+                EXPECT(r->reduce_op() == 9);  // unknown names leave it as it is (ops/Reduce.hpp:42-64)
+            }
+        }
+        {
             auto nm = ops::create_from_type(ops::OpType::NMS);
             EXPECT(nm && nm->get_type() == ops::OpType::NMS && dynamic_cast<ops::Nms *>(nm.get()));
         }
@@ -656,6 +676,62 @@ template <typename T> static void model_head_case(const std::string &file, int r
     EXPECT(ok);
 }
 
+// Reduce "max" along one axis against torch::amax (exact: a maximum has no rounding), and the errors for what is not built.
+template <typename T> static void reduce_case(const std::vector<int> &shape, int axis, int keepdims) {
+    TestCase<T> tc("Reduce");
+    torch::manual_seed(17);
+    std::vector<int64_t> dims(shape.begin(), shape.end());
+    auto x = torch::randn(dims, tc.conf());
+    auto want = torch::amax(x, {axis}, keepdims == 1).contiguous();
+    auto in = std::make_shared<Tensor<T>>(shape);
+    fill_from_torch(in, x);
+    std::vector<int> out_shape(want.sizes().begin(), want.sizes().end());
+    auto expect = std::make_shared<Tensor<T>>(out_shape);
+    fill_from_torch(expect, want);
+    const std::unordered_map<std::string, std::string> attrs = {
+        {"reduce_op", "max"}, {"axes", "[" + std::to_string(axis) + "]"}, {"keepdims", std::to_string(keepdims)}};
+    const bool ok = tc.run_test({in}, {expect}, [&](std::unique_ptr<ops::Operator> &op) { op->setAttribute(attrs); });
+    std::printf("Reduce max %s shape [", std::is_same_v<T, float> ? "fp32" : "fp16");
+    for (size_t i = 0; i < shape.size(); i++) std::printf("%s%d", i ? "," : "", shape[i]);
+    std::printf("] axis %d keepdims %d: %s\n", axis, keepdims, ok ? "ok" : "FAILED");
+    EXPECT(ok);
+}
+
+// The detection-style chain from its model file: Softmax over classes, class maximum, top anchors.
+static void model_chain_case(bool fuse, size_t want_nodes) {
+    auto pool = TestEnv::pool;
+    vkop::core::Runtime rt(pool, g_golden + "/detection_chain.vkopbin", 0);
+    rt.set_postprocess_fusion(fuse);
+    rt.LoadModel();
+    EXPECT(rt.num_nodes() == want_nodes);
+    torch::manual_seed(23);
+    auto x = torch::randn({2, 80, 840}) * 2;
+    auto in = vkop::core::as_tensor<float>(rt.GetInput());
+    fill_from_torch(in, x);
+    in->copyToGPU(pool);
+    rt.Run();
+    rt.ReadResult();
+    auto best = torch::amax(torch::softmax(x.to(torch::kFloat64), 1).to(torch::kFloat32), {1});
+    auto sorted = torch::sort(best, /*stable=*/true, -1, /*descending=*/true);
+    auto ev = std::get<0>(sorted).slice(-1, 0, 30).contiguous();
+    auto ei = std::get<1>(sorted).slice(-1, 0, 30).to(torch::kInt).contiguous();
+    auto values = vkop::core::as_tensor<float>(rt.GetOutput("values"));
+    auto anchors = vkop::core::as_tensor<int>(rt.GetOutput("anchors"));
+    bool ok = values && anchors;
+    int64_t worst = 0;
+    for (int i = 0; ok && i < 60; i++) {
+        const float want = ev.data_ptr<float>()[i];
+        worst = std::max(worst, ulp_distance((*values)[static_cast<size_t>(i)], want));
+        const int j = i % 30;
+        const bool tied = (j > 0 && ev.data_ptr<float>()[i - 1] == want) || (j + 1 < 30 && ev.data_ptr<float>()[i + 1] == want);
+        if (!tied) ok = (*anchors)[static_cast<size_t>(i)] == ei.data_ptr<int>()[i];
+    }
+    ok = ok && worst <= 2;
+    std::printf("Model detection_chain.vkopbin, %zu operator(s): %s, worst distance %lld ulp\n", rt.num_nodes(), ok ? "ok" : "FAILED",
+                static_cast<long long>(worst));
+    EXPECT(ok);
+}
+
 static void model_run_tests() {
     TestEnv::initialize();
     auto pool = TestEnv::pool;
@@ -664,6 +740,8 @@ static void model_run_tests() {
     model_head_case<uint16_t>("classifier_head.vkopbin", 8, 5, true, 1);
     model_head_case<float>("classifier_head_k_input.vkopbin", 4, 7, true, 2);  // probabilities are an output: two operators
     model_head_case<uint16_t>("classifier_head_k_input.vkopbin", 4, 7, true, 2);
+    model_chain_case(true, 2);   // Softmax + Reduce as one operator, then TopK
+    model_chain_case(false, 3);
     {
         vkop::core::Runtime rt(pool, g_golden + "/detection_tail.vkopbin", 0);
         rt.LoadModel();
@@ -728,6 +806,11 @@ int main(int argc, char **argv) {
         nms_case<float>({1, 200, 4}, {1, 1, 200}, 0, 0.7F, 0.4F);
         nms_case<float>({1, 50, 4}, {1, 7, 50}, 0, 0.3F, 0.2F);
         nms_case<uint16_t>({2, 300, 4}, {2, 3, 300}, 0, 0.5F, 0.3F);
+        reduce_case<float>({16, 80, 8400}, 1, 0);
+        reduce_case<float>({16, 80, 8400}, 1, 1);
+        reduce_case<uint16_t>({4, 80, 1000}, -2, 0);
+        reduce_case<float>({4, 1000}, -1, 0);
+        reduce_case<float>({3, 5, 7, 9}, 0, 1);
         model_run_tests();
         // the benchmark's arrangement: full-size outputs, the first k read back
         {
