@@ -141,6 +141,17 @@ size_t vkop_hip_softmax_reduce_max_workspace_bytes(int dtype, const int *shape, 
 int vkop_hip_softmax_reduce_max(const void *in, void *out, int dtype, const int *shape,
                                 int ndim, int axis, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- Nucleus (top-p) cut on the output of a sorted top-k: counts[row] = the
+ * smallest m >= 1 such that values[row][0..m) sum to at least p, or k when they
+ * never do (also when a NaN enters the sum).  The sum is taken in float, front
+ * to back, so the count is reproducible bit for bit.  values: rows x k
+ * probabilities in descending order, rows row_stride elements apart (the
+ * benchmark's arrangement writes top-k into full-width rows,
+ * benchmark/main.cpp:92-94).  No counterpart in the reference: a sampling-style
+ * extension on the softmax -> top-k path. */
+int vkop_hip_topp_count(const void *values, int32_t *counts, int dtype, int rows,
+                        int k, int row_stride, float p, void *stream);
+
 /* ---- Non-maximum suppression: replaces Nms::execute (ops/Nms.hpp:73-118) and
  * shaders/nms.comp, the operator that follows the top-k in the detection-style
  * post-processing.  boxes [B][N][4] and scores [B][C][N] of `dtype`; per (batch,

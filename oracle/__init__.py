@@ -49,6 +49,8 @@ def lib():
         L.vkop_oracle_get_top_k_predictions.restype = c_int
         L.vkop_oracle_get_top_k_predictions.argtypes = [vp, c_int, c_int, vp, vp]
         L.vkop_oracle_nms_f32.restype = c_int
+        L.vkop_oracle_topp_count_f32.argtypes = [vp, c_int, c_int, c_int, c_float, vp]
+        L.vkop_oracle_topp_count_f32.restype = None
         L.vkop_oracle_nms_f32.argtypes = [vp, vp, vp, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int]
         _lib = L
     return _lib
@@ -192,3 +194,14 @@ def nms(boxes, scores, iou_threshold, score_threshold, max_output_boxes_per_clas
                                   int(max_output_boxes_per_class), float(iou_threshold), float(score_threshold),
                                   int(N if max_candidates is None else max_candidates))
     return out[:m].copy()
+
+
+def topp_count(values, p):
+    """Nucleus cut on sorted top-k probabilities [.., k] (float32, or float16 widened): per row the smallest
+    count of leading values whose float sum, front to back, reaches p; k when it never does."""
+    v = np.ascontiguousarray(np.asarray(values).astype(np.float32))
+    k = v.shape[-1]
+    rows = v.size // k if k else 0
+    out = np.empty(v.shape[:-1], dtype=np.int32)
+    lib().vkop_oracle_topp_count_f32(_ptr(v), rows, k, k, float(p), _ptr(out))
+    return out

@@ -527,3 +527,27 @@ int vkop_oracle_nms_f32(const float *boxes, const float *scores, int32_t *out,
     free(active);
     return total;
 }
+
+/* ------------------------------------------------------------------ */
+/* nucleus (top-p) cut on sorted top-k probabilities                   */
+/* ------------------------------------------------------------------ */
+
+/* No counterpart in the reference (a sampling-style extension on its softmax ->
+ * top-k path, benchmark/main.cpp:85-101): the usual sampler rule, keep leading
+ * values until their running float sum reaches p, the one that crosses included. */
+void vkop_oracle_topp_count_f32(const float *values, int rows, int k,
+                                int row_stride, float p, int32_t *counts) {
+    for (int r = 0; r < rows; r++) {
+        const float *v = values + (size_t)r * row_stride;
+        volatile float sum = 0.0f; /* (volatile: every partial sum rounded to float) */
+        int count = k;
+        for (int j = 0; j < k; j++) {
+            sum = sum + v[j];
+            if (sum >= p) {
+                count = j + 1;
+                break;
+            }
+        }
+        counts[r] = count;
+    }
+}

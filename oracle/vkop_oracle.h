@@ -113,6 +113,12 @@ int vkop_oracle_nms_f32(const float *boxes, const float *scores, int32_t *out,
                         float iou_threshold, float score_threshold,
                         int max_candidates);
 
+/* Nucleus (top-p) cut: counts[r] = smallest m >= 1 with values[r][0..m) summing
+ * (float, front to back) to at least p; k when they never do.  Not in the
+ * reference: a sampling-style extension on its softmax -> top-k path. */
+void vkop_oracle_topp_count_f32(const float *values, int rows, int k,
+                                int row_stride, float p, int32_t *counts);
+
 #ifdef __cplusplus
 }
 #endif

@@ -781,6 +781,18 @@ def test_nms_detection_workload_full_size(ops):
     assert not over and np.array_equal(host(got), want) and len(want) == 4 * 20 * 200
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_topp_count_on_fused_output(ops, dtype):
+    x = np.ascontiguousarray(synth.llm_logits(64, 128256, synth.SEEDS["C3"])[:, :32000].astype(dtype))
+    for k in (1, 50, 200, 255):
+        v, _ = ops.softmax_topk(dev(x), k)
+        for p in (0.0, 0.3, 0.9, 0.999, 2.0):
+            assert np.array_equal(host(ops.topp_count(v, p)), oracle.topp_count(host(v), p)), (k, p)
+    wide = np.sort(np.random.default_rng(1).random((3, 5, 2048)).astype(dtype) / 1024, axis=-1)[..., ::-1].copy()
+    got = host(ops.topp_count(dev(wide), 0.75))
+    assert got.shape == (3, 5) and np.array_equal(got, oracle.topp_count(wide, 0.75))
+
+
 # ---- models from .vkopbin files ---------------------------------------------------------------------
 
 GOLDEN_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")

@@ -375,3 +375,29 @@ def test_nms_invariants_and_closed_forms():
                        apart[..., 2] - apart[..., 0], apart[..., 3] - apart[..., 1]], -1).astype(np.float32)
     assert np.array_equal(oracle.nms(centre, sc, 0.5, 0.0, center_point_box=1), oracle.nms(apart, sc, 0.5, 0.0))
     assert oracle.nms(apart, sc, 0.5, 0.0, max_candidates=4)[:, 2].tolist() == [1, 3, 2, 0]
+
+
+# ---- nucleus (top-p) cut: not in the reference, pinned on closed forms and numpy's sequential cumsum --------------
+
+def test_topp_count_closed_forms_and_cumsum():
+    eighths = np.full((1, 8), 0.125, dtype=np.float32)              # every partial sum exact
+    for p, want in [(0.0, 1), (0.125, 1), (0.126, 2), (0.5, 4), (0.51, 5), (1.0, 8), (1.5, 8), (-1.0, 1)]:
+        assert oracle.topp_count(eighths, p).tolist() == [want], p
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((64, 4000)).astype(np.float32) * 3
+    probs = oracle.softmax(x, -1)
+    v, _ = oracle.topk(probs, 50, -1)
+    running = np.cumsum(v, axis=-1, dtype=np.float32)               # numpy accumulates front to back in float32
+    last = 0
+    for p in (0.05, 0.3, 0.5, 0.8, 0.9, 0.99, 1.0):
+        got = oracle.topp_count(v, p)
+        reached = running >= np.float32(p)
+        want = np.where(reached.any(axis=-1), reached.argmax(axis=-1) + 1, 50)
+        assert np.array_equal(got, want), p
+        assert (got >= last).all()                                  # a larger p never needs fewer values
+        last = got
+    bad = v.copy()
+    bad[3, 2] = np.nan                                              # a NaN in the sum: nothing is ever reached after it
+    assert oracle.topp_count(bad, 0.9999)[3] == 50
+    half = v.astype(np.float16)
+    assert np.array_equal(oracle.topp_count(half, 0.7), oracle.topp_count(half.astype(np.float32), 0.7))

@@ -56,6 +56,7 @@ def lib():
     sig = {
         "vkop_hip_nms_workspace_bytes": (sz, [i, i, i, i]),
         "vkop_hip_nms": (i, [vp, vp, vp, i, vp, i, i, i, i, i, i, f, f, vp, sz, vp]),
+        "vkop_hip_topp_count": (i, [vp, vp, i, i, i, i, f, vp]),
         "vkop_hip_init": (i, [i]),
         "vkop_hip_shutdown": (i, []),
         "vkop_hip_last_error": (ctypes.c_char_p, []),
@@ -233,6 +234,10 @@ def softmax_topk(inp, probs, values, indices, dtype, shape, axis, k, largest=1, 
 def reduce_max(inp, out, dtype, shape, axis, stream=0):
     arr, nd = _shape(shape)
     check(lib().vkop_hip_reduce_max(inp, out, dtype, arr, nd, axis, stream))
+
+
+def topp_count(values, counts, dtype, rows, k, row_stride, p, stream=0):
+    check(lib().vkop_hip_topp_count(values, counts, int(dtype), int(rows), int(k), int(row_stride), float(p), stream))
 
 
 def tune(name, value):

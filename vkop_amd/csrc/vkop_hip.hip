@@ -890,6 +890,20 @@ int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape, 
     return reduce_max_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), v, as_stream(stream));
 }
 
+int vkop_hip_topp_count(const void *values, int32_t *counts, int dtype, int rows, int k, int row_stride, float p, void *stream) {
+    if (int rc = check_dtype(dtype)) return rc;
+    if (rows < 0 || k < 1 || row_stride < k) return fail(VKOP_HIP_ERR_INVALID, "rows %d, k %d, row stride %d", rows, k, row_stride);
+    if (rows == 0) return VKOP_HIP_OK;
+    if (values == nullptr || counts == nullptr) return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    if (dtype == VKOP_HIP_F32)
+        vkop::topp_count_kernel<float><<<rows, vkop::kWave, 0, as_stream(stream)>>>(static_cast<const float *>(values), counts,
+                                                                                static_cast<uint32_t>(k), static_cast<size_t>(row_stride), p);
+    else
+        vkop::topp_count_kernel<uint16_t><<<rows, vkop::kWave, 0, as_stream(stream)>>>(static_cast<const uint16_t *>(values), counts,
+                                                                                   static_cast<uint32_t>(k), static_cast<size_t>(row_stride), p);
+    return launched("topp_count_kernel");
+}
+
 int vkop_hip_tune(const char *name, int value) {
     if (name == nullptr) return fail(VKOP_HIP_ERR_INVALID, "name is null");
     if (std::strcmp(name, "rows.threads") == 0) g_rows_threads = value;

@@ -117,6 +117,17 @@ def reduce_max(x, axis):
     return out
 
 
+def topp_count(values, p):
+    """Nucleus cut on sorted top-k probabilities [.., k]: per row the smallest count of leading values whose float
+    sum, taken front to back, reaches p (k when it never does).  -> int32 tensor of the leading shape."""
+    values, dt = _prep(values)
+    k = values.shape[-1]
+    rows = values.numel() // k if k else 0
+    counts = torch.empty(values.shape[:-1], dtype=torch.int32, device=values.device)
+    capi.topp_count(values.data_ptr(), counts.data_ptr(), dt, rows, k, k, p, _stream())
+    return counts
+
+
 def nms(boxes, scores, iou_threshold, score_threshold, max_output_boxes_per_class=0, center_point_box=0,
         out_capacity=None, workspace=None):
     """Non-maximum suppression per (batch, class): boxes [B,N,4], scores [B,C,N] (both float32 or both float16).
