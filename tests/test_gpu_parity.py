@@ -761,6 +761,24 @@ def test_nms_either_workgroup_size(ops, threads):
         capi.tune("nms.threads", 0)
 
 
+def test_nms_pairs_without_candidates_and_tiny_rows(ops):
+    rng = np.random.default_rng(4)
+    for B, C, N in [(2, 3, 4), (1, 5, 3), (2, 2, 64), (1, 1, 2), (3, 1, 8)]:
+        boxes = _nms_boxes(rng, B, N)
+        scores = rng.random((B, C, N)).astype(np.float32)
+        got, over = ops.nms(dev(boxes), dev(scores), 0.5, 2.0)                  # nothing passes the score threshold
+        assert host(got).shape == (0, 3) and not over
+        scores[:, 0] = -1.0                                                     # class 0 has no candidate, the others do
+        got, _ = ops.nms(dev(boxes), dev(scores), 0.5, 0.0)
+        want = oracle.nms(boxes, scores, 0.5, 0.0, 0, max_candidates=2048)
+        assert np.array_equal(host(got), want) and not (want[:, 1] == 0).any()
+        for dt in (np.float16,):
+            got16, _ = ops.nms(dev(boxes.astype(dt)), dev(scores.astype(dt)), 0.5, 0.0)
+            want16 = oracle.nms(boxes.astype(dt).astype(np.float32), scores.astype(dt).astype(np.float32), 0.5, 0.0, 0,
+                                max_candidates=2048)
+            assert np.array_equal(host(got16), want16)
+
+
 def test_nms_detection_workload_full_size(ops):
     """The detection-shaped case of the operator benchmark, and a dense one with a per-class limit, against the oracle."""
     c5 = synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"])
