@@ -779,6 +779,43 @@ def test_nms_pairs_without_candidates_and_tiny_rows(ops):
             assert np.array_equal(host(got16), want16)
 
 
+def test_nms_random_configurations(ops):
+    """Seeded sweep over sizes around the kernel's tile, block and capacity boundaries, quantised scores and boxes
+    (ties, identical and empty boxes), thresholds including negative ones, limits, both box formats and types."""
+    from vkop_amd import capi
+    rng = np.random.default_rng(2026)
+    try:
+        for it in range(80):
+            B, C = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+            N = int(rng.choice([1, 3, 4, 63, 64, 65, 255, 256, 257, 512, 513, 1000, 2047, 2048, 2049, 4096, 9216, 9217, 12289]))
+            ctr = rng.random((B, N, 2)).astype(np.float32)
+            size = (rng.random((B, N, 2)) * float(rng.choice([0.05, 0.2, 0.6, 1.3]))).astype(np.float32)
+            boxes = np.concatenate([ctr - size / 2, ctr + size / 2], -1).astype(np.float32)
+            scores = rng.random((B, C, N)).astype(np.float32)
+            mode = int(rng.integers(0, 4))
+            if mode == 1:
+                scores = np.round(scores * 8) / 8
+            elif mode == 2:
+                boxes = np.round(boxes * 4) / 4
+            elif mode == 3:
+                scores[..., ::3] = scores[..., :1]
+            thr, iou = float(rng.choice([-1.0, 0.0, 0.1, 0.5, 0.9, 0.99])), float(rng.choice([-0.5, 0.0, 0.1, 0.45, 0.7, 1.0]))
+            per, centre = int(rng.choice([0, 0, 1, 7, 100, 3000])), int(rng.integers(0, 2))
+            capi.tune("nms.threads", int(rng.choice([0, 256, 1024])))
+            if centre:
+                boxes = np.stack([(boxes[..., 0] + boxes[..., 2]) / 2, (boxes[..., 1] + boxes[..., 3]) / 2,
+                                  boxes[..., 2] - boxes[..., 0], boxes[..., 3] - boxes[..., 1]], -1).astype(np.float32)
+            if rng.integers(0, 2):
+                boxes, scores = boxes.astype(np.float16), scores.astype(np.float16)
+            got, over = ops.nms(dev(boxes), dev(scores), iou, thr, per, centre)
+            b32, s32 = boxes.astype(np.float32), scores.astype(np.float32)
+            want = oracle.nms(b32, s32, iou, thr, per, centre, max_candidates=2048)
+            assert np.array_equal(host(got), want), (it, B, C, N, mode, thr, iou, per, centre, boxes.dtype)
+            assert over == bool(((s32 > thr).sum(-1) > 2048).any()), it
+    finally:
+        capi.tune("nms.threads", 0)
+
+
 def test_nms_detection_workload_full_size(ops):
     """The detection-shaped case of the operator benchmark, and a dense one with a per-class limit, against the oracle."""
     c5 = synth.detection_scores(16, 80, 8400, synth.SEEDS["C5"])
