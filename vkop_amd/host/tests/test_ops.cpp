@@ -775,11 +775,40 @@ static void model_run_tests() {
     }
 }
 
+// Every single-byte change of every fixture either parses or is refused with std::runtime_error; nothing else
+// is thrown and nothing outside the (exact-size) buffer is touched.
+static void model_file_mutation_tests() {
+    size_t parsed = 0, refused = 0, other = 0;
+    for (const char *name : {"classifier_head.vkopbin", "classifier_head_k_input.vkopbin", "detection_tail.vkopbin",
+                             "detection_chain.vkopbin", "add_conv_model.vkopbin"}) {
+        const auto bytes = file_bytes(g_golden + "/" + name);
+        EXPECT(!bytes.empty());
+        for (size_t at = 0; at < bytes.size(); ++at) {
+            for (uint8_t value : {uint8_t{0x00}, uint8_t{0x7F}, uint8_t{0xFF}, static_cast<uint8_t>(bytes[at] ^ 0x01)}) {
+                if (value == bytes[at]) continue;
+                std::vector<uint8_t> copy(bytes);
+                copy[at] = value;
+                try {
+                    const vkop::load::VkModel m(copy.data(), copy.size());
+                    parsed++;
+                } catch (const std::runtime_error &) {
+                    refused++;
+                } catch (...) {
+                    other++;
+                }
+            }
+        }
+    }
+    std::printf("Model file mutations: %zu parsed, %zu refused, %zu other\n", parsed, refused, other);
+    EXPECT(other == 0 && refused > 1000 && parsed > 1000);
+}
+
 int main(int argc, char **argv) {
     const bool no_gpu = argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0;
     g_golden = (std::filesystem::path(argv[0]).parent_path() / ".." / ".." / ".." / "tests" / "golden").string();
     host_logic_tests();
     model_file_tests();
+    model_file_mutation_tests();
     if (!no_gpu) {
         const std::vector<std::pair<std::vector<int>, int>> softmax_cases = {
             {{1, 10, 7, 7}, 1}, {{1, 6, 8, 8}, 3}, {{2, 4, 10, 10}, 2}, {{1, 8, 6, 6}, 2}, {{1, 16, 5, 5}, 1}, {{4, 1000}, 1},
