@@ -106,3 +106,18 @@ def test_plan_fuses_the_class_maximum_with_its_softmax():
          {"op_type": "Reduce", "name": "r", "attributes": {"reduce_op": "max", "axes": [1], "keepdims": 0},
           "inputs": [{"name": "p", "shape": [4, 8]}], "outputs": [{"name": "y", "shape": [4]}]}]))
     assert [k for k, _, _ in runtime.plan(other_axis)] == ["softmax", "reduce_max"]
+
+
+def test_every_single_byte_change_parses_or_raises_value_error():
+    for name in ("classifier_head.vkopbin", "detection_tail.vkopbin", "add_conv_model.vkopbin", "classifier_head_k_input.vkopbin"):
+        data = open(os.path.join(GOLDEN, name), "rb").read()
+        refused = 0
+        for at in range(len(data)):
+            for value in (0x00, 0x7F, 0xFF, data[at] ^ 1):
+                if value == data[at]:
+                    continue
+                try:
+                    vkopbin.read_model(data[:at] + bytes([value]) + data[at + 1:])
+                except ValueError:
+                    refused += 1
+        assert refused > 100
