@@ -271,7 +271,6 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(NT >= 1024 ?
 #pragma unroll
         for (int r = 0; r < JP; r++) {
             const uint32_t j = wave * JP + static_cast<uint32_t>(r);
-            if (j >= K - base) break;  // (past the block's candidates; the same for the whole wave)
             if (lane > j && nms_iou(bi, box[j]) > iou_threshold) bits |= 1u << r;
         }
         if (bits != 0) atomicOr(&block_cols[lane], static_cast<unsigned long long>(bits) << (wave * JP));
