@@ -90,6 +90,12 @@ def cpu_baseline(x, k, budget_s=12.0):
         torch.topk(torch.softmax(xt, -1), k, -1, True, True)
         n += 1
     t_torch = (time.perf_counter() - t0) / max(n, 1)
+    # the reference's own CPU post-processing, restated: one row at a time, one thread (core/function.cpp:150-183)
+    sample = min(rows, 8)
+    t0 = time.perf_counter()
+    for r in range(sample):
+        oracle.get_top_k_predictions(x[r], k)
+    t_post = (time.perf_counter() - t0) / sample
     return {
         "value": rows / t_oracle, "unit": "rows/s", "cores": int(used), "kind": "port",
         "sample": "whole %dx%d batch, %d repeats of the C oracle (OpenMP over rows)" % (x.shape[0], x.shape[1], reps),
@@ -97,6 +103,9 @@ def cpu_baseline(x, k, budget_s=12.0):
                          "version": torch.__version__, "repeats": n,
                          "what": "torch.topk(torch.softmax(x,-1),k) on the host, as tests/SoftmaxTest.cpp:138 and "
                                  "tests/TopkTest.cpp:73 compute expectations"},
+        "reference_cpu_postproc": {"value": 1.0 / t_post, "unit": "rows/s", "cores": 1, "rows_timed": sample,
+                                   "what": "Function::get_top_k_predictions restated (core/function.cpp:150-183): softmax of "
+                                           "one row, full sort by probability, first k; the CPU code the GPU path replaces"},
     }
 
 
