@@ -18,10 +18,22 @@
  *                     structural invariants on tie-heavy lines.
  *   fused             composition of the two, checked the same way.
  *   get_top_k_predictions  numpy restatement on tie-free rows.
+ *   reduce max        numpy's maximum (a maximum has no rounding), NaN lines.
+ *   nms               the expectation of the reference's own test re-derived
+ *                     in numpy on its three cases (tests/NmsTest.cpp:62-169),
+ *                     invariants (kept boxes of a pair do not overlap above
+ *                     the threshold, every dropped candidate overlaps an
+ *                     earlier kept one), closed forms (disjoint boxes, equal
+ *                     boxes, threshold >= 1, per-class limit = prefix), centre
+ *                     format = corner format after conversion.
+ *   topp_count        not in the reference: closed forms with exact partial
+ *                     sums, numpy's sequential float32 cumsum, monotone in p.
  * Parity unpinned (no reference test or fixture fixes them, the behaviour is a
  * stated choice): the order of tied values (lower index first; libtorch's own
  * tie order is implementation defined), NaN ranking, largest == 0, rank-3
- * shapes, k >= 256.
+ * shapes, k >= 256; for nms the order of equal scores (lower box index first),
+ * more than 1024 candidates per (batch, class) pair (the shader's array ends
+ * there) and scores exactly at the threshold (left out, as the shader's >).
  */
 #include "vkop_oracle.h"
 
