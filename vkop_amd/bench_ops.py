@@ -186,6 +186,8 @@ def main():
     e = np.exp(c5 - c5.max(axis=1, keepdims=True))
     nms_case("C5 nms [16,80,8400] f32 iou 0.45 score 0.25 max 100", boxes, np.ascontiguousarray((e / e.sum(axis=1, keepdims=True))
              .astype(np.float32)), 100, 0.45, 0.25)
+    nms_case("nms one image [1,80,8400] f32 iou 0.45 score 0.25 max 100", boxes[:1], np.ascontiguousarray((e / e.sum(axis=1, keepdims=True))
+             .astype(np.float32)[:1]), 100, 0.45, 0.25)
     # the longest walk one (batch, class) pair can ask for: 2048 candidates, none suppressed early
     nms_case("nms [1,1,2048] f32 all candidates, iou 0.7", boxes[:1, :2048], rng.random((1, 1, 2048), dtype=np.float32), 0,
              0.7, 0.0)
