@@ -13,6 +13,9 @@
   detection_chain.vkopbin   class scores [2,80,840] -> Softmax(axis 1) -> Reduce(max, axes [1], keepdims 0) ->
                             TopK(K 30): the detection-style post-processing (example/yolo/main.cpp:60-127).
 
+  two_heads.vkopbin         a classifier head (probabilities and top-7, the probabilities an output too) beside a
+                            detection tail in one model: two nodes in the first level, a dependency into the second.
+
 add_conv_model.vkopbin is not written here: it is the reference's own model file
 (model/add_conv_model.vkopbin, made by its converter), kept as a reading fixture.
 """
@@ -67,6 +70,17 @@ def main():
          {"op_type": "TopK", "name": "node_topk", "attributes": {"K": 30, "axis": -1},
           "inputs": [shape("best", (2, 840))], "outputs": [shape("values", (2, 30)), shape("anchors", (2, 30))]}])
     open(os.path.join(HERE, "detection_chain.vkopbin"), "wb").write(chain)
+
+    two = vkopbin.write_model(
+        [shape("logits", (4, 1000)), shape("boxes", (1, 200, 4)), shape("scores", (1, 4, 200))],
+        [shape("probs", (4, 1000)), shape("values", (4, 7)), shape("indices", (4, 7)), shape("selected", (800, 3))],
+        [{"op_type": "Softmax", "name": "node_softmax", "attributes": {"axis": -1},
+          "inputs": [shape("logits", (4, 1000))], "outputs": [shape("probs", (4, 1000))]},
+         {"op_type": "Nms", "name": "node_nms", "attributes": {"iou_threshold": 0.4, "score_threshold": 0.5},
+          "inputs": [shape("boxes", (1, 200, 4)), shape("scores", (1, 4, 200))], "outputs": [shape("selected", (800, 3))]},
+         {"op_type": "TopK", "name": "node_topk", "attributes": {"K": 7},
+          "inputs": [shape("probs", (4, 1000))], "outputs": [shape("values", (4, 7)), shape("indices", (4, 7))]}])
+    open(os.path.join(HERE, "two_heads.vkopbin"), "wb").write(two)
 
 
 if __name__ == "__main__":

@@ -44,5 +44,5 @@ def test_reference_case_lists_through_operator_interface():
                    "Model classifier_head_k_input.vkopbin fp16 [4,1000] k 7, 2 operator(s) (node_topk): ok",
                    "Model detection_tail.vkopbin: ok", "Reduce max fp32 shape [16,80,8400] axis 1 keepdims 0: ok",
                    "Reduce max fp16 shape [4,80,1000] axis -2 keepdims 0: ok", "Model detection_chain.vkopbin, 2 operator(s): ok",
-                   "Model detection_chain.vkopbin, 3 operator(s): ok"):
+                   "Model detection_chain.vkopbin, 3 operator(s): ok", "Model two_heads.vkopbin, 3 operators in 2 levels: ok"):
         assert needle in r.stdout

@@ -61,7 +61,7 @@ def test_damaged_files_are_refused():
 
 
 def test_fixture_generator_reproduces_the_committed_files(tmp_path):
-    names = ["classifier_head.vkopbin", "classifier_head_k_input.vkopbin", "detection_tail.vkopbin", "detection_chain.vkopbin"]
+    names = ["classifier_head.vkopbin", "classifier_head_k_input.vkopbin", "detection_tail.vkopbin", "detection_chain.vkopbin", "two_heads.vkopbin"]
     before = {n: open(os.path.join(GOLDEN, n), "rb").read() for n in names}
     src = open(os.path.join(GOLDEN, "make_vkopbin.py")).read().replace("HERE = os.path.dirname(os.path.abspath(__file__))",
                                                                       f"HERE = {str(tmp_path)!r}")
@@ -121,3 +121,10 @@ def test_every_single_byte_change_parses_or_raises_value_error():
                 except ValueError:
                     refused += 1
         assert refused > 100
+
+
+def test_levels_with_two_nodes():
+    two = vkopbin.read_model(os.path.join(GOLDEN, "two_heads.vkopbin"))
+    assert two["levels"] == [["node_softmax", "node_nms"], ["node_topk"]]
+    assert two["nodes"][2]["dependencies"] == ["node_softmax"] and two["nodes"][1]["dependencies"] == []
+    assert [k for k, _, _ in runtime.plan(two)] == ["softmax", "nms", "topk"]      # the probabilities are an output: no fusion

@@ -732,6 +732,51 @@ static void model_chain_case(bool fuse, size_t want_nodes) {
     EXPECT(ok);
 }
 
+// Two heads in one model: two nodes in the first level (one per queue), a dependency from the second level into it.
+static void model_two_heads_case() {
+    auto pool = TestEnv::pool;
+    vkop::core::Runtime rt(pool, g_golden + "/two_heads.vkopbin", 0);
+    rt.LoadModel();
+    EXPECT(rt.num_nodes() == 3);
+    torch::manual_seed(31);
+    auto x = torch::randn({4, 1000}) * 3;
+    auto scores = torch::rand({1, 4, 200});
+    auto centre = torch::rand({1, 200, 2}), size = torch::rand({1, 200, 2}) * 0.4F;
+    auto boxes = torch::cat({centre - size / 2, centre + size / 2}, -1);
+    auto tl = vkop::core::as_tensor<float>(rt.GetInput("logits"));
+    auto tb = vkop::core::as_tensor<float>(rt.GetInput("boxes"));
+    auto ts = vkop::core::as_tensor<float>(rt.GetInput("scores"));
+    fill_from_torch(tl, x);
+    fill_from_torch(tb, boxes);
+    fill_from_torch(ts, scores);
+    tl->copyToGPU(pool);
+    tb->copyToGPU(pool);
+    ts->copyToGPU(pool);
+    for (int i = 0; i < 3; i++) rt.Run();
+    rt.ReadResult();
+    auto p = torch::softmax(x.to(torch::kFloat64), -1).to(torch::kFloat32);
+    auto want_top = torch::topk(p, 7, -1, true, true);
+    auto wi = std::get<1>(want_top).to(torch::kInt).contiguous();
+    auto indices = vkop::core::as_tensor<int>(rt.GetOutput("indices"));
+    auto probs = vkop::core::as_tensor<float>(rt.GetOutput("probs"));
+    auto selected = vkop::core::as_tensor<int>(rt.GetOutput("selected"));
+    bool ok = indices && probs && selected;
+    for (int i = 0; ok && i < 28; i++) ok = (*indices)[static_cast<size_t>(i)] == wi.data_ptr<int>()[i];
+    // (all 4000 probabilities: the small ones carry the rounding of x - max in single precision, which the operator
+    //  shares with libtorch's float kernel; against the double-precision expectation that is a relative 1e-6)
+    double worst = 0;
+    for (int i = 0; ok && i < 4000; i++) {
+        const double w = p.contiguous().data_ptr<float>()[i];
+        worst = std::max(worst, std::fabs((*probs)[static_cast<size_t>(i)] - w) / w);
+    }
+    const auto want = nms_expectation(boxes, scores, 0.4F, 0.5F);
+    for (size_t i = 0; ok && i < want.size(); i++) ok = (*selected)[i] == want[i];
+    ok = ok && worst <= 2e-6 && !want.empty() && (*selected)[want.size()] == -1;
+    std::printf("Model two_heads.vkopbin, 3 operators in 2 levels: %s, %zu records, probabilities within %.1e relative\n", ok ? "ok" : "FAILED",
+                want.size() / 3, worst);
+    EXPECT(ok);
+}
+
 static void model_run_tests() {
     TestEnv::initialize();
     auto pool = TestEnv::pool;
@@ -742,6 +787,7 @@ static void model_run_tests() {
     model_head_case<uint16_t>("classifier_head_k_input.vkopbin", 4, 7, true, 2);
     model_chain_case(true, 2);   // Softmax + Reduce as one operator, then TopK
     model_chain_case(false, 3);
+    model_two_heads_case();
     {
         vkop::core::Runtime rt(pool, g_golden + "/detection_tail.vkopbin", 0);
         rt.LoadModel();
@@ -780,7 +826,7 @@ static void model_run_tests() {
 static void model_file_mutation_tests() {
     size_t parsed = 0, refused = 0, other = 0;
     for (const char *name : {"classifier_head.vkopbin", "classifier_head_k_input.vkopbin", "detection_tail.vkopbin",
-                             "detection_chain.vkopbin", "add_conv_model.vkopbin"}) {
+                             "detection_chain.vkopbin", "two_heads.vkopbin", "add_conv_model.vkopbin"}) {
         const auto bytes = file_bytes(g_golden + "/" + name);
         EXPECT(!bytes.empty());
         for (size_t at = 0; at < bytes.size(); ++at) {
