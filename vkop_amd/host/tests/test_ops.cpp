@@ -336,6 +336,7 @@ static void host_logic_tests() {
     // names and numbering (ops/Ops.hpp)
     EXPECT(static_cast<int>(ops::OpType::SOFTMAX) == 26);
     EXPECT(static_cast<int>(ops::OpType::TOPK) == 30);
+    EXPECT(static_cast<int>(ops::OpType::REDUCE) == 20 && static_cast<int>(ops::OpType::NMS) == 32);  // ops/Ops.hpp:78,90
     EXPECT(static_cast<int>(ops::OpType::WHERE) == 40);
     EXPECT(ops::convert_optype_to_string(ops::OpType::SOFTMAX) == "Softmax");
     EXPECT(ops::convert_optype_to_string(ops::OpType::TOPK) == "TopK");
