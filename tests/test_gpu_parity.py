@@ -885,6 +885,15 @@ def test_model_files_drive_the_operators(ops, dtype):
     for fuse in (True, False):
         out = runtime.run_model(chain, {"scores": dev(sc)}, fuse=fuse)
         assert np.array_equal(host(out["anchors"]), bi) and np.array_equal(host(out["values"]).view(bits), bv.view(bits)), fuse
+    # two heads in one model
+    two = vkopbin.read_model(os.path.join(GOLDEN_DIR, "two_heads.vkopbin"))
+    rng2 = np.random.default_rng(12)
+    tb, tsc = _nms_boxes(rng2, 1, 200, 0.4).astype(dtype), rng2.random((1, 4, 200)).astype(dtype)
+    out = runtime.run_model(two, {"logits": dev(x[:4]), "boxes": dev(tb), "scores": dev(tsc)})
+    ev7, ei7 = oracle.topk(host(out["probs"]), 7, -1)
+    assert np.array_equal(host(out["indices"]), ei7) and np.array_equal(host(out["values"]).view(bits), ev7.view(bits))
+    assert np.array_equal(host(out["selected"]), oracle.nms(tb.astype(np.float32), tsc.astype(np.float32), 0.4, 0.5, 0,
+                                                             max_candidates=2048))
     # detection tail
     tail = vkopbin.read_model(os.path.join(GOLDEN_DIR, "detection_tail.vkopbin"))
     rng = np.random.default_rng(9)
