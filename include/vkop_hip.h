@@ -126,6 +126,24 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
                           int ndim, int axis, int k, int largest,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- The fused post-proc for callers that cannot allocate device memory (work
+ * recorded into a HIP graph, tight serving loops, harnesses that forbid
+ * hipMalloc): vkop_hip_softmax_topk without out_probs and without a workspace
+ * argument.  No counterpart in the reference.  Its scratch is an array of
+ * VKOP_HIP_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs on
+ * until the process ends; the call allocates and frees nothing.  A tensor whose
+ * vkop_hip_softmax_topk_workspace_bytes() exceeds that size is refused with
+ * VKOP_HIP_ERR_WORKSPACE.  Results are bit for bit those of
+ * vkop_hip_softmax_topk.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (different streams or threads) race; calls
+ * on one stream, or ordered by events, are fine.  The stream must belong to the
+ * current device; call vkop_hip_init(device) first (it looks up the array's
+ * address; otherwise the first call on a device does). */
+#define VKOP_HIP_STATIC_SCRATCH_BYTES (4u << 20)
+int vkop_hip_softmax_topk_static(const void *in, void *out_values, int32_t *out_indices,
+                                 int dtype, const int *shape, int ndim, int axis, int k,
+                                 int largest, void *stream);
+
 /* ---- Max along an axis, (.., n, ..) -> (.., ..): the per-anchor class max
  * between softmax and top-k in the detection-style post-proc
  * (example/yolo/main.cpp:60-127; ops/Reduce.hpp covers only 4-D images). */

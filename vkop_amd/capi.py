@@ -86,6 +86,7 @@ def lib():
         "vkop_hip_topk": (i, [vp, vp, vp, i, ip, i, i, i, i, i, vp, sz, vp]),
         "vkop_hip_softmax_topk_workspace_bytes": (sz, [i, ip, i, i, i]),
         "vkop_hip_softmax_topk": (i, [vp, vp, vp, vp, i, ip, i, i, i, i, vp, sz, vp]),
+        "vkop_hip_softmax_topk_static": (i, [vp, vp, vp, i, ip, i, i, i, i, vp]),
         "vkop_hip_reduce_max": (i, [vp, vp, i, ip, i, i, vp]),
         "vkop_hip_softmax_reduce_max_workspace_bytes": (sz, [i, ip, i, i]),
         "vkop_hip_softmax_reduce_max": (i, [vp, vp, i, ip, i, i, vp, sz, vp]),
@@ -229,6 +230,15 @@ def softmax_topk(inp, probs, values, indices, dtype, shape, axis, k, largest=1, 
     arr, nd = _shape(shape)
     check(lib().vkop_hip_softmax_topk(inp, probs, values, indices, dtype, arr, nd, axis, int(k), int(largest),
                                       workspace, workspace_bytes, stream))
+
+
+STATIC_SCRATCH_BYTES = 4 << 20
+
+
+def softmax_topk_static(inp, values, indices, dtype, shape, axis, k, largest=1, stream=0):
+    """The fused call on the library's own static scratch: allocates nothing."""
+    arr, nd = _shape(shape)
+    check(lib().vkop_hip_softmax_topk_static(inp, values, indices, dtype, arr, nd, axis, int(k), int(largest), stream))
 
 
 def reduce_max(inp, out, dtype, shape, axis, stream=0):

@@ -94,6 +94,36 @@ int launched(const char *what) {
     return VKOP_HIP_OK;
 }
 
+// ---- scratch of the entry point that allocates nothing ------------------------
+// One array per GPU, created when the library's code is loaded on that GPU and
+// held until the process ends.  In host code the array's name is only a handle:
+// its device address is looked up once per device (resolve_static_scratch) and
+// that address is what kernels, fills and copies are given.
+static __device__ __align__(256) unsigned char scratch[VKOP_HIP_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+// set when a call on the static scratch may have left a row's arrival counter
+// non-zero (a launch failed half way): the next call clears the counters first
+std::atomic<int> g_scratch_dirty[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call
+// per device, with that device current), and the device's ordinal.
+int resolve_static_scratch(void **ptr, int *device) {
+    int dev = 0;
+    VKOP_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(VKOP_HIP_ERR_UNSUPPORTED, "device ordinal %d beyond %d", dev, kMaxDevices);
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        VKOP_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return fail(VKOP_HIP_ERR_DEVICE, "hipGetSymbolAddress gave no address for the static scratch");
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    *device = dev;
+    return VKOP_HIP_OK;
+}
+
 // vkop_hip_tune state
 std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0}, g_nms_threads{0};
 
@@ -647,6 +677,10 @@ int vkop_hip_init(int device) {
         return fail(VKOP_HIP_ERR_UNSUPPORTED, "device %d is %s; this library is built for gfx950 only", device,
                     prop.gcnArchName);
     VKOP_HIP_TRY(hipFree(nullptr));  // force context creation here, not inside the first timed call
+    // the address of this device's static scratch, for vkop_hip_softmax_topk_static
+    void *sp = nullptr;
+    int dev = 0;
+    if (int rc = resolve_static_scratch(&sp, &dev)) return rc;
     return VKOP_HIP_OK;
 }
 
@@ -876,6 +910,49 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     return fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_probs),
                       static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, workspace,
                       as_stream(stream));
+}
+
+int vkop_hip_softmax_topk_static(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape,
+                                 int ndim, int axis, int k, int largest, void *stream) {
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (v.elems == 0 && k == 0) return VKOP_HIP_OK;
+    if (int rc = check_k(v, k)) return rc;
+    if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
+    if (in == nullptr || out_values == nullptr || out_indices == nullptr)
+        return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    const FusedPlan plan = plan_fused(v, k, dtype, largest, false);
+    const size_t need = rows_layout(v, plan.rows, plan.big).total;
+    if (need > static_cast<size_t>(VKOP_HIP_STATIC_SCRATCH_BYTES))
+        return fail(VKOP_HIP_ERR_WORKSPACE,
+                    "this tensor needs %zu bytes of scratch, the static array holds %zu: use vkop_hip_softmax_topk with a workspace",
+                    need, static_cast<size_t>(VKOP_HIP_STATIC_SCRATCH_BYTES));
+    void *sp = nullptr;
+    int dev = 0;
+    if (int rc = resolve_static_scratch(&sp, &dev)) return rc;
+    // The array keeps what the last call left.  All a call needs to find at zero
+    // are the per-row arrival counters, which every call that completes returns
+    // to zero; after a call that failed half way they are cleared here (a fill
+    // kernel, not a memset, so that the call may be recorded).
+    if (g_scratch_dirty[dev].exchange(0) != 0) {
+        const size_t words = kTicketBytes / 4;
+        vkop::fill_zero_kernel<<<static_cast<unsigned>((words + 255) / 256), 256, 0, as_stream(stream)>>>(
+            static_cast<uint32_t *>(sp), words);
+        if (int rc = launched("fill_zero_kernel")) {
+            g_scratch_dirty[dev].store(1);
+            return rc;
+        }
+    }
+    int rc;
+    if (dtype == VKOP_HIP_F32)
+        rc = fused_impl(static_cast<const float *>(in), static_cast<float *>(nullptr), static_cast<float *>(out_values),
+                        out_indices, v, k, largest, dtype, sp, as_stream(stream));
+    else
+        rc = fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(nullptr),
+                        static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, sp, as_stream(stream));
+    if (rc != VKOP_HIP_OK) g_scratch_dirty[dev].store(1);
+    return rc;
 }
 
 int vkop_hip_reduce_max(const void *in, void *out, int dtype, const int *shape, int ndim, int axis, void *stream) {
