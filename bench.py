@@ -258,7 +258,7 @@ def main():
 
     def timed(stages, nlanes):
         """(device ms, host wall ms) of K steps after W warm-up steps, HIP events on the main stream."""
-        capi.tune("rows.stages", stages)
+        capi.measure_stages(stages)
         graphs = []
         if args.eager:
             fork(nlanes)
@@ -289,7 +289,7 @@ def main():
         torch.cuda.synchronize()
         for g in graphs:
             capi.graph_destroy(g)
-        capi.tune("rows.stages", 3)
+        capi.measure_stages(3)
         return max(capi.event_elapsed_ms(e0, e1), 0.0), wall
 
     # each kernel of the path by itself (same launches, same inputs, the other

@@ -193,30 +193,32 @@ int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_ca
                  int max_output_boxes_per_class, float iou_threshold, float score_threshold,
                  void *workspace, size_t workspace_bytes, void *stream);
 
-/* ---- Tuning and measurement knobs (process-wide; no counterpart in the
- * reference, whose shaders fix their workgroup shapes at compile time).
+/* ---- Tuning knobs (no counterpart in the reference, whose shaders fix their
+ * workgroup shapes at compile time).  Results are identical for every setting;
+ * only the kernels and launch shapes chosen differ.  The settings are
+ * process-wide and read when a call is made: set them before the threads that
+ * call the operators start, not while calls are being made (a call that sees a
+ * setting change between its workspace query and its launch is refused with
+ * VKOP_HIP_ERR_WORKSPACE at worst, never runs out of bounds: *_workspace_bytes()
+ * covers every setting).
+ *   "rows.path": 0 (default) = long last-axis rows go through the scan + pick
+ *       kernel pair where it applies; 1 = never (the chunk + merge kernels).
  *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the
- *       streaming kernel (threads per workgroup, 128-bit loads per thread,
+ *       chunk kernel (threads per workgroup, 128-bit loads per thread,
  *       workgroups per row); all three must be set, 0 = automatic (default).
- *   "rows.fused": 0 (default) = rows split over several workgroups are merged
- *       by a second kernel; 1 = one kernel, whose workgroups merge each row as
- *       its last chunk completes (measured slower on MI355X: the merge then
- *       waits behind the streaming loads).  Results are identical.
- *   "rows.stages": with rows.fused = 0 only: 3 = both kernels (default), 1 =
- *       only the chunk kernel, 2 = only the merge kernel.  1 and 2 exist so
- *       that a benchmark can time each kernel by itself; their results are not
- *       valid top-k output.
+ *   "rows.fused": 0 (default) = rows split over several chunk workgroups are
+ *       merged by a second kernel; 1 = one kernel, whose workgroups merge each
+ *       row as its last chunk completes (measured slower on MI355X).
  *   "nms.threads": threads per workgroup of the Nms kernel: 0 (default) = 256
  *       from 1024 (batch, class) pairs on, else 1024; 256 or 1024 force one.
- *       Results are identical.
  * Unknown names return VKOP_HIP_ERR_INVALID. */
 int vkop_hip_tune(const char *name, int value);
 
 /* Launch shape the fused / top-k entry points would use for this tensor:
  * threads per workgroup, 128-bit loads per thread and workgroups per row of the
- * streaming kernel (a separate merge kernel runs when chunks > 1); all three are
- * 0 when the general one-workgroup-per-line kernels would run.  Any out pointer
- * may be NULL. */
+ * streaming kernel (a second kernel per row follows when chunks > 1); all three
+ * are 0 when the general one-workgroup-per-line kernels would run.  Any out
+ * pointer may be NULL. */
 int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k,
                        int *threads, int *loads, int *chunks);
 

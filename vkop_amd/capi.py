@@ -91,6 +91,7 @@ def lib():
         "vkop_hip_softmax_reduce_max_workspace_bytes": (sz, [i, ip, i, i]),
         "vkop_hip_softmax_reduce_max": (i, [vp, vp, i, ip, i, i, vp, sz, vp]),
         "vkop_hip_tune": (i, [ctypes.c_char_p, i]),
+        "vkop_hip_measure_stages": (i, [i]),
         "vkop_hip_rows_plan": (i, [i, ip, i, i, i, ip, ip, ip]),
     }
     for name, (res, args) in sig.items():
@@ -253,6 +254,12 @@ def topp_count(values, counts, dtype, rows, k, row_stride, p, stream=0):
 def tune(name, value):
     """Process-wide tuning / measurement knob (see include/vkop_hip.h)."""
     check(lib().vkop_hip_tune(name.encode(), int(value)))
+
+
+def measure_stages(stages):
+    """Benchmarks only (vkop_amd/csrc/vkop_hip_internal.h): launch only the first (1) or second (2) kernel of a
+    two-kernel streaming call, or both (3, the normal state).  Results are not valid with 1 or 2."""
+    check(lib().vkop_hip_measure_stages(int(stages)))
 
 
 def rows_plan(dtype, shape, axis, k):

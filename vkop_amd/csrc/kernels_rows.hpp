@@ -56,6 +56,14 @@ constexpr int kMergeWavesMax = 256;   // chunk-kernel waves per row the merge ca
 constexpr int kMergeChunksMax = 64;   // chunks per row
 constexpr int kLocalCap = 1024;       // candidate slots of the LDS-resident list of a one-workgroup row (cap for k = 255)
 
+// f(std::integral_constant<int, I>) for I = B .. E-1, unrolled at compile time
+template <int B, int E, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 // ---- wave-level helpers (all 64 lanes must be active) -----------------------
 
 // max over the wave, returned wave-uniform: four DPP-fused steps inside each
@@ -431,10 +439,13 @@ __device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *ro
 // group of probability 0 (the underflowed tail of the row and its -inf
 // elements), is filled by fill_group_by_scan instead.  Writes those places and
 // returns g0.  All NT threads call.
-template <typename T, int NT, int ES>
-__device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&cv)[ES], const T *rowp, T *ov, int32_t *oi,
-                                               uint32_t n, uint32_t kk, uint32_t per, uint32_t G, uint32_t thr, float p_cut,
-                                               float M, double rinv) {
+// add_missing(xlo): all threads call it; it appends to sh.cand / sh.count (atomicAdd;
+// entries past kFastCap are dropped but counted) every element of the row whose key is
+// at least xlo and that is not among the candidates yet, and returns whether it
+// touched them (the same value in every thread).
+template <typename T, int NT, typename AddMissing>
+__device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_missing, const T *rowp, T *ov, int32_t *oi,
+                                               uint32_t n, uint32_t kk, float p_cut, float M, double rinv) {
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     auto prob_of_key = [&](uint32_t key) {
         return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(key), M)) * rinv));
@@ -477,36 +488,8 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
     }
     __syncthreads();
     const uint32_t g0 = sh.g0, xlo = sh.xlo, xhi = sh.pkey[g0];
-    // Members of the group that are not in the candidate array yet: candidates this
-    // workgroup loaded but left below the merge threshold (still in registers), and
-    // elements their chunk never listed (below the chunk's threshold: those chunks
-    // are read again, which a chunk threshold far below the k-th place never needs).
-    bool added = false;
-    if (xlo < thr) {
-#pragma unroll
-        for (int e = 0; e < ES; e++) {
-            const uint32_t key = static_cast<uint32_t>(cv[e] >> 32);
-            if (key >= xlo && key < thr) {
-                const uint32_t pos = atomicAdd(&sh.count, 1u);
-                if (pos < kFastCap) sh.cand[pos] = cv[e];
-            }
-        }
-        added = true;
-    }
-    for (uint32_t b = 0; b < G; b++) {
-        const uint32_t ct = sh.cthr[b];
-        if (ct <= xlo) continue;  // (same for every thread)
-        const uint32_t c0 = min(b * per, n), c1 = min(c0 + per, n);
-        for (uint32_t j = c0 + tid; j < c1; j += NT) {
-            const uint32_t key = order_key(load_elem(rowp, j));
-            if (key >= xlo && key < ct) {
-                const uint32_t pos = atomicAdd(&sh.count, 1u);
-                if (pos < kFastCap) sh.cand[pos] = composite(key, j);
-            }
-        }
-        added = true;
-    }
-    if (added) __syncthreads();
+    // members of the group that are not in the candidate array yet
+    if (add_missing(xlo)) __syncthreads();
     const uint32_t C3 = sh.count;
     if (C3 > kFastCap) {
         fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, xlo, xhi, p_cut);
@@ -531,6 +514,107 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, const uint64_t (&
         }
     }
     return g0;
+}
+
+// ---- from the candidates above the threshold to the row's result ------------------
+// sh.cand[0..C2) holds every element of the row at or above some threshold (C2 <=
+// kFastCap; `partial`: fewer than k+1 of them, the rest of the row is -inf);
+// sh.rank[0..kFastCap) is zero and a barrier lies behind both; M, s_base: the row's
+// maximum and its sum of fast terms; sh.ref / sh.scale: per summing wave, its reference
+// and exp(ref - M); wave_of(idx): the wave that summed element idx.  Exact ranks (key,
+// then lower index); the fast terms of the k+1 ranked elements are replaced by accurate
+// ones; probabilities for those only; a probability tie across the k-th place is
+// settled over every element of the row with that probability (settle_tie with
+// add_missing); ordered store.  All NT threads call.
+template <typename T, int NT, bool SOFTMAX, typename WaveOf, typename AddMissing>
+__device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool partial, float M, double s_base, const T *rowp,
+                                           T *ov, int32_t *oi, uint32_t n, uint32_t kk, uint32_t want, WaveOf wave_of,
+                                           AddMissing add_missing) {
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1);
+    uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
+    // ---- E. exact ranks; accurate terms for the ranked elements ----------------
+    block_rank<NT>(sh, C2);
+    // only the k+1 largest are used from here on: which other candidates
+    // passed the threshold depends on the order the chunks stored theirs in,
+    // and nothing that reaches the output may
+    const uint32_t ranked = min(C2, want);
+    for (uint32_t t = tid; t < C2; t += NT) {
+        const uint32_t r = sh.rank[t];
+        if (r < ranked) {
+            const uint64_t cmp = sh.cand[t];
+            const uint32_t key = static_cast<uint32_t>(cmp >> 32);
+            const uint32_t idx = composite_index(cmp);
+            sh.pidx[r] = idx;
+            sh.pkey[r] = key;
+            double cr = 0.0;
+            float term = 0.f;  // the element's softmax term, exp(fl(x - M))
+            if (SOFTMAX && key != 0xFFFFFFFFu) {
+                const uint32_t sp = wave_of(idx);
+                const float xv = ordered_to_float(key);
+                // what the element should contribute, exp(fl(x - M)), minus what
+                // its wave added for it, fast_term(x, ref) * exp(ref - M)
+                term = softmax_term(xv, M);
+                cr = static_cast<double>(term) - static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
+            }
+            sh.prob[r] = term;  // scaled to a probability below
+            sh.corr[r] = cr;
+        }
+    }
+    __syncthreads();
+    // every wave adds up the corrections itself (same values, same tree, same
+    // result, run after run), which saves a trip through LDS and a barrier
+    double csum = 0.0;
+    for (uint32_t r = lane; r < ranked; r += kWave) csum += sh.corr[r];
+    const double total = s_base + wave_sum_f64_uniform(csum);
+    if constexpr (SOFTMAX) {
+        // the formula of softmax_prob(): the float term scaled in double, rounded once
+        const double rinv = 1.0 / total;
+        if (tid <= kk && tid < ranked)
+            sh.prob[tid] = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[tid]) * rinv));
+        __syncthreads();
+        // Probabilities are non-increasing along the rank order, so equal
+        // ones are neighbours.  A tie that reaches past the k-th place is
+        // settled by index over every element of the row with that
+        // probability, candidates or not.
+        if (partial) {
+            // the candidates of probability 0, if any, and the -inf elements form one
+            // group behind every positive probability: lowest indices first
+            if (tid == 0) sh.g0 = C2;
+            __syncthreads();
+            if (tid < C2 && sh.prob[tid] == 0.f && (tid == 0 || sh.prob[tid - 1] != 0.f)) sh.g0 = tid;
+            __syncthreads();
+            tie_g0 = sh.g0;
+            fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, tie_g0, kk, 0u,
+                                            tie_g0 < C2 ? sh.pkey[tie_g0] : kKeyNegInf, 0.f);
+        } else if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
+            tie_g0 = settle_tie<T, NT>(sh, add_missing, rowp, ov, oi, n, kk, sh.prob[kk], M, rinv);
+        }
+    } else if (partial) {
+        // the -inf elements follow the candidates, lowest indices first
+        tie_g0 = C2;
+        fill_group_by_scan<T, NT, false>(sh.scan_counts, rowp, ov, oi, n, C2, kk, kKeyNegInf, kKeyNegInf, 0.f);
+    }
+
+    const uint32_t plain = min(kk, tie_g0);  // ranks at or after tie_g0 were written by settle_tie
+    for (uint32_t r = tid; r < plain; r += NT) {
+        const uint32_t idx = sh.pidx[r];
+        if constexpr (SOFTMAX) {
+            const float p = sh.prob[r];
+            // final place inside a run of equal probabilities: by index
+            uint32_t lo = r, hi = r, pos = r;
+            while (lo > 0 && sh.prob[lo - 1] == p) lo--;
+            while (hi + 1 < plain && sh.prob[hi + 1] == p) hi++;
+            if (hi > lo) {
+                pos = lo;
+                for (uint32_t q = lo; q <= hi; q++) pos += (sh.pidx[q] < idx) ? 1u : 0u;
+            }
+            store_elem(ov, pos, p);
+            oi[pos] = static_cast<int32_t>(idx);
+        } else {
+            ov[r] = rowp[idx];  // bit copy (keeps the sign of a zero)
+            oi[r] = static_cast<int32_t>(idx);
+        }
+    }
 }
 
 // ---- merge of one row's chunk results (all NT threads of a workgroup) --------
@@ -687,8 +771,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     }
     if (G == 1) thr = 1u;
     uint32_t merge_thr = thr;  // candidates with keys at or above it are in sh.cand (of equal keys maybe only the first)
-    bool slow = sh.flag != 0u;
-    uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
+    const bool slow = sh.flag != 0u;
     if constexpr (SOFTMAX) {
         if (!(s_base > 0.0 && s_base < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY)) {
             // a NaN or +inf element, or nothing above -inf: every probability of the
@@ -787,101 +870,51 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
             C2 = sh.count;
             merge_thr = cutkey;
         }
-        // Fewer than k+1 candidates: no chunk had k+1 elements above -inf, so every
-        // chunk listed all it has and the rest of the row is -inf (probability 0).
-        const bool partial = C2 < min(want, n);
-        if (C2 > kFastCap) {
-            slow = true;
-        } else {
-            // ---- E. exact ranks; accurate terms for the ranked elements ----------------
-            block_rank<NT>(sh, C2);
-            // only the k+1 largest are used from here on: which other candidates
-            // passed the threshold depends on the order the chunks stored theirs in,
-            // and nothing that reaches the output may
-            const uint32_t ranked = min(C2, want);
-            for (uint32_t t = tid; t < C2; t += NT) {
-                const uint32_t r = sh.rank[t];
-                if (r < ranked) {
-                    const uint64_t cmp = sh.cand[t];
-                    const uint32_t key = static_cast<uint32_t>(cmp >> 32);
-                    const uint32_t idx = composite_index(cmp);
-                    sh.pidx[r] = idx;
-                    sh.pkey[r] = key;
-                    double cr = 0.0;
-                    float term = 0.f;  // the element's softmax term, exp(fl(x - M))
-                    if (SOFTMAX && key != 0xFFFFFFFFu) {
-                        // the chunk-kernel wave that summed this element
-                        const uint32_t b = idx / per, off = idx - b * per;
-                        const uint32_t sp = b * src_nw + ((off / VEC) % src_nt) / kWave;
-                        const float xv = ordered_to_float(key);
-                        // what the element should contribute, exp(fl(x - M)), minus what
-                        // its wave added for it, fast_term(x, ref) * exp(ref - M)
-                        term = softmax_term(xv, M);
-                        cr = static_cast<double>(term) - static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
+        if (C2 <= kFastCap) {
+            // Fewer than k+1 candidates: no chunk had k+1 elements above -inf, so every
+            // chunk listed all it has and the rest of the row is -inf (probability 0).
+            const bool partial = C2 < min(want, n);
+            // Members of a tie across the k-th place that are not candidates yet:
+            // candidates this workgroup loaded but left below the merge threshold (still
+            // in registers), and elements their chunk never listed (below the chunk's
+            // threshold: those chunks are read again, which a chunk threshold far below
+            // the k-th place never needs).
+            auto add_missing = [&](uint32_t xlo) -> bool {
+                bool added = false;
+                if (xlo < merge_thr) {
+#pragma unroll
+                    for (int e = 0; e < ES; e++) {
+                        const uint32_t key = static_cast<uint32_t>(cv[e] >> 32);
+                        if (key >= xlo && key < merge_thr) {
+                            const uint32_t pos = atomicAdd(&sh.count, 1u);
+                            if (pos < kFastCap) sh.cand[pos] = cv[e];
+                        }
                     }
-                    sh.prob[r] = term;  // scaled to a probability below
-                    sh.corr[r] = cr;
+                    added = true;
                 }
-            }
-            __syncthreads();
-            // every wave adds up the corrections itself (same values, same tree, same
-            // result, run after run), which saves a trip through LDS and a barrier
-            double csum = 0.0;
-            for (uint32_t r = lane; r < ranked; r += kWave) csum += sh.corr[r];
-            const double total = s_base + wave_sum_f64_uniform(csum);
-            if constexpr (SOFTMAX) {
-                // the formula of softmax_prob(): the float term scaled in double, rounded once
-                const double rinv = 1.0 / total;
-                if (tid <= kk && tid < ranked)
-                    sh.prob[tid] = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[tid]) * rinv));
-                __syncthreads();
-                // Probabilities are non-increasing along the rank order, so equal
-                // ones are neighbours.  A tie that reaches past the k-th place is
-                // settled by index over every element of the row with that
-                // probability, candidates or not.
-                if (partial) {
-                    // the candidates of probability 0, if any, and the -inf elements form one
-                    // group behind every positive probability: lowest indices first
-                    if (tid == 0) sh.g0 = C2;
-                    __syncthreads();
-                    if (tid < C2 && sh.prob[tid] == 0.f && (tid == 0 || sh.prob[tid - 1] != 0.f)) sh.g0 = tid;
-                    __syncthreads();
-                    tie_g0 = sh.g0;
-                    fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, tie_g0, kk, 0u,
-                                                    tie_g0 < C2 ? sh.pkey[tie_g0] : kKeyNegInf, 0.f);
-                } else if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
-                    tie_g0 = settle_tie<T, NT, ES>(sh, cv, rowp, ov, oi, n, kk, per, G, merge_thr, sh.prob[kk], M, rinv);
+                for (uint32_t b = 0; b < G; b++) {
+                    const uint32_t ct = sh.cthr[b];
+                    if (ct <= xlo) continue;  // (same for every thread)
+                    const uint32_t c0 = min(b * per, n), c1 = min(c0 + per, n);
+                    for (uint32_t j = c0 + tid; j < c1; j += NT) {
+                        const uint32_t key = order_key(load_elem(rowp, j));
+                        if (key >= xlo && key < ct) {
+                            const uint32_t pos = atomicAdd(&sh.count, 1u);
+                            if (pos < kFastCap) sh.cand[pos] = composite(key, j);
+                        }
+                    }
+                    added = true;
                 }
-            } else if (partial) {
-                // the -inf elements follow the candidates, lowest indices first
-                tie_g0 = C2;
-                fill_group_by_scan<T, NT, false>(sh.scan_counts, rowp, ov, oi, n, C2, kk, kKeyNegInf, kKeyNegInf, 0.f);
-            }
+                return added;
+            };
+            // the chunk-kernel wave that summed element idx
+            auto wave_of = [&](uint32_t idx) {
+                const uint32_t b = idx / per, off = idx - b * per;
+                return b * src_nw + ((off / VEC) % src_nt) / kWave;
+            };
+            finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing);
+            return;
         }
-    }
-
-    if (!slow) {
-        const uint32_t plain = min(kk, tie_g0);  // ranks at or after tie_g0 were written by settle_tie
-        for (uint32_t r = tid; r < plain; r += NT) {
-            const uint32_t idx = sh.pidx[r];
-            if constexpr (SOFTMAX) {
-                const float p = sh.prob[r];
-                // final place inside a run of equal probabilities: by index
-                uint32_t lo = r, hi = r, pos = r;
-                while (lo > 0 && sh.prob[lo - 1] == p) lo--;
-                while (hi + 1 < plain && sh.prob[hi + 1] == p) hi++;
-                if (hi > lo) {
-                    pos = lo;
-                    for (uint32_t q = lo; q <= hi; q++) pos += (sh.pidx[q] < idx) ? 1u : 0u;
-                }
-                store_elem(ov, pos, p);
-                oi[pos] = static_cast<int32_t>(idx);
-            } else {
-                ov[r] = rowp[idx];  // bit copy (keeps the sign of a zero)
-                oi[r] = static_cast<int32_t>(idx);
-            }
-        }
-        return;
     }
 
     // ---- exact path: radix select over the whole row ----------------------------

@@ -1,0 +1,451 @@
+// Long contiguous rows split over several workgroups: the streaming pass.
+//
+// rows_scan_kernel reads the input once and does nothing with an element but what
+// every element needs: it goes into the maximum of its BLOCK -- 16 consecutive
+// 128-bit vectors of the row, 256 bytes, what 16 neighbouring lanes read with one
+// load -- and, for the softmax variant, into the wave's sum of exp(x - ref).  It
+// writes one order key per block and one record per wave.  No threshold, no
+// compaction, no barrier: the pass is issue-bound on this chip (every instruction of
+// every wave costs four cycles of its SIMD), so whatever only a few elements need is
+// left to the kernel that follows.
+//
+// rows_pick_kernel (one workgroup per row) finds a value that k+1 block maxima
+// reach, reads again the few blocks that reach it (k+1 of them plus ties, 256
+// contiguous bytes each), and ranks their elements at or above that value exactly
+// (kernels_rows.hpp: finish_row).
+#pragma once
+
+#include "kernels_rows.hpp"
+
+namespace vkop {
+
+constexpr int kScanThreads = 256;
+constexpr int kScanWaves = kScanThreads / kWave;
+constexpr int kBlockLanes = 16;  // lanes (vectors) per block: one row of a wave's cross-lane network
+
+struct ScanWorkspace {
+    uint32_t *bmax;    // [rows][blocks]: order key of the block's maximum (softmax: NaN dropped; plain top-k: all
+                       // ones if the block holds a NaN); block b = elements b * 16 * vector width ... of the row
+    uint64_t *recs;    // [rows][G][kScanWaves][2]: sum of exp(x - ref) over the wave's elements (double bits); ref
+                       // (low half) and the wave's maximum (high half) as float bits
+    uint32_t blocks;   // blocks per row: ceil(n / (16 * vector width))
+};
+
+// Launch: rows * G workgroups of kScanThreads; a chunk is exactly 256 * V vectors
+// (G = ceil(n / that)), so that blocks never straddle chunks.
+template <typename T, int V, bool SOFTMAX, bool ALIGNED>
+__global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__restrict__ in, uint32_t n, uint32_t G,
+                                                                 ScanWorkspace ws) {
+    constexpr int NT = kScanThreads, NW = kScanWaves;
+    constexpr int VEC = Vec128<T>::N;
+    constexpr uint32_t per = static_cast<uint32_t>(NT) * V * VEC;
+    constexpr int WB = V * (kWave / kBlockLanes);  // blocks a wave covers: V vectors x 4 rows of 16 lanes
+    static_assert(WB <= kWave, "a lane per block of the wave");
+    __shared__ float vm_lds[NW][V][kWave];  // per wave: the maximum of every lane's vector i
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
+    const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
+    const T *rowp = in + static_cast<size_t>(row) * n;
+    const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
+
+    // all loads in flight (never a branch around a load: out-of-chunk lanes read the
+    // row's first element(s) instead and are masked where the data is used)
+    Vec128<T> q[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+        q[i].v = make_uint4(0, 0, 0, 0);
+        if constexpr (ALIGNED) {
+            q[i].load(rowp + (e0 < c1 ? e0 : 0u));
+        } else {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < c1 ? e0 + c : 0u));
+        }
+    }
+
+    // The rest exists twice: for a chunk that fills every lane of every vector (no
+    // masking anywhere) and for a ragged one.
+    auto body = [&](auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        auto in_range = [&](uint32_t e) { return FULL || e < c1; };
+        auto elem = [&](auto i_tag, int c) {
+            constexpr int i = decltype(i_tag)::value;
+            const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+            return in_range(ALIGNED ? e0 : e0 + static_cast<uint32_t>(c)) ? q[i].get(c) : -INFINITY;
+        };
+        float ref = 0.f;
+        double acc = 0.0;  // every term is added in double: a dominant term must not swallow what follows it
+        static_for<0, V>([&](auto i_tag) {
+            constexpr int i = decltype(i_tag)::value;
+            float xv[VEC];
+            float vm = -INFINITY;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                xv[c] = elem(i_tag, c);
+                vm = fmaxf(vm, xv[c]);  // (drops NaN)
+            }
+            if constexpr (SOFTMAX) {
+                if constexpr (i == 0) {
+                    // reference of the wave's partial sum: kRefLift above the maximum of its
+                    // first vectors; 0 if they hold no finite element (terms are then 0, or
+                    // NaN, which must survive -- never -inf - -inf)
+                    const float wm0 = wave_max_f32_uniform(vm);
+                    ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
+                }
+#pragma unroll
+                for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(xv[c], ref));
+                // the sum so far exists HERE, under the loads still in flight (or the
+                // compiler moves all of it behind the last load)
+                asm volatile("" : "+v"(acc));
+            } else {
+                // NaN ranks first in a plain top-k: the vector's maximum is then NaN
+                bool has_nan = false;
+#pragma unroll
+                for (int c = 0; c < VEC; c += 2) has_nan = has_nan || __builtin_isunordered(xv[c], xv[c + 1]);
+                vm = has_nan ? __uint_as_float(0x7FC00000u) : vm;
+            }
+            vm_lds[wave][i][lane] = vm;
+        });
+        // ---- block maxima: lane L of the wave takes block L of the wave's WB blocks -----
+        // (block (vector i, lanes 16 r .. 16 r + 15) is the wave's block 4 i + r, and its 16
+        // lane values lie side by side; the wave's blocks are read by the wave that wrote them)
+        __builtin_amdgcn_wave_barrier();
+        float bm = -INFINITY;
+        bool b_nan = false;
+        if (lane < static_cast<uint32_t>(WB)) {
+            const float4 *src = reinterpret_cast<const float4 *>(&vm_lds[wave][0][0] + lane * kBlockLanes);
+#pragma unroll
+            for (int j = 0; j < kBlockLanes / 4; j++) {
+                const float4 v4 = src[j];
+                bm = fmaxf(fmaxf(bm, fmaxf(v4.x, v4.y)), fmaxf(v4.z, v4.w));
+                if constexpr (!SOFTMAX) b_nan = b_nan || __builtin_isunordered(v4.x, v4.y) || __builtin_isunordered(v4.z, v4.w);
+            }
+            // the wave's block L = vector L / 4, lane row L % 4 starts at element
+            // c0 + ((L / 4) * NT + wave * 64 + (L % 4) * 16) * VEC of the row
+            const uint32_t e_block = c0 + ((lane / 4u) * NT + wave * kWave + (lane % 4u) * kBlockLanes) * VEC;
+            if (FULL || e_block < c1) {
+                const uint32_t key = b_nan ? 0xFFFFFFFFu : order_key(bm);
+                ws.bmax[static_cast<size_t>(row) * ws.blocks + e_block / (kBlockLanes * VEC)] = key;
+            }
+        }
+        // ---- the wave's record ---------------------------------------------------------------
+        if constexpr (SOFTMAX) {
+            const float wm = wave_max_f32_uniform(bm);
+            double wsum = wave_sum_f64_uniform(acc);
+            if (wm - ref > kTermSwitch) {  // wave-uniform
+                // an element well above the reference: its fast term is poor (or has
+                // overflowed); everything is in registers, so sum again against the maximum
+                ref = (wm < INFINITY) ? wm : ref;
+                acc = 0.0;
+                static_for<0, V>([&](auto i_tag) {
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(elem(i_tag, c), ref));
+                });
+                wsum = wave_sum_f64_uniform(acc);
+            }
+            if (lane == 0) {
+                uint64_t *record = ws.recs + 2 * (static_cast<size_t>(row * G + chunk) * NW + wave);
+                record[0] = static_cast<uint64_t>(__double_as_longlong(wsum));
+                record[1] = (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref);
+            }
+        }
+    };
+    if (c1 - c0 == per) body(std::true_type{});
+    else body(std::false_type{});
+}
+
+constexpr int kPickHitCap = 1024;  // blocks one gather reads again
+
+struct PickShared {
+    RowsShared fast;
+    uint32_t hits[kPickHitCap];  // the blocks to read again
+};
+union PickSharedUnion {
+    PickShared pick;
+    SelectShared exact;
+    __device__ PickSharedUnion() {}
+};
+
+// One workgroup of NT threads per row, after rows_scan_kernel on the same stream.
+// GE: block keys a thread takes in (GE * NT >= blocks per row); G, per: chunks per
+// row and elements per chunk of the scan kernel (which wave summed which element).
+//   A. one round trip: the wave records and the row's block keys (GE per thread);
+//   B. the row's maximum and sum of terms from the wave records;
+//   C. a value that at least k+1 block maxima reach: ballot descents over the
+//      per-thread maxima of the keys (every block maximum is an element);
+//   D. the blocks that reach it -- k+1 and a few -- are read again, 16 lanes a block,
+//      several loads per thread in flight; their elements at or above the value are
+//      the candidates (everything else in the row is below k+1 elements);
+//   E. finish_row: exact ranks, accurate terms, probabilities, ties, ordered store.
+// A probability tie across the k-th place that reaches below the value gathers again
+// with the tied interval's lower end (settle_tie); what that cannot hold (rows full of
+// equal values) goes to the scan from the row's start or, from D, to the exact radix
+// select over the whole row.
+constexpr int kPickThreads = 512;
+
+template <typename T, bool SOFTMAX, bool ALIGNED, int GE, int NT = kPickThreads>
+__global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                                  int32_t *__restrict__ indices, uint32_t n, uint32_t k,
+                                                                  uint32_t G, uint32_t per, ScanWorkspace ws) {
+    constexpr int NW = NT / kWave;
+    constexpr int VEC = Vec128<T>::N;
+    constexpr int U = NT >= 1024 ? 2 : NT >= 512 ? 4 : 8;  // loads per thread in flight while blocks are read again (128 blocks a round)
+    constexpr uint32_t BE = kBlockLanes * VEC;  // elements per block
+    __shared__ PickSharedUnion smem;
+    __shared__ float fscratch[NW];
+    __shared__ double dscratch[NW];
+    RowsShared &sh = smem.pick.fast;
+    uint32_t *hits = smem.pick.hits;
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t row = blockIdx.x;
+    const T *rowp = in + static_cast<size_t>(row) * n;
+    T *ov = values + static_cast<size_t>(row) * k;
+    int32_t *oi = indices + static_cast<size_t>(row) * k;
+    const uint32_t want = k + 1;
+    const uint32_t kk = min(k, n);
+    const uint32_t waves = G * kScanWaves;
+    // ---- A. everything the kernel reads first, in one round trip --------------------
+    // (never a branch around a load: out-of-range threads re-read entry 0)
+    const uint64_t *recs = ws.recs + 2 * static_cast<size_t>(row) * waves;
+    const uint32_t wq = tid < waves ? tid : 0u;
+    uint64_t s_bits = 0, rm_bits = 0;
+    if constexpr (SOFTMAX) {
+        s_bits = recs[2 * wq];
+        rm_bits = recs[2 * wq + 1];
+    }
+    const uint32_t blocks = ws.blocks;
+    const uint32_t *bmax = ws.bmax + static_cast<size_t>(row) * blocks;
+    uint32_t gk[GE];
+#pragma unroll
+    for (int e = 0; e < GE; e++) {
+        const uint32_t b = static_cast<uint32_t>(e) * NT + tid;
+        gk[e] = bmax[b < blocks ? b : 0u];
+    }
+
+    // ---- B. the row's maximum and sum from the wave partials --------------------------
+    for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;  // for block_rank, barriers away
+    if (tid == 0) sh.count = 0;
+    if constexpr (SOFTMAX) {
+        SumPartial p0{0.0, 0.f, -INFINITY};
+        if (tid < waves) {
+            p0.s = __longlong_as_double(static_cast<long long>(s_bits));
+            p0.ref = __uint_as_float(static_cast<uint32_t>(rm_bits));
+            p0.m = __uint_as_float(static_cast<uint32_t>(rm_bits >> 32));
+            sh.ref[tid] = p0.ref;
+        }
+        // With at most 64 wave records (one per lane of wave 0) that wave alone combines
+        // them, by cross-lane steps, while the others go on to the threshold; the
+        // results are published by the barrier there.
+        if (waves <= static_cast<uint32_t>(kWave)) {
+            if (wave == 0) {
+                const float m = wave_max_f32_uniform(p0.m);
+                double acc = 0.0;
+                if (tid < waves) {
+                    const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+                    sh.scale[tid] = sc;
+                    if (p0.s != 0.0) acc = p0.s * sc;
+                }
+                const double total = wave_sum_f64_uniform(acc);
+                if (lane == 0) {
+                    sh.row_max = m;
+                    sh.total = total;
+                }
+            }
+        } else {
+            const float m = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.ref is published)
+            double acc = 0.0;
+            if (tid < waves) {
+                const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+                sh.scale[tid] = sc;
+                if (p0.s != 0.0) acc = p0.s * sc;
+            }
+            const double total = block_sum_fast<NT>(acc, dscratch);  // (barrier: sh.scale is published)
+            if (tid == 0) {
+                sh.row_max = m;
+                sh.total = total;
+            }
+        }
+    }
+
+    // ---- C. a value that k+1 block maxima reach ---------------------------------------------
+    uint32_t lmk = 0;
+#pragma unroll
+    for (int e = 0; e < GE; e++) {
+        if (static_cast<uint32_t>(e) * NT + tid >= blocks) gk[e] = 0;  // (block 0 was read instead)
+        lmk = max(lmk, gk[e]);
+    }
+    // Every wave takes, by a ballot descent over its own 64 thread maxima (18 bits),
+    // the largest value that its share of k+1 of them reach: the smallest of these
+    // bounds is reached by k+1 thread maxima in all, hence by k+1 blocks.  A share of
+    // more than half a wave, or a wave without enough live threads, leaves it to one
+    // wave and all the maxima.
+    const uint32_t quota = (want + NW - 1) / NW;
+    uint32_t mine_q = 0;
+    if (quota <= 32u) {
+        for (int bit = 31; bit > 13; bit--) {
+            const uint32_t trial = mine_q | (1u << bit);
+            if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= quota) mine_q = trial;
+        }
+    }
+    sh.lane_key[tid] = lmk;
+    if (lane == 0) sh.wave_thr[wave] = mine_q;
+    __syncthreads();
+    float M = 0.f;
+    double s_base = 0.0;
+    if constexpr (SOFTMAX) {
+        M = sh.row_max;
+        s_base = sh.total;
+    }
+    uint32_t thr = sh.wave_thr[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) thr = min(thr, sh.wave_thr[w]);
+    if (thr <= 1u) {  // (the same for every thread)
+        if (wave == 0) {
+            const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
+            if (lane == 0) sh.thr = t;
+        }
+        __syncthreads();
+        thr = sh.thr;
+    }
+    // -inf never becomes a candidate: a row with k+1 larger elements does not need it,
+    // and finish_row fills any other row's last places from the row itself
+    thr = max(thr, kKeyNegInf + 1u);
+    if constexpr (SOFTMAX) {
+        if (!(s_base > 0.0 && s_base < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY)) {
+            // a NaN or +inf element, or nothing above -inf: every probability of the
+            // row is NaN, all of them tie, the lowest indices win
+            for (uint32_t r = tid; r < kk; r += NT) {
+                store_elem(ov, r, __uint_as_float(0x7FC00000u));
+                oi[r] = static_cast<int32_t>(r);
+            }
+            return;
+        }
+    }
+
+    // ---- D. the elements with keys in [lo, hi) of the blocks whose maximum reaches lo -> sh.cand ----
+    // All threads call; ends with a barrier.  Returns true (in every thread) when more
+    // than kPickHitCap blocks reach lo: nothing was gathered then.
+    uint32_t round = 0;
+    // (always inlined: a call would put the block keys, captured by reference, into scratch memory)
+    auto gather = [&](uint32_t lo, uint64_t hi) __attribute__((always_inline)) -> bool {
+        uint32_t wave_n = 0;  // wave-uniform
+#pragma unroll
+        for (int e = 0; e < GE; e++) wave_n += static_cast<uint32_t>(__popcll(__ballot(gk[e] >= lo)));
+        uint32_t *wc = sh.scan_counts + (round & 1u) * NW;
+        round++;
+        if (lane == 0) wc[wave] = wave_n;
+        __syncthreads();
+        uint32_t H = 0, pos = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const uint32_t c = wc[w];
+            pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
+            H += c;
+        }
+        if (H > static_cast<uint32_t>(kPickHitCap)) return true;
+#pragma unroll
+        for (int e = 0; e < GE; e++) {
+            const bool pass = gk[e] >= lo;
+            const uint64_t mask = __ballot(pass);
+            if (mask != 0ull) {
+                if (pass) hits[pos + lanes_below(mask)] = static_cast<uint32_t>(e) * NT + tid;
+                pos += static_cast<uint32_t>(__popcll(mask));
+            }
+        }
+        __syncthreads();
+        const uint32_t items = H * kBlockLanes;  // one per vector of a block that is read again
+        for (uint32_t j0 = 0; j0 < items; j0 += NT * U) {
+            Vec128<T> r[U];
+            uint32_t e0[U], cend[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint32_t j = j0 + static_cast<uint32_t>(u) * NT + tid;
+                const uint32_t b = hits[j < items ? j / kBlockLanes : 0u];
+                e0[u] = b * BE + (j % kBlockLanes) * VEC;
+                cend[u] = j < items ? n : 0u;  // (0: nothing of this slot counts)
+                r[u].v = make_uint4(0, 0, 0, 0);
+                if constexpr (ALIGNED) {
+                    r[u].load(rowp + (e0[u] < cend[u] ? e0[u] : 0u));
+                } else {
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) r[u].set(c, load_elem(rowp, e0[u] + c < cend[u] ? e0[u] + c : 0u));
+                }
+            }
+            const float lo_f = ordered_to_float(lo);  // (lo > key of -inf: a number or +inf)
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                // a vector without an element at or above lo (15 of a block's 16) costs one test
+                float vm = -INFINITY;
+                bool any_nan = false;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    const float x = r[u].get(c);
+                    vm = fmaxf(vm, x);
+                    if constexpr (!SOFTMAX) any_nan = any_nan || x != x;
+                }
+                if (!(vm < lo_f) || any_nan) {
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        const float x = r[u].get(c);
+                        const uint32_t idx = e0[u] + static_cast<uint32_t>(c);
+                        const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
+                        if (idx < cend[u] && key >= lo && static_cast<uint64_t>(key) < hi) {
+                            const uint32_t at = atomicAdd(&sh.count, 1u);
+                            if (at < static_cast<uint32_t>(kFastCap)) sh.cand[at] = composite(key, idx);
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        return false;
+    };
+    const bool many_groups = gather(thr, 1ull << 32);
+    const uint32_t C2 = sh.count;
+    if (!many_groups && C2 <= static_cast<uint32_t>(kFastCap)) {
+        // Fewer than k+1 candidates: fewer than k+1 blocks hold an element above -inf,
+        // every one of them was read again, and the rest of the row is -inf.
+        const bool partial = C2 < min(want, n);
+        // members of a tie across the k-th place below the value used above
+        auto add_missing = [&](uint32_t xlo) -> bool {
+            if (xlo >= thr) return false;
+            if (gather(xlo, thr)) {
+                if (tid == 0) sh.count = kFastCap + 1;  // too many to collect: the scan from the row's start
+                __syncthreads();
+            }
+            return true;
+        };
+        // the scan-kernel wave that summed element idx
+        auto wave_of = [&](uint32_t idx) {
+            const uint32_t b = idx / per, off = idx - b * per;
+            return b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;
+        };
+        finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing);
+        return;
+    }
+
+    // ---- exact path: radix select over the whole row ----------------------------
+    __syncthreads();  // LDS changes owner
+    SelectShared &exact = smem.exact;
+    if constexpr (SOFTMAX) {
+        // the statistics the way the general kernels define them
+        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch);
+        select_topk_line<NT>(exact, n, kk, [&](uint32_t j) {
+            return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
+        });
+        for (uint32_t r = tid; r < kk; r += NT) {
+            const uint32_t idx = composite_index(exact.sel[r]);
+            store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
+            oi[r] = static_cast<int32_t>(idx);
+        }
+    } else {
+        select_topk_line<NT>(exact, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
+        for (uint32_t r = tid; r < kk; r += NT) {
+            const uint32_t idx = composite_index(exact.sel[r]);
+            ov[r] = rowp[idx];
+            oi[r] = static_cast<int32_t>(idx);
+        }
+    }
+}
+
+}  // namespace vkop

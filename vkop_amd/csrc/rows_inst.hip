@@ -65,6 +65,47 @@ template <typename T, bool SOFTMAX> void launch_rows_merge(const RowsLaunch &a) 
 #undef VKOP_MERGE_LAUNCH
 }
 
+template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
+    const T *in = static_cast<const T *>(a.in);
+    constexpr uint32_t VEC = 16 / sizeof(T);
+    const uint32_t per = kScanThreads * a.v * VEC;
+    const uint32_t ge = (a.ws.blocks + kPickThreads - 1) / kPickThreads;
+    if (ge > 16) return false;
+    bool scanned = (a.stages & 1) == 0;
+#define VKOP_SCAN_CASE(V)                                                                                      \
+    if (!scanned && a.v == V) {                                                                                \
+        if (a.aligned) rows_scan_kernel<T, V, SOFTMAX, true><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws); \
+        else rows_scan_kernel<T, V, SOFTMAX, false><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws);          \
+        scanned = true;                                                                                        \
+    }
+    VKOP_SCAN_CASE(2)
+    VKOP_SCAN_CASE(4)
+    VKOP_SCAN_CASE(8)
+    if constexpr (sizeof(T) == 4) {
+        VKOP_SCAN_CASE(16)
+    }
+#undef VKOP_SCAN_CASE
+    if (!scanned) return false;
+    if ((a.stages & 2) == 0) return true;
+#define VKOP_PICK_LAUNCH(GE, AL)                                                      \
+    rows_pick_kernel<T, SOFTMAX, AL, GE><<<a.rows, kPickThreads, 0, a.stream>>>(      \
+        in, static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, per, a.ws)
+#define VKOP_PICK_CASE(GE)                         \
+    if (ge <= GE) {                                \
+        if (a.aligned) VKOP_PICK_LAUNCH(GE, true); \
+        else VKOP_PICK_LAUNCH(GE, false);          \
+        return true;                               \
+    }
+    VKOP_PICK_CASE(2)
+    VKOP_PICK_CASE(4)
+    VKOP_PICK_CASE(8)
+    VKOP_PICK_CASE(16)
+#undef VKOP_PICK_CASE
+#undef VKOP_PICK_LAUNCH
+    return false;
+}
+
+template bool launch_rows_scan<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const ScanLaunch &);
 template bool launch_rows_chunk<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
 template void launch_rows_merge<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
 

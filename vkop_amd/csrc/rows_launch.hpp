@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels_rows.hpp"
+#include "kernels_stream.hpp"
 
 namespace vkop {
 
@@ -23,6 +24,26 @@ struct RowsLaunch {
     RowsWorkspace ws;
     hipStream_t stream;
 };
+
+// Launch of the streaming pair rows_scan_kernel + rows_pick_kernel (kernels_stream.hpp).
+struct ScanLaunch {
+    const void *in;
+    void *values;
+    int32_t *indices;
+    uint32_t rows, n, k;
+    uint32_t v;        // 128-bit loads per thread of the scan kernel (a chunk is 256 * v vectors)
+    uint32_t g;        // chunks per row
+    bool aligned;      // rows start on 16 bytes and n is a multiple of the vector width
+    int stages;        // 1 = scan only, 2 = pick only, 3 = both (1 and 2: measurements)
+    ScanWorkspace ws;
+    hipStream_t stream;
+};
+// Enqueues rows_scan_kernel and rows_pick_kernel; false if no kernel is built for the shape.
+template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a);
+extern template bool launch_rows_scan<float, true>(const ScanLaunch &);
+extern template bool launch_rows_scan<float, false>(const ScanLaunch &);
+extern template bool launch_rows_scan<uint16_t, true>(const ScanLaunch &);
+extern template bool launch_rows_scan<uint16_t, false>(const ScanLaunch &);
 
 // Enqueues rows_chunk_kernel; false if no kernel is built for (nt, v).
 template <typename T, bool SOFTMAX> bool launch_rows_chunk(const RowsLaunch &a);

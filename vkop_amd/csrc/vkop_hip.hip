@@ -1,6 +1,7 @@
 // C ABI of the softmax / top-k library (declared in include/vkop_hip.h):
 // argument checking, kernel selection and launches (the only kernel here clears a workspace).
 #include "../../include/vkop_hip.h"
+#include "vkop_hip_internal.h"
 
 #include <hip/hip_runtime.h>
 
@@ -125,7 +126,8 @@ int resolve_static_scratch(void **ptr, int *device) {
 }
 
 // vkop_hip_tune state
-std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0}, g_nms_threads{0};
+std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0}, g_rows_path{0},
+    g_nms_threads{0};
 
 // The per-row arrival counters of the one-kernel top-k variant sit at a fixed
 // place, the first kTicketRows words of every workspace, whatever the operator
@@ -377,8 +379,55 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     return c;
 }
 
+// Launch shape of the streaming pair rows_scan_kernel + rows_pick_kernel: 256 threads,
+// V 128-bit loads per thread, G chunks per row; blocks = 256-byte blocks per row.
+struct ScanCfg {
+    bool ok = false;
+    int v = 0;
+    uint32_t g = 0, blocks = 0;
+};
+
+// Long last-axis rows, largest first, k up to kFastMaxK: the scan + pick pair.  The
+// largest chunk that still leaves 512 workgroups (else the smallest); rows too short
+// to be split, or with fewer than 4 (k + 1) blocks, or with more blocks than the pick
+// kernel takes in (16 per thread), are left to the other kernels.
+// (for_size: what a call could use whatever the tuning knobs say at that time)
+ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) {
+    ScanCfg c;
+    if (v.g.inner != 1 || k > vkop::kFastMaxK || v.g.n == 0 || v.g.outer == 0) return c;
+    if (!for_size) {
+        if (g_rows_path.load() == 1) return c;
+        // a forced shape of the other streaming kernels
+        if (g_rows_threads.load() > 0 && g_rows_loads.load() > 0 && g_rows_chunks.load() > 0) return c;
+    }
+    const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
+    const uint32_t n = v.g.n, rows = v.g.outer;
+    const uint32_t blocks = (n + vkop::kBlockLanes * vec - 1) / (vkop::kBlockLanes * vec);
+    if (blocks < 4u * (static_cast<uint32_t>(k) + 1u)) return c;
+    if ((blocks + vkop::kPickThreads - 1) / vkop::kPickThreads > 16u) return c;
+    const int vmax = dtype == VKOP_HIP_F32 ? 16 : 8;
+    int pick = 0;
+    for (int vv = 2; vv <= vmax; vv *= 2) {
+        const uint32_t per = static_cast<uint32_t>(vkop::kScanThreads) * vv * vec;
+        const uint32_t g = (n + per - 1) / per;
+        if (g < 2 || g * vkop::kScanWaves > static_cast<uint32_t>(vkop::kMergeWavesMax)) continue;
+        if (static_cast<uint64_t>(rows) * g >= (1ull << 31)) continue;
+        if (pick == 0) pick = vv;
+        if (static_cast<uint64_t>(rows) * g >= 512) pick = vv;
+    }
+    if (pick == 0) return c;
+    c.v = pick;
+    const uint32_t per = static_cast<uint32_t>(vkop::kScanThreads) * pick * vec;
+    c.g = (n + per - 1) / per;
+    c.blocks = blocks;
+    c.ok = true;
+    return c;
+}
+
 struct RowsLayout {
     size_t tickets = 0, sums = 0, cand = 0, stats = 0, total = 0;
+    // scan + pick pair (kernels_stream.hpp)
+    size_t bmax = 0, recs = 0;
     // multi-workgroup radix select (kernels_bigk.hpp)
     size_t hist = 0, hist_bytes = 0, state = 0, counts = 0, sel = 0, chunkstats = 0;
 };
@@ -406,7 +455,7 @@ BigKCfg choose_bigk_cfg(const View &v, int k, int dtype) {
 // the size does not depend on which of them a call ends up taking.
 // (the arrival counters come first, see kTicketRows)
 
-RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKCfg{}) {
+RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKCfg{}, const ScanCfg &sc = ScanCfg{}) {
     RowsLayout l;
     const size_t lines = static_cast<size_t>(v.g.outer) * v.g.inner;
     size_t off = 0;
@@ -414,7 +463,12 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
     off += kTicketBytes;
     l.stats = off;
     off += align_up(lines * sizeof(vkop::LineStats));
-    if (c.ok) {
+    if (sc.ok) {
+        l.bmax = off;
+        off += align_up(lines * sc.blocks * sizeof(uint32_t));
+        l.recs = off;
+        off += align_up(lines * sc.g * vkop::kScanWaves * 2 * sizeof(uint64_t));
+    } else if (c.ok) {
         const size_t chunks = lines * c.g;
         l.sums = off;
         off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * 3 * sizeof(uint64_t));
@@ -481,6 +535,31 @@ int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, 
 }
 
 template <typename T, bool SOFTMAX>
+int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, const ScanCfg &c, void *ws,
+                const RowsLayout &l, hipStream_t st) {
+    auto *base = static_cast<unsigned char *>(ws);
+    const uint32_t vec = 16 / sizeof(T);
+    vkop::ScanLaunch a;
+    a.in = in;
+    a.values = values;
+    a.indices = indices;
+    a.rows = v.g.outer;
+    a.n = v.g.n;
+    a.k = static_cast<uint32_t>(k);
+    a.v = static_cast<uint32_t>(c.v);
+    a.g = c.g;
+    a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
+    a.stages = g_rows_stages.load();
+    a.ws.bmax = reinterpret_cast<uint32_t *>(base + l.bmax);
+    a.ws.recs = reinterpret_cast<uint64_t *>(base + l.recs);
+    a.ws.blocks = c.blocks;
+    a.stream = st;
+    if (!vkop::launch_rows_scan<T, SOFTMAX>(a))
+        return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_scan_kernel / rows_pick_kernel for %d loads, %u blocks", c.v, c.blocks);
+    return launched("rows_scan_kernel / rows_pick_kernel");
+}
+
+template <typename T, bool SOFTMAX>
 int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, const RowsCfg &c, void *ws,
                 const RowsLayout &l, hipStream_t st) {
     vkop::RowsWorkspace w;
@@ -528,14 +607,16 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
 template <typename T>
 int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int dtype, void *ws,
               size_t ws_bytes, hipStream_t st) {
-    const RowsCfg c = largest ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
-    const BigKCfg b = c.ok ? BigKCfg{} : choose_bigk_cfg(v, k, dtype);
-    if (c.ok || b.ok) {
-        const RowsLayout l = rows_layout(v, c, b);
+    const ScanCfg sc = largest ? choose_scan_cfg(v, k, dtype) : ScanCfg{};
+    const RowsCfg c = (largest && !sc.ok) ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
+    const BigKCfg b = (c.ok || sc.ok) ? BigKCfg{} : choose_bigk_cfg(v, k, dtype);
+    if (sc.ok || c.ok || b.ok) {
+        const RowsLayout l = rows_layout(v, c, b, sc);
         if (ws == nullptr || ws_bytes < l.total)
             return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, l.total);
         if ((reinterpret_cast<uintptr_t>(ws) & (kAlign - 1)) != 0)
             return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
+        if (sc.ok) return launch_scan<T, false>(in, values, indices, v, k, sc, ws, l, st);
         if (c.ok) return launch_rows<T, false>(in, values, indices, v, k, c, ws, l, st);
         return launch_bigk<T, false>(in, values, indices, v, k, largest, b, ws, l, st);
     }
@@ -552,14 +633,16 @@ int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, in
 // ------------------------------------------------------------------ fused ----
 // Which route a fused call takes; the workspace size follows from it.
 struct FusedPlan {
+    ScanCfg scan;
     RowsCfg rows;
     BigKCfg big;
 };
 FusedPlan plan_fused(const View &v, int k, int dtype, int largest, bool want_probs) {
     FusedPlan p;
     if (want_probs) return p;  // the softmax tensor is written by the general kernels
-    if (largest) p.rows = choose_rows_cfg(v, k, dtype);
-    if (!p.rows.ok) p.big = choose_bigk_cfg(v, k, dtype);
+    if (largest) p.scan = choose_scan_cfg(v, k, dtype);
+    if (largest && !p.scan.ok) p.rows = choose_rows_cfg(v, k, dtype);
+    if (!p.scan.ok && !p.rows.ok) p.big = choose_bigk_cfg(v, k, dtype);
     return p;
 }
 
@@ -567,7 +650,8 @@ template <typename T>
 int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, int dtype,
                void *ws, hipStream_t st) {
     const FusedPlan p = plan_fused(v, k, dtype, largest, probs != nullptr);
-    const RowsLayout l = rows_layout(v, p.rows, p.big);
+    const RowsLayout l = rows_layout(v, p.rows, p.big, p.scan);
+    if (p.scan.ok) return launch_scan<T, true>(in, values, indices, v, k, p.scan, ws, l, st);
     if (p.rows.ok) return launch_rows<T, true>(in, values, indices, v, k, p.rows, ws, l, st);
     if (p.big.ok) return launch_bigk<T, true>(in, values, indices, v, k, largest, p.big, ws, l, st);
     // general path: line statistics (and the softmax tensor when asked for), then
@@ -586,7 +670,8 @@ int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v
 size_t selection_workspace(const View &v, int k, int dtype) {
     const size_t a = rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
     const size_t b = rows_layout(v, RowsCfg{}, choose_bigk_cfg(v, k, dtype)).total;
-    return a > b ? a : b;
+    const size_t c = rows_layout(v, RowsCfg{}, BigKCfg{}, choose_scan_cfg(v, k, dtype, true)).total;
+    return a > b ? (a > c ? a : c) : (b > c ? b : c);
 }
 
 // max over `axis` of the softmax along `axis`, without the softmax tensor
@@ -898,7 +983,7 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     if (in == nullptr || out_values == nullptr || out_indices == nullptr)
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
     const FusedPlan plan = plan_fused(v, k, dtype, largest, out_probs != nullptr);
-    const size_t need = rows_layout(v, plan.rows, plan.big).total;
+    const size_t need = rows_layout(v, plan.rows, plan.big, plan.scan).total;
     if (workspace == nullptr || workspace_bytes < need)
         return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
@@ -923,7 +1008,7 @@ int vkop_hip_softmax_topk_static(const void *in, void *out_values, int32_t *out_
     if (in == nullptr || out_values == nullptr || out_indices == nullptr)
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
     const FusedPlan plan = plan_fused(v, k, dtype, largest, false);
-    const size_t need = rows_layout(v, plan.rows, plan.big).total;
+    const size_t need = rows_layout(v, plan.rows, plan.big, plan.scan).total;
     if (need > static_cast<size_t>(VKOP_HIP_STATIC_SCRATCH_BYTES))
         return fail(VKOP_HIP_ERR_WORKSPACE,
                     "this tensor needs %zu bytes of scratch, the static array holds %zu: use vkop_hip_softmax_topk with a workspace",
@@ -987,15 +1072,22 @@ int vkop_hip_tune(const char *name, int value) {
     else if (std::strcmp(name, "rows.loads") == 0) g_rows_loads = value;
     else if (std::strcmp(name, "rows.chunks") == 0) g_rows_chunks = value;
     else if (std::strcmp(name, "rows.fused") == 0) g_rows_fused = value != 0;
+    else if (std::strcmp(name, "rows.path") == 0) {
+        if (value != 0 && value != 1) return fail(VKOP_HIP_ERR_INVALID, "rows.path must be 0 or 1");
+        g_rows_path = value;
+    }
     else if (std::strcmp(name, "nms.threads") == 0) {
         if (value != 0 && value != vkop::kNmsThreadsNarrow && value != vkop::kNmsThreadsWide)
             return fail(VKOP_HIP_ERR_INVALID, "nms.threads must be 0, %d or %d", vkop::kNmsThreadsNarrow, vkop::kNmsThreadsWide);
         g_nms_threads = value;
     }
-    else if (std::strcmp(name, "rows.stages") == 0) {
-        if (value < 1 || value > 3) return fail(VKOP_HIP_ERR_INVALID, "rows.stages must be 1, 2 or 3");
-        g_rows_stages = value;
-    } else return fail(VKOP_HIP_ERR_INVALID, "unknown tuning name '%s'", name);
+    else return fail(VKOP_HIP_ERR_INVALID, "unknown tuning name '%s'", name);
+    return VKOP_HIP_OK;
+}
+
+int vkop_hip_measure_stages(int stages) {
+    if (stages < 1 || stages > 3) return fail(VKOP_HIP_ERR_INVALID, "stages must be 1, 2 or 3");
+    g_rows_stages = stages;
     return VKOP_HIP_OK;
 }
 
@@ -1004,6 +1096,13 @@ int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k, i
     View v;
     if (int rc = check_dtype(dtype)) return rc;
     if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    const ScanCfg sc = k >= 1 ? choose_scan_cfg(v, k, dtype) : ScanCfg{};
+    if (sc.ok) {
+        if (threads != nullptr) *threads = vkop::kScanThreads;
+        if (loads != nullptr) *loads = sc.v;
+        if (chunks != nullptr) *chunks = static_cast<int>(sc.g);
+        return VKOP_HIP_OK;
+    }
     const RowsCfg c = k >= 1 ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
     if (threads != nullptr) *threads = c.ok ? c.nt : 0;
     if (loads != nullptr) *loads = c.ok ? c.v : 0;

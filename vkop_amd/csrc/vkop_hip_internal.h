@@ -1,0 +1,23 @@
+/*
+ * Measurement hooks of libvkop_hip.so that are NOT part of its public interface
+ * (include/vkop_hip.h): exported for this repository's benchmarks only.
+ */
+#ifndef VKOP_HIP_INTERNAL_H_
+#define VKOP_HIP_INTERNAL_H_
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Which kernels of a two-kernel streaming call are launched from now on, in every
+ * thread of the process: 3 = both (the state the library starts in), 1 = only the
+ * first, 2 = only the second (it reads the workspace an earlier whole call left).
+ * With 1 or 2 the top-k and fused entry points do NOT produce valid results: the
+ * settings exist so that a benchmark can time each kernel by itself with the
+ * launches a real call makes.  Not thread-safe; set it back to 3. */
+int vkop_hip_measure_stages(int stages);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VKOP_HIP_INTERNAL_H_ */
