@@ -7,7 +7,22 @@ A step is one call of the fused entry point (vkop_hip_softmax_topk, through the 
 ABI) over one batch of synthetic logits already resident in HBM.  The default
 workload is the one the metric is quoted on: [64,128256] float32, k = 50.  The
 batches rotate over enough distinct device buffers (> 256 MB in total) that the
-Infinity Cache cannot serve the reads.  Prints ONE JSON line.
+Infinity Cache cannot serve the reads; the figure with one buffer (cache
+resident) is reported beside it.  Prints ONE JSON line.
+
+How the K steps are timed.  Step i runs on lane i % L (L independent calls in
+flight, each lane with its own stream, workspace and outputs); every lane's
+share of the K steps is recorded once (a HIP graph) and the recordings are
+replayed: W warm-up steps, then the K-step recordings once untimed (their first
+launch uploads them), then timed: back to back until at least 400 steps are in
+the timed region (one replay of 20 steps on 4 lanes is five calls a lane that
+all start in the same phase: a pipeline filling, not running), lanes running
+free.  The timed replays are enqueued behind a spin kernel on the launch
+stream, so that all lanes are queued before the first of them starts and the
+host's submission time is not inside the timed region; HIP events on that
+stream bracket the region, with a device synchronize on both sides.  The host
+wall clock of the same replays without the gate is reported as well
+(`host_wall_ms_per_step`).
 
 The CPU baseline leg times, on the host cores of the same machine, the CPU
 oracle (test infrastructure, used here only as the thing being timed against)
@@ -17,6 +32,7 @@ treat as truth.
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -25,28 +41,25 @@ sys.path.insert(0, ROOT)
 
 # Four calls in flight need four hardware queues of their own; with four queues
 # per process (HIP's default, and what this pool exports) two of the streams end
-# up sharing one: 11.4 us per step measured instead of 7.3.  --hw-queues sets
-# GPU_MAX_HW_QUEUES for this process before the HIP runtime starts.
+# up sharing one.  --hw-queues sets GPU_MAX_HW_QUEUES for this process before the
+# HIP runtime starts.  More than four calls in flight run slower on this part.
 DEFAULT_HW_QUEUES = 8
 
 HBM_PEAK_GBS = 8000.0   # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this script scaled by the same counters over a copy kernel
-# of known size (profiles/ holds the runs); None = not measured for the workload.
-TRAFFIC = {"C3": 34599831}   # rows_chunk_kernel: 33011902 B read + 1587929 B written
-
 WORKLOADS = {
-    # name: (description, generator kwargs, k, axis)
+    # name: (description, generator kwargs, k)
     "C1": ("[1,1000] f32 softmax+topk k=5", dict(kind="cls", rows=1, cols=1000), 5),
     "C2": ("[256,1000] f32 softmax+topk k=5", dict(kind="cls", rows=256, cols=1000), 5),
     "C3": ("[64,128256] f32 softmax+topk k=50", dict(kind="llm", rows=64, cols=128256), 50),
     "C4": ("[8,262144] f32 softmax+topk k=1024", dict(kind="grid", rows=8, cols=262144), 1024),
     # a variant of C3, not one of the reference's configurations: its logits truncated to bfloat16 precision
-    # (what a bf16 LM head hands over);
-    # equal logits then straddle the k-th place in most rows and the merge settles a tie per row
+    # (what a bf16 LM head hands over); equal logits then straddle the k-th place in most rows
     "C3bf16": ("[64,128256] f32 softmax+topk k=50, bf16-valued logits", dict(kind="llm_bf16", rows=64, cols=128256), 50),
 }
+
+# kernels of a two-kernel streaming call, by the path the library takes (vkop_hip_measure_path)
+PATH_KERNELS = {1: ("rows_chunk_kernel", "rows_merge_kernel"), 2: ("rows_scan_kernel", "rows_pick_kernel")}
 
 
 def make_input(spec, seed):
@@ -62,9 +75,31 @@ def make_input(spec, seed):
     return synth.grid_values(spec["rows"], spec["cols"], seed)
 
 
-def cpu_baseline(x, k, budget_s=12.0):
+def traffic_from_profiles(workload, kernel):
+    """HBM bytes per launch of `kernel`, from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE and WRITE_SIZE scaled by the same counters over a copy of known size);
+    None if profiles/ holds no such line."""
+    path = os.path.join(ROOT, "profiles", "softmax_topk_%s_hbm_traffic.txt" % workload)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"^%s: read (\d+) B \+ written (\d+) B = (\d+) B of HBM traffic per launch" % re.escape(kernel), text, re.M)
+    return int(m.group(3)) if m else None
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(x, k, budget_s=14.0):
     """Times the CPU side on a bounded sample of the same workload."""
-    import numpy as np
     import torch
 
     import oracle
@@ -74,35 +109,43 @@ def cpu_baseline(x, k, budget_s=12.0):
     t0 = time.perf_counter()
     _, _, used = oracle.softmax_topk_mt(x, k, threads=cores)
     once = time.perf_counter() - t0
-    reps = max(1, min(50, int(budget_s / 2 / max(once, 1e-6))))
+    reps = max(1, min(50, int(budget_s / 3 / max(once, 1e-6))))
     t0 = time.perf_counter()
     for _ in range(reps):
         oracle.softmax_topk_mt(x, k, threads=cores)
     t_oracle = (time.perf_counter() - t0) / reps
-    # libtorch CPU: at::softmax + at::topk, the reference tests' expectation source
-    torch.set_num_threads(cores)
+    # libtorch CPU: at::softmax + at::topk, the reference tests' expectation source,
+    # on all host threads and on one
     xt = torch.from_numpy(x)
-    for _ in range(2):
-        torch.topk(torch.softmax(xt, -1), k, -1, True, True)
-    t0 = time.perf_counter()
-    n = 0
-    while time.perf_counter() - t0 < budget_s / 2 and n < 200:
-        torch.topk(torch.softmax(xt, -1), k, -1, True, True)
-        n += 1
-    t_torch = (time.perf_counter() - t0) / max(n, 1)
+
+    def time_torch(threads, budget):
+        torch.set_num_threads(threads)
+        for _ in range(2):
+            torch.topk(torch.softmax(xt, -1), k, -1, True, True)
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < budget and n < 200:
+            torch.topk(torch.softmax(xt, -1), k, -1, True, True)
+            n += 1
+        return (time.perf_counter() - t0) / max(n, 1), n, torch.get_num_threads()
+    t_torch, n_torch, thr_torch = time_torch(cores, budget_s / 3)
+    t_torch1, n_torch1, _ = time_torch(1, budget_s / 4)
+    torch.set_num_threads(cores)
     # the reference's own CPU post-processing, restated: one row at a time, one thread (core/function.cpp:150-183)
     sample = min(rows, 8)
     t0 = time.perf_counter()
     for r in range(sample):
         oracle.get_top_k_predictions(x[r], k)
     t_post = (time.perf_counter() - t0) / sample
+    what = ("torch.topk(torch.softmax(x,-1),k) on the host, as tests/SoftmaxTest.cpp:138 and tests/TopkTest.cpp:73 "
+            "compute expectations")
     return {
         "value": rows / t_oracle, "unit": "rows/s", "cores": int(used), "kind": "port",
         "sample": "whole %dx%d batch, %d repeats of the C oracle (OpenMP over rows)" % (x.shape[0], x.shape[1], reps),
-        "libtorch_cpu": {"value": rows / t_torch, "unit": "rows/s", "threads": torch.get_num_threads(),
-                         "version": torch.__version__, "repeats": n,
-                         "what": "torch.topk(torch.softmax(x,-1),k) on the host, as tests/SoftmaxTest.cpp:138 and "
-                                 "tests/TopkTest.cpp:73 compute expectations"},
+        "cpu_model": cpu_model(), "host_threads": cores,
+        "libtorch_cpu": {"value": rows / t_torch, "unit": "rows/s", "threads": thr_torch, "version": torch.__version__,
+                         "cpu_capability": torch.backends.cpu.get_cpu_capability(), "repeats": n_torch, "what": what},
+        "libtorch_cpu_1_thread": {"value": rows / t_torch1, "unit": "rows/s", "threads": 1, "repeats": n_torch1},
         "reference_cpu_postproc": {"value": 1.0 / t_post, "unit": "rows/s", "cores": 1, "rows_timed": sample,
                                    "what": "Function::get_top_k_predictions restated (core/function.cpp:150-183): softmax of "
                                            "one row, full sort by probability, first k; the CPU code the GPU path replaces"},
@@ -123,25 +166,28 @@ def copy_calibration(nbytes=256 << 20, launches=20):
                       "launches": launches, "kernel": "__amd_rocclr_copyBuffer, the runtime's device copy kernel behind dst.copy_(src)"}))
 
 
+def ulps(a, b):
+    import numpy as np
+    ia = a.view(np.int32).astype(np.int64)
+    ib = b.view(np.int32).astype(np.int64)
+    return np.abs(ia - ib)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-host", action="store_true", help="skip the host-buffer (PCIe) round-trip leg")
-    ap.add_argument("--resident", action="store_true", help="reuse one input buffer (Infinity-Cache resident figure)")
     ap.add_argument("--hw-queues", type=int, default=DEFAULT_HW_QUEUES,
                     help="hardware queues this process may use (GPU_MAX_HW_QUEUES); 0 = leave the environment as it is")
     ap.add_argument("--inflight", type=int, default=0,
                     help="independent calls in flight (each on its own stream with its own workspace and outputs)")
-    ap.add_argument("--launch-shape", default="",
-                    help="threads,loads,chunks for the streaming kernel instead of the library's choice (experiments)")
-    ap.add_argument("--fused", action="store_true",
-                    help="run the streaming path as one kernel (the last chunk of a row merges it) instead of two")
-    ap.add_argument("--eager", action="store_true",
-                    help="issue every call from the host loop instead of replaying a recording of the K calls")
+    ap.add_argument("--rows-path", type=int, default=0, choices=(0, 1),
+                    help="0 = the library's choice of streaming kernels, 1 = the chunk + merge kernels (vkop_hip_tune rows.path)")
+    ap.add_argument("--no-gate", action="store_true", help="do not hold the timed replay behind a spin kernel")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of known size (the yardstick for the FETCH_SIZE / "
                          "WRITE_SIZE counters) and print its size")
@@ -167,22 +213,16 @@ def main():
 
     capi.lib()
     capi.init(0)
-    capi.tune("rows.fused", 1 if args.fused else 0)
-    if args.launch_shape:
-        for name, value in zip(("rows.threads", "rows.loads", "rows.chunks"), args.launch_shape.split(",")):
-            capi.tune(name, int(value))
+    capi.tune("rows.path", args.rows_path)
     desc, spec, k = WORKLOADS[args.workload]
     rows, cols = spec["rows"], spec["cols"]
     shape = (rows, cols)
     in_bytes = rows * cols * 4
     algo_bytes = in_bytes + rows * k * 8
-    nbuf = 1 if args.resident else max(2, -(-(288 << 20) // in_bytes))
-    nbuf = min(nbuf, 64)
+    nbuf = min(64, max(2, -(-(288 << 20) // in_bytes)))
     seed0 = synth.SEEDS.get(args.workload[:2], 1)
     host_inputs = [make_input(spec, seed0 + 7919 * b) for b in range(min(nbuf, 3))]
-    bufs = []
-    for b in range(nbuf):
-        bufs.append(torch.from_numpy(host_inputs[b % len(host_inputs)]).cuda())
+    bufs = [torch.from_numpy(host_inputs[b % len(host_inputs)]).cuda() for b in range(nbuf)]
     # One "lane" per call in flight: its own stream, workspace and outputs, like the
     # reference's kInflight = 2 queues (core/runtime.cpp:408-446).  Step i runs on
     # lane i % L; steps on one lane are serialized, lanes overlap.
@@ -199,26 +239,32 @@ def main():
         capi.stream_sync(ln["stream"])
     torch.cuda.synchronize()
     main_stream = lanes[0]["stream"]
+    torch_main = torch.cuda.ExternalStream(main_stream)
 
-    def step(i, nlanes):
-        ln = lanes[i % nlanes]
-        capi.softmax_topk(bufs[i % nbuf].data_ptr(), 0, ln["vals"].data_ptr(), ln["idx"].data_ptr(), capi.F32, shape,
-                          -1, k, 1, ln["ws_ptr"], ws_bytes, ln["stream"])
+    def call(buf, ln):
+        capi.softmax_topk(buf.data_ptr(), 0, ln["vals"].data_ptr(), ln["idx"].data_ptr(), capi.F32, shape, -1, k, 1,
+                          ln["ws_ptr"], ws_bytes, ln["stream"])
 
-    # parity of what is about to be timed, on every lane
+    # parity of what is about to be timed, on every lane: against the oracle (the bar)
+    # and against libtorch's CPU result on the same tensor (reported)
     parity = {"indices_exact": True, "max_ulp_vs_oracle": 0}
     ov, oix = oracle.softmax_topk(host_inputs[0], k)
-    for j, ln in enumerate(lanes):
-        capi.softmax_topk(bufs[0].data_ptr(), 0, ln["vals"].data_ptr(), ln["idx"].data_ptr(), capi.F32, shape, -1, k, 1,
-                          ln["ws_ptr"], ws_bytes, ln["stream"])
+    for ln in lanes:
+        call(bufs[0], ln)
         capi.stream_sync(ln["stream"])
         gi, gv = ln["idx"].cpu().numpy(), ln["vals"].cpu().numpy()
-        ulp = int(np.abs(gv.view(np.int32).astype(np.int64) - ov.view(np.int32).astype(np.int64)).max())
         parity["indices_exact"] = parity["indices_exact"] and bool(np.array_equal(gi, oix))
-        parity["max_ulp_vs_oracle"] = max(parity["max_ulp_vs_oracle"], ulp)
+        parity["max_ulp_vs_oracle"] = max(parity["max_ulp_vs_oracle"], int(ulps(gv, ov).max()))
     if not parity["indices_exact"] or parity["max_ulp_vs_oracle"] > 2:
         print("bench.py: parity check failed: %s" % parity, file=sys.stderr)
         sys.exit(1)
+    tv, ti = torch.topk(torch.softmax(torch.from_numpy(host_inputs[0]), -1), k, -1, True, True)
+    same = ti.numpy().astype(np.int32) == gi
+    d = ulps(gv, tv.numpy())[same]
+    parity["vs_libtorch_cpu"] = {"indices_equal_fraction": float(same.mean()),
+                                 "max_ulp": int(d.max()) if d.size else None, "mean_ulp": float(d.mean()) if d.size else None,
+                                 "what": "values at the places where libtorch's index agrees; libtorch sums a long row in "
+                                         "ISA-dependent float lanes and is itself several ulp from the exact sum"}
 
     def fork(nlanes):
         """The other lanes' streams start after everything already on the main stream."""
@@ -237,14 +283,14 @@ def main():
     # side, the way the reference records each operator into a command buffer and
     # Runtime::Run submits one batch per queue (core/runtime.cpp:404-458); a host
     # loop of ~10 us Python calls could not keep a ~10 us kernel fed.
-    def record(count, first, nlanes):
+    def record(count, first, nlanes, nb):
         """One recording per lane: the lane's share of steps first .. first+count-1, in order."""
         graphs = []
         for j in range(nlanes):
             capi.graph_begin(lanes[j]["stream"])
             for i in range(first, first + count):
                 if i % nlanes == j:
-                    step(i, nlanes)
+                    call(bufs[i % nb], lanes[j])
             graphs.append(capi.graph_end(lanes[j]["stream"]))
         return graphs
 
@@ -256,80 +302,134 @@ def main():
 
     e0, e1 = capi.event_create(), capi.event_create()
 
-    def timed(stages, nlanes):
-        """(device ms, host wall ms) of K steps after W warm-up steps, HIP events on the main stream."""
+    # spin kernel that holds the timed replay back until every lane is queued: sized
+    # from a measurement of its own rate to about 2 ms (the host needs a few hundred
+    # microseconds to queue the lanes from Python)
+    gate_cycles, gate_ms = 0, 0.0
+    if not args.no_gate and hasattr(torch.cuda, "_sleep"):
+        probe = 1000000
+        with torch.cuda.stream(torch_main):
+            torch.cuda._sleep(probe)
+            capi.event_record(e0, main_stream)
+            torch.cuda._sleep(probe)
+            capi.event_record(e1, main_stream)
+        capi.event_sync(e1)
+        per_cycle_ms = max(capi.event_elapsed_ms(e0, e1), 1e-6) / probe
+        gate_ms = 4.0
+        gate_cycles = int(gate_ms / per_cycle_ms)
+
+    def gate():
+        if gate_cycles:
+            with torch.cuda.stream(torch_main):
+                torch.cuda._sleep(gate_cycles)
+
+    # The K-step recordings are replayed back to back until at least MIN_TIMED steps are
+    # inside the timed region, lanes running free (no join between replays): with 20
+    # steps and 4 lanes a single replay is five calls a lane, all lanes starting in the
+    # same phase, which is the pipeline filling, not running.
+    MIN_TIMED = 400
+    replays = max(1, -(-MIN_TIMED // args.steps))
+
+    def timed(stages, nlanes, nb=nbuf, prime=False):
+        """(device ms per step, host wall ms per step of ungated replays) after W warm-up steps."""
+        capi.measure_stages(3)
+        if prime:   # leave in every lane's workspace what a whole call on the (single) buffer leaves
+            for ln in lanes[:nlanes]:
+                call(bufs[0], ln)
+                capi.stream_sync(ln["stream"])
         capi.measure_stages(stages)
         graphs = []
-        if args.eager:
+        if args.warmup > 0:
+            gw = record(args.warmup, 0, nlanes, nb)
+            graphs += gw
+            submit(gw, nlanes)
+        gk = record(args.steps, args.warmup, nlanes, nb)
+        graphs += gk
+
+        def replay_all():
             fork(nlanes)
-            for i in range(args.warmup):
-                step(i, nlanes)
+            for _ in range(replays):
+                for j in range(nlanes):
+                    capi.graph_launch(gk[j], lanes[j]["stream"])
             join(nlanes)
-        else:
-            if args.warmup > 0:
-                gw = record(args.warmup, 0, nlanes)
-                graphs += gw
-                submit(gw, nlanes)
-            gk = record(args.steps, args.warmup, nlanes)
-            graphs += gk
+        # the recordings that are timed, once untimed: their first launch is not what is measured
         capi.stream_sync(main_stream)
         torch.cuda.synchronize()
+        submit(gk, nlanes)
+        capi.stream_sync(main_stream)
+        torch.cuda.synchronize()
+        # host wall clock of the same replays without the gate (submission time included)
         t0 = time.perf_counter()
-        capi.event_record(e0, main_stream)
-        if args.eager:
-            fork(nlanes)
-            for i in range(args.steps):
-                step(args.warmup + i, nlanes)
-            join(nlanes)
-        else:
-            submit(gk, nlanes)
-        capi.event_record(e1, main_stream)
-        capi.event_sync(e1)
+        replay_all()
+        capi.stream_sync(main_stream)
         wall = (time.perf_counter() - t0) * 1e3
+        torch.cuda.synchronize()
+        # the timed replays: queued behind the gate, HIP events on the launch stream
+        t0 = time.perf_counter()
+        gate()
+        capi.event_record(e0, main_stream)
+        replay_all()
+        capi.event_record(e1, main_stream)
+        queued_ms = (time.perf_counter() - t0) * 1e3
+        if gate_cycles and queued_ms > gate_ms:
+            print("bench.py: queueing the lanes took %.2f ms, longer than the %.1f ms gate: the timed region "
+                  "includes host submission time" % (queued_ms, gate_ms), file=sys.stderr)
+        capi.event_sync(e1)
         torch.cuda.synchronize()
         for g in graphs:
             capi.graph_destroy(g)
         capi.measure_stages(3)
-        return max(capi.event_elapsed_ms(e0, e1), 0.0), wall
+        n = replays * args.steps
+        return max(capi.event_elapsed_ms(e0, e1), 0.0) / n, wall / n
 
-    # each kernel of the path by itself (same launches, same inputs, the other
-    # kernel left out), then the whole step, which is the figure reported
+    # each kernel of the path by itself (same launches, same inputs, the other kernel
+    # left out), then the whole step, which is the figure reported
     stage_ms = {}
     stage_overlapped = None
     plan = capi.rows_plan(capi.F32, shape, -1, k)
-    two_kernels = plan[2] > 1 and not args.fused
+    path = capi.measure_path(capi.F32, shape, -1, k)
+    names = PATH_KERNELS.get(path)
+    two_kernels = names is not None and plan[2] > 1
+    serial_ms = timed(3, 1)[0]
     if two_kernels:
-        # one call in flight; the merge-only run reads the workspace the whole-step run left
-        serial_ms = timed(3, 1)[0] / args.steps
-        stage_ms["rows_chunk_kernel"] = timed(1, 1)[0] / args.steps
-        stage_ms["rows_merge_kernel"] = timed(2, 1)[0] / args.steps
+        # one call in flight.  The second kernel by itself reads the workspace an earlier whole call
+        # left; the pick kernel also reads the input again, so it is timed on one buffer with
+        # that buffer's workspace (its few re-reads then come from the cache)
+        stage_ms[names[0]] = timed(1, 1)[0]
+        stage_ms[names[1]] = timed(2, 1, 1, True)[0] if path == 2 else timed(2, 1)[0]
         if len(lanes) > 1:
-            stage_overlapped = {"rows_chunk_kernel": timed(1, len(lanes))[0] / args.steps * 1e3,
-                                "rows_merge_kernel": timed(2, len(lanes))[0] / args.steps * 1e3}
-    else:
-        serial_ms = timed(3, 1)[0] / args.steps
-    dev_ms, wall_ms = timed(3, len(lanes))
-    ms_per_step = dev_ms / args.steps
-    wall_per_step = wall_ms / args.steps
-    dominant = max(stage_ms, key=stage_ms.get) if stage_ms else "rows_chunk_kernel (the step's only kernel)"
-    dom_ms = stage_ms.get(dominant, ms_per_step)
+            stage_overlapped = {names[0]: timed(1, len(lanes))[0] * 1e3,
+                                names[1]: (timed(2, len(lanes), 1, True)[0] if path == 2 else timed(2, len(lanes))[0]) * 1e3}
+    ms_per_step, wall_per_step = timed(3, len(lanes))
+    resident_ms = timed(3, len(lanes), 1)[0]
+    # the kernel that moves the bytes (the first of the pair; the second reads a few kilobytes per row)
+    dominant = names[0] if two_kernels else "the step's only kernel"
+    dom_ms = stage_ms.get(dominant, serial_ms)
 
     achieved = algo_bytes / (dom_ms * 1e-3) / 1e9
     out = {
         "metric": "softmax+topk rows/s and % HBM roofline at [64,128256] fp32, k=50" if args.workload == "C3"
         else "softmax+topk rows/s, " + desc,
-        "value": rows / (wall_per_step * 1e-3),
+        "value": rows / (ms_per_step * 1e-3),
         "unit": "rows/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": wall_per_step,
+        "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": desc, "k": k, "calls_in_flight": len(lanes), "hw_queues": hw_queues, "kernels_per_call": 2 if two_kernels else 1, "input_buffers_rotated": nbuf,
-                   "input_set_bytes": nbuf * in_bytes, "device": capi.device_info()[0],
-                   "launch_shape": {"threads": plan[0], "loads_per_thread": plan[1], "chunks_per_row": plan[2]}},
-        "device_ms_per_step": ms_per_step,
+        "config": {"workload": desc, "k": k, "calls_in_flight": len(lanes), "hw_queues": hw_queues,
+                   "kernels_per_call": 2 if two_kernels else 1, "kernels": list(names) if two_kernels else None,
+                   "input_buffers_rotated": nbuf, "input_set_bytes": nbuf * in_bytes, "device": capi.device_info()[0],
+                   "launch_shape": {"threads": plan[0], "loads_per_thread": plan[1], "chunks_per_row": plan[2]},
+                   "timing": "HIP events on the launch stream around back-to-back replays of the recorded K steps (at least "
+                             "400 steps in all, lanes running free), queued behind a spin kernel (%s); W warm-up steps and "
+                             "one untimed replay of the same recordings before them"
+                             % ("%.1f ms" % gate_ms if gate_cycles else "off")},
+        "steps_in_timed_region": replays * args.steps,
+        "host_wall_ms_per_step": wall_per_step,
+        "cache_resident_ms_per_step": resident_ms,
+        "cache_resident_rows_per_s": rows / (resident_ms * 1e-3),
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": TRAFFIC.get(args.workload),
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic_from_profiles(args.workload, dominant),
                      "kernel": dominant,
                      "algorithmic_bytes_per_launch": algo_bytes,
                      "launch_us": dom_ms * 1e3,
@@ -338,9 +438,9 @@ def main():
                      "whole_step_us": ms_per_step * 1e3,
                      "whole_step_frac": algo_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "whole_step_us_one_in_flight": serial_ms * 1e3,
+                     "whole_step_frac_one_in_flight": algo_bytes / (serial_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "timing": "HIP events on the launch stream around %d back-to-back launches of that kernel alone, one "
-                               "call in flight (%s); includes the gap between launches"
-                               % (args.steps, "host loop" if args.eager else "one recorded submission")},
+                               "call in flight (recorded submissions); includes the gap between launches" % (replays * args.steps)},
         "parity": parity,
     }
     # For a caller whose logits sit in host memory: upload over PCIe from pinned
@@ -357,8 +457,7 @@ def main():
 
         def host_round_trip():
             capi.memcpy_h2d(bufs[0].data_ptr(), pin_in.data_ptr(), in_bytes, ln["stream"])
-            capi.softmax_topk(bufs[0].data_ptr(), 0, ln["vals"].data_ptr(), ln["idx"].data_ptr(), capi.F32, shape, -1,
-                              k, 1, ln["ws_ptr"], ws_bytes, ln["stream"])
+            call(bufs[0], ln)
             capi.memcpy_d2h(pin_v.data_ptr(), ln["vals"].data_ptr(), rows * k * 4, ln["stream"])
             capi.memcpy_d2h(pin_i.data_ptr(), ln["idx"].data_ptr(), rows * k * 4, ln["stream"])
         host_round_trip()

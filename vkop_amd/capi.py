@@ -92,6 +92,7 @@ def lib():
         "vkop_hip_softmax_reduce_max": (i, [vp, vp, i, ip, i, i, vp, sz, vp]),
         "vkop_hip_tune": (i, [ctypes.c_char_p, i]),
         "vkop_hip_measure_stages": (i, [i]),
+        "vkop_hip_measure_path": (i, [i, ip, i, i, i]),
         "vkop_hip_rows_plan": (i, [i, ip, i, i, i, ip, ip, ip]),
     }
     for name, (res, args) in sig.items():
@@ -260,6 +261,12 @@ def measure_stages(stages):
     """Benchmarks only (vkop_amd/csrc/vkop_hip_internal.h): launch only the first (1) or second (2) kernel of a
     two-kernel streaming call, or both (3, the normal state).  Results are not valid with 1 or 2."""
     check(lib().vkop_hip_measure_stages(int(stages)))
+
+
+def measure_path(dtype, shape, axis, k):
+    """Benchmarks only: 2 = scan + pick kernels, 1 = chunk (+ merge) kernels, 0 = other kernels for this tensor."""
+    arr, nd = _shape(shape)
+    return lib().vkop_hip_measure_path(dtype, arr, nd, axis, int(k))
 
 
 def rows_plan(dtype, shape, axis, k):

@@ -1085,6 +1085,14 @@ int vkop_hip_tune(const char *name, int value) {
     return VKOP_HIP_OK;
 }
 
+int vkop_hip_measure_path(int dtype, const int *shape, int ndim, int axis, int k) {
+    View v;
+    if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return -1;
+    if (choose_scan_cfg(v, k, dtype).ok) return 2;
+    if (choose_rows_cfg(v, k, dtype).ok) return 1;
+    return 0;
+}
+
 int vkop_hip_measure_stages(int stages) {
     if (stages < 1 || stages > 3) return fail(VKOP_HIP_ERR_INVALID, "stages must be 1, 2 or 3");
     g_rows_stages = stages;

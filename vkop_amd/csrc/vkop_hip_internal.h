@@ -17,6 +17,12 @@ extern "C" {
  * launches a real call makes.  Not thread-safe; set it back to 3. */
 int vkop_hip_measure_stages(int stages);
 
+/* Which streaming kernels a fused / top-k (largest) call on this tensor would run
+ * with the current tuning settings: 2 = rows_scan_kernel + rows_pick_kernel, 1 =
+ * rows_chunk_kernel (+ rows_merge_kernel when a row is split), 0 = other kernels,
+ * -1 = bad arguments. */
+int vkop_hip_measure_path(int dtype, const int *shape, int ndim, int axis, int k);
+
 #ifdef __cplusplus
 }
 #endif
