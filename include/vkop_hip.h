@@ -126,6 +126,23 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
                           int ndim, int axis, int k, int largest,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* ---- Sampling-style variant of the fused post-proc (no counterpart in the
+ * reference; its TopK parses k, axis, largest and sorted, ops/Topk.hpp:62-79, and
+ * the benchmark scales nothing, benchmark/main.cpp:85-101).  Every logit is first
+ * multiplied by `scale` (1 / temperature; positive and finite) in single
+ * precision, x' = fl32(x * scale); out_values / out_indices are the fused
+ * softmax -> top-k, largest first, of x', to the bars of vkop_hip_softmax_topk
+ * on a tensor holding x' (bit for bit its result on long last-axis rows, where
+ * both run the same streaming kernels; to the same bar against an exact softmax elsewhere, where this entry
+ * point runs the one-workgroup-per-line kernels).  out_counts (int32 per
+ * row, may be NULL; last axis only) receives the nucleus cut of each row's
+ * result for top_p, the number vkop_hip_topp_count gives on out_values.
+ * Workspace: vkop_hip_softmax_topk_workspace_bytes(). */
+int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *out_indices,
+                                   int32_t *out_counts, int dtype, const int *shape, int ndim,
+                                   int axis, int k, float scale, float top_p, void *workspace,
+                                   size_t workspace_bytes, void *stream);
+
 /* ---- The fused post-proc for callers that cannot allocate device memory (work
  * recorded into a HIP graph, tight serving loops, harnesses that forbid
  * hipMalloc): vkop_hip_softmax_topk without out_probs and without a workspace

@@ -44,6 +44,9 @@ def lib():
             getattr(L, name).argtypes = [vp, vp, vp, vp, c_int, c_int, c_int, c_int, c_int]
         L.vkop_oracle_softmax_topk_f32_mt.restype = c_int
         L.vkop_oracle_softmax_topk_f32_mt.argtypes = [vp, vp, vp, c_int, c_int, c_int, c_int, c_int, c_int]
+        for name in ("vkop_oracle_softmax_topk_sampling_f32", "vkop_oracle_softmax_topk_sampling_f16"):
+            getattr(L, name).restype = None
+            getattr(L, name).argtypes = [vp, c_float, c_float, vp, vp, vp, c_int, c_int, c_int, c_int]
         L.vkop_oracle_reduce_max_f32.restype = None
         L.vkop_oracle_reduce_max_f32.argtypes = [vp, vp, c_int, c_int, c_int]
         L.vkop_oracle_get_top_k_predictions.restype = c_int
@@ -138,6 +141,28 @@ def softmax_topk(x, k, axis=-1, largest=True, return_probs=False):
         vals = vals.view(np.float16)
         probs = probs.view(np.float16) if probs is not None else None
     return (vals, idx, probs) if return_probs else (vals, idx)
+
+
+def softmax_topk_sampling(x, k, scale=1.0, top_p=None, axis=-1):
+    """Fused softmax -> top-k of fl32(x * scale); with top_p also the nucleus counts.
+    -> (values, indices) or (values, indices, counts)."""
+    a, half = _canon(x)
+    outer, n, inner, ax = _split(a.shape, axis)
+    if not 0 <= k <= n:
+        raise ValueError("k out of range")
+    oshape = list(a.shape)
+    oshape[ax] = k
+    vals = np.empty(oshape, dtype=a.dtype)
+    idx = np.empty(oshape, dtype=np.int32)
+    cshape = list(a.shape)
+    del cshape[ax]
+    counts = np.empty(cshape, dtype=np.int32) if top_p is not None else None
+    fn = lib().vkop_oracle_softmax_topk_sampling_f16 if half else lib().vkop_oracle_softmax_topk_sampling_f32
+    fn(_ptr(a), float(np.float32(scale)), float(np.float32(top_p if top_p is not None else 0.0)), _ptr(vals), _ptr(idx),
+       _ptr(counts), outer, n, inner, int(k))
+    if half:
+        vals = vals.view(np.float16)
+    return (vals, idx, counts) if top_p is not None else (vals, idx)
 
 
 def softmax_topk_mt(x, k, axis=-1, largest=True, threads=0):

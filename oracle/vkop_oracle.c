@@ -393,6 +393,95 @@ void vkop_oracle_softmax_topk_f16(const uint16_t *in, uint16_t *probs,
 }
 
 /* ------------------------------------------------------------------ */
+/* sampling-style variant of the fused post-proc                        */
+/* ------------------------------------------------------------------ */
+
+/* No counterpart in the reference (extensions on its softmax -> top-k path,
+ * benchmark/main.cpp:85-101; the attribute parsing they would hang on is
+ * ops/Topk.hpp:62-79): every logit is first multiplied by `scale` (1 /
+ * temperature) in single precision, x' = fl32(x * scale); the result is the
+ * fused softmax -> top-k (largest first) of x'; counts, when given, receives
+ * per line the nucleus cut of vkop_oracle_topp_count_f32 on that line's k
+ * sorted probabilities for top_p. */
+void vkop_oracle_softmax_topk_sampling_f32(const float *in, float scale,
+                                           float top_p, float *values,
+                                           int32_t *indices, int32_t *counts,
+                                           int outer, int n, int inner,
+                                           int k) {
+    if (outer <= 0 || n <= 0 || inner <= 0 || k <= 0)
+        return;
+    if (k > n)
+        k = n;
+    float *x = (float *)malloc(sizeof(float) * ((size_t)2 * n + 2 * (size_t)k));
+    float *y = x + n, *v = x + 2 * (size_t)n, *pv = v + k;
+    int32_t *ix = (int32_t *)malloc(sizeof(int32_t) * (size_t)k);
+    for (int o = 0; o < outer; o++)
+        for (int i = 0; i < inner; i++) {
+            size_t ibase = (size_t)o * n * inner + i;
+            size_t obase = (size_t)o * k * inner + i;
+            for (int j = 0; j < n; j++) {
+                volatile float t = in[ibase + (size_t)j * inner] * scale;
+                x[j] = t; /* (volatile: the product rounded to float) */
+            }
+            softmax_line(x, y, n);
+            topk_line(y, n, k, 1, v, ix);
+            for (int j = 0; j < k; j++) {
+                pv[j] = y[ix[j]];
+                values[obase + (size_t)j * inner] = pv[j];
+                indices[obase + (size_t)j * inner] = ix[j];
+            }
+            if (counts)
+                vkop_oracle_topp_count_f32(pv, 1, k, k, top_p,
+                                           counts + (size_t)o * inner + i);
+        }
+    free(x);
+    free(ix);
+}
+
+void vkop_oracle_softmax_topk_sampling_f16(const uint16_t *in, float scale,
+                                           float top_p, uint16_t *values,
+                                           int32_t *indices, int32_t *counts,
+                                           int outer, int n, int inner,
+                                           int k) {
+    if (outer <= 0 || n <= 0 || inner <= 0 || k <= 0)
+        return;
+    if (k > n)
+        k = n;
+    float *x = (float *)malloc(sizeof(float) * ((size_t)2 * n + 2 * (size_t)k));
+    float *y = x + n, *v = x + 2 * (size_t)n, *pv = v + k;
+    uint16_t *yh = (uint16_t *)malloc(sizeof(uint16_t) * (size_t)n);
+    int32_t *ix = (int32_t *)malloc(sizeof(int32_t) * (size_t)k);
+    for (int o = 0; o < outer; o++)
+        for (int i = 0; i < inner; i++) {
+            size_t ibase = (size_t)o * n * inner + i;
+            size_t obase = (size_t)o * k * inner + i;
+            for (int j = 0; j < n; j++) {
+                volatile float t =
+                    vkop_oracle_half_to_float(in[ibase + (size_t)j * inner]) * scale;
+                x[j] = t;
+            }
+            softmax_line(x, y, n);
+            /* the softmax operator stores halves; top-k sees those halves */
+            for (int j = 0; j < n; j++) {
+                yh[j] = vkop_oracle_float_to_half(y[j]);
+                y[j] = vkop_oracle_half_to_float(yh[j]);
+            }
+            topk_line(y, n, k, 1, v, ix);
+            for (int j = 0; j < k; j++) {
+                pv[j] = y[ix[j]];
+                values[obase + (size_t)j * inner] = yh[ix[j]];
+                indices[obase + (size_t)j * inner] = ix[j];
+            }
+            if (counts)
+                vkop_oracle_topp_count_f32(pv, 1, k, k, top_p,
+                                           counts + (size_t)o * inner + i);
+        }
+    free(x);
+    free(yh);
+    free(ix);
+}
+
+/* ------------------------------------------------------------------ */
 /* reduce max, CPU post-proc restatement                               */
 /* ------------------------------------------------------------------ */
 

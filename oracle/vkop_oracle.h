@@ -67,6 +67,21 @@ void vkop_oracle_softmax_topk_f16(const uint16_t *in, uint16_t *probs,
                                   int outer, int n, int inner, int k,
                                   int largest);
 
+/* Sampling-style variant (no counterpart in the reference; the attribute
+ * parsing such options would hang on is ops/Topk.hpp:62-79): every logit is
+ * first multiplied by `scale` (1 / temperature) in single precision, then the
+ * fused softmax -> top-k, largest first, of the scaled logits; counts (may be
+ * NULL) receives per line the nucleus cut of vkop_oracle_topp_count_f32 for
+ * top_p on the line's k sorted probabilities (halves widened for f16). */
+void vkop_oracle_softmax_topk_sampling_f32(const float *in, float scale,
+                                           float top_p, float *values,
+                                           int32_t *indices, int32_t *counts,
+                                           int outer, int n, int inner, int k);
+void vkop_oracle_softmax_topk_sampling_f16(const uint16_t *in, float scale,
+                                           float top_p, uint16_t *values,
+                                           int32_t *indices, int32_t *counts,
+                                           int outer, int n, int inner, int k);
+
 /* Same as vkop_oracle_softmax_topk_f32 with the (outer*inner) lines spread
  * over OpenMP threads; used only to time a multi-core CPU baseline.
  * Returns the number of threads used. */

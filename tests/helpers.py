@@ -102,3 +102,54 @@ def reference_half_tolerance_ok(out, exp):
     a = np.abs(exp)
     thr = np.where(a > 1.0, a * 0.02, 0.02)
     return bool(np.all(~np.isnan(out)) and np.all(np.abs(out - exp) <= thr))
+
+
+def check_fused_invariants(x_row, vals_row, idx_row):
+    """What any correct fused softmax -> top-k (largest first) of one row satisfies,
+    whatever row sum the implementation arrived at, because a probability is a
+    non-decreasing function of its logit: returned probabilities do not increase;
+    equal returned probabilities come in increasing index order; a larger logit never
+    has a smaller returned probability; nothing left out has a logit at or above that
+    of a returned entry whose probability exceeds the last one; and anything left out
+    whose logit reaches the smallest logit of the last probability's group (it then
+    has that same probability) has a higher index than every returned member of the
+    group.  Rows holding NaN / +inf (all-NaN results) are not for this check.
+    Raises AssertionError naming the property that fails."""
+    x = np.asarray(x_row, dtype=np.float32)
+    p = np.asarray(vals_row, dtype=np.float32)
+    ix = np.asarray(idx_row).astype(np.int64)
+    k = len(ix)
+    assert len(set(ix.tolist())) == k and ix.min() >= 0 and ix.max() < len(x), "indices not distinct / in range"
+    assert np.all(p[:-1] >= p[1:]), "probabilities increase along the result"
+    same = p[:-1] == p[1:]
+    assert np.all(ix[1:][same] > ix[:-1][same]), "equal probabilities not in increasing index order"
+    lx = x[ix]
+    order = np.argsort(-lx, kind="stable")
+    assert np.all(np.diff(p[order]) <= 0), "a larger logit has a smaller probability"
+    rest = np.ones(len(x), bool)
+    rest[ix] = False
+    if not rest.any():
+        return
+    last = p[-1]
+    group = p == last
+    above = ~group
+    if above.any():
+        assert x[rest].max() < lx[above].min(), "an element left out beats a returned one with a larger probability"
+    reach = rest & (x >= lx[group].min())
+    if reach.any():
+        assert np.nonzero(reach)[0].min() > ix[group].max(), "a tie at the last place was not settled by lower index"
+
+
+def well_separated_cut(probs_row, logits_row, k, min_ulp=4):
+    """True when the row's k+1 largest probabilities (an oracle's) are pairwise either at
+    least min_ulp apart or equal with equal logits: then an implementation within a
+    couple of ulp of them must return exactly the oracle's indices."""
+    pr = np.asarray(probs_row, dtype=np.float32)
+    lg = np.asarray(logits_row, dtype=np.float32)
+    if np.isnan(pr).any():
+        return False
+    order = np.lexsort((np.arange(len(pr)), -pr))[:k + 1]
+    top, tl = pr[order], lg[order]
+    d = ulp_diff(top[:-1], top[1:])
+    ok = (d >= min_ulp) | ((d == 0) & (tl[:-1] == tl[1:]))
+    return bool(np.all(ok))

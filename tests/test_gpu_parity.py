@@ -13,8 +13,8 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (check_topk_invariants, half_ulp_diff, reference_float_tolerance_ok,
-                     reference_half_tolerance_ok, ulp_diff)
+from helpers import (check_fused_invariants, check_topk_invariants, half_ulp_diff, reference_float_tolerance_ok,
+                     reference_half_tolerance_ok, ulp_diff, well_separated_cut)
 from vkop_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -254,14 +254,28 @@ def assert_fused(ops, x, k, axis=-1, largest=True):
         assert half_ulp_diff(v2, v).max() <= 1
     else:
         assert ulp_diff(v2, v).max() <= 1
+    pm = np.moveaxis(p, axis, -1).reshape(-1, x.shape[axis])
+    i2 = np.moveaxis(ix2, axis, -1).reshape(-1, k)
+    i1 = np.moveaxis(ix, axis, -1).reshape(-1, k)
     if not same:
         # only a probability tie that the 1-ulp difference opens or closes may
         # reorder: the ranking must still be exact for the values it returned
-        pm = np.moveaxis(p, axis, -1).reshape(-1, x.shape[axis])
-        i2 = np.moveaxis(ix2, axis, -1).reshape(-1, k)
-        i1 = np.moveaxis(ix, axis, -1).reshape(-1, k)
+        tolerant = 0
         for r in range(pm.shape[0]):
-            assert sorted(pm[r][i2[r]].tolist()) == sorted(pm[r][i1[r]].tolist()), r
+            if not np.array_equal(i2[r], i1[r]):
+                tolerant += 1
+                assert sorted(pm[r][i2[r]].tolist()) == sorted(pm[r][i1[r]].tolist()), r
+        print("assert_fused %s k=%d: %d of %d rows differ from the tensor route by a tie the row sum opened or closed"
+              % (x.shape, k, tolerant, pm.shape[0]))
+        assert tolerant <= max(1, pm.shape[0] // 5), (tolerant, pm.shape[0])
+    if largest:
+        # whichever way such a tie went, the result is ranked by (probability, then lower
+        # index) of a monotone function of the logits: checked on the logits themselves
+        xm = np.moveaxis(x, axis, -1).reshape(-1, x.shape[axis]).astype(np.float32)
+        v2m = np.moveaxis(v2, axis, -1).reshape(-1, k).astype(np.float32)
+        for r in range(pm.shape[0]):
+            if np.isfinite(v2m[r]).all():
+                check_fused_invariants(xm[r], v2m[r], i2[r])
     # (4) against the oracle's own fused result: values to the softmax bar,
     # indices wherever the oracle's probabilities around the cut are distinct
     ov, oix, op = oracle.softmax_topk(x, k, axis, largest, return_probs=True)
@@ -275,6 +289,10 @@ def assert_fused(ops, x, k, axis=-1, largest=True):
             ptop = np.sort(pm[r])[::-1][:k + 1] if largest else np.sort(pm[r])[:k + 1]
             if len(np.unique(top)) == len(top) and len(np.unique(ptop)) == len(ptop) and not np.isnan(ptop).any():
                 assert np.array_equal(im[r], om[r]), r
+            # the streaming result: exactly the oracle's indices wherever the oracle's
+            # probabilities around the cut are well apart (or tie through equal logits)
+            if largest and well_separated_cut(pm[r], xm[r], k):
+                assert np.array_equal(i2[r], om[r]), r
     return v, ix
 
 
@@ -674,7 +692,23 @@ def test_awkward_rows_against_the_oracle(ops, n, k):
             d = half_ulp_diff(v[r], ev[r]) if dtype == np.float16 else ulp_diff(v[r], ev[r])
             assert d.max() <= 1, (r, n, k)
             assert len(set(ix[r].tolist())) == k
+        print("awkward rows n=%d k=%d %s: %d of %d rows differ from the tensor route by a tie the row sum opened or closed"
+              % (n, k, np.dtype(dtype).name, int((~rows_equal).sum()), len(rows_equal)))
         assert rows_equal.mean() > 0.8
+        # every row, tolerant branch or not: ranked by (probability, then lower index) of a
+        # monotone function of the logits; and exactly the oracle's indices wherever its
+        # probabilities around the cut are well apart (or tie through equal logits)
+        op_full = oracle.softmax(x)
+        xf = x.astype(np.float32)
+        exact_rows = 0
+        for r in range(x.shape[0]):
+            vr = v[r].astype(np.float32)
+            if np.isfinite(vr).all():
+                check_fused_invariants(xf[r], vr, ix[r])
+            if well_separated_cut(op_full[r].astype(np.float32), xf[r], k, 4 if dtype == np.float32 else 1 << 14):
+                exact_rows += 1
+                assert np.array_equal(ix[r], oix[r]), (r, n, k)
+        print("   ... %d rows with a well separated cut match the oracle's indices exactly" % exact_rows)
         for largest in (True, False):
             t, j = ops.topk(dev(x), k, -1, largest)
             et, ej = oracle.topk(x, k, -1, largest)

@@ -1,0 +1,284 @@
+"""The scan + pick kernel pair (long last-axis rows) and the sampling-style entry
+point, on the GPU, through the C ABI.
+
+* The pair against the chunk + merge kernels it stands in for (vkop_hip_tune
+  "rows.path"): bit-identical results -- both implement "top-k by (probability, then
+  lower index) of the row's softmax" and sum the row's terms in orders of their own,
+  so a value may differ by an ulp where the sums round apart; indices, and values
+  where the sums agree, are compared exactly, values otherwise to one ulp -- and
+  against the oracle: the monotone-ranking invariants on every row, exact indices
+  wherever the oracle's probabilities around the cut are well apart.
+* vkop_hip_softmax_topk_sampling against the oracle's sampling variant and against
+  the plain entry point on a tensor scaled on the host.
+* The NaN replacement option of the softmax on axes other than the last.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import check_fused_invariants, check_topk_invariants, half_ulp_diff, ulp_diff, well_separated_cut
+from vkop_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from vkop_amd import capi, ops as _ops
+    capi.lib()              # raises if the HIP library is not built: no fallback
+    capi.init(0)
+    yield _ops
+    capi.tune("rows.path", 0)
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint16:
+        a = a.view(np.float16)
+    return torch.from_numpy(a).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def _rows(kind, rows, n, rng):
+    if kind == "llm":
+        return synth.llm_logits(rows, n, seed=int(rng.integers(1, 1 << 30)))
+    x = (rng.standard_normal((rows, n)) * 1.5).astype(np.float32)
+    if kind == "bf16":        # what a bf16 head hands over: equal logits straddle the cut
+        return np.ascontiguousarray((x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32))
+    if kind == "levels":      # 64 levels: massive ties
+        return (np.round(x * 8) / 8).astype(np.float32)
+    if kind == "sorted":
+        x = np.sort(x, axis=1)
+        x[1::2] = x[1::2, ::-1]
+        return np.ascontiguousarray(x)
+    if kind == "masked":      # a few allowed tokens per row, the rest -inf
+        m = rng.random((rows, n)) < (40.0 / n)
+        x[~m] = -np.inf
+        x[0, :] = -np.inf
+        x[0, 5] = 1.0
+        return x
+    if kind == "constant":
+        x[:] = np.float32(-2.5)
+        x[1, n // 2:] = np.float32(3.0)
+        return x
+    if kind == "spikes":      # elements far above their wave's first vectors, and a dominant one
+        x[:, n // 3] += 40.0
+        x[2, 17::4099] += 25.0
+        return x
+    raise ValueError(kind)
+
+
+KINDS = ["llm", "bf16", "levels", "sorted", "masked", "constant", "spikes"]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("n,k", [(128256, 50), (128256, 1), (128256, 255), (40000, 7), (16385, 20), (13057, 50),
+                                 (262144, 64), (100003, 33), (500000, 100), (300000, 511)])
+def test_scan_pick_pair_equals_chunk_merge_and_oracle(ops, n, k, dtype):
+    from vkop_amd import capi
+    rng = np.random.default_rng(n * 31 + k)
+    rows = 6
+    dt = capi.F32 if dtype == np.float32 else capi.F16
+    capi.tune("rows.path", 0)
+    if capi.measure_path(dt, (rows, n), -1, k) != 2:
+        pytest.skip("not a shape the scan + pick pair takes in this element type")
+    for kind in KINDS:
+        x = np.ascontiguousarray(_rows(kind, rows, n, rng).astype(dtype))
+        xd = dev(x)
+        capi.tune("rows.path", 0)
+        v, ix = ops.softmax_topk(xd, k)
+        t, tj = ops.topk(xd, k)
+        v, ix, t, tj = host(v), host(ix), host(t), host(tj)
+        capi.tune("rows.path", 1)
+        v1, ix1 = ops.softmax_topk(xd, k)
+        t1, tj1 = ops.topk(xd, k)
+        v1, ix1, t1, tj1 = host(v1), host(ix1), host(t1), host(tj1)
+        capi.tune("rows.path", 0)
+        bits = np.uint16 if dtype == np.float16 else np.uint32
+        what = (kind, n, k, np.dtype(dtype).name)
+        # plain top-k: no arithmetic, everything exact, both pairs and the oracle
+        et, ej = oracle.topk(x, k)
+        assert np.array_equal(tj, ej) and np.array_equal(t.view(bits), et.view(bits)), what
+        assert np.array_equal(tj1, ej) and np.array_equal(t1.view(bits), et.view(bits)), what
+        # fused: values within an ulp of the other pair's, to the bar against the oracle
+        ov, oix, op = oracle.softmax_topk(x, k, return_probs=True)
+        if dtype == np.float16:
+            assert half_ulp_diff(v, v1).max() <= 1 and half_ulp_diff(v, ov).max() <= 1, what
+        else:
+            assert ulp_diff(v, v1).max() <= 1 and ulp_diff(v, ov).max() <= 2, what
+        differ = 0
+        xf = x.astype(np.float32)
+        for r in range(rows):
+            vr = v[r].astype(np.float32)
+            if not np.array_equal(ix[r], ix1[r]):
+                differ += 1      # only where the two row sums round a tie open or closed
+                assert not np.array_equal(v[r].view(bits), v1[r].view(bits)) or \
+                    sorted(ix[r].tolist()) != sorted(ix1[r].tolist()), what
+            if np.isfinite(vr).all():
+                check_fused_invariants(xf[r], vr, ix[r])
+            else:
+                assert np.array_equal(ix[r], np.arange(k)), what       # all-NaN row: lowest indices
+            if well_separated_cut(op[r].astype(np.float32), xf[r], k, 4 if dtype == np.float32 else 1 << 14):
+                assert np.array_equal(ix[r], oix[r]), (what, r)
+        assert differ <= 2, (what, differ)
+
+
+@pytest.mark.parametrize("n", [16388, 40002, 128255])
+def test_scan_pick_pair_on_rows_that_do_not_start_on_16_bytes(ops, n):
+    """n not a multiple of the vector width (rows after the first are unaligned), and a
+    tensor that starts two elements into an allocation: the element-wise load variants."""
+    rng = np.random.default_rng(n)
+    for dtype in (np.float32, np.float16):
+        x = np.ascontiguousarray((rng.standard_normal((5, n)) * 2).astype(dtype))
+        x[3, ::5] = x[3, 1]
+        big = torch.empty(5 * n + 8, dtype=torch.float32 if dtype == np.float32 else torch.float16, device="cuda")
+        xd = big[2:2 + 5 * n].view(5, n)
+        xd.copy_(dev(x))
+        for k in (5, 60):
+            v, ix = ops.softmax_topk(xd, k)
+            t, tj = ops.topk(xd, k)
+            v, ix, t, tj = host(v), host(ix), host(t), host(tj)
+            et, ej = oracle.topk(x, k)
+            bits = np.uint16 if dtype == np.float16 else np.uint32
+            assert np.array_equal(tj, ej) and np.array_equal(t.view(bits), et.view(bits)), (n, k)
+            ov, oix, op = oracle.softmax_topk(x, k, return_probs=True)
+            if dtype == np.float16:
+                assert half_ulp_diff(v, ov).max() <= 1
+            else:
+                assert ulp_diff(v, ov).max() <= 2
+            for r in range(5):
+                check_fused_invariants(x[r].astype(np.float32), v[r].astype(np.float32), ix[r])
+                if well_separated_cut(op[r].astype(np.float32), x[r].astype(np.float32), k, 4 if dtype == np.float32 else 1 << 14):
+                    assert np.array_equal(ix[r], oix[r]), (n, k, r)
+
+
+def test_plain_topk_nan_ranks_first_through_the_scan_pick_pair(ops):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((4, 70000)).astype(np.float32)
+    x[0, [5, 69999, 30000]] = np.nan
+    x[1, ::3] = np.nan                       # more NaN than k
+    x[2, 1000] = np.inf
+    x[2, 2000] = -np.inf
+    x[3, :] = np.nan
+    for k in (1, 4, 100):
+        t, tj = ops.topk(dev(x), k)
+        et, ej = oracle.topk(x, k)
+        assert np.array_equal(host(tj), ej) and np.array_equal(host(t).view(np.uint32), et.view(np.uint32)), k
+
+
+# ------------------------------------------------------------ sampling variant --
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("shape,k", [((16, 128256), 50), ((3, 40000), 7), ((256, 1000), 5), ((2, 33), 33), ((5, 2, 4097), 9)])
+def test_sampling_variant_against_the_oracle(ops, shape, k, dtype):
+    rng = np.random.default_rng(shape[-1] + k)
+    x = synth.llm_logits(int(np.prod(shape[:-1])), shape[-1], seed=shape[-1], temperature=1.0).reshape(shape)
+    x = np.ascontiguousarray(x.astype(dtype))
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    for scale, top_p in ((1.25, 0.9), (1.0, 0.5), (0.5, 0.999), (3.0, 0.2)):
+        v, ix, c = ops.softmax_topk_sampling(dev(x), k, scale, top_p)
+        v, ix, c = host(v), host(ix), host(c)
+        ov, oix, oc = oracle.softmax_topk_sampling(x, k, scale, top_p)
+        what = (shape, k, scale, top_p)
+        if dtype == np.float16:
+            assert half_ulp_diff(v, ov).max() <= 1, what
+        else:
+            assert ulp_diff(v, ov).max() <= 2, what
+        # the count is a function of the stored values: exact against the pinned CPU rule on them,
+        # and equal to the separate entry point's
+        vf = v.astype(np.float32).reshape(-1, k)
+        assert np.array_equal(c.reshape(-1), oracle.topp_count(vf, top_p)), what
+        same_values = np.array_equal(v.view(bits), ov.view(bits))
+        if same_values:
+            assert np.array_equal(c, oc), what
+        # bit for bit the plain entry point on a tensor scaled on the host (one float32 product per element)
+        xs = (x.astype(np.float32) * np.float32(scale)).astype(np.float32)
+        # (bit for bit where both run the scan + pick kernels; other shapes take the line kernels here and the
+        # one-workgroup streaming kernels there, which add up the row in different orders: both within the 2-ulp bar of the oracle)
+        if dtype == np.float32:
+            from vkop_amd import capi
+            pv, pix = ops.softmax_topk(dev(xs), k)
+            pv, pix = host(pv), host(pix)
+            if capi.measure_path(capi.F32, shape, -1, k) == 2:
+                assert np.array_equal(pix, ix) and np.array_equal(pv.view(np.uint32), v.view(np.uint32)), what
+            else:
+                assert ulp_diff(pv, v).max() <= 2, what
+        xf = (x.astype(np.float32) * np.float32(scale)).reshape(-1, shape[-1])
+        op = oracle.softmax(xf)
+        for r in range(xf.shape[0]):
+            check_fused_invariants(xf[r], vf[r], ix.reshape(-1, k)[r])
+            if dtype == np.float32 and well_separated_cut(op[r], xf[r], k):
+                assert np.array_equal(ix.reshape(-1, k)[r], oix.reshape(-1, k)[r]), (what, r)
+
+
+def test_sampling_variant_ties_special_rows_and_errors(ops):
+    from vkop_amd import capi
+    rng = np.random.default_rng(9)
+    x = (np.round(rng.standard_normal((6, 50000)) * 4) / 4).astype(np.float32)   # ties across the cut
+    x[1, 10:] = -np.inf                     # fewer elements above -inf than k
+    x[2, 77] = np.nan                       # an all-NaN result
+    x[3] = 1.5                              # a constant row
+    k = 40
+    v, ix, c = ops.softmax_topk_sampling(dev(x), k, 0.75, 0.8)
+    v, ix, c = host(v), host(ix), host(c)
+    with np.errstate(invalid="ignore"):
+        ov, oix, oc = oracle.softmax_topk_sampling(x, k, 0.75, 0.8)
+    assert np.array_equal(np.isnan(v), np.isnan(ov))
+    assert ulp_diff(v, ov).max() <= 2
+    assert np.array_equal(ix[2], np.arange(k)) and c[2] == k
+    assert np.array_equal(ix[3], np.arange(k)) and np.array_equal(ix[1][:10], oix[1][:10])
+    ok = ~np.isnan(v).any(axis=1)
+    assert np.array_equal(c[ok], oracle.topp_count(v[ok], 0.8))
+    xs = (x * np.float32(0.75)).astype(np.float32)
+    for r in np.nonzero(ok)[0]:
+        check_fused_invariants(xs[r], v[r], ix[r])
+    xd = dev(x)
+    out = torch.empty((6, k), dtype=torch.float32, device="cuda")
+    oi = torch.empty((6, k), dtype=torch.int32, device="cuda")
+    ws = torch.zeros(1 << 22, dtype=torch.uint8, device="cuda")
+    ptr = (ws.data_ptr() + 255) // 256 * 256
+    for bad in (0.0, -1.0, float("inf"), float("nan")):
+        with pytest.raises(capi.VkopHipError) as e:
+            capi.softmax_topk_sampling(xd.data_ptr(), out.data_ptr(), oi.data_ptr(), 0, capi.F32, x.shape, -1, k, bad, 0.5, ptr,
+                                       1 << 21, 0)
+        assert e.value.code == capi.ERR_INVALID
+    with pytest.raises(capi.VkopHipError) as e:   # the count along an axis that is not the last
+        capi.softmax_topk_sampling(xd.data_ptr(), out.data_ptr(), oi.data_ptr(), oi.data_ptr(), capi.F32, x.shape, 0, 3, 1.0, 0.5,
+                                   ptr, 1 << 21, 0)
+    assert e.value.code == capi.ERR_UNSUPPORTED
+
+
+# ------------------------------------------ softmax: NaN option on the other axes --
+
+@pytest.mark.parametrize("shape,axis", [((130, 70), 0), ((5, 130, 70), 1), ((2, 3, 40, 9), 2), ((80, 8400), 0), ((3, 4, 5, 6), 0),
+                                        ((4, 3000, 3), 1)])
+def test_nan_replacement_on_axes_other_than_the_last(ops, shape, axis):
+    """shaders/softmax2.comp:177-181 implements the option for axis 0 of a matrix; here every axis."""
+    rng = np.random.default_rng(sum(shape) + axis)
+    for dtype in (np.float32, np.float16):
+        x = rng.standard_normal(shape).astype(np.float32)
+        idx = tuple(rng.integers(0, s, size=6) for s in shape)
+        x[idx] = np.nan                                     # lines holding a NaN: all of the line's outputs are NaN
+        line = [0] * len(shape)
+        line[axis] = slice(None)
+        x[tuple(line)] = -np.inf                            # a line of -inf: NaN too
+        x = np.ascontiguousarray(x.astype(dtype))
+        with np.errstate(invalid="ignore"):
+            exp = oracle.softmax(x, axis)
+            expn = oracle.softmax(x, axis, nan_where=1, nan_value=0.25)
+        assert np.isnan(exp.astype(np.float32)).any()
+        got = host(ops.softmax(dev(x), axis))
+        gotn = host(ops.softmax(dev(x), axis, nan_where=True, nan_value=0.25))
+        assert np.array_equal(np.isnan(got.astype(np.float32)), np.isnan(exp.astype(np.float32)))
+        assert not np.isnan(gotn.astype(np.float32)).any()
+        assert np.array_equal(gotn.astype(np.float32) == 0.25, (expn.astype(np.float32) == 0.25))
+        if dtype == np.float16:
+            assert half_ulp_diff(gotn, expn).max() <= 1
+        else:
+            assert ulp_diff(gotn, expn).max() <= 2

@@ -401,3 +401,82 @@ def test_topp_count_closed_forms_and_cumsum():
     assert oracle.topp_count(bad, 0.9999)[3] == 50
     half = v.astype(np.float16)
     assert np.array_equal(oracle.topp_count(half, 0.7), oracle.topp_count(half.astype(np.float32), 0.7))
+
+
+# ------------------------------------------------ sampling-style fused variant --
+
+def test_sampling_variant_scale_and_count_pins():
+    """vkop_oracle_softmax_topk_sampling_*: not the formula retyped, but facts that fix it.
+    scale = 1 is the plain fused oracle bit for bit; a power-of-two scale multiplies
+    exactly, so the result is the plain oracle's on numpy's ldexp of the input; any scale
+    is the plain oracle on numpy's own float32 product (one rounding per element, done by
+    another implementation); the counts are topp_count (pinned above) on the returned
+    values, with its closed forms: p <= first value -> 1, p above the total -> k."""
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((6, 3000)) * 2).astype(np.float32)
+    x[1, ::7] = x[1, 3]                      # ties
+    x[2, 100:] = -np.inf                     # fewer finite elements than most k
+    for k in (1, 7, 50):
+        v1, i1 = oracle.softmax_topk_sampling(x, k, 1.0)
+        ev, ei = oracle.softmax_topk(x, k)
+        assert np.array_equal(i1, ei) and np.array_equal(v1.view(np.uint32), ev.view(np.uint32))
+        for j in (-2, 1, 3):
+            v2, i2 = oracle.softmax_topk_sampling(x, k, 2.0 ** j)
+            ev, ei = oracle.softmax_topk(np.ldexp(x, j).astype(np.float32), k)
+            assert np.array_equal(i2, ei) and np.array_equal(v2.view(np.uint32), ev.view(np.uint32)), (k, j)
+        for scale in (1.25, 0.7, 3.3333333):
+            v3, i3, c3 = oracle.softmax_topk_sampling(x, k, scale, top_p=0.9)
+            xs = (x * np.float32(scale)).astype(np.float32)
+            ev, ei = oracle.softmax_topk(xs, k)
+            assert np.array_equal(i3, ei) and np.array_equal(v3.view(np.uint32), ev.view(np.uint32)), (k, scale)
+            assert np.array_equal(c3, oracle.topp_count(v3, 0.9))
+        _, _, c = oracle.softmax_topk_sampling(x, k, 1.25, top_p=0.0)
+        assert np.all(c == 1)
+        _, _, c = oracle.softmax_topk_sampling(x, k, 1.25, top_p=1.5)
+        assert np.all(c == k)
+    # half precision: the same facts on the widened halves
+    xh = x[:3].astype(np.float16)
+    v, i = oracle.softmax_topk_sampling(xh, 9, 1.0)
+    ev, ei = oracle.softmax_topk(xh, 9)
+    assert np.array_equal(i, ei) and np.array_equal(v.view(np.uint16), ev.view(np.uint16))
+    v, i, c = oracle.softmax_topk_sampling(xh, 9, 2.0, top_p=0.5)
+    x2 = (xh.astype(np.float32) * np.float32(2.0)).astype(np.float16)   # exact in half away from overflow
+    ev, ei = oracle.softmax_topk(x2, 9)
+    assert np.array_equal(i, ei) and np.array_equal(v.view(np.uint16), ev.view(np.uint16))
+    assert np.array_equal(c, oracle.topp_count(v.astype(np.float32), 0.5))
+
+
+def test_fused_invariant_check_catches_a_wrong_tie_break():
+    """tests/helpers.py: check_fused_invariants accepts the oracle's results and refuses a
+    result whose tie at the last place went to a higher index, an entry left out that
+    beats a returned one, and equal probabilities out of index order."""
+    from helpers import check_fused_invariants, well_separated_cut
+    rng = np.random.default_rng(0)
+    x = (np.round(rng.standard_normal((4, 5000)) * 8) / 8).astype(np.float32)   # many equal logits
+    v, ix = oracle.softmax_topk(x, 50)
+    for r in range(4):
+        check_fused_invariants(x[r], v[r], ix[r])
+    r = 0
+    group = np.nonzero(v[r] == v[r, -1])[0]
+    level = x[r, ix[r, group]].min()
+    left_out = [j for j in np.nonzero(x[r] == level)[0] if j not in ix[r]]
+    assert left_out, "the case needs a tie across the last place"
+    wrong = ix[r].copy()
+    wrong[-1] = max(left_out)                               # same probability, higher index
+    with pytest.raises(AssertionError, match="lower index"):
+        check_fused_invariants(x[r], v[r], wrong)
+    wrong = ix[r].copy()
+    wrong[0] = int(np.argmin(x[r]))                         # the row's best element left out for its worst
+    with pytest.raises(AssertionError):
+        check_fused_invariants(x[r], v[r], wrong)
+    pair = np.nonzero(v[r][:-1] == v[r][1:])[0]
+    if pair.size:
+        wrong = ix[r].copy()
+        a = pair[0]
+        wrong[a], wrong[a + 1] = wrong[a + 1], wrong[a]
+        with pytest.raises(AssertionError, match="increasing index"):
+            check_fused_invariants(x[r], v[r], wrong)
+    y = rng.standard_normal((1, 4000)).astype(np.float32)
+    assert well_separated_cut(oracle.softmax(y)[0], y[0], 10, 1) in (True, False)
+    y[0, :20] = 9.0                                          # ties through equal logits count as separated
+    assert well_separated_cut(oracle.softmax(y)[0], y[0], 10)

@@ -38,6 +38,13 @@ def declared_symbols():
     return sorted(set(re.findall(r"\b(vkop_hip_[a-z0-9_]+)\s*\(", text)))
 
 
+def internal_symbols():
+    """Names of the measurement hooks vkop_amd/csrc/vkop_hip_internal.h declares (not part of the public interface)."""
+    text = open(os.path.join(_HERE, "csrc", "vkop_hip_internal.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vkop_hip_[a-z0-9_]+)\s*\(", text)))
+
+
 _lib = None
 
 
@@ -87,6 +94,7 @@ def lib():
         "vkop_hip_softmax_topk_workspace_bytes": (sz, [i, ip, i, i, i]),
         "vkop_hip_softmax_topk": (i, [vp, vp, vp, vp, i, ip, i, i, i, i, vp, sz, vp]),
         "vkop_hip_softmax_topk_static": (i, [vp, vp, vp, i, ip, i, i, i, i, vp]),
+        "vkop_hip_softmax_topk_sampling": (i, [vp, vp, vp, vp, i, ip, i, i, i, f, f, vp, sz, vp]),
         "vkop_hip_reduce_max": (i, [vp, vp, i, ip, i, i, vp]),
         "vkop_hip_softmax_reduce_max_workspace_bytes": (sz, [i, ip, i, i]),
         "vkop_hip_softmax_reduce_max": (i, [vp, vp, i, ip, i, i, vp, sz, vp]),
@@ -232,6 +240,14 @@ def softmax_topk(inp, probs, values, indices, dtype, shape, axis, k, largest=1, 
     arr, nd = _shape(shape)
     check(lib().vkop_hip_softmax_topk(inp, probs, values, indices, dtype, arr, nd, axis, int(k), int(largest),
                                       workspace, workspace_bytes, stream))
+
+
+def softmax_topk_sampling(inp, values, indices, counts, dtype, shape, axis, k, scale, top_p, workspace=0, workspace_bytes=0,
+                          stream=0):
+    """Fused softmax -> top-k of fl32(x * scale); counts (0 = none): nucleus cut per row for top_p."""
+    arr, nd = _shape(shape)
+    check(lib().vkop_hip_softmax_topk_sampling(inp, values, indices, counts, dtype, arr, nd, axis, int(k), float(scale),
+                                               float(top_p), workspace, workspace_bytes, stream))
 
 
 STATIC_SCRATCH_BYTES = 4 << 20

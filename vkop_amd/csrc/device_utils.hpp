@@ -34,6 +34,18 @@ template <> __device__ __forceinline__ float round_to_storage<uint16_t>(float v)
     return __half2float(__float2half_rn(v));
 }
 
+// x * scale rounded to float on its own: never contracted into a fused multiply-add
+// with what follows, so that a kernel given a scale computes on exactly the values
+// a tensor scaled beforehand would hold.
+// (the empty asm hides the product from the optimizer; `__fmul_rn` alone is a plain
+// multiplication to this compiler and does get contracted)
+__device__ __forceinline__ float scaled(float x, float scale) {
+#pragma clang fp contract(off)
+    float p = x * scale;
+    asm volatile("" : "+v"(p));
+    return p;
+}
+
 // ------------------------------------------------------------ ordering ----
 
 // Maps a float to a uint32 whose unsigned order is the ranking top-k uses:

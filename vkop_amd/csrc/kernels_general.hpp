@@ -26,22 +26,23 @@ struct LineStats {
 };
 
 // max and sum of exp(x - max) of one line, by all NT threads of the block.
+// scale: every element counts times scale (1: as it is).
 template <typename T, int NT>
 __device__ __forceinline__ LineStats line_stats(const T *x, size_t base, uint32_t n, uint32_t stride,
-                                                float *fscratch, double *dscratch) {
+                                                float *fscratch, double *dscratch, float scale = 1.f) {
     const uint32_t tid = threadIdx.x;
     float m = -INFINITY;
-    for (uint32_t j = tid; j < n; j += NT) m = fmaxf(m, load_elem(x, base + static_cast<size_t>(j) * stride));
+    for (uint32_t j = tid; j < n; j += NT) m = fmaxf(m, scaled(load_elem(x, base + static_cast<size_t>(j) * stride), scale));
     m = block_max<NT>(m, fscratch);
     // every term is a float (as the softmax definition rounds it); the sum of
     // the terms is exact to double rounding, in a fixed order
     double a0 = 0.0, a1 = 0.0;
     uint32_t j = tid;
     for (; j + NT < n; j += 2u * NT) {
-        a0 += static_cast<double>(softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m));
-        a1 += static_cast<double>(softmax_term(load_elem(x, base + static_cast<size_t>(j + NT) * stride), m));
+        a0 += static_cast<double>(softmax_term(scaled(load_elem(x, base + static_cast<size_t>(j) * stride), scale), m));
+        a1 += static_cast<double>(softmax_term(scaled(load_elem(x, base + static_cast<size_t>(j + NT) * stride), scale), m));
     }
-    if (j < n) a0 += static_cast<double>(softmax_term(load_elem(x, base + static_cast<size_t>(j) * stride), m));
+    if (j < n) a0 += static_cast<double>(softmax_term(scaled(load_elem(x, base + static_cast<size_t>(j) * stride), scale), m));
     const double s = block_sum<NT>(a0 + a1, dscratch);
     return LineStats{m, 0.f, 1.0 / s};
 }
@@ -56,17 +57,17 @@ __device__ __forceinline__ float softmax_prob(float x, LineStats st) {
 // ---- softmax, one workgroup per line ---------------------------------------
 template <typename T, int NT>
 __global__ __launch_bounds__(NT) void softmax_lines_kernel(const T *in, T *out, LineGeom g, int nan_where,
-                                                           float nan_value, LineStats *stats_out) {
+                                                           float nan_value, LineStats *stats_out, float scale = 1.f) {
     __shared__ float fscratch[NT / kWave];
     __shared__ double dscratch[NT / kWave];
     const uint32_t line = blockIdx.x;
     const size_t base = g.base(line);
-    const LineStats st = line_stats<T, NT>(in, base, g.n, g.inner, fscratch, dscratch);
+    const LineStats st = line_stats<T, NT>(in, base, g.n, g.inner, fscratch, dscratch, scale);
     if (stats_out != nullptr && threadIdx.x == 0) stats_out[line] = st;
     if (out == nullptr) return;
     for (uint32_t j = threadIdx.x; j < g.n; j += NT) {
         const size_t at = base + static_cast<size_t>(j) * g.inner;
-        float p = round_to_storage<T>(softmax_prob(load_elem(in, at), st));
+        float p = round_to_storage<T>(softmax_prob(scaled(load_elem(in, at), scale), st));
         if (nan_where && p != p) p = nan_value;
         store_elem(out, at, p);
     }
@@ -206,21 +207,21 @@ template <typename T, int NT>
 __global__ __launch_bounds__(NT) void softmax_topk_lines_kernel(const T *__restrict__ in,
                                                                 const LineStats *__restrict__ stats,
                                                                 T *__restrict__ values, int32_t *__restrict__ indices,
-                                                                LineGeom g, uint32_t k, int largest) {
+                                                                LineGeom g, uint32_t k, int largest, float scale = 1.f) {
     __shared__ SelectShared sh;
     const uint32_t line = blockIdx.x;
     const size_t base = g.base(line);
     const LineStats st = stats[line];
     const uint32_t flip = largest ? 0u : 0xFFFFFFFFu;
     select_topk_line<NT>(sh, g.n, k, [&](uint32_t j) {
-        const float p = softmax_prob(load_elem(in, base + static_cast<size_t>(j) * g.inner), st);
+        const float p = softmax_prob(scaled(load_elem(in, base + static_cast<size_t>(j) * g.inner), scale), st);
         return order_key(round_to_storage<T>(p)) ^ flip;
     });
     const uint32_t o = line / g.inner, i = line - o * g.inner;
     const size_t obase = static_cast<size_t>(o) * k * g.inner + i;
     for (uint32_t r = threadIdx.x; r < k; r += NT) {
         const uint32_t idx = composite_index(sh.sel[r]);
-        const float p = softmax_prob(load_elem(in, base + static_cast<size_t>(idx) * g.inner), st);
+        const float p = softmax_prob(scaled(load_elem(in, base + static_cast<size_t>(idx) * g.inner), scale), st);
         store_elem(values, obase + static_cast<size_t>(r) * g.inner, p);
         indices[obase + static_cast<size_t>(r) * g.inner] = static_cast<int32_t>(idx);
     }

@@ -380,10 +380,12 @@ template <> struct Vec128<uint16_t> {
 // read from its start, NT * 4 elements at a time, until enough members are found
 // -- soon, for a group that large.  SOFTMAX: every member's value is tie_value (the
 // group's probability); otherwise the element itself.  counts: 2 * NT / 64 words
-// of LDS.  All NT threads call.
+// of LDS.  scale: the keys are those of the elements times scale (1: as they are).
+// All NT threads call.
 template <typename T, int NT, bool SOFTMAX>
 __device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *rowp, T *ov, int32_t *oi, uint32_t n,
-                                                   uint32_t g0, uint32_t kk, uint32_t xlo, uint32_t xhi, float tie_value) {
+                                                   uint32_t g0, uint32_t kk, uint32_t xlo, uint32_t xhi, float tie_value,
+                                                   float scale = 1.f) {
     constexpr int NW = NT / kWave;
     constexpr int U = 4;
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -397,7 +399,7 @@ __device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *ro
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const uint32_t j = j0 + u;
-            const uint32_t key = order_key(load_elem(rowp, j < n ? j : 0u));
+            const uint32_t key = order_key(scaled(load_elem(rowp, j < n ? j : 0u), scale));
             member[u] = j < n && key >= xlo && key <= xhi;
             const uint64_t mask = __ballot(member[u]);
             below += lanes_below(mask);
@@ -445,7 +447,7 @@ __device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *ro
 // touched them (the same value in every thread).
 template <typename T, int NT, typename AddMissing>
 __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_missing, const T *rowp, T *ov, int32_t *oi,
-                                               uint32_t n, uint32_t kk, float p_cut, float M, double rinv) {
+                                               uint32_t n, uint32_t kk, float p_cut, float M, double rinv, float scale = 1.f) {
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     auto prob_of_key = [&](uint32_t key) {
         return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(key), M)) * rinv));
@@ -455,7 +457,7 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_mi
         // probability 0: every element from the group's largest logit down
         __syncthreads();
         const uint32_t g0 = sh.g0;
-        fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, 0u, sh.pkey[g0], p_cut);
+        fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, 0u, sh.pkey[g0], p_cut, scale);
         return g0;
     }
     if (tid == 0) sh.members = 0;
@@ -492,7 +494,7 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_mi
     if (add_missing(xlo)) __syncthreads();
     const uint32_t C3 = sh.count;
     if (C3 > kFastCap) {
-        fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, xlo, xhi, p_cut);
+        fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, g0, kk, xlo, xhi, p_cut, scale);
         return g0;
     }
     // the group's members (their indices) side by side, then each counts the members before it
@@ -525,11 +527,17 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_mi
 // then lower index); the fast terms of the k+1 ranked elements are replaced by accurate
 // ones; probabilities for those only; a probability tie across the k-th place is
 // settled over every element of the row with that probability (settle_tie with
-// add_missing); ordered store.  All NT threads call.
+// add_missing); ordered store.  scale: the row's elements count times scale (the keys
+// of the candidates are those of the scaled elements already).  count_out (softmax
+// variant, may be null): receives the nucleus cut of the row's result for top_p -- the
+// smallest m >= 1 whose first m probabilities, added in float front to back, reach
+// top_p, else kk -- the number topp_count_kernel gives on the stored values.
+// All NT threads call.
 template <typename T, int NT, bool SOFTMAX, typename WaveOf, typename AddMissing>
 __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool partial, float M, double s_base, const T *rowp,
                                            T *ov, int32_t *oi, uint32_t n, uint32_t kk, uint32_t want, WaveOf wave_of,
-                                           AddMissing add_missing) {
+                                           AddMissing add_missing, float scale = 1.f, int32_t *count_out = nullptr,
+                                           float top_p = 0.f) {
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1);
     uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
     // ---- E. exact ranks; accurate terms for the ranked elements ----------------
@@ -585,9 +593,9 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
             __syncthreads();
             tie_g0 = sh.g0;
             fill_group_by_scan<T, NT, true>(sh.scan_counts, rowp, ov, oi, n, tie_g0, kk, 0u,
-                                            tie_g0 < C2 ? sh.pkey[tie_g0] : kKeyNegInf, 0.f);
+                                            tie_g0 < C2 ? sh.pkey[tie_g0] : kKeyNegInf, 0.f, scale);
         } else if (C2 > kk && sh.prob[kk - 1] == sh.prob[kk]) {
-            tie_g0 = settle_tie<T, NT>(sh, add_missing, rowp, ov, oi, n, kk, sh.prob[kk], M, rinv);
+            tie_g0 = settle_tie<T, NT>(sh, add_missing, rowp, ov, oi, n, kk, sh.prob[kk], M, rinv, scale);
         }
     } else if (partial) {
         // the -inf elements follow the candidates, lowest indices first
@@ -613,6 +621,31 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
         } else {
             ov[r] = rowp[idx];  // bit copy (keeps the sign of a zero)
             oi[r] = static_cast<int32_t>(idx);
+        }
+    }
+    if constexpr (SOFTMAX) {
+        if (count_out != nullptr && tid < static_cast<uint32_t>(kWave)) {
+            // The stored values in output order: equal probabilities only change places
+            // among themselves, so rank order gives the same sequence; from tie_g0 on every
+            // place holds the tied group's probability (0 when the row ran out of elements
+            // above -inf).  Walked through the lanes in order, as topp_count_kernel does.
+            const float tail = (!partial && kk < C2) ? sh.prob[kk] : 0.f;
+            float sum = 0.f;
+            uint32_t count = kk;
+            for (uint32_t base = 0; base < kk && count == kk; base += kWave) {
+                const uint32_t r = base + lane;
+                const float v = r < kk ? (r < plain ? sh.prob[r] : tail) : 0.f;
+                const uint32_t m = min(static_cast<uint32_t>(kWave), kk - base);
+                for (uint32_t j = 0; j < m; j++) {
+                    sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(
+                                             __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
+                    if (sum >= top_p) {
+                        count = base + j + 1;
+                        break;
+                    }
+                }
+            }
+            if (lane == 0) *count_out = static_cast<int32_t>(count);
         }
     }
 }

@@ -33,9 +33,11 @@ struct ScanWorkspace {
 
 // Launch: rows * G workgroups of kScanThreads; a chunk is exactly 256 * V vectors
 // (G = ceil(n / that)), so that blocks never straddle chunks.
-template <typename T, int V, bool SOFTMAX, bool ALIGNED>
+// SCALED: every element counts times `scale` (a temperature; > 0), one multiplication
+// in single precision before anything else sees it.
+template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED = false>
 __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__restrict__ in, uint32_t n, uint32_t G,
-                                                                 ScanWorkspace ws) {
+                                                                 ScanWorkspace ws, float scale = 1.f) {
     constexpr int NT = kScanThreads, NW = kScanWaves;
     constexpr int VEC = Vec128<T>::N;
     constexpr uint32_t per = static_cast<uint32_t>(NT) * V * VEC;
@@ -71,7 +73,9 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
         auto elem = [&](auto i_tag, int c) {
             constexpr int i = decltype(i_tag)::value;
             const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-            return in_range(ALIGNED ? e0 : e0 + static_cast<uint32_t>(c)) ? q[i].get(c) : -INFINITY;
+            float x = q[i].get(c);
+            if constexpr (SCALED) x = scaled(x, scale);
+            return in_range(ALIGNED ? e0 : e0 + static_cast<uint32_t>(c)) ? x : -INFINITY;
         };
         float ref = 0.f;
         double acc = 0.0;  // every term is added in double: a dominant term must not swallow what follows it
@@ -183,10 +187,13 @@ union PickSharedUnion {
 // select over the whole row.
 constexpr int kPickThreads = 512;
 
+// scale: as in the scan kernel (1 when that ran unscaled); counts (softmax variant,
+// may be null): per row the nucleus cut of its result for top_p (finish_row).
 template <typename T, bool SOFTMAX, bool ALIGNED, int GE, int NT = kPickThreads>
 __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in, T *__restrict__ values,
-                                                                  int32_t *__restrict__ indices, uint32_t n, uint32_t k,
-                                                                  uint32_t G, uint32_t per, ScanWorkspace ws) {
+                                                       int32_t *__restrict__ indices, uint32_t n, uint32_t k, uint32_t G,
+                                                       uint32_t per, ScanWorkspace ws, float scale = 1.f,
+                                                       int32_t *__restrict__ counts = nullptr, float top_p = 0.f) {
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
     constexpr int U = NT >= 1024 ? 2 : NT >= 512 ? 4 : 8;  // loads per thread in flight while blocks are read again (128 blocks a round)
@@ -318,6 +325,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                 store_elem(ov, r, __uint_as_float(0x7FC00000u));
                 oi[r] = static_cast<int32_t>(r);
             }
+            if (counts != nullptr && tid == 0) counts[row] = static_cast<int32_t>(kk);  // (a sum of NaN reaches nothing)
             return;
         }
     }
@@ -379,14 +387,14 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                 bool any_nan = false;
 #pragma unroll
                 for (int c = 0; c < VEC; c++) {
-                    const float x = r[u].get(c);
+                    const float x = scaled(r[u].get(c), scale);
                     vm = fmaxf(vm, x);
                     if constexpr (!SOFTMAX) any_nan = any_nan || x != x;
                 }
                 if (!(vm < lo_f) || any_nan) {
 #pragma unroll
                     for (int c = 0; c < VEC; c++) {
-                        const float x = r[u].get(c);
+                        const float x = scaled(r[u].get(c), scale);
                         const uint32_t idx = e0[u] + static_cast<uint32_t>(c);
                         const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
                         if (idx < cend[u] && key >= lo && static_cast<uint64_t>(key) < hi) {
@@ -420,7 +428,8 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             const uint32_t b = idx / per, off = idx - b * per;
             return b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;
         };
-        finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing);
+        finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing, scale,
+                                   counts != nullptr ? counts + row : nullptr, top_p);
         return;
     }
 
@@ -429,14 +438,36 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     SelectShared &exact = smem.exact;
     if constexpr (SOFTMAX) {
         // the statistics the way the general kernels define them
-        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch);
+        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch, scale);
         select_topk_line<NT>(exact, n, kk, [&](uint32_t j) {
-            return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
+            return order_key(round_to_storage<T>(softmax_prob(scaled(load_elem(rowp, j), scale), st)));
         });
         for (uint32_t r = tid; r < kk; r += NT) {
             const uint32_t idx = composite_index(exact.sel[r]);
-            store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
+            store_elem(ov, r, softmax_prob(scaled(load_elem(rowp, idx), scale), st));
             oi[r] = static_cast<int32_t>(idx);
+        }
+        if (counts != nullptr) {
+            // (rare path: the stored values are read back by the first wave, walked in order)
+            __syncthreads();
+            if (tid < static_cast<uint32_t>(kWave)) {
+                float sum = 0.f;
+                uint32_t count = kk;
+                for (uint32_t base = 0; base < kk && count == kk; base += kWave) {
+                    const uint32_t r = base + lane;
+                    const float v = r < kk ? round_to_storage<T>(softmax_prob(scaled(load_elem(rowp, composite_index(exact.sel[r < kk ? r : 0u])), scale), st)) : 0.f;
+                    const uint32_t m = min(static_cast<uint32_t>(kWave), kk - base);
+                    for (uint32_t j = 0; j < m; j++) {
+                        sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(
+                                                 __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
+                        if (sum >= top_p) {
+                            count = base + j + 1;
+                            break;
+                        }
+                    }
+                }
+                if (lane == 0) counts[row] = static_cast<int32_t>(count);
+            }
         }
     } else {
         select_topk_line<NT>(exact, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });

@@ -72,11 +72,18 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
     const uint32_t ge = (a.ws.blocks + kPickThreads - 1) / kPickThreads;
     if (ge > 16) return false;
     bool scanned = (a.stages & 1) == 0;
-#define VKOP_SCAN_CASE(V)                                                                                      \
-    if (!scanned && a.v == V) {                                                                                \
-        if (a.aligned) rows_scan_kernel<T, V, SOFTMAX, true><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws); \
-        else rows_scan_kernel<T, V, SOFTMAX, false><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws);          \
-        scanned = true;                                                                                        \
+    const bool scaled = SOFTMAX && a.scale != 1.f;
+#define VKOP_SCAN_LAUNCH(V, AL, SC) \
+    rows_scan_kernel<T, V, SOFTMAX, AL, SC><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws, a.scale)
+#define VKOP_SCAN_CASE(V)                                             \
+    if (!scanned && a.v == V) {                                       \
+        if constexpr (SOFTMAX) {                                      \
+            if (scaled && a.aligned) VKOP_SCAN_LAUNCH(V, true, true); \
+            else if (scaled) VKOP_SCAN_LAUNCH(V, false, true);        \
+        }                                                             \
+        if (!scaled && a.aligned) VKOP_SCAN_LAUNCH(V, true, false);   \
+        else if (!scaled) VKOP_SCAN_LAUNCH(V, false, false);          \
+        scanned = true;                                               \
     }
     VKOP_SCAN_CASE(2)
     VKOP_SCAN_CASE(4)
@@ -85,11 +92,12 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
         VKOP_SCAN_CASE(16)
     }
 #undef VKOP_SCAN_CASE
+#undef VKOP_SCAN_LAUNCH
     if (!scanned) return false;
     if ((a.stages & 2) == 0) return true;
 #define VKOP_PICK_LAUNCH(GE, AL)                                                      \
     rows_pick_kernel<T, SOFTMAX, AL, GE><<<a.rows, kPickThreads, 0, a.stream>>>(      \
-        in, static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, per, a.ws)
+        in, static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, per, a.ws, SOFTMAX ? a.scale : 1.f, a.counts, a.top_p)
 #define VKOP_PICK_CASE(GE)                         \
     if (ge <= GE) {                                \
         if (a.aligned) VKOP_PICK_LAUNCH(GE, true); \

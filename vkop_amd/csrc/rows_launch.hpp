@@ -35,6 +35,9 @@ struct ScanLaunch {
     uint32_t g;        // chunks per row
     bool aligned;      // rows start on 16 bytes and n is a multiple of the vector width
     int stages;        // 1 = scan only, 2 = pick only, 3 = both (1 and 2: measurements)
+    float scale;       // softmax variant: every logit times this (1 = the unscaled kernels)
+    int32_t *counts;   // softmax variant: per-row nucleus cut for top_p, or null
+    float top_p;
     ScanWorkspace ws;
     hipStream_t stream;
 };

@@ -536,7 +536,7 @@ int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, 
 
 template <typename T, bool SOFTMAX>
 int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, const ScanCfg &c, void *ws,
-                const RowsLayout &l, hipStream_t st) {
+                const RowsLayout &l, hipStream_t st, float scale = 1.f, int32_t *counts = nullptr, float top_p = 0.f) {
     auto *base = static_cast<unsigned char *>(ws);
     const uint32_t vec = 16 / sizeof(T);
     vkop::ScanLaunch a;
@@ -550,6 +550,9 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.g = c.g;
     a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
     a.stages = g_rows_stages.load();
+    a.scale = scale;
+    a.counts = counts;
+    a.top_p = top_p;
     a.ws.bmax = reinterpret_cast<uint32_t *>(base + l.bmax);
     a.ws.recs = reinterpret_cast<uint64_t *>(base + l.recs);
     a.ws.blocks = c.blocks;
@@ -995,6 +998,52 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     return fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_probs),
                       static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, workspace,
                       as_stream(stream));
+}
+
+int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *out_indices, int32_t *out_counts, int dtype,
+                                   const int *shape, int ndim, int axis, int k, float scale, float top_p, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+    View v;
+    if (int rc = check_dtype(dtype)) return rc;
+    if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (!(scale > 0.f) || !(scale < INFINITY)) return fail(VKOP_HIP_ERR_INVALID, "scale must be positive and finite");
+    if (v.elems == 0 && k == 0) return VKOP_HIP_OK;
+    if (int rc = check_k(v, k)) return rc;
+    if (v.g.outer == 0 || v.g.inner == 0) return VKOP_HIP_OK;
+    if (in == nullptr || out_values == nullptr || out_indices == nullptr)
+        return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
+    if (out_counts != nullptr && v.g.inner != 1)
+        return fail(VKOP_HIP_ERR_UNSUPPORTED, "the nucleus count is defined along the last axis only");
+    const size_t need = selection_workspace(v, k, dtype);
+    if (workspace == nullptr || workspace_bytes < need)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if ((reinterpret_cast<uintptr_t>(workspace) & (kAlign - 1)) != 0)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
+    const hipStream_t st = as_stream(stream);
+    const ScanCfg sc = choose_scan_cfg(v, k, dtype);
+    auto run = [&](auto tag) -> int {
+        using T = decltype(tag);
+        const T *x = static_cast<const T *>(in);
+        T *values = static_cast<T *>(out_values);
+        if (sc.ok) {
+            const RowsLayout l = rows_layout(v, RowsCfg{}, BigKCfg{}, sc);
+            return launch_scan<T, true>(x, values, out_indices, v, k, sc, workspace, l, st, scale, out_counts, top_p);
+        }
+        // every other shape: the line kernels on the scaled elements, then the count on their sorted result
+        const RowsLayout l = rows_layout(v, RowsCfg{}, BigKCfg{});
+        const uint32_t lines = v.g.outer * v.g.inner;
+        auto *stats = reinterpret_cast<vkop::LineStats *>(static_cast<unsigned char *>(workspace) + l.stats);
+        vkop::softmax_lines_kernel<T, kLineThreads>
+            <<<lines, kLineThreads, 0, st>>>(x, static_cast<T *>(nullptr), v.g, 0, 0.f, stats, scale);
+        vkop::softmax_topk_lines_kernel<T, kLineThreads>
+            <<<lines, kLineThreads, 0, st>>>(x, stats, values, out_indices, v.g, static_cast<uint32_t>(k), 1, scale);
+        if (out_counts != nullptr)
+            vkop::topp_count_kernel<T><<<lines, vkop::kWave, 0, st>>>(values, out_counts, static_cast<uint32_t>(k),
+                                                                      static_cast<size_t>(k), top_p);
+        return launched("softmax_lines_kernel / softmax_topk_lines_kernel / topp_count_kernel");
+    };
+    if (dtype == VKOP_HIP_F32) return run(float{});
+    return run(uint16_t{});
 }
 
 int vkop_hip_softmax_topk_static(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape,

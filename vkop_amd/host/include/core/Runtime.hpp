@@ -70,6 +70,14 @@ class Runtime {
             if (ops::convert_opstring_to_enum(n.op_type) == ops::OpType::UNKNOWN || !ops::create_from_type(ops::convert_opstring_to_enum(n.op_type)))
                 throw std::runtime_error("LoadModel: node " + n.name + " needs operator " + n.op_type + ", which this library does not have");
         }
+        // every initializer's data is as long as its dimensions promise (checked before any device work)
+        auto elem_size = [](const std::string &dtype) -> size_t {
+            if (dtype == "int8" || dtype == "uint8" || dtype == "bool") return 1;
+            if (dtype == "float16" || dtype == "bfloat16" || dtype == "int16" || dtype == "uint16") return 2;
+            if (dtype == "int64" || dtype == "uint64" || dtype == "float64") return 8;
+            return 4;
+        };
+        for (const auto &it : model.initializers) (void)model.initializer_data(it.first, elem_size(it.second.dtype));
         auto dev = m_cmdpool_->getVulkanDevice();
         auto make = [this](const std::vector<uint32_t> &dims, bool index, bool on_device = true) -> std::shared_ptr<ITensor> {
             if (index) return std::make_shared<Tensor<int>>(dims, on_device);
@@ -97,7 +105,7 @@ class Runtime {
         }
         for (const auto &it : model.initializers) {
             const auto &init = it.second;
-            const uint8_t *src = model.initializer_data(init.name);
+            const uint8_t *src = model.initializer_data(init.name, elem_size(init.dtype));  // (length checked again)
             auto host_only = [&](auto t, const auto *data) {
                 t->set_ref_cnt_forever();
                 t->fillToCPU(data);

@@ -90,6 +90,20 @@ class VkModel {
     const uint8_t *initializer_data(const std::string &name) const {
         return initializer_memory.data() + initializer_offsets.at(name);
     }
+    // The same, after checking that the initializer's data holds what its dimensions
+    // promise (product of dims elements of elem_size bytes); throws if it is shorter.
+    const uint8_t *initializer_data(const std::string &name, size_t elem_size) const {
+        const auto &init = initializers.at(name);
+        uint64_t elems = 1;
+        for (uint32_t d : init.dims) {
+            elems *= d;
+            if (elems > (1ull << 40)) throw std::runtime_error("Initializer " + name + ": dimensions too large");
+        }
+        if (elems * elem_size > initializer_bytes.at(name))
+            throw std::runtime_error("Initializer " + name + ": " + std::to_string(initializer_bytes.at(name)) + " bytes of data for " +
+                                     std::to_string(elems) + " elements of " + std::to_string(elem_size) + " bytes");
+        return initializer_data(name);
+    }
 
     void dump_model(std::ostream &os = std::cout) const {
         auto shapes = [&os](const char *title, const std::vector<Shape> &list) {
@@ -223,7 +237,7 @@ class VkModel {
         // initializers, packed into one block at 64-byte steps (model/load.cpp:132-178)
         const uint32_t num_init = c.count("initializer list", 20);
         struct Piece {
-            std::string name;
+            size_t at;  // where the piece goes in initializer_memory
             const uint8_t *bytes;
             size_t size;
         };
@@ -237,16 +251,18 @@ class VkModel {
             const int64_t bytes = c.value<int64_t>("initializer size");
             if (bytes < 0) throw std::runtime_error("Negative size of initializer " + init.name);
             const uint8_t *p = c.take(static_cast<uint64_t>(bytes), "initializer data");
+            // (two initializers of one name would leave one offset for two pieces of different sizes)
+            if (initializers.count(init.name)) throw std::runtime_error("Initializer " + init.name + " appears twice");
             const size_t at = (total + 63) & ~static_cast<size_t>(63);
             initializer_offsets[init.name] = at;
             initializer_bytes[init.name] = static_cast<size_t>(bytes);
             total = at + static_cast<size_t>(bytes);
-            pieces.push_back({init.name, p, static_cast<size_t>(bytes)});
+            pieces.push_back({at, p, static_cast<size_t>(bytes)});
             initializers[init.name] = std::move(init);
         }
         initializer_memory.assign(total, 0);
         for (const auto &p : pieces)
-            if (p.size) std::memcpy(initializer_memory.data() + initializer_offsets[p.name], p.bytes, p.size);
+            if (p.size) std::memcpy(initializer_memory.data() + p.at, p.bytes, p.size);
         const uint32_t num_levels = c.count("level list", 4);
         concurrent_execution_levels.resize(num_levels);
         for (auto &level : concurrent_execution_levels)

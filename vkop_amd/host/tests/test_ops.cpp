@@ -624,6 +624,71 @@ static void model_file_tests() {
         EXPECT(it != bytes.end());
         if (it != bytes.end()) EXPECT(broken(static_cast<size_t>(it - bytes.begin()) + 4, 9));  // attribute tag 9
     }
+    {
+        // Files nothing but their initializers: two of one name (the second, shorter one would
+        // leave its offset to the first one's bytes) are refused by the reader; data shorter than
+        // the dimensions promise is refused when a runtime loads the model (it copies
+        // product-of-dims elements); both from exact-size heap blocks.
+        struct Init {
+            std::string name, dtype;
+            std::vector<uint32_t> dims;
+            std::vector<uint8_t> data;
+        };
+        auto file_of = [](const std::vector<Init> &inits) {
+            std::vector<uint8_t> b;
+            auto u32 = [&b](uint32_t v) { for (int i = 0; i < 4; i++) b.push_back(static_cast<uint8_t>(v >> (8 * i))); };
+            auto str = [&](const std::string &t) { u32(static_cast<uint32_t>(t.size())); b.insert(b.end(), t.begin(), t.end()); };
+            u32(0);  // inputs
+            u32(0);  // outputs
+            u32(0);  // nodes
+            u32(static_cast<uint32_t>(inits.size()));
+            for (const auto &i : inits) {
+                str(i.name);
+                str(i.dtype);
+                u32(static_cast<uint32_t>(i.dims.size()));
+                for (uint32_t d : i.dims) u32(d);
+                const uint64_t n = i.data.size();
+                for (int k = 0; k < 8; k++) b.push_back(static_cast<uint8_t>(n >> (8 * k)));
+                b.insert(b.end(), i.data.begin(), i.data.end());
+            }
+            u32(0);  // levels
+            return b;
+        };
+        const auto good = file_of({{"a", "float32", {1024}, std::vector<uint8_t>(4096, 1)}, {"b", "float32", {1}, std::vector<uint8_t>(4, 2)}});
+        const VkModel m(good.data(), good.size());
+        EXPECT(m.initializer_bytes.at("a") == 4096 && m.initializer_offsets.at("b") == 4096 && m.initializer_data("b")[0] == 2);
+        EXPECT(m.initializer_data("a", 4)[4095] == 1);
+        const auto twice = file_of({{"a", "float32", {1024}, std::vector<uint8_t>(4096, 1)}, {"a", "float32", {1}, std::vector<uint8_t>(4, 2)}});
+        bool refused = false;
+        try {
+            const VkModel m2(twice.data(), twice.size());
+        } catch (const std::runtime_error &e) {
+            refused = std::string(e.what()).find("twice") != std::string::npos;
+        }
+        EXPECT(refused);
+        const auto shorter = file_of({{"w", "float32", {1024}, std::vector<uint8_t>(16, 3)}});
+        const VkModel m3(shorter.data(), shorter.size());  // the reader takes it: dims and data are separate fields
+        refused = false;
+        try {
+            (void)m3.initializer_data("w", 4);
+        } catch (const std::runtime_error &e) {
+            refused = std::string(e.what()).find("16 bytes of data for 1024 elements") != std::string::npos;
+        }
+        EXPECT(refused);
+        const std::string tmp = "build/short_initializer.vkopbin";
+        {
+            std::ofstream f(tmp, std::ios::binary);
+            f.write(reinterpret_cast<const char *>(shorter.data()), static_cast<std::streamsize>(shorter.size()));
+        }
+        refused = false;
+        try {
+            vkop::core::Runtime rt(nullptr, tmp, 0);
+            rt.LoadModel();
+        } catch (const std::runtime_error &e) {
+            refused = std::string(e.what()).find("bytes of data for") != std::string::npos;
+        }
+        EXPECT(refused);
+    }
 }
 
 // Models from .vkopbin files through Runtime::LoadModel / Run / ReadResult.

@@ -96,6 +96,23 @@ def softmax_topk(x, k, axis=-1, largest=True, return_probs=False, workspace=None
     return (values, indices, probs) if return_probs else (values, indices)
 
 
+def softmax_topk_sampling(x, k, scale=1.0, top_p=None, axis=-1, workspace=None):
+    """Sampling-style fused call: top-k of softmax(fl32(x * scale)); with top_p also the nucleus count per row.
+    -> (values, indices) or (values, indices, counts)."""
+    x, dt = _prep(x)
+    shape = _out_shape(x, axis, k)
+    values = torch.empty(shape, dtype=x.dtype, device=x.device)
+    indices = torch.empty(shape, dtype=torch.int32, device=x.device)
+    cshape = list(x.shape)
+    del cshape[axis if axis >= 0 else axis + x.dim()]
+    counts = torch.empty(cshape, dtype=torch.int32, device=x.device) if top_p is not None else None
+    ws = workspace or _default_ws
+    ptr, size = ws.get(capi.softmax_topk_workspace_bytes(dt, x.shape, axis, k))
+    capi.softmax_topk_sampling(x.data_ptr(), values.data_ptr(), indices.data_ptr(), counts.data_ptr() if counts is not None else 0,
+                               dt, x.shape, axis, k, scale, top_p if top_p is not None else 0.0, ptr, size, _stream())
+    return (values, indices, counts) if top_p is not None else (values, indices)
+
+
 def softmax_reduce_max(x, axis, workspace=None):
     """max over `axis` of softmax along `axis`, in one read (bit-equal to reduce_max(softmax(x, axis), axis))."""
     x, dt = _prep(x)
