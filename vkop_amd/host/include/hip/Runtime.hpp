@@ -26,6 +26,28 @@
 
 #include "vkop_hip.h"
 
+// The two words of Vulkan vocabulary the reference's operator sources spell out when
+// they call their base class (ops/Softmax.hpp:33-44, ops/Topk.hpp:33-37): the kind of
+// each binding (values as in vulkan_core.h).  Nothing here acts on them; they are kept
+// so that an operator written against the reference's base class compiles.  Global, as
+// in vulkan_core.h, and skipped when that header is already in.
+#ifndef VULKAN_CORE_H_
+enum VkDescriptorType {
+    VK_DESCRIPTOR_TYPE_SAMPLER = 0,
+    VK_DESCRIPTOR_TYPE_COMBINED_IMAGE_SAMPLER = 1,
+    VK_DESCRIPTOR_TYPE_SAMPLED_IMAGE = 2,
+    VK_DESCRIPTOR_TYPE_STORAGE_IMAGE = 3,
+    VK_DESCRIPTOR_TYPE_UNIFORM_TEXEL_BUFFER = 4,
+    VK_DESCRIPTOR_TYPE_STORAGE_TEXEL_BUFFER = 5,
+    VK_DESCRIPTOR_TYPE_UNIFORM_BUFFER = 6,
+    VK_DESCRIPTOR_TYPE_STORAGE_BUFFER = 7
+};
+#endif
+#ifndef DESCRIPTOR_TYPE_STORAGE
+#define DESCRIPTOR_TYPE_STORAGE VK_DESCRIPTOR_TYPE_STORAGE_BUFFER        /* vulkan/VulkanResource.hpp:11 */
+#define DESCRIPTOR_TYPE_UNIFORM VK_DESCRIPTOR_TYPE_UNIFORM_TEXEL_BUFFER  /* vulkan/VulkanResource.hpp:12 */
+#endif
+
 namespace vkop {
 
 constexpr int kInflight = 2;  // queues in flight, as vulkan/VulkanDevice.hpp:13
@@ -165,6 +187,7 @@ class HipCommandBuffer {
 
 // The reference's names, so that caller code written against it still compiles.
 using VulkanDevice = HipDevice;
+using VulkanResource = HipBuffer;  // what a tensor binds (vulkan/VulkanResource.hpp): here always a device buffer
 using VulkanCommandPool = HipCommandPool;
 using VulkanCommandBuffer = HipCommandBuffer;
 using VulkanBuffer = HipBuffer;

@@ -4,10 +4,18 @@
 //   create -> set_runtime_device -> setAttribute -> onExecute (records) ->
 //   caller submits get_record() and waits.
 //
-// What has no counterpart is gone: SPIR-V blobs, descriptor types and sets,
-// push-constant size (the constructor therefore takes only the operator kind
-// and the fp16 flag), the dummy buffer statics.  Errors are C++ exceptions and
-// asserts, as in the reference; the factory returns nullptr for unknown kinds.
+// The constructor and `submit` keep the reference's signatures
+// (ops/Operator.hpp:21-23, 225-238), so an operator written against the reference's
+// base class compiles against this one: the SPIR-V blob, the binding kinds and the
+// push-constant size are taken and kept (types_, pc_size_) but nothing acts on them,
+// and `submit` -- where the reference binds a pipeline, pushes constants and records
+// a dispatch -- has nothing to dispatch here: the operators of this library call the
+// C ABI from execute(), and the base `submit` refuses with an exception naming the
+// operator, so that one ported without a HIP kernel fails loudly instead of doing
+// nothing.  The short constructor (kind, fp16) is what the operators here use.
+// Descriptor sets, pipelines and the dummy buffer statics have no counterpart.
+// Errors are C++ exceptions and asserts, as in the reference; the factory returns
+// nullptr for unknown kinds.
 #ifndef VKOP_HIP_OPS_OPERATOR_HPP_
 #define VKOP_HIP_OPS_OPERATOR_HPP_
 
@@ -31,6 +39,14 @@ namespace ops {
 class Operator {
   public:
     explicit Operator(OpType type, int fp16 = 0) : type_(type), fp16_(fp16) { instance_count_.fetch_add(1); }
+    // the reference's signature (ops/Operator.hpp:21-31)
+    explicit Operator(OpType type, uint8_t *spv, uint32_t spv_len, const std::vector<VkDescriptorType> &types,
+                      size_t pc_size = 0, int fp16 = 0)
+        : type_(type), fp16_(fp16), pc_size_(pc_size), spv_(spv), spv_len_(spv_len), types_(types) {
+        assert(pc_size_ <= 128);
+        instance_count_.fetch_add(1);
+        objs_.reserve(types_.size());
+    }
     virtual ~Operator() { instance_count_.fetch_sub(1); }
     Operator(const Operator &) = delete;
     Operator &operator=(const Operator &) = delete;
@@ -79,6 +95,7 @@ class Operator {
         if (!m_dev_ || !m_cmdpool_) throw std::runtime_error("onExecute before set_runtime_device");
         if (!m_cmd_ || m_cmd_->queue_id() != id) m_cmd_ = std::make_shared<VulkanCommandBuffer>(m_cmdpool_, id);
         m_id_ = id;
+        objs_.clear();  // (ops/Operator.hpp:131)
         m_cmd_->begin();
         execute(inputs, outputs);
         m_cmd_->end();
@@ -106,6 +123,24 @@ class Operator {
     bool trace_ = false;
     std::string name_;
     int fp16_ = 0;  // 0: fp32, 1: fp16
+    // what the reference's constructor is given (kept, not acted on) and what its
+    // operators collect per call before they submit (ops/Operator.hpp:176-199)
+    size_t pc_size_ = 0;
+    uint8_t *spv_ = nullptr;
+    uint32_t spv_len_ = 0;
+    std::vector<VkDescriptorType> types_;
+    std::vector<std::shared_ptr<VulkanResource>> objs_;
+
+    // ops/Operator.hpp:225-238 binds the pipeline and its descriptor set, pushes pc_size_
+    // bytes at `ptr` and records a dispatch of width x height x layers workgroups.  There
+    // is no pipeline here: an operator either overrides this or, like the ones of this
+    // library, calls the C ABI from execute() and never gets here.
+    virtual void submit(void *ptr, int width, int height, int layers) {
+        (void)ptr;
+        throw std::runtime_error("Operator::submit: " + convert_optype_to_string(type_) + " (" + std::to_string(width) + "x" +
+                                 std::to_string(height) + "x" + std::to_string(layers) +
+                                 " workgroups) has no HIP kernel behind it in this library");
+    }
 
     // Calls func(T{}) for the element type `dtype` names; throws for a type no
     // operator here handles (ops/Operator.hpp:198-222).

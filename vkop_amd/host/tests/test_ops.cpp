@@ -332,6 +332,90 @@ void nms_case(const std::vector<int> &box_shape, const std::vector<int> &score_s
     EXPECT(ok);
 }
 
+// An operator written against the reference's base class as it stands
+// (ops/Operator.hpp:21-23 constructor, 225-238 submit; the calling pattern of
+// ops/Softmax.hpp:33-44,120-128): a SPIR-V blob, the kinds of its bindings and the size
+// of its push constants go to the base constructor, execute() collects the bound
+// resources in objs_ and ends in submit(&pc, gx, gy, gz).  It has to compile and run
+// against this library's base unchanged.
+namespace {
+struct DummyPush {
+    int n;
+    float alpha;
+};
+uint8_t g_dummy_spv[8] = {0x03, 0x02, 0x23, 0x07, 0, 0, 1, 0};
+
+class ReferenceStyleOp : public ops::Operator {
+  public:
+    explicit ReferenceStyleOp(bool own_submit)
+        : Operator(ops::OpType::RELU, g_dummy_spv, sizeof(g_dummy_spv),
+                   {VK_DESCRIPTOR_TYPE_STORAGE_IMAGE, VK_DESCRIPTOR_TYPE_COMBINED_IMAGE_SAMPLER, DESCRIPTOR_TYPE_STORAGE},
+                   sizeof(DummyPush)),
+          own_submit_(own_submit) {}
+
+    // what execute() does between collecting its resources and returning, callable
+    // without a device
+    void record(int n) {
+        DummyPush pc{n, 0.5F};
+        objs_.emplace_back(std::shared_ptr<vkop::VulkanResource>());
+        if (types_[2] == DESCRIPTOR_TYPE_STORAGE) submit(&pc, (n + 255) / 256, 1, 1);
+        else submit(&pc, (n + 15) / 16, 16, 1);
+    }
+    size_t pc_size() const { return pc_size_; }
+    size_t bindings() const { return types_.size(); }
+    size_t collected() const { return objs_.size(); }
+    DummyPush seen_pc{};
+    int seen_grid[3] = {0, 0, 0};
+
+  protected:
+    void submit(void *ptr, int width, int height, int layers) override {
+        if (!own_submit_) {
+            Operator::submit(ptr, width, height, layers);
+            return;
+        }
+        std::memcpy(&seen_pc, ptr, pc_size_);
+        seen_grid[0] = width;
+        seen_grid[1] = height;
+        seen_grid[2] = layers;
+    }
+
+  private:
+    void execute(const std::vector<std::shared_ptr<ITensor>> &inputs,
+                 const std::vector<std::shared_ptr<ITensor>> &outputs) override {
+        (void)outputs;
+        record(inputs[0]->size() / 4);
+    }
+    bool own_submit_;
+};
+}  // namespace
+
+static void reference_base_class_tests() {
+    const int before = ops::Operator::instance_count_.load();
+    {
+        ReferenceStyleOp op(true);
+        EXPECT(ops::Operator::instance_count_.load() == before + 1);
+        EXPECT(op.get_type() == ops::OpType::RELU);
+        EXPECT(op.pc_size() == sizeof(DummyPush) && op.bindings() == 3);
+        op.record(1000);
+        EXPECT(op.seen_pc.n == 1000 && op.seen_pc.alpha == 0.5F);
+        EXPECT(op.seen_grid[0] == 4 && op.seen_grid[1] == 1 && op.seen_grid[2] == 1);
+        EXPECT(op.collected() == 1);
+    }
+    {
+        // the base submit has no pipeline to dispatch: it refuses, naming the operator
+        ReferenceStyleOp op(false);
+        std::string msg;
+        try {
+            op.record(64);
+        } catch (const std::runtime_error &e) {
+            msg = e.what();
+        }
+        EXPECT(msg.find("Relu") != std::string::npos);
+        EXPECT(msg.find("1x1x1") != std::string::npos);
+    }
+    EXPECT(ops::Operator::instance_count_.load() == before);
+}
+
 static void host_logic_tests() {
     // names and numbering (ops/Ops.hpp)
     EXPECT(static_cast<int>(ops::OpType::SOFTMAX) == 26);
@@ -919,6 +1003,7 @@ int main(int argc, char **argv) {
     const bool no_gpu = argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0;
     g_golden = (std::filesystem::path(argv[0]).parent_path() / ".." / ".." / ".." / "tests" / "golden").string();
     host_logic_tests();
+    reference_base_class_tests();
     model_file_tests();
     model_file_mutation_tests();
     if (!no_gpu) {
