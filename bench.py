@@ -188,6 +188,9 @@ def main():
     ap.add_argument("--rows-path", type=int, default=0, choices=(0, 1),
                     help="0 = the library's choice of streaming kernels, 1 = the chunk + merge kernels (vkop_hip_tune rows.path)")
     ap.add_argument("--no-gate", action="store_true", help="do not hold the timed replay behind a spin kernel")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch every call from the host instead of replaying recordings (for counter runs under "
+                         "rocprofv3 --pmc, which collects per dispatch; the timings of such a run are not the metric)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of known size (the yardstick for the FETCH_SIZE / "
                          "WRITE_SIZE counters) and print its size")
@@ -287,17 +290,27 @@ def main():
         """One recording per lane: the lane's share of steps first .. first+count-1, in order."""
         graphs = []
         for j in range(nlanes):
+            mine = [i for i in range(first, first + count) if i % nlanes == j]
+            if args.eager:
+                graphs.append(mine)
+                continue
             capi.graph_begin(lanes[j]["stream"])
-            for i in range(first, first + count):
-                if i % nlanes == j:
-                    call(bufs[i % nb], lanes[j])
+            for i in mine:
+                call(bufs[i % nb], lanes[j])
             graphs.append(capi.graph_end(lanes[j]["stream"]))
         return graphs
 
-    def submit(graphs, nlanes):
+    def launch(graph, j, nb):
+        if args.eager:
+            for i in graph:
+                call(bufs[i % nb], lanes[j])
+        else:
+            capi.graph_launch(graph, lanes[j]["stream"])
+
+    def submit(graphs, nlanes, nb):
         fork(nlanes)
         for j in range(nlanes):
-            capi.graph_launch(graphs[j], lanes[j]["stream"])
+            launch(graphs[j], j, nb)
         join(nlanes)
 
     e0, e1 = capi.event_create(), capi.event_create()
@@ -342,7 +355,7 @@ def main():
         if args.warmup > 0:
             gw = record(args.warmup, 0, nlanes, nb)
             graphs += gw
-            submit(gw, nlanes)
+            submit(gw, nlanes, nb)
         gk = record(args.steps, args.warmup, nlanes, nb)
         graphs += gk
 
@@ -350,12 +363,12 @@ def main():
             fork(nlanes)
             for _ in range(replays):
                 for j in range(nlanes):
-                    capi.graph_launch(gk[j], lanes[j]["stream"])
+                    launch(gk[j], j, nb)
             join(nlanes)
         # the recordings that are timed, once untimed: their first launch is not what is measured
         capi.stream_sync(main_stream)
         torch.cuda.synchronize()
-        submit(gk, nlanes)
+        submit(gk, nlanes, nb)
         capi.stream_sync(main_stream)
         torch.cuda.synchronize()
         # host wall clock of the same replays without the gate (submission time included)
@@ -376,8 +389,9 @@ def main():
                   "includes host submission time" % (queued_ms, gate_ms), file=sys.stderr)
         capi.event_sync(e1)
         torch.cuda.synchronize()
-        for g in graphs:
-            capi.graph_destroy(g)
+        if not args.eager:
+            for g in graphs:
+                capi.graph_destroy(g)
         capi.measure_stages(3)
         n = replays * args.steps
         return max(capi.event_elapsed_ms(e0, e1), 0.0) / n, wall / n
@@ -423,7 +437,8 @@ def main():
                    "timing": "HIP events on the launch stream around back-to-back replays of the recorded K steps (at least "
                              "400 steps in all, lanes running free), queued behind a spin kernel (%s); W warm-up steps and "
                              "one untimed replay of the same recordings before them"
-                             % ("%.1f ms" % gate_ms if gate_cycles else "off")},
+                             % ("%.1f ms" % gate_ms if gate_cycles else "off")
+                             if not args.eager else "EAGER host launches (a counter run): these timings are not the metric"},
         "steps_in_timed_region": replays * args.steps,
         "host_wall_ms_per_step": wall_per_step,
         "cache_resident_ms_per_step": resident_ms,

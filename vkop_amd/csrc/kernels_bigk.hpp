@@ -156,11 +156,11 @@ __global__ __launch_bounds__(kBigThreads) void bigk_hist_kernel(const T *__restr
     bigk_load_striped<T, V, ALIGNED>(q, rowp, c0, c1);
     for (uint32_t b = tid; b < BINS; b += kBigThreads) lh[b] = 0;
 
-    uint32_t *state = ws.state + row * 8;
+    uint32_t *state = ws.state + static_cast<size_t>(row) * 8;
     uint32_t want_hi = 0;  // the digits found so far, as the high bits of a key
     if constexpr (PASS == 1) {
         uint32_t d, need;
-        resolve_digit<kBigBins>(ws.hist + (0 * rows + row) * kBigBins, k, scratch, answer, d, need);
+        resolve_digit<kBigBins>(ws.hist + (static_cast<size_t>(0) * rows + row) * kBigBins, k, scratch, answer, d, need);
         if (chunk == 0 && tid == 0) {
             state[0] = d;
             state[1] = need;
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(kBigThreads) void bigk_hist_kernel(const T *__restr
     } else if constexpr (PASS == 2) {
         const uint32_t d0 = state[0], need0 = state[1];
         uint32_t d, need;
-        resolve_digit<kBigBins>(ws.hist + (1 * rows + row) * kBigBins, need0, scratch, answer, d, need);
+        resolve_digit<kBigBins>(ws.hist + (static_cast<size_t>(1) * rows + row) * kBigBins, need0, scratch, answer, d, need);
         if (chunk == 0 && tid == 0) {
             state[2] = d;
             state[3] = need;
@@ -216,10 +216,10 @@ __global__ __launch_bounds__(kBigThreads) void bigk_count_kernel(const T *__rest
     const T *rowp = in + static_cast<size_t>(row) * n;
     Vec128<T> q[V];
     bigk_load_striped<T, V, ALIGNED>(q, rowp, c0, c1);
-    uint32_t *state = ws.state + row * 8;
+    uint32_t *state = ws.state + static_cast<size_t>(row) * 8;
     const uint32_t d0 = state[0], d1 = state[2], need1 = state[3];
     uint32_t d2, need_eq;
-    resolve_digit<1024>(ws.hist + (2 * rows + row) * kBigBins, need1, scratch, answer, d2, need_eq);
+    resolve_digit<1024>(ws.hist + (static_cast<size_t>(2) * rows + row) * kBigBins, need1, scratch, answer, d2, need_eq);
     const uint32_t thr = (d0 << 21) | (d1 << 10) | d2;  // the key of the k-th element
     if (chunk == 0 && tid == 0) {
         state[4] = thr;
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(kBigThreads) void bigk_gather_kernel(const T *__res
             for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < c1 ? e0 + c : 0u));
         }
     }
-    const uint32_t *state = ws.state + row * 8;
+    const uint32_t *state = ws.state + static_cast<size_t>(row) * 8;
     const uint32_t thr = state[4], need_eq = state[5];
     // elements above / equal to the threshold in earlier chunks of the row
     uint32_t cg = 0, ce = 0;
