@@ -29,6 +29,8 @@ struct ScanWorkspace {
     uint64_t *recs;    // [rows][G][kScanWaves][2]: sum of exp(x - ref) over the wave's elements (double bits); ref
                        // (low half) and the wave's maximum (high half) as float bits
     uint32_t blocks;   // blocks per row: ceil(n / (16 * vector width))
+    uint32_t *zero;    // null, or [rows][zero_words] words the scan kernel clears for the kernels behind it
+    uint32_t zero_words;  // (at most 256)
 };
 
 // Launch: rows * G workgroups of kScanThreads; a chunk is exactly 256 * V vectors
@@ -49,6 +51,7 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
     const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
     const T *rowp = in + static_cast<size_t>(row) * n;
     const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
+    if (ws.zero != nullptr && chunk == 0 && tid < ws.zero_words) ws.zero[static_cast<size_t>(row) * ws.zero_words + tid] = 0;
 
     // all loads in flight (never a branch around a load: out-of-chunk lanes read the
     // row's first element(s) instead and are masked where the data is used)

@@ -70,7 +70,8 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
     constexpr uint32_t VEC = 16 / sizeof(T);
     const uint32_t per = kScanThreads * a.v * VEC;
     const uint32_t ge = (a.ws.blocks + kPickThreads - 1) / kPickThreads;
-    if (ge > 16) return false;
+    const uint32_t ge_big = (a.ws.blocks + kBigPickThreads - 1) / kBigPickThreads;
+    if (a.g2 == 0 ? ge > 16 : ge_big > 32) return false;
     bool scanned = (a.stages & 1) == 0;
     const bool scaled = SOFTMAX && a.scale != 1.f;
 #define VKOP_SCAN_LAUNCH(V, AL, SC) \
@@ -95,6 +96,27 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
 #undef VKOP_SCAN_LAUNCH
     if (!scanned) return false;
     if ((a.stages & 2) == 0) return true;
+    if (a.g2 != 0) {
+#define VKOP_BIG_LAUNCH(GE, AL)                                                                  \
+    bigpick_gather_kernel<T, SOFTMAX, AL, GE><<<a.rows * a.g2, kBigPickThreads, 0, a.stream>>>( \
+        in, a.n, a.k, a.g2, a.g, per, a.ws, a.bw)
+#define VKOP_BIG_CASE(GE)                         \
+    if (!gathered && ge_big <= GE) {              \
+        if (a.aligned) VKOP_BIG_LAUNCH(GE, true); \
+        else VKOP_BIG_LAUNCH(GE, false);          \
+        gathered = true;                          \
+    }
+        bool gathered = false;
+        VKOP_BIG_CASE(4)
+        VKOP_BIG_CASE(8)
+        VKOP_BIG_CASE(16)
+        VKOP_BIG_CASE(32)
+#undef VKOP_BIG_CASE
+#undef VKOP_BIG_LAUNCH
+        bigpick_rank_kernel<T, SOFTMAX><<<a.rows * (kBigPickCap / kBigPickMine), kBigPickThreads, 0, a.stream>>>(
+            in, static_cast<T *>(a.values), a.indices, a.n, a.k, a.bw);
+        return true;
+    }
 #define VKOP_PICK_LAUNCH(GE, AL)                                                      \
     rows_pick_kernel<T, SOFTMAX, AL, GE><<<a.rows, kPickThreads, 0, a.stream>>>(      \
         in, static_cast<T *>(a.values), a.indices, a.n, a.k, a.g, per, a.ws, SOFTMAX ? a.scale : 1.f, a.counts, a.top_p)
@@ -118,3 +140,9 @@ template bool launch_rows_chunk<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch
 template void launch_rows_merge<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
 
 }  // namespace vkop
+
+#ifdef VKOP_STAMPS
+extern "C" int VKOP_STAMPS(unsigned long long *out) {
+    return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(vkop::g_bp_stamps), 64 * sizeof(unsigned long long)));
+}
+#endif

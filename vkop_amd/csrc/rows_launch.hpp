@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels_rows.hpp"
+#include "kernels_bigpick.hpp"
 #include "kernels_stream.hpp"
 
 namespace vkop {
@@ -39,9 +40,12 @@ struct ScanLaunch {
     int32_t *counts;   // softmax variant: per-row nucleus cut for top_p, or null
     float top_p;
     ScanWorkspace ws;
+    uint32_t g2;          // 0, or (k beyond the pick kernel's list) workgroups a row of bigpick_gather_kernel
+    BigPickWorkspace bw;  // ... and its candidate lists
     hipStream_t stream;
 };
-// Enqueues rows_scan_kernel and rows_pick_kernel; false if no kernel is built for the shape.
+// Enqueues rows_scan_kernel and rows_pick_kernel (or, with g2 set, the bigpick pair
+// behind the scan); false if no kernel is built for the shape.
 template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a);
 extern template bool launch_rows_scan<float, true>(const ScanLaunch &);
 extern template bool launch_rows_scan<float, false>(const ScanLaunch &);

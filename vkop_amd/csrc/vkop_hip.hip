@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
@@ -385,6 +386,7 @@ struct ScanCfg {
     bool ok = false;
     int v = 0;
     uint32_t g = 0, blocks = 0;
+    uint32_t g2 = 0;  // k beyond the pick kernel's list: workgroups a row of the gather kernel (kernels_bigpick.hpp)
 };
 
 // Long last-axis rows, largest first, k up to kFastMaxK: the scan + pick pair.  The
@@ -394,7 +396,8 @@ struct ScanCfg {
 // (for_size: what a call could use whatever the tuning knobs say at that time)
 ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) {
     ScanCfg c;
-    if (v.g.inner != 1 || k > vkop::kFastMaxK || v.g.n == 0 || v.g.outer == 0) return c;
+    if (v.g.inner != 1 || k > vkop::kMaxK || v.g.n == 0 || v.g.outer == 0) return c;
+    const bool big = k > vkop::kFastMaxK;
     if (!for_size) {
         if (g_rows_path.load() == 1) return c;
         // a forced shape of the other streaming kernels
@@ -403,14 +406,17 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
     const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
     const uint32_t n = v.g.n, rows = v.g.outer;
     const uint32_t blocks = (n + vkop::kBlockLanes * vec - 1) / (vkop::kBlockLanes * vec);
-    if (blocks < 4u * (static_cast<uint32_t>(k) + 1u)) return c;
-    if ((blocks + vkop::kPickThreads - 1) / vkop::kPickThreads > 16u) return c;
+    if (blocks < (big ? 2u : 4u) * (static_cast<uint32_t>(k) + 1u)) return c;
+    if (!big && (blocks + vkop::kPickThreads - 1) / vkop::kPickThreads > 16u) return c;
+    if (big && (blocks + vkop::kBigPickThreads - 1) / vkop::kBigPickThreads > 32u) return c;
+    if (big && static_cast<uint64_t>(rows) * (vkop::kBigPickCap / vkop::kBigPickMine) >= (1ull << 31)) return c;
+    const uint32_t waves_max = big ? static_cast<uint32_t>(vkop::kBigPickRecsMax) : static_cast<uint32_t>(vkop::kMergeWavesMax);
     const int vmax = dtype == VKOP_HIP_F32 ? 16 : 8;
     int pick = 0;
     for (int vv = 2; vv <= vmax; vv *= 2) {
         const uint32_t per = static_cast<uint32_t>(vkop::kScanThreads) * vv * vec;
         const uint32_t g = (n + per - 1) / per;
-        if (g < 2 || g * vkop::kScanWaves > static_cast<uint32_t>(vkop::kMergeWavesMax)) continue;
+        if (g < 2 || g * vkop::kScanWaves > waves_max) continue;
         if (static_cast<uint64_t>(rows) * g >= (1ull << 31)) continue;
         if (pick == 0) pick = vv;
         if (static_cast<uint64_t>(rows) * g >= 512) pick = vv;
@@ -420,6 +426,14 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
     const uint32_t per = static_cast<uint32_t>(vkop::kScanThreads) * pick * vec;
     c.g = (n + per - 1) / per;
     c.blocks = blocks;
+    if (big) {
+        // a share of at most 256 blocks (a thread each) and, rows permitting, of at least 32;
+        // about 512 workgroups in all
+        const uint32_t least = (blocks + 255u) / 256u, most = (blocks + 31u) / 32u;
+        const uint32_t fill = (512u + rows - 1u) / rows;
+        c.g2 = std::max(least, std::min(fill, most));
+        if (static_cast<uint64_t>(rows) * c.g2 >= (1ull << 31)) return c;
+    }
     c.ok = true;
     return c;
 }
@@ -427,7 +441,7 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
 struct RowsLayout {
     size_t tickets = 0, sums = 0, cand = 0, stats = 0, total = 0;
     // scan + pick pair (kernels_stream.hpp)
-    size_t bmax = 0, recs = 0;
+    size_t bmax = 0, recs = 0, bcand = 0, bterm = 0, bhead = 0, bstat = 0;
     // multi-workgroup radix select (kernels_bigk.hpp)
     size_t hist = 0, hist_bytes = 0, state = 0, counts = 0, sel = 0, chunkstats = 0;
 };
@@ -468,6 +482,16 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
         off += align_up(lines * sc.blocks * sizeof(uint32_t));
         l.recs = off;
         off += align_up(lines * sc.g * vkop::kScanWaves * 2 * sizeof(uint64_t));
+        if (sc.g2 != 0) {
+            l.bcand = off;
+            off += align_up(lines * vkop::kBigPickLists * vkop::kBigPickListCap * sizeof(uint64_t));
+            l.bterm = off;
+            off += align_up(lines * vkop::kBigPickLists * vkop::kBigPickListCap * sizeof(float));
+            l.bhead = off;
+            off += align_up(lines * vkop::kBigPickHeadWords * sizeof(uint32_t));
+            l.bstat = off;
+            off += align_up(2 * lines * sizeof(double));
+        }
     } else if (c.ok) {
         const size_t chunks = lines * c.g;
         l.sums = off;
@@ -556,6 +580,18 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.ws.bmax = reinterpret_cast<uint32_t *>(base + l.bmax);
     a.ws.recs = reinterpret_cast<uint64_t *>(base + l.recs);
     a.ws.blocks = c.blocks;
+    a.ws.zero = nullptr;
+    a.ws.zero_words = 0;
+    a.g2 = c.g2;
+    a.bw = vkop::BigPickWorkspace{nullptr, nullptr, nullptr, nullptr};
+    if (c.g2 != 0) {
+        a.bw.cand = reinterpret_cast<uint64_t *>(base + l.bcand);
+        a.bw.term = reinterpret_cast<float *>(base + l.bterm);
+        a.bw.head = reinterpret_cast<uint32_t *>(base + l.bhead);
+        a.bw.stat = reinterpret_cast<double *>(base + l.bstat);
+        a.ws.zero = a.bw.head;
+        a.ws.zero_words = vkop::kBigPickHeadWords;
+    }
     a.stream = st;
     if (!vkop::launch_rows_scan<T, SOFTMAX>(a))
         return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_scan_kernel / rows_pick_kernel for %d loads, %u blocks", c.v, c.blocks);
@@ -1025,7 +1061,7 @@ int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *ou
         using T = decltype(tag);
         const T *x = static_cast<const T *>(in);
         T *values = static_cast<T *>(out_values);
-        if (sc.ok) {
+        if (sc.ok && sc.g2 == 0) {
             const RowsLayout l = rows_layout(v, RowsCfg{}, BigKCfg{}, sc);
             return launch_scan<T, true>(x, values, out_indices, v, k, sc, workspace, l, st, scale, out_counts, top_p);
         }
@@ -1137,7 +1173,8 @@ int vkop_hip_tune(const char *name, int value) {
 int vkop_hip_measure_path(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return -1;
-    if (choose_scan_cfg(v, k, dtype).ok) return 2;
+    const ScanCfg sc = choose_scan_cfg(v, k, dtype);
+    if (sc.ok) return sc.g2 != 0 ? 3 : 2;
     if (choose_rows_cfg(v, k, dtype).ok) return 1;
     return 0;
 }
