@@ -63,7 +63,7 @@ def _rows(kind, rows, n, rng):
         m = rng.random((rows, n)) < (40.0 / n)
         x[~m] = -np.inf
         x[0, :] = -np.inf
-        x[0, 5] = 1.0
+        x[0, min(5, n - 1)] = 1.0
         return x
     if kind == "constant":
         x[:] = np.float32(-2.5)
@@ -147,6 +147,16 @@ def test_scan_with_spread_out_pick_for_large_k_equals_radix_select_and_oracle(op
     select (rows.path = 1) and the oracle -- the regular rows, and the ones the pair hands
     to its exact fallback (constant and masked rows, levels with thousands of equals)."""
     _compare_paths(ops, n, k, dtype, 4, KINDS + ["grid"], 3)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("n,k", [(1000, 5), (1000, 16), (33, 5), (5, 5), (1024, 1), (2048, 7), (777, 10), (256, 3), (64, 16),
+                                 (1001, 5), (130, 2)])
+def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k, dtype):
+    """Short rows, small k (a classifier head): the one-wave-per-row kernel against the
+    chunk kernel (rows.path = 1) and the oracle, on regular rows and on the ones it hands
+    to its exact fallback (ties en masse, masked rows, constant rows)."""
+    _compare_paths(ops, n, k, dtype, 6, KINDS, 4)
 
 
 @pytest.mark.parametrize("n", [16388, 40002, 128255])

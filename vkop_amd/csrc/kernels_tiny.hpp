@@ -1,0 +1,191 @@
+// Short last-axis rows and small k (a classifier head: [batch, 1000], k = 5): one
+// wave per row, the row in its registers, nothing but cross-lane operations between
+// the load and the store -- a latency path: what a call costs here is the launch and
+// one chain of dependent instructions, so the chain is kept short.
+//
+//   1. V 128-bit loads per lane (the row striped over the lanes);
+//   2. the row's maximum; (softmax) the sum of fast terms exp2((x - M) log2 e);
+//   3. the (k+1)-th largest of the 64 lane maxima, by a ballot descent: at least k+1
+//      elements reach it (a probability tie that runs off the end of the candidates:
+//      again with 2 (k+1) + 2 lane maxima, and once more);
+//   4. the elements that reach it -- the candidates, at most 64 -- one per lane;
+//   5. (softmax) their accurate terms replace the fast ones in the sum; each gets its
+//      probability, float(term / sum) rounded to the tensor's type;
+//   6. every candidate counts the candidates that rank before it (larger probability,
+//      or key for a plain top-k; then lower index) and stores itself at that place if
+//      it is below k.
+// A row this cannot settle goes to the exact single-workgroup select over the row
+// (select.hpp) in the same kernel: more than 64 candidates or fewer than k+1 (equal
+// values en masse, rows of -inf), a sum that is not a positive finite number, a tie in
+// probability that runs from the k-th place to the last candidate (an element below
+// the candidates might share it).
+#pragma once
+
+#include "kernels_general.hpp"
+#include "kernels_rows.hpp"
+#include "kernels_softmax.hpp"
+#include "select.hpp"
+
+namespace vkop {
+
+constexpr int kTinyMaxK = 16;
+
+template <typename T, int V, bool SOFTMAX, bool ALIGNED>
+__global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                          int32_t *__restrict__ indices, uint32_t n, uint32_t k) {
+    constexpr int VEC = Vec128<T>::N;
+    constexpr int ELEMS = V * VEC;
+    __shared__ union U {
+        uint64_t cand[kWave];
+        SelectShared exact;
+        __device__ U() {}
+    } smem;
+    __shared__ float fscratch[1];
+    __shared__ double dscratch[1];
+    const uint32_t lane = threadIdx.x;
+    const uint32_t row = blockIdx.x;
+    const T *rowp = in + static_cast<size_t>(row) * n;
+    T *ov = values + static_cast<size_t>(row) * k;
+    int32_t *oi = indices + static_cast<size_t>(row) * k;
+    const uint32_t want = k + 1, kk = min(k, n);
+
+    // ---- 1. the row: element c of vector i of this lane is element (i * 64 + lane) * VEC + c
+    Vec128<T> q[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        const uint32_t e0 = (static_cast<uint32_t>(i) * kWave + lane) * VEC;
+        q[i].v = make_uint4(0, 0, 0, 0);
+        if constexpr (ALIGNED) {
+            q[i].load(rowp + (e0 < n ? e0 : 0u));
+        } else {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < n ? e0 + c : 0u));
+        }
+    }
+    // ---- 2. keys, maximum, sum of fast terms
+    uint32_t key[ELEMS];  // 0: not an element (past the row, or a NaN of the softmax variant)
+    uint32_t lmk = 0;
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+#pragma unroll
+        for (int c = 0; c < VEC; c++) {
+            const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
+            const float x = q[i].get(c);
+            const bool live = e < n && !(SOFTMAX && x != x);
+            key[i * VEC + c] = live ? order_key(x) : 0u;
+            lmk = max(lmk, key[i * VEC + c]);
+            if (e < n) m = fmaxf(m, x);  // (drops NaN)
+        }
+    }
+    float M = 0.f, ref = 0.f;
+    double s_fast = 0.0;
+    bool bad = false;
+    if constexpr (SOFTMAX) {
+        M = wave_max_f32_uniform(m);
+        ref = (M > -INFINITY && M < INFINITY) ? M : 0.f;
+        double acc = 0.0;
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
+                if (e < n) acc += static_cast<double>(fast_term_unbiased(q[i].get(c), ref));  // (a NaN element makes the sum NaN)
+            }
+        }
+        s_fast = wave_sum_f64_uniform(acc);
+        bad = !(s_fast > 0.0 && s_fast < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY);
+    }
+    // Steps 3 to 6, at most three times: with k+1 lane maxima, then with twice and four
+    // times as many when a probability tie runs off the end of the candidates.
+    bool exact = bad;
+    for (uint32_t lanes_wanted = want; !exact; lanes_wanted = 2u * lanes_wanted + 2u) {
+        // ---- 3. the lanes_wanted-th largest lane maximum, to 22 bits (-inf never becomes a candidate)
+        uint32_t thr = 0;
+        for (int bit = 31; bit >= 10; bit--) {
+            const uint32_t trial = thr | (1u << bit);
+            if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= lanes_wanted) thr = trial;
+        }
+        thr = max(thr, kKeyNegInf + 1u);
+        // ---- 4. the candidates, in LDS one after the other, then one per lane
+        uint32_t C = 0;  // wave-uniform
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const bool pass = key[i * VEC + c] >= thr;
+                const uint64_t mask = __ballot(pass);
+                if (mask != 0ull) {  // (wave-uniform)
+                    const uint32_t at = C + lanes_below(mask);
+                    const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
+                    if (pass && at < static_cast<uint32_t>(kWave)) smem.cand[at] = composite(key[i * VEC + c], e);
+                    C += static_cast<uint32_t>(__popcll(mask));
+                }
+            }
+        }
+        __syncthreads();  // (one wave: the list is written)
+        if (C > static_cast<uint32_t>(kWave) || C < min(want, n)) break;
+        const bool have = lane < C;
+        uint64_t mine = have ? smem.cand[lane] : 0ull;
+        __syncthreads();  // (the list may be written again)
+        if constexpr (SOFTMAX) {
+            // ---- 5. accurate terms for the candidates, the corrected sum, probabilities
+            const float xv = ordered_to_float(static_cast<uint32_t>(mine >> 32));
+            const float term = have ? softmax_term(xv, M) : 0.f;
+            const double cr = have ? static_cast<double>(term) - static_cast<double>(fast_term_unbiased(xv, ref)) : 0.0;
+            const double total = s_fast + wave_sum_f64_uniform(cr);
+            const float p = round_to_storage<T>(static_cast<float>(static_cast<double>(term) * (1.0 / total)));
+            mine = have ? ((static_cast<uint64_t>(order_key(p)) << 32) | (mine & 0xFFFFFFFFull)) : 0ull;
+        }
+        // ---- 6. ranks among the candidates
+        const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
+        uint32_t before = 0;
+        for (uint32_t c = 0; c < C; c++) {
+            const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), static_cast<int>(c)))) << 32) |
+                                   static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_lo), static_cast<int>(c)));
+            before += (other > mine) ? 1u : 0u;
+        }
+        if constexpr (SOFTMAX) {
+            // a probability shared by the k-th place and the last candidate may go on below the candidates
+            if (C < n && C > kk) {
+                const uint64_t at_cut = __ballot(have && before == kk - 1u), at_end = __ballot(have && before == C - 1u);
+                const uint32_t p_cut = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), __builtin_ctzll(at_cut)));
+                const uint32_t p_end = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), __builtin_ctzll(at_end)));
+                if (p_cut == p_end) {
+                    if (lanes_wanted >= static_cast<uint32_t>(kWave)) break;
+                    continue;  // more candidates
+                }
+            }
+        }
+        if (have && before < kk) {
+            const uint32_t idx = composite_index(mine);
+            if constexpr (SOFTMAX) store_elem(ov, before, ordered_to_float(mine_hi));
+            else ov[before] = rowp[idx];  // bit copy (keeps the sign of a zero)
+            oi[before] = static_cast<int32_t>(idx);
+        }
+        return;
+    }
+    // ---- the exact select over the whole row -----------------------------------------------
+    __syncthreads();  // LDS changes owner
+    SelectShared &ex = smem.exact;
+    if constexpr (SOFTMAX) {
+        const LineStats st = line_stats<T, kWave>(rowp, 0, n, 1, fscratch, dscratch, 1.f);
+        select_topk_line<kWave>(ex, n, kk, [&](uint32_t j) {
+            return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
+        });
+        for (uint32_t r = lane; r < kk; r += kWave) {
+            const uint32_t idx = composite_index(ex.sel[r]);
+            store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
+            oi[r] = static_cast<int32_t>(idx);
+        }
+    } else {
+        select_topk_line<kWave>(ex, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
+        for (uint32_t r = lane; r < kk; r += kWave) {
+            const uint32_t idx = composite_index(ex.sel[r]);
+            ov[r] = rowp[idx];
+            oi[r] = static_cast<int32_t>(idx);
+        }
+    }
+}
+
+}  // namespace vkop

@@ -135,6 +135,28 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
     return false;
 }
 
+template <typename T, bool SOFTMAX> bool launch_rows_tiny(const TinyLaunch &a) {
+#define VKOP_TINY_CASE(V)                                                                              \
+    if (a.v == V) {                                                                                    \
+        if (a.aligned)                                                                                 \
+            rows_tiny_kernel<T, V, SOFTMAX, true><<<a.rows, kWave, 0, a.stream>>>(                     \
+                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k);        \
+        else                                                                                           \
+            rows_tiny_kernel<T, V, SOFTMAX, false><<<a.rows, kWave, 0, a.stream>>>(                    \
+                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k);        \
+        return true;                                                                                   \
+    }
+    VKOP_TINY_CASE(1)
+    VKOP_TINY_CASE(2)
+    VKOP_TINY_CASE(4)
+    if constexpr (sizeof(T) == 4) {
+        VKOP_TINY_CASE(8)
+    }
+#undef VKOP_TINY_CASE
+    return false;
+}
+
+template bool launch_rows_tiny<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const TinyLaunch &);
 template bool launch_rows_scan<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const ScanLaunch &);
 template bool launch_rows_chunk<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);
 template void launch_rows_merge<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch &);

@@ -10,6 +10,7 @@
 #include "kernels_rows.hpp"
 #include "kernels_bigpick.hpp"
 #include "kernels_stream.hpp"
+#include "kernels_tiny.hpp"
 
 namespace vkop {
 
@@ -51,6 +52,21 @@ extern template bool launch_rows_scan<float, true>(const ScanLaunch &);
 extern template bool launch_rows_scan<float, false>(const ScanLaunch &);
 extern template bool launch_rows_scan<uint16_t, true>(const ScanLaunch &);
 extern template bool launch_rows_scan<uint16_t, false>(const ScanLaunch &);
+
+// Enqueues rows_tiny_kernel (one wave per row, v 128-bit loads per lane); false if no kernel is built for v.
+struct TinyLaunch {
+    const void *in;
+    void *values;
+    int32_t *indices;
+    uint32_t rows, n, k, v;
+    bool aligned;
+    hipStream_t stream;
+};
+template <typename T, bool SOFTMAX> bool launch_rows_tiny(const TinyLaunch &a);
+extern template bool launch_rows_tiny<float, true>(const TinyLaunch &);
+extern template bool launch_rows_tiny<float, false>(const TinyLaunch &);
+extern template bool launch_rows_tiny<uint16_t, true>(const TinyLaunch &);
+extern template bool launch_rows_tiny<uint16_t, false>(const TinyLaunch &);
 
 // Enqueues rows_chunk_kernel; false if no kernel is built for (nt, v).
 template <typename T, bool SOFTMAX> bool launch_rows_chunk(const RowsLaunch &a);

@@ -380,6 +380,35 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
     return c;
 }
 
+// Short last-axis rows, largest first, k up to kTinyMaxK: one wave per row
+// (kernels_tiny.hpp); v = 128-bit loads per lane, 0 = not for this tensor.
+int choose_tiny_loads(const View &v, int k, int dtype) {
+    if (v.g.inner != 1 || k < 1 || k > vkop::kTinyMaxK || v.g.n == 0 || v.g.outer == 0) return 0;
+    if (g_rows_path.load() == 1) return 0;
+    if (g_rows_threads.load() > 0 && g_rows_loads.load() > 0 && g_rows_chunks.load() > 0) return 0;
+    const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
+    const int vmax = dtype == VKOP_HIP_F32 ? 8 : 4;
+    for (int vv = 1; vv <= vmax; vv *= 2)
+        if (static_cast<uint32_t>(vkop::kWave) * vv * vec >= v.g.n) return vv;
+    return 0;
+}
+
+template <typename T, bool SOFTMAX>
+int launch_tiny(const T *in, T *values, int32_t *indices, const View &v, int k, int loads, hipStream_t st) {
+    vkop::TinyLaunch a;
+    a.in = in;
+    a.values = values;
+    a.indices = indices;
+    a.rows = v.g.outer;
+    a.n = v.g.n;
+    a.k = static_cast<uint32_t>(k);
+    a.v = static_cast<uint32_t>(loads);
+    a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % (16 / sizeof(T)) == 0);
+    a.stream = st;
+    if (!vkop::launch_rows_tiny<T, SOFTMAX>(a)) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_tiny_kernel for %d loads", loads);
+    return launched("rows_tiny_kernel");
+}
+
 // Launch shape of the streaming pair rows_scan_kernel + rows_pick_kernel: 256 threads,
 // V 128-bit loads per thread, G chunks per row; blocks = 256-byte blocks per row.
 struct ScanCfg {
@@ -646,6 +675,7 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
 template <typename T>
 int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int dtype, void *ws,
               size_t ws_bytes, hipStream_t st) {
+    if (const int tiny = largest ? choose_tiny_loads(v, k, dtype) : 0) return launch_tiny<T, false>(in, values, indices, v, k, tiny, st);
     const ScanCfg sc = largest ? choose_scan_cfg(v, k, dtype) : ScanCfg{};
     const RowsCfg c = (largest && !sc.ok) ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
     const BigKCfg b = (c.ok || sc.ok) ? BigKCfg{} : choose_bigk_cfg(v, k, dtype);
@@ -688,6 +718,8 @@ FusedPlan plan_fused(const View &v, int k, int dtype, int largest, bool want_pro
 template <typename T>
 int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, int dtype,
                void *ws, hipStream_t st) {
+    if (const int tiny = (largest && probs == nullptr) ? choose_tiny_loads(v, k, dtype) : 0)
+        return launch_tiny<T, true>(in, values, indices, v, k, tiny, st);
     const FusedPlan p = plan_fused(v, k, dtype, largest, probs != nullptr);
     const RowsLayout l = rows_layout(v, p.rows, p.big, p.scan);
     if (p.scan.ok) return launch_scan<T, true>(in, values, indices, v, k, p.scan, ws, l, st);
@@ -1173,6 +1205,7 @@ int vkop_hip_tune(const char *name, int value) {
 int vkop_hip_measure_path(int dtype, const int *shape, int ndim, int axis, int k) {
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v) || k < 1) return -1;
+    if (choose_tiny_loads(v, k, dtype) != 0) return 4;
     const ScanCfg sc = choose_scan_cfg(v, k, dtype);
     if (sc.ok) return sc.g2 != 0 ? 3 : 2;
     if (choose_rows_cfg(v, k, dtype).ok) return 1;
@@ -1190,6 +1223,12 @@ int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k, i
     View v;
     if (int rc = check_dtype(dtype)) return rc;
     if (int rc = make_view(shape, ndim, axis, &v)) return rc;
+    if (const int tiny = choose_tiny_loads(v, k, dtype)) {
+        if (threads != nullptr) *threads = vkop::kWave;
+        if (loads != nullptr) *loads = tiny;
+        if (chunks != nullptr) *chunks = 1;
+        return VKOP_HIP_OK;
+    }
     const ScanCfg sc = k >= 1 ? choose_scan_cfg(v, k, dtype) : ScanCfg{};
     if (sc.ok) {
         if (threads != nullptr) *threads = vkop::kScanThreads;
