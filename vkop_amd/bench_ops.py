@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Times every operator of the library on the five reference workloads.
 
-  python -m vkop_amd.bench_ops [--steps K] [--warmup W] [--only NAME_SUBSTRING]
+  python -m vkop_amd.bench_ops [--steps K] [--warmup W] [--only NAME_SUBSTRING] [--eager]
 
 bench.py at the repository root measures the headline (fused softmax -> top-k on
 [64,128256]); this script covers the rest: plain softmax, plain top-k, the fused
@@ -25,6 +25,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--only", default="")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch every call from the host instead of replaying a recording (for counter runs under "
+                         "rocprofv3 --pmc; the timings of such a run mean nothing)")
     args = ap.parse_args()
 
     import numpy as np
@@ -49,6 +52,12 @@ def main():
         return ws, ptr
 
     def timed(call, nbuf):
+        if args.eager:
+            for i in range(args.warmup + args.steps):
+                call(i % nbuf)
+            capi.stream_sync(stream)
+            return None
+
         def record(count, first):
             capi.graph_begin(stream)
             for i in range(first, first + count):
@@ -68,6 +77,9 @@ def main():
         return ms / args.steps * 1e3
 
     def report(name, us, algo_bytes):
+        if us is None:
+            print(json.dumps({"case": name, "eager": True, "algorithmic_bytes": algo_bytes}), flush=True)
+            return
         print(json.dumps({"case": name, "us_per_call": round(us, 2), "algorithmic_bytes": algo_bytes,
                           "algorithmic_GBps": round(algo_bytes / us / 1e3, 1),
                           "frac_of_8TBps": round(algo_bytes / us / 1e3 / 8000.0, 4)}), flush=True)
@@ -175,6 +187,9 @@ def main():
         us = timed(lambda b: capi.nms(bx.data_ptr(), sc.data_ptr(), out.data_ptr(), cap, count.data_ptr(), F32, B, C, N, 0,
                                       per_class, iou_thr, score_thr, ptr, nb + 256, stream), 1)
         m = int(count.cpu()[0])
+        if us is None:
+            print(json.dumps({"case": name, "eager": True, "selected": m}), flush=True)
+            return
         print(json.dumps({"case": name, "us_per_call": round(us, 2), "selected": m,
                           "algorithmic_bytes": boxes.nbytes + scores.nbytes + 12 * m,
                           "algorithmic_GBps": round((boxes.nbytes + scores.nbytes + 12 * m) / us / 1e3, 1)}), flush=True)

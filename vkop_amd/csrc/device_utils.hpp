@@ -65,6 +65,22 @@ __device__ __forceinline__ uint32_t composite_index(uint64_t c) {
     return 0xFFFFFFFFu - static_cast<uint32_t>(c);
 }
 
+// ------------------------------------------------------- block order ----
+// Workgroups are handed to the chip's 8 XCDs in turn (workgroup b runs on XCD b mod 8),
+// and each XCD has an L2 of its own: two workgroups with neighbouring blockIdx never
+// share one.  For kernels whose neighbouring pieces of work touch the same cache lines
+// (rows of a slab that do not start on a line boundary), this gives the position in
+// the work's own order that workgroup blockIdx.x should take so that neighbouring
+// pieces run on one XCD: XCD x takes the x-th eighth of the pieces.  A bijection on
+// [0, gridDim.x).
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ uint32_t xcd_grouped_block() {
+    const uint32_t nb = gridDim.x, b = blockIdx.x;
+    const uint32_t xcd = b % kXcds, local = b / kXcds;
+    const uint32_t each = nb / kXcds, rem = nb % kXcds;  // the first `rem` XCDs get one piece more
+    return xcd * each + min(xcd, rem) + local;
+}
+
 // ---------------------------------------------------------- reductions ----
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -106,7 +106,7 @@ __global__ __launch_bounds__(NT) void reduce_max_strided_kernel(const T *__restr
     constexpr uint32_t P = 4, LPW = kWave / P, U = 8;
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t part = lane / LPW;
-    const uint32_t wave_id = (blockIdx.x * NT + threadIdx.x) / kWave;
+    const uint32_t wave_id = (xcd_grouped_block() * NT + threadIdx.x) / kWave;  // (neighbouring lines share cache lines)
     const uint32_t lines = g.outer * g.inner;
     const uint32_t line_raw = wave_id * LPW + (lane % LPW);
     const bool live = line_raw < lines;

@@ -229,7 +229,8 @@ __global__ __launch_bounds__(kStridedThreads) void softmax_strided_reg_kernel(co
     constexpr int NPER = NMAX / P;  // elements per lane
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t part = lane / LPW;
-    const uint32_t wave_id = (blockIdx.x * kStridedThreads + threadIdx.x) / kWave;
+    // (neighbouring groups of lines share cache lines where rows of the slab start off a line boundary)
+    const uint32_t wave_id = (xcd_grouped_block() * kStridedThreads + threadIdx.x) / kWave;
     const uint32_t lines = g.outer * g.inner;
     const uint32_t line_raw = wave_id * LPW + (lane % LPW);
     const bool live = line_raw < lines;

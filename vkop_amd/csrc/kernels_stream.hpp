@@ -289,33 +289,41 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // bounds is reached by k+1 thread maxima in all, hence by k+1 blocks.  A share of
     // more than half a wave, or a wave without enough live threads, leaves it to one
     // wave and all the maxima.
-    const uint32_t quota = (want + NW - 1) / NW;
-    uint32_t mine_q = 0;
-    if (quota <= 32u) {
-        for (int bit = 31; bit > 13; bit--) {
-            const uint32_t trial = mine_q | (1u << bit);
-            if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= quota) mine_q = trial;
+    // (all threads call, each with its own maximum; the first barrier inside also
+    // publishes the row's maximum and sum of phase B)
+    // by_quota false: one wave and all the maxima at once (waves that are not alike -- a
+    // sorted row -- make the smallest of the waves' bounds far too low).
+    auto threshold_of_thread_maxima = [&](uint32_t mine_max, bool by_quota) -> uint32_t {
+        const uint32_t quota = (want + NW - 1) / NW;
+        uint32_t mine_q = 0;
+        if (by_quota && quota <= 32u) {
+            for (int bit = 31; bit > 13; bit--) {
+                const uint32_t trial = mine_q | (1u << bit);
+                if (static_cast<uint32_t>(__popcll(__ballot(mine_max >= trial))) >= quota) mine_q = trial;
+            }
         }
-    }
-    sh.lane_key[tid] = lmk;
-    if (lane == 0) sh.wave_thr[wave] = mine_q;
-    __syncthreads();
+        sh.lane_key[tid] = mine_max;
+        if (lane == 0) sh.wave_thr[wave] = mine_q;
+        __syncthreads();
+        uint32_t t = sh.wave_thr[0];
+#pragma unroll
+        for (int w = 1; w < NW; w++) t = min(t, sh.wave_thr[w]);
+        if (t <= 1u) {  // (the same for every thread)
+            if (wave == 0) {
+                const uint32_t f = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
+                if (lane == 0) sh.thr = f;
+            }
+            __syncthreads();
+            t = sh.thr;
+        }
+        return t;
+    };
+    uint32_t thr = threshold_of_thread_maxima(lmk, true);
     float M = 0.f;
     double s_base = 0.0;
     if constexpr (SOFTMAX) {
         M = sh.row_max;
         s_base = sh.total;
-    }
-    uint32_t thr = sh.wave_thr[0];
-#pragma unroll
-    for (int w = 1; w < NW; w++) thr = min(thr, sh.wave_thr[w]);
-    if (thr <= 1u) {  // (the same for every thread)
-        if (wave == 0) {
-            const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
-            if (lane == 0) sh.thr = t;
-        }
-        __syncthreads();
-        thr = sh.thr;
     }
     // -inf never becomes a candidate: a row with k+1 larger elements does not need it,
     // and finish_row fills any other row's last places from the row itself
@@ -338,7 +346,10 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // than kPickHitCap blocks reach lo: nothing was gathered then.
     uint32_t round = 0;
     // (always inlined: a call would put the block keys, captured by reference, into scratch memory)
-    auto gather = [&](uint32_t lo, uint64_t hi) __attribute__((always_inline)) -> bool {
+    // dry_tag true: nothing is appended; dry_max becomes the largest key this thread saw in [lo, hi).
+    uint32_t dry_max = 0;
+    auto gather = [&](uint32_t lo, uint64_t hi, auto dry_tag) __attribute__((always_inline)) -> bool {
+        constexpr bool DRY = decltype(dry_tag)::value;
         uint32_t wave_n = 0;  // wave-uniform
 #pragma unroll
         for (int e = 0; e < GE; e++) wave_n += static_cast<uint32_t>(__popcll(__ballot(gk[e] >= lo)));
@@ -401,8 +412,12 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                         const uint32_t idx = e0[u] + static_cast<uint32_t>(c);
                         const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
                         if (idx < cend[u] && key >= lo && static_cast<uint64_t>(key) < hi) {
-                            const uint32_t at = atomicAdd(&sh.count, 1u);
-                            if (at < static_cast<uint32_t>(kFastCap)) sh.cand[at] = composite(key, idx);
+                            if constexpr (DRY) {
+                                dry_max = max(dry_max, key);
+                            } else {
+                                const uint32_t at = atomicAdd(&sh.count, 1u);
+                                if (at < static_cast<uint32_t>(kFastCap)) sh.cand[at] = composite(key, idx);
+                            }
                         }
                     }
                 }
@@ -411,8 +426,26 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         __syncthreads();
         return false;
     };
-    const bool many_groups = gather(thr, 1ull << 32);
-    const uint32_t C2 = sh.count;
+    bool many_groups = gather(thr, 1ull << 32, std::false_type{});
+    uint32_t C2 = sh.count;
+    if (!many_groups && C2 > static_cast<uint32_t>(kFastCap)) {
+        // More elements at or above thr than the list holds although only k+1 and a few
+        // blocks reach it: those blocks' maxima are alike and so are their other elements
+        // (a sorted row; the waves' shares of the block maxima are then not alike either, and
+        // thr is lower than it need be).  The same step once more, a level down: every
+        // thread takes the largest of the elements it reads from those blocks, and the
+        // (k+1)-th largest of these thread maxima is a threshold as good as thr -- k+1
+        // elements reach it, and whatever reaches it lies in a block whose maximum does --
+        // and far tighter.
+        dry_max = 0;
+        gather(thr, 1ull << 32, std::true_type{});
+        const uint32_t tight = threshold_of_thread_maxima(dry_max, false);  // (the barrier at the end of gather lies between this and the last use of its LDS)
+        if (tid == 0) sh.count = 0;
+        __syncthreads();
+        thr = max(thr, tight);
+        many_groups = gather(thr, 1ull << 32, std::false_type{});
+        C2 = sh.count;
+    }
     if (!many_groups && C2 <= static_cast<uint32_t>(kFastCap)) {
         // Fewer than k+1 candidates: fewer than k+1 blocks hold an element above -inf,
         // every one of them was read again, and the rest of the row is -inf.
@@ -420,7 +453,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         // members of a tie across the k-th place below the value used above
         auto add_missing = [&](uint32_t xlo) -> bool {
             if (xlo >= thr) return false;
-            if (gather(xlo, thr)) {
+            if (gather(xlo, thr, std::false_type{})) {
                 if (tid == 0) sh.count = kFastCap + 1;  // too many to collect: the scan from the row's start
                 __syncthreads();
             }
