@@ -183,6 +183,13 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
         const uint32_t b = static_cast<uint32_t>(e) * NT + tid;
         gk[e] = bmax[b < blocks ? b : 0u];
     }
+    const uint32_t *bmin = ws.bmin + static_cast<size_t>(row) * blocks;
+    uint32_t gn[GE];  // the same blocks' minima
+#pragma unroll
+    for (int e = 0; e < GE; e++) {
+        const uint32_t b = static_cast<uint32_t>(e) * NT + tid;
+        gn[e] = bmin[b < blocks ? b : 0u];
+    }
     const uint32_t share = (blocks + G2 - 1) / G2;
     const uint32_t myb = part * share + tid;  // this thread's block of the workgroup's share
     const bool mine_live = tid < share && myb < blocks;
@@ -202,6 +209,7 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
     for (int e = 0; e < GE; e++) {
         const bool live = static_cast<uint32_t>(e) * NT + tid < blocks && gk[e] > kKeyNegInf;
         if (!live) gk[e] = 0;  // (0: not a key)
+        if (!live) gn[e] = 0;
         kmax = max(kmax, gk[e]);
         kmin = live ? min(kmin, gk[e]) : kmin;
         nlive += static_cast<uint32_t>(__popcll(__ballot(live)));  // wave-uniform
@@ -288,12 +296,87 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
             floor_key = cand_thr;
         }
     }
-    const uint32_t lo = bigpick_lowered<T, SOFTMAX>(thr);
+    uint32_t lo = bigpick_lowered<T, SOFTMAX>(thr);
+    // ---- clustered rows -------------------------------------------------------------------------
+    // Blocks whose MINIMUM reaches thr hold 16 * VEC elements that do.  When the blocks that
+    // reach lo are known to hold more candidates than a row's lists (a sorted row: k+1 blocks
+    // reach thr and all but one are such blocks; a row of one value: every block is), two
+    // facts about the block minima make the candidates few again without a look at the
+    // elements:
+    //  * m = ceil((k+1) / (16 * VEC)) block minima reach their m-th largest, so k+1 elements
+    //    reach it: a threshold as valid as thr and, on such rows, far higher;
+    //  * in index order, let B be the first block at which the count "all of a block whose
+    //    minimum reaches thr, one of a block whose maximum does" comes to k+1: k+1 elements
+    //    at or above thr lie in blocks up to B, so an element at or below thr in a later
+    //    block has k+1 elements in front of it that rank no lower and come first -- it is
+    //    not part of the result, nor of any tie that decides it, and is left out.
+    uint32_t last_block_for_equals = 0xFFFFFFFFu;
+    {
+        uint32_t c2 = 0;  // (wave-uniform) blocks whose minimum reaches thr, high half; blocks whose maximum reaches lo, low half
+#pragma unroll
+        for (int e = 0; e < GE; e++)
+            c2 += (static_cast<uint32_t>(__popcll(__ballot(gn[e] >= thr && gk[e] != 0u))) << 16) +
+                  static_cast<uint32_t>(__popcll(__ballot(gk[e] >= lo)));
+        flip ^= 1u;
+        const uint32_t both = bigpick_count_sum(c2, cslots[flip]);
+        const uint32_t nfull = both >> 16, nhit = both & 0xFFFFu;
+        if (nfull * BE + (nhit - nfull) > static_cast<uint32_t>(kBigPickCap)) {  // (the same for every thread of every workgroup of the row)
+            const uint32_t m = (want + BE - 1) / BE;
+            uint32_t tmin = 0;
+            for (int bit = 31; bit >= 10; bit--) {
+                const uint32_t trial = tmin | (1u << bit);
+                uint32_t c = 0;
+#pragma unroll
+                for (int e = 0; e < GE; e++) c += static_cast<uint32_t>(__popcll(__ballot(gn[e] >= trial && gk[e] != 0u)));
+                flip ^= 1u;
+                if (bigpick_count_sum(c, cslots[flip]) >= m) tmin = trial;
+            }
+            if (tmin > thr) {
+                thr = tmin;
+                lo = bigpick_lowered<T, SOFTMAX>(thr);
+            }
+            // per block, in index order, how many elements at or above thr it is KNOWN to hold
+            uint16_t *known = reinterpret_cast<uint16_t *>(lcand);  // (8192 entries; the list is not in use yet)
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < GE; e++) {
+                const uint32_t b = static_cast<uint32_t>(e) * NT + tid;
+                if (b < 8192u) known[b] = static_cast<uint16_t>(gk[e] == 0u ? 0u : gn[e] >= thr ? BE : gk[e] >= thr ? 1u : 0u);
+            }
+            for (uint32_t b = static_cast<uint32_t>(GE) * NT + tid; b < 8192u; b += NT) known[b] = 0;
+            if (tid == 0) answer[0] = 0xFFFFFFFFu;
+            __syncthreads();
+            if (tid < static_cast<uint32_t>(kWave)) {
+                // lane L owns blocks 128 L .. 128 L + 127 (summed in rotated order: lanes on different banks)
+                uint32_t sum = 0;
+                for (uint32_t j = 0; j < 128u; j++) sum += known[lane * 128u + ((j + 2u * lane) & 127u)];
+                uint32_t incl = sum;  // sum over lanes <= this one
+#pragma unroll
+                for (int o = 1; o < kWave; o <<= 1) {
+                    const uint32_t t = __shfl_up(incl, o, kWave);
+                    if (lane >= static_cast<uint32_t>(o)) incl += t;
+                }
+                uint32_t before = incl - sum;
+                if (before < want && want <= incl) {
+                    for (uint32_t j = 0; j < 128u; j++) {
+                        before += known[lane * 128u + j];
+                        if (before >= want) {
+                            answer[0] = lane * 128u + j;
+                            break;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+            last_block_for_equals = answer[0];
+            __syncthreads();  // (the list's LDS is free again)
+        }
+    }
     if (part == 0 && tid == 0) head[16 * kBigPickLists] = thr;
     BPS(3);
 
     // ---- the blocks of this workgroup's share that reach lo --------------------------------
-    const bool pass = mine_live && mykey >= lo;
+    const bool pass = mine_live && mykey >= lo && (myb <= last_block_for_equals || mykey > thr);
     const uint64_t mask = __ballot(pass);
     if (lane == 0) wave_hits[wave] = static_cast<uint32_t>(__popcll(mask));
     __syncthreads();
@@ -344,7 +427,7 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
                     const float x = r[u].get(c);
                     const uint32_t idx = e0[u] + static_cast<uint32_t>(c);
                     const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
-                    if (idx < cend[u] && key >= lo) {
+                    if (idx < cend[u] && key >= lo && (key > thr || idx / BE <= last_block_for_equals)) {
                         const uint32_t at = atomicAdd(&lcount, 1u);
                         if (at < static_cast<uint32_t>(kBigPickListCap)) lcand[at] = composite(key, idx);
                     }

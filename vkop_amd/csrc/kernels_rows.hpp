@@ -375,21 +375,19 @@ template <> struct Vec128<uint16_t> {
     }
 };
 
-// Places g0 .. kk-1 of a row's result go to the lowest-index elements whose order
-// key lies in [xlo, xhi] (a group of equal rank too large to collect): the row is
-// read from its start, NT * 4 elements at a time, until enough members are found
-// -- soon, for a group that large.  SOFTMAX: every member's value is tie_value (the
-// group's probability); otherwise the element itself.  counts: 2 * NT / 64 words
-// of LDS.  scale: the keys are those of the elements times scale (1: as they are).
-// All NT threads call.
-template <typename T, int NT, bool SOFTMAX>
-__device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *rowp, T *ov, int32_t *oi, uint32_t n,
-                                                   uint32_t g0, uint32_t kk, uint32_t xlo, uint32_t xhi, float tie_value,
-                                                   float scale = 1.f) {
+// The first `places` elements of a row, in index order, whose order key lies in
+// [xlo, xhi]: the row is read from its start, NT * 4 elements at a time, until enough
+// are found -- soon, when they are many, which is when this is used.  emit(pos, j) is
+// called by the thread that read element j, the pos-th such element (pos < places).
+// counts: 2 * NT / 64 words of LDS.  scale: the keys are those of the elements times
+// scale (1: as they are).  All NT threads call; returns how many were found (the same
+// in every thread; at least `places` unless the row has fewer).
+template <typename T, int NT, typename Emit>
+__device__ __forceinline__ uint32_t first_members_by_scan(uint32_t *counts, const T *rowp, uint32_t n, uint32_t places,
+                                                          uint32_t xlo, uint32_t xhi, float scale, Emit emit) {
     constexpr int NW = NT / kWave;
     constexpr int U = 4;
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t places = kk - g0;
     uint32_t found = 0;  // the same in every thread
     uint32_t round = 0;
     for (uint32_t base = 0; base < n && found < places; base += NT * U, round++) {
@@ -419,16 +417,28 @@ __device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *ro
 #pragma unroll
         for (int u = 0; u < U; u++) {
             if (member[u]) {
-                if (pos < places) {
-                    if constexpr (SOFTMAX) store_elem(ov, g0 + pos, tie_value);
-                    else ov[g0 + pos] = rowp[j0 + u];
-                    oi[g0 + pos] = static_cast<int32_t>(j0 + u);
-                }
+                if (pos < places) emit(pos, j0 + static_cast<uint32_t>(u));
                 pos++;
             }
         }
         found += in_tile;
     }
+    return found;
+}
+
+// Places g0 .. kk-1 of a row's result go to the lowest-index elements whose order
+// key lies in [xlo, xhi] (a group of equal rank too large to collect).  SOFTMAX:
+// every member's value is tie_value (the group's probability); otherwise the element
+// itself.  All NT threads call.
+template <typename T, int NT, bool SOFTMAX>
+__device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *rowp, T *ov, int32_t *oi, uint32_t n,
+                                                   uint32_t g0, uint32_t kk, uint32_t xlo, uint32_t xhi, float tie_value,
+                                                   float scale = 1.f) {
+    first_members_by_scan<T, NT>(counts, rowp, n, kk - g0, xlo, xhi, scale, [&](uint32_t pos, uint32_t j) {
+        if constexpr (SOFTMAX) store_elem(ov, g0 + pos, tie_value);
+        else ov[g0 + pos] = rowp[j];
+        oi[g0 + pos] = static_cast<int32_t>(j);
+    });
 }
 
 // A probability tie across the k-th place.  Probability is monotone in the logit,

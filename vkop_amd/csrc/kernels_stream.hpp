@@ -29,6 +29,8 @@ struct ScanWorkspace {
     uint64_t *recs;    // [rows][G][kScanWaves][2]: sum of exp(x - ref) over the wave's elements (double bits); ref
                        // (low half) and the wave's maximum (high half) as float bits
     uint32_t blocks;   // blocks per row: ceil(n / (16 * vector width))
+    uint32_t *bmin;    // null, or (WITH_MIN) [rows][blocks]: order key of the block's minimum (NaN dropped; the key
+                       // of -inf for a block that reaches past the row's end or holds -inf)
     uint32_t *zero;    // null, or [rows][zero_words] words the scan kernel clears for the kernels behind it
     uint32_t zero_words;  // (at most 256)
 };
@@ -37,7 +39,9 @@ struct ScanWorkspace {
 // (G = ceil(n / that)), so that blocks never straddle chunks.
 // SCALED: every element counts times `scale` (a temperature; > 0), one multiplication
 // in single precision before anything else sees it.
-template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED = false>
+// WITH_MIN: the blocks' minima as well (for the large-k kernels behind it: a block whose
+// minimum reaches a value holds 16 * vector width elements that do).
+template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED = false, bool WITH_MIN = false>
 __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__restrict__ in, uint32_t n, uint32_t G,
                                                                  ScanWorkspace ws, float scale = 1.f) {
     constexpr int NT = kScanThreads, NW = kScanWaves;
@@ -46,6 +50,7 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
     constexpr int WB = V * (kWave / kBlockLanes);  // blocks a wave covers: V vectors x 4 rows of 16 lanes
     static_assert(WB <= kWave, "a lane per block of the wave");
     __shared__ float vm_lds[NW][V][kWave];  // per wave: the maximum of every lane's vector i
+    __shared__ float vmin_lds[WITH_MIN ? NW : 1][WITH_MIN ? V : 1][kWave];
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
     const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
@@ -91,6 +96,12 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                 xv[c] = elem(i_tag, c);
                 vm = fmaxf(vm, xv[c]);  // (drops NaN)
             }
+            if constexpr (WITH_MIN) {
+                float vn = INFINITY;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) vn = fminf(vn, xv[c]);  // (an element past the chunk's end counts as -inf)
+                vmin_lds[wave][i][lane] = vn;
+            }
             if constexpr (SOFTMAX) {
                 if constexpr (i == 0) {
                     // reference of the wave's partial sum: kRefLift above the maximum of its
@@ -133,6 +144,16 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
             if (FULL || e_block < c1) {
                 const uint32_t key = b_nan ? 0xFFFFFFFFu : order_key(bm);
                 ws.bmax[static_cast<size_t>(row) * ws.blocks + e_block / (kBlockLanes * VEC)] = key;
+                if constexpr (WITH_MIN) {
+                    const float4 *srcn = reinterpret_cast<const float4 *>(&vmin_lds[wave][0][0] + lane * kBlockLanes);
+                    float bn = INFINITY;
+#pragma unroll
+                    for (int j = 0; j < kBlockLanes / 4; j++) {
+                        const float4 v4 = srcn[j];
+                        bn = fminf(fminf(bn, fminf(v4.x, v4.y)), fminf(v4.z, v4.w));
+                    }
+                    ws.bmin[static_cast<size_t>(row) * ws.blocks + e_block / (kBlockLanes * VEC)] = order_key(bn);
+                }
             }
         }
         // ---- the wave's record ---------------------------------------------------------------
@@ -446,12 +467,53 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         many_groups = gather(thr, 1ull << 32, std::false_type{});
         C2 = sh.count;
     }
+    // Still too many: equal values en masse AT the threshold (rows of few distinct
+    // values, constant rows).  k+1 elements reach thr, so the row's k+1 largest are the
+    // elements above it -- fewer than k+1, or thr + 1 is the threshold to use -- and then
+    // the first elements equal to it, in index order: those are found by reading the row
+    // from its start, where a value this frequent turns up at once.
+    bool first_equals_only = false;  // the candidates hold only some of the elements equal to thr
+    if ((many_groups || C2 > static_cast<uint32_t>(kFastCap)) && thr < 0xFFFFFFFFu) {
+        __syncthreads();
+        if (tid == 0) sh.count = 0;
+        __syncthreads();
+        const bool many_above = gather(thr + 1u, 1ull << 32, std::false_type{});
+        const uint32_t above = sh.count;
+        many_groups = true;  // (the exact select, unless one of the two cases below applies)
+        if (!many_above && above <= static_cast<uint32_t>(kFastCap)) {
+            if (above >= want) {
+                thr += 1u;
+                C2 = above;
+                many_groups = false;
+            } else {
+                const uint32_t need = want - above, at = thr;
+                const uint32_t found = first_members_by_scan<T, NT>(sh.scan_counts, rowp, n, need, at, at, scale,
+                                                                    [&](uint32_t pos, uint32_t j) { sh.cand[above + pos] = composite(at, j); });
+                __syncthreads();
+                if (found >= need) {
+                    if (tid == 0) sh.count = want;
+                    __syncthreads();
+                    C2 = want;
+                    first_equals_only = true;
+                    many_groups = false;
+                }
+            }
+        }
+    }
     if (!many_groups && C2 <= static_cast<uint32_t>(kFastCap)) {
         // Fewer than k+1 candidates: fewer than k+1 blocks hold an element above -inf,
         // every one of them was read again, and the rest of the row is -inf.
         const bool partial = C2 < min(want, n);
         // members of a tie across the k-th place below the value used above
         auto add_missing = [&](uint32_t xlo) -> bool {
+            if (first_equals_only) {
+                // the tied group reaches into values the candidates hold only in part: its
+                // places are filled from the row's start, whatever the list holds
+                __syncthreads();
+                if (tid == 0) sh.count = kFastCap + 1;
+                __syncthreads();
+                return true;
+            }
             if (xlo >= thr) return false;
             if (gather(xlo, thr, std::false_type{})) {
                 if (tid == 0) sh.count = kFastCap + 1;  // too many to collect: the scan from the row's start

@@ -76,7 +76,14 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
     const bool scaled = SOFTMAX && a.scale != 1.f;
 #define VKOP_SCAN_LAUNCH(V, AL, SC) \
     rows_scan_kernel<T, V, SOFTMAX, AL, SC><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws, a.scale)
+#define VKOP_SCAN_MIN_LAUNCH(V, AL) \
+    rows_scan_kernel<T, V, SOFTMAX, AL, false, true><<<a.rows * a.g, kScanThreads, 0, a.stream>>>(in, a.n, a.g, a.ws, 1.f)
 #define VKOP_SCAN_CASE(V)                                             \
+    if (!scanned && a.v == V && a.g2 != 0) {                          \
+        if (a.aligned) VKOP_SCAN_MIN_LAUNCH(V, true);                 \
+        else VKOP_SCAN_MIN_LAUNCH(V, false);                          \
+        scanned = true;                                               \
+    }                                                                 \
     if (!scanned && a.v == V) {                                       \
         if constexpr (SOFTMAX) {                                      \
             if (scaled && a.aligned) VKOP_SCAN_LAUNCH(V, true, true); \
@@ -93,6 +100,7 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
         VKOP_SCAN_CASE(16)
     }
 #undef VKOP_SCAN_CASE
+#undef VKOP_SCAN_MIN_LAUNCH
 #undef VKOP_SCAN_LAUNCH
     if (!scanned) return false;
     if ((a.stages & 2) == 0) return true;

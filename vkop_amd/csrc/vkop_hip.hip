@@ -470,7 +470,7 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
 struct RowsLayout {
     size_t tickets = 0, sums = 0, cand = 0, stats = 0, total = 0;
     // scan + pick pair (kernels_stream.hpp)
-    size_t bmax = 0, recs = 0, bcand = 0, bterm = 0, bhead = 0, bstat = 0;
+    size_t bmax = 0, recs = 0, bmin = 0, bcand = 0, bterm = 0, bhead = 0, bstat = 0;
     // multi-workgroup radix select (kernels_bigk.hpp)
     size_t hist = 0, hist_bytes = 0, state = 0, counts = 0, sel = 0, chunkstats = 0;
 };
@@ -512,6 +512,8 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
         l.recs = off;
         off += align_up(lines * sc.g * vkop::kScanWaves * 2 * sizeof(uint64_t));
         if (sc.g2 != 0) {
+            l.bmin = off;
+            off += align_up(lines * sc.blocks * sizeof(uint32_t));
             l.bcand = off;
             off += align_up(lines * vkop::kBigPickLists * vkop::kBigPickListCap * sizeof(uint64_t));
             l.bterm = off;
@@ -609,6 +611,7 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.ws.bmax = reinterpret_cast<uint32_t *>(base + l.bmax);
     a.ws.recs = reinterpret_cast<uint64_t *>(base + l.recs);
     a.ws.blocks = c.blocks;
+    a.ws.bmin = nullptr;
     a.ws.zero = nullptr;
     a.ws.zero_words = 0;
     a.g2 = c.g2;
@@ -618,6 +621,7 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
         a.bw.term = reinterpret_cast<float *>(base + l.bterm);
         a.bw.head = reinterpret_cast<uint32_t *>(base + l.bhead);
         a.bw.stat = reinterpret_cast<double *>(base + l.bstat);
+        a.ws.bmin = reinterpret_cast<uint32_t *>(base + l.bmin);
         a.ws.zero = a.bw.head;
         a.ws.zero_words = vkop::kBigPickHeadWords;
     }
