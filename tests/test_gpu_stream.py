@@ -73,10 +73,30 @@ def _rows(kind, rows, n, rng):
         x[:, n // 3] += 40.0
         x[2, 17::4099] += 25.0
         return x
+    if kind == "tenth":       # one value everywhere, not a round one (its key has low bits set)
+        x[:] = np.float32(0.1)
+        x[rows - 1, :] = np.float32(-7.3)
+        return x
+    if kind == "two_values":
+        return np.where(rng.random((rows, n)) < 0.5, np.float32(1.7), np.float32(1.7000002)).astype(np.float32)
+    if kind == "sorted_desc":
+        return np.ascontiguousarray(np.sort(x, axis=1)[:, ::-1])
+    if kind == "flat_with_peaks":   # one value, and a few larger ones scattered over the row
+        x[:] = np.float32(-0.3)
+        for r in range(rows):
+            at = rng.choice(n, size=min(n, 3 + 2 * r), replace=False)
+            x[r, at] = np.float32(2.0) + rng.random(at.size).astype(np.float32)
+        return x
+    if kind == "runs":        # sorted inside runs of 4096: clustered, not sorted as a whole
+        x = x.copy()
+        for s0 in range(0, n, 4096):
+            x[:, s0:s0 + 4096] = np.sort(x[:, s0:s0 + 4096], axis=1)
+        return x
     raise ValueError(kind)
 
 
 KINDS = ["llm", "bf16", "levels", "sorted", "masked", "constant", "spikes"]
+TIE_KINDS = ["tenth", "two_values", "sorted_desc", "flat_with_peaks", "runs"]
 
 
 def _compare_paths(ops, n, k, dtype, rows, kinds, path):
@@ -157,6 +177,17 @@ def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k
     chunk kernel (rows.path = 1) and the oracle, on regular rows and on the ones it hands
     to its exact fallback (ties en masse, masked rows, constant rows)."""
     _compare_paths(ops, n, k, dtype, 6, KINDS, 4)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (262144, 1024, 3), (300000, 600, 3), (1000, 5, 4), (2048, 16, 4)])
+def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtype):
+    """Rows that defeat a threshold taken from block or lane maxima -- one value everywhere
+    (with a key that is not a round number), two values a float apart, rows sorted
+    downwards, a flat row with a few peaks, rows sorted in runs -- settled by each route's
+    own means (a second threshold, the first elements equal to the tie value, block
+    minima), against the other kernels and the oracle."""
+    _compare_paths(ops, n, k, dtype, 4, TIE_KINDS, path)
 
 
 @pytest.mark.parametrize("n", [16388, 40002, 128255])

@@ -292,6 +292,31 @@ __device__ __forceinline__ float fast_term(float x, float m) {
     return __builtin_amdgcn_exp2f((x - m) * 1.44269504088896341f);
 }
 
+// The same term with the argument's rounding taken back out: a = fl(d log2 e) goes to
+// the hardware unit, and what the rounding dropped (from a fused multiply-add, plus the
+// low part of log2 e) comes back as a first-order factor: 2^(a + l) = 2^a (1 + l ln 2),
+// |l| < 1e-6.  The hardware unit's one ulp is then all the error there is (fast_term's
+// argument alone is good to about |d| 2^-24 absolute: 1.4 ulp of the term at d = -3).
+// For rows that few waves sum: one repeated value that carries most of a row's sum and
+// is not among the ranked elements puts its term's error, the same every time, into
+// every probability of the row -- a flat row with a few peaks came out 4 ulp off with
+// fast_term, against a bar of 2; on long rows hundreds of waves with references of their
+// own spread that error.  Four instructions more per element.
+__device__ __forceinline__ float fast_term_reduced(float x, float m) {
+    const float d = x - m;
+    constexpr float kHi = 1.44269502162933349609375f;  // float(log2 e)
+    constexpr float kLo = 1.925963033500011e-8f;       // log2 e - kHi
+    const float a = d * kHi;
+    const float l = fmaf(d, kLo, fmaf(d, kHi, -a));  // (d = -inf: NaN, and so is the product below -- see the select)
+    const float e = __builtin_amdgcn_exp2f(a);
+    const float t = fmaf(e, l * 0.693147180559945309f, e);
+    return e > 0.f && e < INFINITY ? t : e;  // (0, inf and NaN as the hardware unit gives them)
+}
+template <bool REDUCED> __device__ __forceinline__ float fast_term_as(float x, float m) {
+    if constexpr (REDUCED) return fast_term_reduced(x, m);
+    else return fast_term(x, m);
+}
+
 // A wave sums its terms against a reference taken from the first vectors it
 // receives, so that the exponentials overlap the loads still in flight: kRefLift
 // above the maximum of those vectors.  Should a later element lie more than
@@ -441,6 +466,39 @@ __device__ __forceinline__ void fill_group_by_scan(uint32_t *counts, const T *ro
     });
 }
 
+// The smallest order key whose probability (prob_of_key, non-decreasing in the key) is
+// still p_cut, given one key `member` that has it: a 64-way search, one evaluation per
+// lane and round.  Called by all 64 lanes of one wave; the same answer in every lane.
+template <typename ProbOfKey>
+__device__ __forceinline__ uint32_t lowest_key_of_probability(uint32_t member, float p_cut, ProbOfKey prob_of_key) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    // invariant: probability(b) == p_cut, probability(a) < p_cut (a = 0 stands for "below everything")
+    uint64_t a = 0, b = member;
+    {
+        // First the keys b - 1, b - 2, b - 4, ...: the interval is usually a few keys
+        // wide (one, for float logits away from 0), and this finds its size class at once.
+        const uint32_t off = lane < 32 ? (1u << lane) : 0xFFFFFFFFu;
+        const uint64_t probe = b > off ? b - off : 0;
+        const bool in = probe != 0 && prob_of_key(static_cast<uint32_t>(probe)) >= p_cut;  // true ... true false ... false
+        const int f = __ffsll(static_cast<long long>(~__ballot(in))) - 1;                   // lanes 32.. are false: f >= 0
+        a = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f));
+        if (f > 0) b = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f > 0 ? f - 1 : 0));
+    }
+    while (b - a > 1) {
+        const uint64_t step = (b - a + 63) / 64;
+        uint64_t probe = a + step * (lane + 1);
+        probe = probe < b ? probe : b;
+        const bool in = prob_of_key(static_cast<uint32_t>(probe)) >= p_cut;  // false ... false true ... true
+        const int f = __ffsll(static_cast<long long>(__ballot(in))) - 1;      // lane 63 probes b: f >= 0
+        const uint32_t blo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f));
+        const uint32_t alo = f > 0 ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f > 0 ? f - 1 : 0))
+                                   : static_cast<uint32_t>(a);
+        b = blo;
+        a = alo;
+    }
+    return static_cast<uint32_t>(b);
+}
+
 // A probability tie across the k-th place.  Probability is monotone in the logit,
 // so the tied group is an interval of logits [x_lo, x_hi]: x_hi is the logit at
 // the group's first rank g0, x_lo is found by a 64-way search over order keys (six
@@ -472,30 +530,7 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_mi
     }
     if (tid == 0) sh.members = 0;
     if (wave == 0) {
-        // invariant: probability(b) == p_cut, probability(a) < p_cut (a = 0 stands for "below everything")
-        uint64_t a = 0, b = sh.pkey[kk];
-        {
-            // First the keys b - 1, b - 2, b - 4, ...: the interval is usually a few keys
-            // wide (one, for float logits away from 0), and this finds its size class at once.
-            const uint32_t off = lane < 32 ? (1u << lane) : 0xFFFFFFFFu;
-            const uint64_t probe = b > off ? b - off : 0;
-            const bool in = probe != 0 && prob_of_key(static_cast<uint32_t>(probe)) >= p_cut;  // true ... true false ... false
-            const int f = __ffsll(static_cast<long long>(~__ballot(in))) - 1;                   // lanes 32.. are false: f >= 0
-            a = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f));
-            if (f > 0) b = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f > 0 ? f - 1 : 0));
-        }
-        while (b - a > 1) {
-            const uint64_t step = (b - a + 63) / 64;
-            uint64_t probe = a + step * (lane + 1);
-            probe = probe < b ? probe : b;
-            const bool in = prob_of_key(static_cast<uint32_t>(probe)) >= p_cut;  // false ... false true ... true
-            const int f = __ffsll(static_cast<long long>(__ballot(in))) - 1;      // lane 63 probes b: f >= 0
-            const uint32_t blo = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f));
-            const uint32_t alo = f > 0 ? static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(static_cast<uint32_t>(probe)), f > 0 ? f - 1 : 0))
-                                       : static_cast<uint32_t>(a);
-            b = blo;
-            a = alo;
-        }
+        const uint32_t b = lowest_key_of_probability(sh.pkey[kk], p_cut, prob_of_key);
         if (lane == 0) sh.xlo = static_cast<uint32_t>(b);
     }
     __syncthreads();
@@ -543,7 +578,8 @@ __device__ __forceinline__ uint32_t settle_tie(RowsShared &sh, AddMissing add_mi
 // smallest m >= 1 whose first m probabilities, added in float front to back, reach
 // top_p, else kk -- the number topp_count_kernel gives on the stored values.
 // All NT threads call.
-template <typename T, int NT, bool SOFTMAX, typename WaveOf, typename AddMissing>
+// REDUCED: the waves summed fast_term_reduced (else fast_term).
+template <typename T, int NT, bool SOFTMAX, bool REDUCED = false, typename WaveOf, typename AddMissing>
 __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool partial, float M, double s_base, const T *rowp,
                                            T *ov, int32_t *oi, uint32_t n, uint32_t kk, uint32_t want, WaveOf wave_of,
                                            AddMissing add_missing, float scale = 1.f, int32_t *count_out = nullptr,
@@ -572,7 +608,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
                 // what the element should contribute, exp(fl(x - M)), minus what
                 // its wave added for it, fast_term(x, ref) * exp(ref - M)
                 term = softmax_term(xv, M);
-                cr = static_cast<double>(term) - static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
+                cr = static_cast<double>(term) - static_cast<double>(fast_term_as<REDUCED>(xv, sh.ref[sp])) * sh.scale[sp];
             }
             sh.prob[r] = term;  // scaled to a probability below
             sh.corr[r] = cr;
@@ -665,7 +701,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
 // threads; G << cap_shift <= kMergeRecsMax, G <= kMergeChunksMax,
 // G * src_nt / 64 <= kMergeWavesMax (the host checks all three).
 // RECS: candidate slots the merge can take in (a multiple of NT).
-template <typename T, int NT, bool SOFTMAX, int RECS = kMergeRecsMax>
+template <typename T, int NT, bool SOFTMAX, int RECS = kMergeRecsMax, bool REDUCED = false>
 __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, float *fscratch, double *dscratch,
                                           const T *rowp, T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
                                           uint32_t per, uint32_t src_nt, const uint64_t *sums,
@@ -955,7 +991,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                 const uint32_t b = idx / per, off = idx - b * per;
                 return b * src_nw + ((off / VEC) % src_nt) / kWave;
             };
-            finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing);
+            finish_row<T, NT, SOFTMAX, REDUCED>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing);
             return;
         }
     }
@@ -1062,6 +1098,23 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         float lmax = -INFINITY, ref = 0.f;
         double acc = 0.0;
         uint32_t lkey = 0u;
+        if constexpr (SOFTMAX && LOCAL) {
+            // A row in one workgroup is summed by a few waves, and against the ROW's maximum:
+            // fl(x - ref) is then the subtraction the softmax definition itself rounds.  (Against
+            // a reference of the wave's own, that rounding -- up to 2 ulp of the term at
+            // x - ref = -5 -- is an error, the same for every element of one value; where
+            // hundreds of waves share a row their references differ and it averages out, here
+            // it would not.)  The row is short: waiting for all of it costs little.
+            float pm = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) pm = fmaxf(pm, in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY);
+            }
+            const float row_max = block_max_fast<NT>(pm, fscratch);
+            ref = (row_max > -INFINITY && row_max < INFINITY) ? row_max : 0.f;
+        }
 #pragma unroll
         for (int i = 0; i < V; i++) {
             const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
@@ -1079,7 +1132,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             lmax = fmaxf(lmax, vm);
             lkey = max(lkey, vk);
             if constexpr (SOFTMAX) {
-                if (i == 0) {
+                if (i == 0 && !LOCAL) {
                     // reference of the wave's partial sum: the maximum of its first
                     // vectors; 0 if they hold no finite element (terms are then 0, or
                     // NaN, which must survive -- never -inf - -inf)
@@ -1087,7 +1140,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
                 }
 #pragma unroll
-                for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(xv[c], ref));
+                for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term_as<LOCAL>(xv[c], ref));  // (a row in one workgroup: few waves)
             }
         }
         if constexpr (SOFTMAX) lkey = in_range(e_first) ? order_key(lmax) : 0u;
@@ -1252,7 +1305,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
 #pragma unroll
                     for (int c = 0; c < VEC; c++) {
                         const float x = in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY;
-                        acc += static_cast<double>(fast_term(x, ref));
+                        acc += static_cast<double>(fast_term_as<LOCAL>(x, ref));
                     }
                 }
                 wsum = wave_sum_f64_uniform(acc);
@@ -1417,7 +1470,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
     }
     if constexpr (LOCAL) {
         __syncthreads();  // the list and the records are in LDS; so is what the merge builds, in other arrays
-        merge_row<T, NT, SOFTMAX, kLocalCap>(smem.fast, smem.exact, fscratch, dscratch, rowp,
+        merge_row<T, NT, SOFTMAX, kLocalCap, true>(smem.fast, smem.exact, fscratch, dscratch, rowp,
                                              values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k, n, k,
                                              1u, per, NT, local_ws + kLocalCap, local_ws, ws.cap_shift);
         (void)s_last;

@@ -314,7 +314,9 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // publishes the row's maximum and sum of phase B)
     // by_quota false: one wave and all the maxima at once (waves that are not alike -- a
     // sorted row -- make the smallest of the waves' bounds far too low).
-    auto threshold_of_thread_maxima = [&](uint32_t mine_max, bool by_quota) -> uint32_t {
+    // bits: how many leading bits of the answer are worked out when one wave does it (32:
+    // the exact (k+1)-th largest, the key of an element).
+    auto threshold_of_thread_maxima = [&](uint32_t mine_max, bool by_quota, int bits = 20) -> uint32_t {
         const uint32_t quota = (want + NW - 1) / NW;
         uint32_t mine_q = 0;
         if (by_quota && quota <= 32u) {
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         for (int w = 1; w < NW; w++) t = min(t, sh.wave_thr[w]);
         if (t <= 1u) {  // (the same for every thread)
             if (wave == 0) {
-                const uint32_t f = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
+                const uint32_t f = block_kth_largest_floor<NW>(sh.lane_key, want, bits);
                 if (lane == 0) sh.thr = f;
             }
             __syncthreads();
@@ -449,6 +451,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     };
     bool many_groups = gather(thr, 1ull << 32, std::false_type{});
     uint32_t C2 = sh.count;
+    uint32_t level_max = lmk;  // the thread maxima the current threshold was taken from
     if (!many_groups && C2 > static_cast<uint32_t>(kFastCap)) {
         // More elements at or above thr than the list holds although only k+1 and a few
         // blocks reach it: those blocks' maxima are alike and so are their other elements
@@ -460,6 +463,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         // and far tighter.
         dry_max = 0;
         gather(thr, 1ull << 32, std::true_type{});
+        level_max = dry_max;
         const uint32_t tight = threshold_of_thread_maxima(dry_max, false);  // (the barrier at the end of gather lies between this and the last use of its LDS)
         if (tid == 0) sh.count = 0;
         __syncthreads();
@@ -473,6 +477,12 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // the first elements equal to it, in index order: those are found by reading the row
     // from its start, where a value this frequent turns up at once.
     bool first_equals_only = false;  // the candidates hold only some of the elements equal to thr
+    if (many_groups || C2 > static_cast<uint32_t>(kFastCap)) {
+        // (thr so far is a value rounded down; this needs the key of an element: the exact
+        // (k+1)-th largest of the thread maxima it came from)
+        __syncthreads();
+        thr = max(thr, threshold_of_thread_maxima(level_max, false, 32));
+    }
     if ((many_groups || C2 > static_cast<uint32_t>(kFastCap)) && thr < 0xFFFFFFFFu) {
         __syncthreads();
         if (tid == 0) sh.count = 0;

@@ -14,11 +14,12 @@
 //   6. every candidate counts the candidates that rank before it (larger probability,
 //      or key for a plain top-k; then lower index) and stores itself at that place if
 //      it is below k.
-// A row this cannot settle goes to the exact single-workgroup select over the row
-// (select.hpp) in the same kernel: more than 64 candidates or fewer than k+1 (equal
-// values en masse, rows of -inf), a sum that is not a positive finite number, a tie in
-// probability that runs from the k-th place to the last candidate (an element below
-// the candidates might share it).
+// More than 64 candidates or fewer than k+1 (equal values en masse at the k-th place,
+// rows of mostly -inf): the elements above the tie value and the first elements equal to
+// it, in index order, and a tie in probability across the k-th place filled from every
+// element of the row that has that probability.  What is left -- a sum that is not a
+// positive finite number, more than k distinct larger values crowded into few lanes --
+// goes to the exact single-workgroup select over the row (select.hpp) in the same kernel.
 #pragma once
 
 #include "kernels_general.hpp"
@@ -90,19 +91,28 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
 #pragma unroll
             for (int c = 0; c < VEC; c++) {
                 const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
-                if (e < n) acc += static_cast<double>(fast_term_unbiased(q[i].get(c), ref));  // (a NaN element makes the sum NaN)
+                if (e < n) acc += static_cast<double>(fast_term_reduced(q[i].get(c), ref));  // (a NaN element makes the sum NaN)
             }
         }
         s_fast = wave_sum_f64_uniform(acc);
         bad = !(s_fast > 0.0 && s_fast < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY);
+        if (bad) {
+            // a NaN or +inf element, or nothing above -inf: every probability of the row is
+            // NaN, all of them tie, the lowest indices win
+            for (uint32_t r = lane; r < kk; r += kWave) {
+                store_elem(ov, r, __uint_as_float(0x7FC00000u));
+                oi[r] = static_cast<int32_t>(r);
+            }
+            return;
+        }
     }
     // Steps 3 to 6, at most three times: with k+1 lane maxima, then with twice and four
     // times as many when a probability tie runs off the end of the candidates.
     bool exact = bad;
     for (uint32_t lanes_wanted = want; !exact; lanes_wanted = 2u * lanes_wanted + 2u) {
-        // ---- 3. the lanes_wanted-th largest lane maximum, to 22 bits (-inf never becomes a candidate)
+        // ---- 3. the lanes_wanted-th largest lane maximum, to 16 bits (-inf never becomes a candidate)
         uint32_t thr = 0;
-        for (int bit = 31; bit >= 10; bit--) {
+        for (int bit = 31; bit >= 16; bit--) {
             const uint32_t trial = thr | (1u << bit);
             if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= lanes_wanted) thr = trial;
         }
@@ -132,7 +142,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             // ---- 5. accurate terms for the candidates, the corrected sum, probabilities
             const float xv = ordered_to_float(static_cast<uint32_t>(mine >> 32));
             const float term = have ? softmax_term(xv, M) : 0.f;
-            const double cr = have ? static_cast<double>(term) - static_cast<double>(fast_term_unbiased(xv, ref)) : 0.0;
+            const double cr = have ? static_cast<double>(term) - static_cast<double>(fast_term_reduced(xv, ref)) : 0.0;
             const double total = s_fast + wave_sum_f64_uniform(cr);
             const float p = round_to_storage<T>(static_cast<float>(static_cast<double>(term) * (1.0 / total)));
             mine = have ? ((static_cast<uint64_t>(order_key(p)) << 32) | (mine & 0xFFFFFFFFull)) : 0ull;
@@ -164,6 +174,148 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             oi[before] = static_cast<int32_t>(idx);
         }
         return;
+    }
+    // ---- equal values en masse at the k-th place, or a row of mostly -inf ---------------------------
+    // The row's k+1 largest are then the elements above the tie value T -- the exact
+    // (k+1)-th largest lane maximum; -inf when fewer than k+1 lanes hold anything -- and the
+    // first elements equal to T in index order.  A probability that the k-th place shares
+    // with the place behind it (equal values do, and different values can) is settled over
+    // every element of the row that has it.
+    if (!bad) {
+        uint32_t tie = 0;
+        for (int bit = 31; bit >= 0; bit--) {
+            const uint32_t trial = tie | (1u << bit);
+            if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= want) tie = trial;
+        }
+        tie = max(tie, kKeyNegInf);
+        // the elements above T, as in step 4
+        uint32_t above = 0;  // wave-uniform
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const bool pass = key[i * VEC + c] > tie;
+                const uint64_t mask = __ballot(pass);
+                if (mask != 0ull) {
+                    const uint32_t at = above + lanes_below(mask);
+                    const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
+                    if (pass && at < static_cast<uint32_t>(kWave)) smem.cand[at] = composite(key[i * VEC + c], e);
+                    above += static_cast<uint32_t>(__popcll(mask));
+                }
+            }
+        }
+        if (above < want) {
+            // the first want - above elements equal to T: vector by vector, lane by lane, element by element
+            const uint32_t need = want - above;
+            uint32_t taken = 0;  // wave-uniform
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                if (taken < need) {
+                    uint32_t mine_eq = 0;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) mine_eq += (key[i * VEC + c] == tie) ? 1u : 0u;
+                    uint32_t incl = mine_eq;  // over the lanes up to this one
+#pragma unroll
+                    for (int o = 1; o < kWave; o <<= 1) {
+                        const uint32_t t = __shfl_up(incl, o, kWave);
+                        if (lane >= static_cast<uint32_t>(o)) incl += t;
+                    }
+                    uint32_t pos = taken + incl - mine_eq;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        if (key[i * VEC + c] == tie) {
+                            const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
+                            if (pos < need) smem.cand[above + pos] = composite(tie, e);
+                            pos++;
+                        }
+                    }
+                    taken += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
+                }
+            }
+            __syncthreads();
+            // (a row shorter than k+1 has them all)
+            const uint32_t C = above + min(taken, need);
+            if (C >= min(want, n)) {
+                const bool have = lane < C;
+                uint64_t mine = have ? smem.cand[lane] : 0ull;
+                const uint32_t xkey = static_cast<uint32_t>(mine >> 32);
+                double rinv = 0.0;
+                auto prob_of_key = [&](uint32_t kx) {
+                    return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(kx), M)) * rinv));
+                };
+                if constexpr (SOFTMAX) {
+                    const float xv = ordered_to_float(xkey);
+                    const float term = have ? softmax_term(xv, M) : 0.f;
+                    const double cr = have ? static_cast<double>(term) - static_cast<double>(fast_term_reduced(xv, ref)) : 0.0;
+                    rinv = 1.0 / (s_fast + wave_sum_f64_uniform(cr));
+                    const float p = round_to_storage<T>(static_cast<float>(static_cast<double>(term) * rinv));
+                    mine = have ? ((static_cast<uint64_t>(order_key(p)) << 32) | (mine & 0xFFFFFFFFull)) : 0ull;
+                }
+                const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
+                uint32_t before = 0;
+                for (uint32_t c = 0; c < C; c++) {
+                    const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), static_cast<int>(c)))) << 32) |
+                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_lo), static_cast<int>(c)));
+                    before += (other > mine) ? 1u : 0u;
+                }
+                uint32_t g0 = kk;  // ranks from here on are filled as one group of equal probability
+                if constexpr (SOFTMAX) {
+                    if (C > kk) {
+                        const uint64_t at_cut = __ballot(have && before == kk - 1u), at_next = __ballot(have && before == kk);
+                        const uint32_t p_cut = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), __builtin_ctzll(at_cut)));
+                        const uint32_t p_next = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), __builtin_ctzll(at_next)));
+                        if (p_cut == p_next) {
+                            // The probability at the k-th place goes on behind it.  It belongs to an
+                            // interval of values [lo, hi]: hi is the largest candidate that has it
+                            // (everything above the tie value is a candidate), lo is searched for; the
+                            // places from the group's first rank on go to the interval's first
+                            // elements in index order -- all of them are in this wave's registers.
+                            const float pc = ordered_to_float(p_cut);
+                            g0 = static_cast<uint32_t>(__popcll(__ballot(have && mine_hi > p_cut)));
+                            uint32_t hi_key = (have && mine_hi == p_cut) ? xkey : 0u;
+#pragma unroll
+                            for (int o = 32; o > 0; o >>= 1) hi_key = max(hi_key, static_cast<uint32_t>(__shfl_xor(static_cast<int>(hi_key), o, kWave)));
+                            const uint32_t lo_key = pc > 0.f ? lowest_key_of_probability(hi_key, pc, prob_of_key) : 1u;
+                            const uint32_t places = kk - g0;
+                            uint32_t filled = 0;  // wave-uniform
+#pragma unroll
+                            for (int i = 0; i < V; i++) {
+                                if (filled < places) {
+                                    uint32_t mine_in = 0;
+#pragma unroll
+                                    for (int c = 0; c < VEC; c++) mine_in += (key[i * VEC + c] >= lo_key && key[i * VEC + c] <= hi_key) ? 1u : 0u;
+                                    uint32_t incl = mine_in;
+#pragma unroll
+                                    for (int o = 1; o < kWave; o <<= 1) {
+                                        const uint32_t t = __shfl_up(incl, o, kWave);
+                                        if (lane >= static_cast<uint32_t>(o)) incl += t;
+                                    }
+                                    uint32_t pos = filled + incl - mine_in;
+#pragma unroll
+                                    for (int c = 0; c < VEC; c++) {
+                                        if (key[i * VEC + c] >= lo_key && key[i * VEC + c] <= hi_key) {
+                                            if (pos < places) {
+                                                store_elem(ov, g0 + pos, pc);
+                                                oi[g0 + pos] = static_cast<int32_t>((static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c));
+                                            }
+                                            pos++;
+                                        }
+                                    }
+                                    filled += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
+                                }
+                            }
+                        }
+                    }
+                }
+                if (have && before < min(kk, g0)) {
+                    const uint32_t idx = composite_index(mine);
+                    if constexpr (SOFTMAX) store_elem(ov, before, ordered_to_float(mine_hi));
+                    else ov[before] = rowp[idx];  // bit copy (keeps the sign of a zero)
+                    oi[before] = static_cast<int32_t>(idx);
+                }
+                return;
+            }
+        }
     }
     // ---- the exact select over the whole row -----------------------------------------------
     __syncthreads();  // LDS changes owner
