@@ -92,11 +92,36 @@ def _rows(kind, rows, n, rng):
         for s0 in range(0, n, 4096):
             x[:, s0:s0 + 4096] = np.sort(x[:, s0:s0 + 4096], axis=1)
         return x
+    if kind == "half_half":   # two values, either one in half of the places: the threshold's value is everywhere
+        return np.where(rng.random((rows, n)) < 0.5, np.float32(1.0), np.float32(-1.0)).astype(np.float32)
+    if kind == "three_allowed":   # three finite elements a row: the rest of the result is -inf, in index order
+        x[:] = -np.inf
+        x[:, [n // 7, n // 2, n - 3]] = np.float32(0.5)
+        return x
+    if kind == "nan_and_inf":  # rows of NaN probabilities (NaN ranks first in the plain top-k)
+        x[0, n // 2] = np.nan
+        x[1, n // 3] = np.inf
+        x[2, 5] = np.nan
+        x[2, n - 1] = np.nan
+        return x
+    if kind == "huge":        # differences of thousands: all but a few probabilities are 0 and tie
+        return (x * np.float32(1e4)).astype(np.float32)
+    if kind == "masked90":    # nine in ten -inf: block maxima of both signs (coarse histogram bins)
+        x[rng.random((rows, n)) < 0.9] = -np.inf
+        return x
+    if kind == "coarse_levels":   # a dozen levels, thousands of elements on the one at the cut
+        return (np.round(x) / 2).astype(np.float32)
+    if kind == "signed_zeros":    # -0 == +0: one rank group, in index order
+        x = np.where(rng.random((rows, n)) < 0.5, np.float32(0.0), np.float32(-0.0)).astype(np.float32)
+        x[:, ::1000] = np.float32(1.0)
+        return x
     raise ValueError(kind)
 
 
 KINDS = ["llm", "bf16", "levels", "sorted", "masked", "constant", "spikes"]
 TIE_KINDS = ["tenth", "two_values", "sorted_desc", "flat_with_peaks", "runs"]
+WALK_KINDS = ["half_half", "three_allowed", "nan_and_inf", "huge", "masked90", "coarse_levels", "signed_zeros", "sorted", "runs",
+              "flat_with_peaks"]
 
 
 def _compare_paths(ops, n, k, dtype, rows, kinds, path):
@@ -188,6 +213,17 @@ def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtyp
     own means (a second threshold, the first elements equal to the tie value, block
     minima), against the other kernels and the oracle."""
     _compare_paths(ops, n, k, dtype, 4, TIE_KINDS, path)
+
+
+@pytest.mark.parametrize("n,k", [(262144, 1024), (262144, 2000), (524288, 2048), (300000, 600), (300001, 700)])
+def test_large_k_rows_whose_cut_falls_into_a_crowd(ops, n, k):
+    """The large-k kernels on rows where the threshold's own rank group is too large for the
+    candidate lists (one value in half of the places, -inf nearly everywhere, probabilities
+    that underflow to 0, -0 and +0, a dozen levels) -- its first members come from a walk over
+    the row in index order, also on rows that do not start on 16 bytes -- on rows of NaN
+    probabilities, on block maxima of both signs and on sorted rows at a k close to the
+    lists' capacity; against the radix select and the oracle."""
+    _compare_paths(ops, n, k, np.float32, 4, WALK_KINDS, 3)
 
 
 @pytest.mark.parametrize("n", [16388, 40002, 128255])

@@ -50,7 +50,12 @@ constexpr int kBigPickWaves = kBigPickThreads / kWave;
 constexpr int kBigPickCap = 4096;       // candidates of a row that are ranked
 constexpr int kBigPickLists = 8;        // lists a row's candidates are appended to (gather workgroup p uses list p % 8:
                                         // eight counters instead of one that every workgroup of the row queues for)
-constexpr int kBigPickListCap = 2048;   // entries per list; also what one gather workgroup can hold
+constexpr int kBigPickListCap = 2048;   // entries per list
+constexpr int kBigPickLocalCap = 4096;  // candidates one gather workgroup can hold (a sorted row's are all in one or two shares)
+constexpr int kBigPickSpread = 512;     // a gather workgroup with more candidates than this deals them over all the lists
+constexpr int kBigPickZoneQuota = 32;   // elements at or below the threshold (down to the margin) one gather workgroup
+                                        // passes on at most (fewer for a large k: bigpick_zone_quota); with more the
+                                        // threshold's own rank group comes from a walk over the row (below)
 constexpr int kBigPickMine = 32;        // candidates one rank workgroup places
 constexpr int kBigPickRecsMax = 1024;   // wave records of a row (chunks * kScanWaves)
 constexpr int kBigPickHeadWords = 16 * kBigPickLists + 16;  // per row: 16 words per list, then 16 for the row
@@ -61,8 +66,9 @@ struct BigPickWorkspace {
     float *term;     // same shape, softmax variant: exp(x - M) of the same elements
     uint32_t *head;  // [rows][kBigPickHeadWords].  List j of a row: word 16 j = entries appended (more than the
                      // capacity = incomplete), words 16 j + 2, 3 = its part of the row's correction (64-bit integer);
-                     // word 128 = the threshold the gather kernel found, before the margin.  All zero when the
-                     // gather kernel starts (the scan kernel clears them).
+                     // word 128 = the threshold the gather kernel found, before the margin; word 129 != 0: some
+                     // workgroup left out its elements at or below the threshold (more than its quota).  All
+                     // zero when the gather kernel starts (the scan kernel clears them).
     double *stat;    // [rows][2] softmax variant: the row's sum of fast terms, scaled to its maximum; that maximum
 };
 
@@ -74,6 +80,14 @@ struct BigPickWorkspace {
 // (at most half an ulp of thr, and then adjacent floats are further apart than the
 // margin anyway) cannot eat it.
 template <typename T> __device__ __forceinline__ float bigpick_margin() { return sizeof(T) == 2 ? 4e-3f : 1e-5f; }
+
+// What one of a row's G2 gather workgroups passes on of elements at or below the
+// threshold: so that these and 1.5 (k+1) elements above it (the usual excess is 1.2 to
+// 1.5) stay within what the rank kernel holds.
+__device__ __forceinline__ uint32_t bigpick_zone_quota(uint32_t want, uint32_t G2) {
+    const uint32_t room = static_cast<uint32_t>(kBigPickCap) > want + want / 2u ? static_cast<uint32_t>(kBigPickCap) - want - want / 2u : 0u;
+    return min(static_cast<uint32_t>(kBigPickZoneQuota), max(4u, room / G2));
+}
 
 // thr: key of a finite number or +inf (never below kKeyNegInf + 1)
 template <typename T, bool SOFTMAX> __device__ __forceinline__ uint32_t bigpick_lowered(uint32_t thr) {
@@ -160,9 +174,10 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
     __shared__ uint32_t wave_hits[NW];
     __shared__ uint32_t wtot[NW];
     __shared__ uint32_t cslots[2][NW];
-    __shared__ uint32_t lcount, lbase;
-    __shared__ uint64_t lcand[kBigPickListCap];
-    __shared__ float lterm[SOFTMAX ? kBigPickListCap : 1];
+    __shared__ uint32_t lcount, zcount, lbase[kBigPickLists];
+    __shared__ uint64_t lcand[kBigPickLocalCap];
+    __shared__ uint64_t zcand[kBigPickZoneQuota];
+    __shared__ float lterm[SOFTMAX ? kBigPickLocalCap : 1];
     __shared__ float fscratch[NW];
     __shared__ double dscratch[NW];
     __shared__ long long iscratch[NW];
@@ -224,7 +239,10 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
         wred[wave][1] = kmin;
         wred[wave][2] = nlive;
     }
-    if (tid == 0) lcount = 0;
+    if (tid == 0) {
+        lcount = 0;
+        zcount = 0;
+    }
     __syncthreads();
     kmax = wred[0][0];
     kmin = wred[0][1];
@@ -247,7 +265,9 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
     };
     uint32_t thr;
     if (nlive < want) {
-        thr = kKeyNegInf + 1u;  // every element above -inf is a candidate
+        // fewer than k+1 blocks hold anything above -inf: every element above -inf is a
+        // candidate, and the -inf elements (the threshold's own) follow in index order
+        thr = kKeyNegInf;
     } else if (kmax == kmin) {
         thr = kmin;
     } else {
@@ -256,32 +276,44 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
         // sample's (k+1)/4-th largest, and a few more for the sampling error, gives a value,
         // and the count over ALL keys says whether k+1 reach it -- if not, lower bins are
         // tried (1, 2, 4 .. further down; the floor itself is reached by enough).  A value
-        // that far more than k+1 reach (coarse bins: an outlier stretches the range)
-        // becomes the floor of a second round.
+        // that clearly more than k+1 reach (coarse bins: keys of both signs, an outlier, a NaN
+        // stretch the range) is followed by a second round over one bin alone, with all of
+        // its keys and the exact number still wanted there.
         const uint32_t quarter = (want + 3u) / 4u;
         const uint32_t need_s = quarter + 2u * static_cast<uint32_t>(sqrtf(static_cast<float>(quarter))) + 8u;
-        uint32_t floor_key = kmin;
+        uint32_t floor_key = kmin, ceil_key = kmax, need_all = want;
+        bool all_keys = false;  // the second round after coarse bins: every key of one bin, the exact number wanted there
         thr = kmin;
         for (int round = 0; round < 2; round++) {  // (every condition below is the same for every thread)
-            const uint32_t range = kmax - floor_key;
+            const uint32_t range = ceil_key - floor_key;
             const uint32_t s = range < 2048u ? 0u : (32u - static_cast<uint32_t>(__clz(range))) - 11u;
             __syncthreads();
             reinterpret_cast<uint4 *>(hist)[2 * tid] = make_uint4(0, 0, 0, 0);
             reinterpret_cast<uint4 *>(hist)[2 * tid + 1] = make_uint4(0, 0, 0, 0);
             __syncthreads();
-            uint32_t ns = 0;  // keys in the sample (wave-uniform)
+            uint32_t ns = 0;  // keys that went in (wave-uniform)
+            if (!all_keys) {
 #pragma unroll
-            for (int i = 0; i < GE / 4; i++) {
-                const uint32_t sel = tid & 3u;
-                const uint32_t key = sel == 0u ? gk[4 * i] : sel == 1u ? gk[4 * i + 1] : sel == 2u ? gk[4 * i + 2] : gk[4 * i + 3];
-                const bool on = key != 0u && key >= floor_key;
-                ns += static_cast<uint32_t>(__popcll(__ballot(on)));
-                bigpick_hist_add(hist, on, (key - floor_key) >> s);
+                for (int i = 0; i < GE / 4; i++) {
+                    const uint32_t sel = tid & 3u;
+                    const uint32_t key = sel == 0u ? gk[4 * i] : sel == 1u ? gk[4 * i + 1] : sel == 2u ? gk[4 * i + 2] : gk[4 * i + 3];
+                    const bool on = key != 0u && key >= floor_key;
+                    ns += static_cast<uint32_t>(__popcll(__ballot(on)));
+                    bigpick_hist_add(hist, on, (key - floor_key) >> s);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < GE; e++) {
+                    const bool on = gk[e] >= floor_key && gk[e] <= ceil_key;  // (floor_key > 0: never "not a key")
+                    ns += static_cast<uint32_t>(__popcll(__ballot(on)));
+                    bigpick_hist_add(hist, on, (gk[e] - floor_key) >> s);
+                }
             }
-            const uint32_t sampled = bigpick_count_sum(ns, cslots[0]);  // (barrier: the histogram is complete)
+            const uint32_t went_in = bigpick_count_sum(ns, cslots[0]);  // (barrier: the histogram is complete)
+            const uint32_t need = all_keys ? need_all : need_s;
             uint32_t d = 0;
-            if (sampled >= need_s) {
-                bigpick_resolve(hist, need_s, answer, wtot);
+            if (went_in >= need) {
+                bigpick_resolve(hist, need, answer, wtot);
                 d = answer[0];
             }
             uint32_t cand_thr = floor_key + (d << s), got = 0;
@@ -292,11 +324,51 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
                 cand_thr = floor_key + (d << s);
             }
             thr = cand_thr;
-            if (d == 0u || s == 0u || got <= 2u * want + 64u) break;
+            // (bins of 2^16 keys and more are coarse -- 1 % of a float's value; finer ones
+            // are rarely worth a second round: tied keys stay tied)
+            const uint32_t tight = s >= 16u ? want + want / 8u + 32u : 2u * want + 64u;
+            if (round == 1 || s == 0u || got <= tight) break;
+            // The bin [cand_thr, cand_thr + 2^s) alone -- or a bin further up: the sample's
+            // allowance makes the choice err downwards, and where k+1 keys still reach a
+            // higher bin's lower end, that is the better value.  The highest such bin: the
+            // next one first (the usual answer: not that one either), then in doubling
+            // steps and by bisection (keys of few distinct values leave most bins empty).
+            const uint32_t nbins = (range >> s) + 1u;
+            uint32_t dlo = d, dhi = nbins, above = 0;  // reach(bin dlo) >= k+1 > reach(bin dhi) = above (bin nbins: nothing)
+            // (fine bins: one bin too low is harmless, the second round starts from here)
+            for (uint32_t step = 1; s >= 16u && dlo + step < nbins; step <<= 1) {
+                const uint32_t c = reach(floor_key + ((dlo + step) << s));
+                if (c < want) {
+                    dhi = dlo + step;
+                    above = c;
+                    break;
+                }
+                dlo += step;
+                got = c;
+            }
+            while (s >= 16u && dhi - dlo > 1u) {
+                const uint32_t mid = dlo + (dhi - dlo) / 2u;
+                const uint32_t c = reach(floor_key + (mid << s));
+                if (c < want) {
+                    dhi = mid;
+                    above = c;
+                } else {
+                    dlo = mid;
+                    got = c;
+                }
+            }
+            cand_thr = floor_key + (dlo << s);
+            thr = cand_thr;
+            if (got <= tight) break;
+            const uint32_t c1 = dhi < nbins ? floor_key + (dhi << s) - 1u : ceil_key;
             floor_key = cand_thr;
+            ceil_key = c1;
+            need_all = want - above;
+            all_keys = s >= 16u;
         }
     }
-    uint32_t lo = bigpick_lowered<T, SOFTMAX>(thr);
+    // (thr == kKeyNegInf: the -inf elements are the threshold's own)
+    uint32_t lo = thr > kKeyNegInf ? bigpick_lowered<T, SOFTMAX>(thr) : thr;
     // ---- clustered rows -------------------------------------------------------------------------
     // Blocks whose MINIMUM reaches thr hold 16 * VEC elements that do.  When the blocks that
     // reach lo are known to hold more candidates than a row's lists (a sorted row: k+1 blocks
@@ -333,7 +405,7 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
             }
             if (tmin > thr) {
                 thr = tmin;
-                lo = bigpick_lowered<T, SOFTMAX>(thr);
+                lo = thr > kKeyNegInf ? bigpick_lowered<T, SOFTMAX>(thr) : thr;
             }
             // per block, in index order, how many elements at or above thr it is KNOWN to hold
             uint16_t *known = reinterpret_cast<uint16_t *>(lcand);  // (8192 entries; the list is not in use yet)
@@ -428,8 +500,14 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
                     const uint32_t idx = e0[u] + static_cast<uint32_t>(c);
                     const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
                     if (idx < cend[u] && key >= lo && (key > thr || idx / BE <= last_block_for_equals)) {
-                        const uint32_t at = atomicAdd(&lcount, 1u);
-                        if (at < static_cast<uint32_t>(kBigPickListCap)) lcand[at] = composite(key, idx);
+                        // above the threshold: wanted whatever else happens; at or below it: up to the quota
+                        if (key > thr) {
+                            const uint32_t at = atomicAdd(&lcount, 1u);
+                            if (at < static_cast<uint32_t>(kBigPickLocalCap)) lcand[at] = composite(key, idx);
+                        } else {
+                            const uint32_t at = atomicAdd(&zcount, 1u);
+                            if (at < static_cast<uint32_t>(kBigPickZoneQuota)) zcand[at] = composite(key, idx);
+                        }
                     }
                 }
             }
@@ -437,8 +515,17 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
     }
     __syncthreads();
     BPS(5);
-    const uint32_t cnt = lcount;  // (the same for every thread)
-    const uint32_t held = min(cnt, static_cast<uint32_t>(kBigPickListCap));
+    // Elements at or below the threshold: within the quota they join the candidates; beyond
+    // it (equal values en masse, rows of mostly -inf) none of this workgroup's do, the row
+    // is marked, and the rank kernel takes the threshold's own rank group from a walk over
+    // the row in index order -- everything ABOVE the threshold is in the lists either way.
+    const uint32_t cnt_a = lcount, cnt_z = zcount;  // (the same for every thread)
+    const bool trimmed = cnt_z > bigpick_zone_quota(want, G2);
+    if (!trimmed && tid < cnt_z && cnt_a + tid < static_cast<uint32_t>(kBigPickLocalCap)) lcand[cnt_a + tid] = zcand[tid];
+    if (trimmed && tid == 0) atomicOr(&head[16 * kBigPickLists + 1], 1u);
+    __syncthreads();
+    const uint32_t cnt = cnt_a + (trimmed ? 0u : cnt_z);
+    const uint32_t held = min(cnt, static_cast<uint32_t>(kBigPickLocalCap));
 
     // ---- softmax: the candidates' accurate terms; what they add to the row's sum ------------
     long long fix = 0;
@@ -463,28 +550,40 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
         if (lane == 0) iscratch[wave] = fix;
     }
     if (cnt != 0) {
-        const uint32_t list = part % kBigPickLists;
+        // Few candidates (the rule): all to list part % 8.  Many (a sorted row's candidates lie
+        // in one or two shares): candidate t to list t % 8, so that no list carries them alone.
+        const bool spread = cnt > static_cast<uint32_t>(kBigPickSpread) && cnt <= static_cast<uint32_t>(kBigPickLocalCap);
+        const uint32_t list0 = part % kBigPickLists;
         __syncthreads();
-        if (tid == 0) {
-            // more than the workgroup can hold: the list's count is pushed past its capacity
-            lbase = atomicAdd(&head[16 * list], cnt <= static_cast<uint32_t>(kBigPickListCap) ? cnt : kBigPickListCap + 1u);
+        if (tid < static_cast<uint32_t>(kBigPickLists)) {
+            if (spread) {
+                lbase[tid] = atomicAdd(&head[16 * tid], (cnt + (kBigPickLists - 1u) - tid) / kBigPickLists);
+            } else if (tid == list0) {
+                // more than the workgroup can hold: the list's count is pushed past its capacity
+                lbase[tid] = atomicAdd(&head[16 * tid], cnt <= static_cast<uint32_t>(kBigPickLocalCap) ? cnt : kBigPickListCap + 1u);
+            }
             if constexpr (SOFTMAX) {
-                long long total = 0;
+                if (tid == list0) {
+                    long long total = 0;
 #pragma unroll
-                for (int w = 0; w < NW; w++) total += iscratch[w];
-                atomicAdd(reinterpret_cast<unsigned long long *>(head + 16 * list + 2), static_cast<unsigned long long>(total));
+                    for (int w = 0; w < NW; w++) total += iscratch[w];
+                    atomicAdd(reinterpret_cast<unsigned long long *>(head + 16 * tid + 2), static_cast<unsigned long long>(total));
+                }
             }
         }
         __syncthreads();
         BPS(6);
-        const uint32_t base = lbase;
-        if (cnt <= static_cast<uint32_t>(kBigPickListCap)) {
-            const size_t at0 = (static_cast<size_t>(row) * kBigPickLists + list) * kBigPickListCap;
-            for (uint32_t t = tid; t < cnt; t += NT)
-                if (base + t < static_cast<uint32_t>(kBigPickListCap)) {
-                    bw.cand[at0 + base + t] = lcand[t];
-                    if constexpr (SOFTMAX) bw.term[at0 + base + t] = lterm[t];
+        if (cnt <= static_cast<uint32_t>(kBigPickLocalCap)) {
+            const size_t row_at = static_cast<size_t>(row) * kBigPickLists * kBigPickListCap;
+            for (uint32_t t = tid; t < cnt; t += NT) {
+                const uint32_t list = spread ? t % kBigPickLists : list0;
+                const uint32_t slot = lbase[list] + (spread ? t / kBigPickLists : t);
+                if (slot < static_cast<uint32_t>(kBigPickListCap)) {  // (a list past its capacity: the rank kernel sees its count)
+                    const size_t at = row_at + static_cast<size_t>(list) * kBigPickListCap + slot;
+                    bw.cand[at] = lcand[t];
+                    if constexpr (SOFTMAX) bw.term[at] = lterm[t];
                 }
+            }
         }
     }
     BPS(7);
@@ -502,6 +601,33 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
                 bw.stat[2 * static_cast<size_t>(row)] = s_base;
                 bw.stat[2 * static_cast<size_t>(row) + 1] = static_cast<double>(M);
             }
+        }
+    }
+}
+
+// The exact single-workgroup select over a whole row (select.hpp): what the lists could
+// not hold or decide.  All threads of the workgroup call.
+template <typename T, bool SOFTMAX>
+__device__ __forceinline__ void bigpick_exact_row(SelectShared &ex, const T *rowp, T *ov, int32_t *oi, uint32_t n, uint32_t kk,
+                                                  float *fscratch, double *dscratch) {
+    constexpr int NT = kBigPickThreads;
+    const uint32_t tid = threadIdx.x;
+    if constexpr (SOFTMAX) {
+        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch, 1.f);
+        select_topk_line<NT>(ex, n, kk, [&](uint32_t j) {
+            return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
+        });
+        for (uint32_t r = tid; r < kk; r += NT) {
+            const uint32_t idx = composite_index(ex.sel[r]);
+            store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
+            oi[r] = static_cast<int32_t>(idx);
+        }
+    } else {
+        select_topk_line<NT>(ex, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
+        for (uint32_t r = tid; r < kk; r += NT) {
+            const uint32_t idx = composite_index(ex.sel[r]);
+            ov[r] = rowp[idx];
+            oi[r] = static_cast<int32_t>(idx);
         }
     }
 }
@@ -524,6 +650,7 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_rank_kernel(const T *
     } smem;
     __shared__ float fscratch[NW];
     __shared__ double dscratch[NW];
+    __shared__ uint32_t walk_slots[NW], walk_counts[2 * NW], walk_keys[2];
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t row = blockIdx.x / G3, g = blockIdx.x - row * G3;
     const T *rowp = in + static_cast<size_t>(row) * n;
@@ -546,51 +673,55 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_rank_kernel(const T *
     }
     const uint32_t C = start[kBigPickLists];
     const uint32_t thr = head[16 * kBigPickLists];
-    exact = exact || C > static_cast<uint32_t>(kBigPickCap) || C < want;
-    if (!exact && g * kBigPickMine >= C) return;  // nothing of the sequence is this workgroup's
+    exact = exact || C > static_cast<uint32_t>(kBigPickCap);
+    // Walk mode: the lists hold every element above the threshold, but of the elements at
+    // or below it not all that the result may need (a gather workgroup met more than its
+    // quota of them; fewer than k+1 candidates; a margin that does not separate
+    // probabilities).  Then everything that ranks with the threshold forms ONE group of equal
+    // rank, taken in index order: the ranking below places what ranks above that group, and
+    // the row's last workgroup fills the remaining places with the group's first members
+    // from a walk over the row.
+    bool walk = !exact && (head[16 * kBigPickLists + 1] != 0u || C < want);
+    uint32_t star = thr;  // what ranks with the threshold: this key (softmax: this probability's key)
     double rinv = 0.0;
+    float M = 0.f;
     if constexpr (SOFTMAX) {
         if (!exact) {
             const double s_base = bw.stat[2 * static_cast<size_t>(row)];
-            const float M = static_cast<float>(bw.stat[2 * static_cast<size_t>(row) + 1]);
+            M = static_cast<float>(bw.stat[2 * static_cast<size_t>(row) + 1]);
+            if (!(s_base > 0.0 && s_base < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY)) {
+                // a NaN or +inf element, or nothing above -inf: every probability of the row is
+                // NaN, all of them tie, the lowest indices win
+                if (g == 0)
+                    for (uint32_t r = tid; r < kk; r += NT) {
+                        store_elem(ov, r, __uint_as_float(0x7FC00000u));
+                        oi[r] = static_cast<int32_t>(r);
+                    }
+                return;
+            }
             long long fix = 0;
 #pragma unroll
             for (int j = 0; j < kBigPickLists; j++)
                 fix += static_cast<long long>(*reinterpret_cast<const unsigned long long *>(head + 16 * j + 2));
             const double total = s_base + static_cast<double>(fix) * (1.0 / kBigPickFixUnit);
-            exact = !(s_base > 0.0 && s_base < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY) ||
-                    !(total > 0.0 && total < static_cast<double>(INFINITY));
+            exact = !(total > 0.0 && total < static_cast<double>(INFINITY));
             if (!exact) {
                 rinv = 1.0 / total;
-                // the margin has to separate what is below it from the k+1 at or above the threshold
                 auto prob = [&](float xv) {
                     return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(xv, M)) * rinv));
                 };
-                exact = !(prob(ordered_to_float(thr)) > prob(ordered_to_float(bigpick_lowered<T, true>(thr))));
+                const float p_star = prob(ordered_to_float(thr));
+                star = order_key(p_star);
+                // the margin has to separate what is below it from the k+1 at or above the threshold
+                if (thr > kKeyNegInf) walk = walk || !(p_star > prob(ordered_to_float(bigpick_lowered<T, true>(thr))));
             }
         }
     }
+    const bool walker = walk && !exact && g == G3 - 1;
+    if (!exact && !walker && g * kBigPickMine >= C) return;  // nothing of the sequence is this workgroup's
     if (exact) {
         if (g != 0) return;
-        SelectShared &ex = smem.exact;
-        if constexpr (SOFTMAX) {
-            const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch, 1.f);
-            select_topk_line<NT>(ex, n, kk, [&](uint32_t j) {
-                return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
-            });
-            for (uint32_t r = tid; r < kk; r += NT) {
-                const uint32_t idx = composite_index(ex.sel[r]);
-                store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
-                oi[r] = static_cast<int32_t>(idx);
-            }
-        } else {
-            select_topk_line<NT>(ex, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
-            for (uint32_t r = tid; r < kk; r += NT) {
-                const uint32_t idx = composite_index(ex.sel[r]);
-                ov[r] = rowp[idx];
-                oi[r] = static_cast<int32_t>(idx);
-            }
-        }
+        bigpick_exact_row<T, SOFTMAX>(smem.exact, rowp, ov, oi, n, kk, fscratch, dscratch);
         return;
     }
     BPS(17);
@@ -612,74 +743,144 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_rank_kernel(const T *
         }
         return live ? c : 0ull;
     };
-    // this wave's quarter of the sequence, entry e of lane L = candidate w Q + 64 e + L; all loads first
-    const uint32_t Q = (C + NW - 1) / NW;
-    const uint32_t steps = (Q + kWave - 1) / kWave;  // (<= kBigRankPerLane)
-    uint64_t ent[kBigRankPerLane];
-    float eterm[kBigRankPerLane];
+    if (g * kBigPickMine < C) {  // (the same for every thread; false only for a walker without candidates of its own)
+        // this wave's quarter of the sequence, entry e of lane L = candidate w Q + 64 e + L; all loads first
+        const uint32_t Q = (C + NW - 1) / NW;
+        const uint32_t steps = (Q + kWave - 1) / kWave;  // (<= kBigRankPerLane)
+        uint64_t ent[kBigRankPerLane];
+        float eterm[kBigRankPerLane];
 #pragma unroll
-    for (int e = 0; e < kBigRankPerLane; e++) {
-        const uint32_t o = static_cast<uint32_t>(e) * kWave + lane;
-        const uint32_t f = wave * Q + o;
-        const bool live = o < Q && f < C;
-        ent[e] = 0;
-        eterm[e] = 0.f;
-        if (static_cast<uint32_t>(e) < steps) {  // (wave-uniform)
-            const size_t at = where(live ? f : 0u);
-            ent[e] = bw.cand[at];
-            if constexpr (SOFTMAX) eterm[e] = bw.term[at];
+        for (int e = 0; e < kBigRankPerLane; e++) {
+            const uint32_t o = static_cast<uint32_t>(e) * kWave + lane;
+            const uint32_t f = wave * Q + o;
+            const bool live = o < Q && f < C;
+            ent[e] = 0;
+            eterm[e] = 0.f;
+            if (static_cast<uint32_t>(e) < steps) {  // (wave-uniform)
+                const size_t at = where(live ? f : 0u);
+                ent[e] = bw.cand[at];
+                if constexpr (SOFTMAX) eterm[e] = bw.term[at];
+            }
         }
-    }
-    // this workgroup's own candidates: lane L < 32 of every wave holds candidate 32 g + L
-    const uint32_t my_at = g * kBigPickMine + (lane & 31u);
-    const bool my_live = my_at < C;
-    const size_t mat = where(my_live ? my_at : 0u);
-    uint64_t mine = bw.cand[mat];
-    float mterm = 0.f;
-    if constexpr (SOFTMAX) mterm = bw.term[mat];
-    mine = keyed(mine, mterm, my_live);
+        // this workgroup's own candidates: lane L < 32 of every wave holds candidate 32 g + L
+        const uint32_t my_at = g * kBigPickMine + (lane & 31u);
+        const bool my_live = my_at < C;
+        const size_t mat = where(my_live ? my_at : 0u);
+        uint64_t mine = bw.cand[mat];
+        float mterm = 0.f;
+        if constexpr (SOFTMAX) mterm = bw.term[mat];
+        mine = keyed(mine, mterm, my_live);
 #pragma unroll
-    for (int e = 0; e < kBigRankPerLane; e++) {
-        const uint32_t o = static_cast<uint32_t>(e) * kWave + lane;
-        ent[e] = keyed(ent[e], eterm[e], static_cast<uint32_t>(e) < steps && o < Q && wave * Q + o < C);
-    }
-    BPS(18);
-    // ---- how many of this wave's entries rank before each of the 32: one compare of the
-    // wave's 64 entries against the candidate (a scalar), and the population count of the result
-    const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
-    uint32_t before = 0;  // lane j: the count for candidate j
-    // (entries past the wave's share are 0 and count for nothing: the loop over them is
-    // compiled for 4, 8, 12 and 16 entries a lane, without a branch inside)
-    auto count_all = [&](auto steps_tag) __attribute__((always_inline)) {
-        constexpr int STEPS = decltype(steps_tag)::value;
-        for (int j = 0; j < kBigPickMine; j++) {
-            const uint64_t m = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), j))) << 32) |
-                               static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_lo), j));
-            uint32_t c = 0;
-#pragma unroll
-            for (int e = 0; e < STEPS; e++) c += static_cast<uint32_t>(__popcll(__ballot(ent[e] > m)));
-            before = (lane == static_cast<uint32_t>(j)) ? c : before;
+        for (int e = 0; e < kBigRankPerLane; e++) {
+            const uint32_t o = static_cast<uint32_t>(e) * kWave + lane;
+            ent[e] = keyed(ent[e], eterm[e], static_cast<uint32_t>(e) < steps && o < Q && wave * Q + o < C);
         }
-    };
-    if (steps <= 4u) count_all(std::integral_constant<int, 4>{});
-    else if (steps <= 8u) count_all(std::integral_constant<int, 8>{});
-    else if (steps <= 12u) count_all(std::integral_constant<int, 12>{});
-    else count_all(std::integral_constant<int, 16>{});
-    if (lane < static_cast<uint32_t>(kBigPickMine)) smem.part[wave][lane] = before;
+        BPS(18);
+        // ---- how many of this wave's entries rank before each of the 32: one compare of the
+        // wave's 64 entries against the candidate (a scalar), and the population count of the result
+        const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
+        uint32_t before = 0;  // lane j: the count for candidate j
+        // (entries past the wave's share are 0 and count for nothing: the loop over them is
+        // compiled for 4, 8, 12 and 16 entries a lane, without a branch inside)
+        auto count_all = [&](auto steps_tag) __attribute__((always_inline)) {
+            constexpr int STEPS = decltype(steps_tag)::value;
+            for (int j = 0; j < kBigPickMine; j++) {
+                const uint64_t m = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), j))) << 32) |
+                                   static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_lo), j));
+                uint32_t c = 0;
+#pragma unroll
+                for (int e = 0; e < STEPS; e++) c += static_cast<uint32_t>(__popcll(__ballot(ent[e] > m)));
+                before = (lane == static_cast<uint32_t>(j)) ? c : before;
+            }
+        };
+        if (steps <= 4u) count_all(std::integral_constant<int, 4>{});
+        else if (steps <= 8u) count_all(std::integral_constant<int, 8>{});
+        else if (steps <= 12u) count_all(std::integral_constant<int, 12>{});
+        else count_all(std::integral_constant<int, 16>{});
+        if (lane < static_cast<uint32_t>(kBigPickMine)) smem.part[wave][lane] = before;
+        __syncthreads();
+        BPS(19);
+        // (walk mode: only what ranks above the threshold's group is placed here)
+        if (tid < static_cast<uint32_t>(kBigPickMine) && my_live && (!walk || mine_hi > star)) {
+            uint32_t rank = 0;
+#pragma unroll
+            for (int w = 0; w < NW; w++) rank += smem.part[w][tid];
+            if (rank < kk) {
+                const uint32_t idx = composite_index(mine);
+                if constexpr (SOFTMAX) store_elem(ov, rank, ordered_to_float(mine_hi));
+                else ov[rank] = rowp[idx];  // bit copy (keeps the sign of a zero)
+                oi[rank] = static_cast<int32_t>(idx);
+            }
+        }
+        BPS(20);
+    }
+    if (!walker) return;  // (the same for every thread)
+
+    // ---- walk mode, the row's last workgroup: the group that ranks with the threshold ---------
+    // n_above entries of the lists rank above it and are placed by the ranking; its members
+    // (an interval of order keys: probability does not decrease with the logit) take the
+    // places behind them in index order.
     __syncthreads();
-    BPS(19);
-    if (tid < static_cast<uint32_t>(kBigPickMine) && my_live) {
-        uint32_t rank = 0;
-#pragma unroll
-        for (int w = 0; w < NW; w++) rank += smem.part[w][tid];
-        if (rank < kk) {
-            const uint32_t idx = composite_index(mine);
-            if constexpr (SOFTMAX) store_elem(ov, rank, ordered_to_float(mine_hi));
-            else ov[rank] = rowp[idx];  // bit copy (keeps the sign of a zero)
-            oi[rank] = static_cast<int32_t>(idx);
-        }
+    uint32_t c_above = 0;  // (wave-uniform)
+    for (uint32_t f0 = 0; f0 < C; f0 += NT) {
+        const uint32_t f = f0 + tid;
+        const bool live = f < C;
+        const size_t at = where(live ? f : 0u);
+        float term = 0.f;
+        if constexpr (SOFTMAX) term = bw.term[at];
+        const uint64_t c = keyed(bw.cand[at], term, live);
+        c_above += static_cast<uint32_t>(__popcll(__ballot(static_cast<uint32_t>(c >> 32) > star)));
     }
-    BPS(20);
+    const uint32_t n_above = bigpick_count_sum(c_above, walk_slots);
+    if (n_above >= kk) return;
+    uint32_t xlo = thr, xhi = thr;
+    float p_star = 0.f;
+    if constexpr (SOFTMAX) {
+        p_star = ordered_to_float(star);
+        if (wave == 0) {
+            auto prob_of_key = [&](uint32_t key) {
+                return round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(key), M)) * rinv));
+            };
+            // down to the smallest key of that probability (probability 0: everything below as well) ...
+            const uint32_t lo_key = (p_star > 0.f && thr > kKeyNegInf) ? lowest_key_of_probability(thr, p_star, prob_of_key) : 0u;
+            // ... and up to the largest: one below the smallest key of a larger probability
+            const float p_next = __uint_as_float(__float_as_uint(p_star) + 1u);
+            const uint32_t top = order_key(M);
+            const uint32_t hi_key = prob_of_key(top) >= p_next ? lowest_key_of_probability(top, p_next, prob_of_key) - 1u : top;
+            if (lane == 0) {
+                walk_keys[0] = lo_key;
+                walk_keys[1] = hi_key;
+            }
+        }
+        __syncthreads();
+        xlo = walk_keys[0];
+        xhi = walk_keys[1];
+    }
+    const uint32_t places = kk - n_above;
+    auto place = [&](uint32_t pos, uint32_t j, float x) {
+        if constexpr (SOFTMAX) store_elem(ov, n_above + pos, p_star);
+        else store_elem(ov, n_above + pos, x);  // (the element's own bits: a half widened to float narrows back exactly)
+        oi[n_above + pos] = static_cast<int32_t>(j);
+    };
+    const bool row_aligned = (reinterpret_cast<uintptr_t>(rowp) & 15u) == 0;  // (the same for every thread)
+#ifdef VKOP_STAMPS
+    const unsigned long long walk_t0 = wall_clock64();
+#endif
+    const uint32_t found = (row_aligned && xhi != 0xFFFFFFFFu) ? first_members_by_vectors<T, NT>(walk_counts, rowp, n, places, xlo, xhi, place)
+                                       : first_members_by_scan<T, NT>(walk_counts, rowp, n, places, xlo, xhi, 1.f,
+                                                                      [&](uint32_t pos, uint32_t j) { place(pos, j, load_elem(rowp, j)); });
+#ifdef VKOP_STAMPS
+    if (tid == 0 && row < 8) {  // per row: (found << 40 | places << 20 | n_above), nanoseconds
+        g_bp_stamps[32 + 2 * row] = (static_cast<unsigned long long>(found) << 40) | (static_cast<unsigned long long>(places) << 20) | n_above;
+        g_bp_stamps[33 + 2 * row] = (wall_clock64() - walk_t0) * 10;
+    }
+#endif
+    if (found < places) {
+        // the group does not fill the places: elements that rank below it are part of the
+        // result, and of those the lists say nothing
+        __syncthreads();
+        bigpick_exact_row<T, SOFTMAX>(smem.exact, rowp, ov, oi, n, kk, fscratch, dscratch);
+    }
 }
 
 }  // namespace vkop

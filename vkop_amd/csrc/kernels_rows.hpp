@@ -451,6 +451,99 @@ __device__ __forceinline__ uint32_t first_members_by_scan(uint32_t *counts, cons
     return found;
 }
 
+// The same for a row that starts on a 16-byte boundary and is walked far (members
+// may be sparse): a thread takes 16 consecutive elements a round (128-bit loads), the
+// next round's loads in flight while the current tile is counted, membership by
+// two-sided float comparison (a median instruction), one prefix sum over the wave's
+// lanes a round.  emit(pos, j, x) also gets the element.  counts: 2 * NT / 64 words of
+// LDS.  Keys of the elements as they are (no scale); xhi must not be a NaN's key.
+template <typename T, int NT, typename Emit>
+__device__ __forceinline__ uint32_t first_members_by_vectors(uint32_t *counts, const T *rowp, uint32_t n, uint32_t places,
+                                                             uint32_t xlo, uint32_t xhi, Emit emit) {
+    constexpr int NW = NT / kWave, VEC = Vec128<T>::N, U = 16 / VEC;
+    constexpr uint32_t per_thread = 16, tile = static_cast<uint32_t>(NT) * per_thread;  // (more a round was measured slower)
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t nv = n - n % VEC;  // the elements that lie in whole vectors
+    // x is a member iff flo <= x <= fhi (keys at or below that of -inf: no lower bound); -0 == +0 as in the keys
+    const float flo = xlo <= kKeyNegInf ? -INFINITY : ordered_to_float(xlo), fhi = ordered_to_float(xhi);
+    Vec128<T> cur[U], nxt[U];
+    auto load_tile = [&](Vec128<T>(&q)[U], uint32_t base) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t e0 = base + tid * per_thread + static_cast<uint32_t>(u) * VEC;
+            q[u].v = make_uint4(0, 0, 0, 0);
+            q[u].load(rowp + (e0 < nv ? e0 : 0u));
+        }
+    };
+    load_tile(cur, 0);
+    uint32_t found = 0, round = 0;  // (found: the same in every thread)
+    for (uint32_t base = 0; base < nv && found < places; base += tile, round++) {
+        const bool more = base + tile < nv;
+        if (more) load_tile(nxt, base + tile);
+        // index order inside the tile: thread, then its elements
+        const uint32_t e_first = base + tid * per_thread;
+        uint32_t bits = 0;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const float x = cur[u].get(c);
+                const bool member = __builtin_amdgcn_fmed3f(x, flo, fhi) == x;  // (false for NaN)
+                bits |= member ? (1u << (u * VEC + c)) : 0u;
+            }
+        }
+        // (vectors past the row's end were read from its start)
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (e_first + static_cast<uint32_t>(u) * VEC >= nv) bits &= ~(((1u << VEC) - 1u) << (u * VEC));  // (VEC <= 8)
+        const uint32_t mine = static_cast<uint32_t>(__popc(bits));
+        uint32_t incl = mine;  // members in this lane and the lanes below it
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const uint32_t t = __shfl_up(incl, o, kWave);
+            if (lane >= static_cast<uint32_t>(o)) incl += t;
+        }
+        uint32_t *wc = counts + (round & 1u) * NW;
+        if (lane == kWave - 1) wc[wave] = incl;
+        __syncthreads();
+        uint32_t pos = found + incl - mine, in_tile = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const uint32_t c = wc[w];
+            pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
+            in_tile += c;
+        }
+        if (bits != 0u && pos < places) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    if ((bits >> (u * VEC + c)) & 1u) {
+                        if (pos < places) emit(pos, e_first + static_cast<uint32_t>(u * VEC + c), cur[u].get(c));
+                        pos++;
+                    }
+                }
+            }
+        }
+        found += in_tile;
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < U; u++) cur[u] = nxt[u];
+        }
+    }
+    if (found < places && nv < n) {
+        // the row's last elements, fewer than a vector: every wave counts them, the first one places them
+        const uint32_t j = nv + lane;
+        const float x = load_elem(rowp, j < n ? j : 0u);
+        const bool member = j < n && __builtin_amdgcn_fmed3f(x, flo, fhi) == x;
+        const uint64_t mask = __ballot(member);
+        const uint32_t pos = found + lanes_below(mask);
+        if (member && wave == 0 && pos < places) emit(pos, j, x);
+        found += static_cast<uint32_t>(__popcll(mask));
+    }
+    return found;
+}
+
 // Places g0 .. kk-1 of a row's result go to the lowest-index elements whose order
 // key lies in [xlo, xhi] (a group of equal rank too large to collect).  SOFTMAX:
 // every member's value is tie_value (the group's probability); otherwise the element
