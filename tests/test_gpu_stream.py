@@ -156,9 +156,10 @@ def _compare_paths(ops, n, k, dtype, rows, kinds, path):
         if dtype == np.float16:
             assert half_ulp_diff(v, v1).max() <= 1 and half_ulp_diff(v, ov).max() <= 1, what
         else:
-            # (the radix select behind rows.path = 1 at large k sums accurate terms only; the
-            # scan's fast terms may put the two row sums an ulp apart on either side of the oracle's)
-            assert ulp_diff(v, v1).max() <= (1 if path == 2 else 2) and ulp_diff(v, ov).max() <= 2, what
+            # (the bar is the distance to the oracle; the radix select behind rows.path = 1 at
+            # large k sums accurate terms only, the scan sums fast ones: on rows of few distinct
+            # values the two row sums may lie an ulp from the oracle's on either side)
+            assert ulp_diff(v, ov).max() <= 2 and ulp_diff(v1, ov).max() <= 2 and ulp_diff(v, v1).max() <= 2, what
         differ = 0
         xf = x.astype(np.float32)
         for r in range(rows):
@@ -205,7 +206,8 @@ def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
-@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (262144, 1024, 3), (300000, 600, 3), (1000, 5, 4), (2048, 16, 4)])
+@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (1048576, 100, 2), (262144, 1024, 3), (300000, 600, 3), (1000, 5, 4),
+                                      (2048, 16, 4)])
 def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtype):
     """Rows that defeat a threshold taken from block or lane maxima -- one value everywhere
     (with a key that is not a round number), two values a float apart, rows sorted

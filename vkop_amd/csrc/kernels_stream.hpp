@@ -450,6 +450,32 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         return false;
     };
     bool many_groups = gather(thr, 1ull << 32, std::false_type{});
+    if (many_groups) {
+        // More than kPickHitCap blocks reach thr: the threads' shares of the block maxima are
+        // not alike (rows sorted in runs as long as the stride between a thread's blocks put
+        // every run's top block into the same few threads, and the (k+1)-th largest THREAD
+        // maximum is then far below the (k+1)-th largest block maximum).  That one exactly,
+        // by a descent over all the keys, a barrier a bit: a dozen microseconds, on such rows.
+        uint32_t exact_thr = 0;
+        for (int bit = 31; bit >= 0; bit--) {
+            const uint32_t trial = exact_thr | (1u << bit);
+            uint32_t c = 0;  // wave-uniform
+#pragma unroll
+            for (int e = 0; e < GE; e++) c += static_cast<uint32_t>(__popcll(__ballot(gk[e] >= trial)));
+            uint32_t *wc = sh.scan_counts + (round & 1u) * NW;
+            round++;
+            if (lane == 0) wc[wave] = c;
+            __syncthreads();
+            uint32_t total = 0;
+#pragma unroll
+            for (int w = 0; w < NW; w++) total += wc[w];
+            if (total >= want) exact_thr = trial;
+        }
+        if (exact_thr > thr) {
+            thr = exact_thr;
+            many_groups = gather(thr, 1ull << 32, std::false_type{});
+        }
+    }
     uint32_t C2 = sh.count;
     uint32_t level_max = lmk;  // the thread maxima the current threshold was taken from
     if (!many_groups && C2 > static_cast<uint32_t>(kFastCap)) {

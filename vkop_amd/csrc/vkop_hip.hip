@@ -310,7 +310,8 @@ uint32_t rows_cap(int k) {
 constexpr int kWaveRowMaxK = 32;  // largest k served by the one-wave-per-row launch
 constexpr int kWideRowMinK = 64;  // above it a row that fits one workgroup is given to one (of enough threads)
 
-RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
+// (for_size: what a call could use whatever rows.path says at that time)
+RowsCfg choose_rows_cfg(const View &v, int k, int dtype, bool for_size = false) {
     RowsCfg c;
     if (v.g.inner != 1 || k > vkop::kFastMaxK || v.g.n == 0 || v.g.outer == 0) return c;
     const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
@@ -355,6 +356,12 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype) {
         c.nt = 64, c.g = 1;
         c.v = wave_loads <= 1 ? 1 : wave_loads <= 2 ? 2 : wave_loads <= 4 ? 4 : 8;
     } else {
+        // Several chunks a row.  With a k above 64 (only rows the scan kernels do not take
+        // get here: half-precision rows of 32K to 64K elements, rows beyond 8192 blocks) the
+        // chunks' lists overflow on anything but well-spread data and are made again from an
+        // exact select, 70 to 700 us measured; the multi-pass radix select takes 50 us
+        // whatever the data.  (rows.path = 1 keeps these kernels on every shape they can do.)
+        if (!for_size && k > kWideRowMinK && g_rows_path.load() != 1) return c;
         // largest per-workgroup chunk that still leaves >= 1024 workgroups; if the
         // tensor is too small for that, the smallest shape that covers a row
         int pick = -1;
@@ -420,7 +427,7 @@ struct ScanCfg {
 
 // Long last-axis rows, largest first, k up to kFastMaxK: the scan + pick pair.  The
 // largest chunk that still leaves 512 workgroups (else the smallest); rows too short
-// to be split, or with fewer than 4 (k + 1) blocks, or with more blocks than the pick
+// to be split, or with fewer than 2 (k + 1) blocks (4 (k + 1) for k > 255), or with more blocks than the pick
 // kernel takes in (16 per thread), are left to the other kernels.
 // (for_size: what a call could use whatever the tuning knobs say at that time)
 ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) {
@@ -435,7 +442,11 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
     const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
     const uint32_t n = v.g.n, rows = v.g.outer;
     const uint32_t blocks = (n + vkop::kBlockLanes * vec - 1) / (vkop::kBlockLanes * vec);
-    if (blocks < (big ? 2u : 4u) * (static_cast<uint32_t>(k) + 1u)) return c;
+    // (the pick kernel's threshold is the (k+1)-th largest of its 512 threads' maxima: at or
+    // above their median -- k + 1 <= 256, twice as many blocks -- few blocks and elements reach
+    // it; closer to the smallest of them, more blocks have to stand behind every thread)
+    const uint32_t blocks_per_place = big ? 2u : (k + 1 <= 256 ? 2u : 4u);
+    if (blocks < blocks_per_place * (static_cast<uint32_t>(k) + 1u)) return c;
     if (!big && (blocks + vkop::kPickThreads - 1) / vkop::kPickThreads > 16u) return c;
     if (big && (blocks + vkop::kBigPickThreads - 1) / vkop::kBigPickThreads > 32u) return c;
     if (big && static_cast<uint64_t>(rows) * (vkop::kBigPickCap / vkop::kBigPickMine) >= (1ull << 31)) return c;
@@ -743,7 +754,7 @@ int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v
 // Workspace that serves whichever route a top-k or fused call on this tensor can
 // take (largest or smallest, with or without the softmax tensor).
 size_t selection_workspace(const View &v, int k, int dtype) {
-    const size_t a = rows_layout(v, choose_rows_cfg(v, k, dtype)).total;
+    const size_t a = rows_layout(v, choose_rows_cfg(v, k, dtype, true)).total;
     const size_t b = rows_layout(v, RowsCfg{}, choose_bigk_cfg(v, k, dtype)).total;
     const size_t c = rows_layout(v, RowsCfg{}, BigKCfg{}, choose_scan_cfg(v, k, dtype, true)).total;
     return a > b ? (a > c ? a : c) : (b > c ? b : c);
