@@ -2,6 +2,7 @@
 """Times every operator of the library on the five reference workloads.
 
   python -m vkop_amd.bench_ops [--steps K] [--warmup W] [--only NAME_SUBSTRING] [--eager]
+  python -m vkop_amd.bench_ops --data-sweep [--only NAME_SUBSTRING]
 
 bench.py at the repository root measures the headline (fused softmax -> top-k on
 [64,128256]); this script covers the rest: plain softmax, plain top-k, the fused
@@ -10,6 +11,12 @@ K calls recorded once and replayed, HIP events around the replay.  Inputs rotate
 over enough device buffers (> 288 MB) that the Infinity Cache cannot serve them.
 Prints one JSON line per case: microseconds per call and the algorithmic rate
 (compulsory reads + final writes over time).
+
+--data-sweep instead times top-k (largest, smallest) and the fused call on a dozen
+shapes x fourteen kinds of rows (sorted, constant, two values, a dozen levels, masked,
+NaN / +inf rows, one value with peaks, sorted runs, ...) in single and half precision and
+flags every case that takes more than three times the same shape's normal rows: the
+places where a selection kernel falls off a cliff.
 """
 import argparse
 import json
@@ -25,6 +32,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--only", default="")
+    ap.add_argument("--data-sweep", action="store_true",
+                    help="time top-k and the fused call on shapes x kinds of awkward rows instead of the workloads")
     ap.add_argument("--eager", action="store_true",
                     help="launch every call from the host instead of replaying a recording (for counter runs under "
                          "rocprofv3 --pmc; the timings of such a run mean nothing)")
@@ -114,6 +123,47 @@ def main():
                                        ptr, nb + 256, stream)
         us = timed(call, len(bufs))
         report(name, us, x.nbytes + rows * k * (x.itemsize + 4))
+
+    if args.data_sweep:
+        shapes = [(256, 1000, 5), (8192, 256, 8), (4096, 1024, 32), (1024, 4096, 64), (256, 8192, 100), (16, 8400, 300),
+                  (64, 32000, 40), (32, 50257, 200), (64, 128256, 50), (16, 100000, 600), (8, 262144, 1024), (8, 262144, 2000),
+                  (4, 1048576, 100)]
+        for rows, n, k in shapes:
+            for dt, tdt, dname in ((F32, torch.float32, "f32"), (F16, torch.float16, "f16")):
+                base = None
+                names = {kind: "[%d,%d] k=%d %s %s" % (rows, n, k, dname, kind) for kind in synth.AWKWARD_KINDS}
+                if not any(args.only in nm for nm in names.values()):
+                    continue
+                for kind in synth.AWKWARD_KINDS:
+                    name = names[kind]
+                    if args.only not in name and kind != "normal":  # (the normal rows are every case's yardstick)
+                        continue
+                    x = synth.awkward_rows(kind, rows, n, seed=rows + n + k)
+                    nb = max(2, min(16, (64 << 20) // x.nbytes))
+                    bufs = [torch.from_numpy(x).cuda().to(tdt) for _ in range(nb)]
+                    vals = torch.empty((rows, k), dtype=tdt, device="cuda")
+                    idx = torch.empty((rows, k), dtype=torch.int32, device="cuda")
+                    wsb = max(capi.topk_workspace_bytes(dt, (rows, n), -1, k), capi.softmax_topk_workspace_bytes(dt, (rows, n), -1, k))
+                    ws, ptr = workspace(wsb + 256)
+                    sh = (rows, n)
+                    us = [timed(lambda b: capi.topk(bufs[b].data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, sh, -1, k, 1, 1, ptr,
+                                                    wsb + 256, stream), nb),
+                          timed(lambda b: capi.softmax_topk(bufs[b].data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), dt, sh, -1, k, 1,
+                                                            ptr, wsb + 256, stream), nb),
+                          timed(lambda b: capi.topk(bufs[b].data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, sh, -1, k, 0, 1, ptr,
+                                                    wsb + 256, stream), nb)]
+                    if args.eager:
+                        continue
+                    if kind == "normal":
+                        base = us
+                    line = {"case": name, "path": capi.measure_path(dt, sh, -1, k), "topk_us": round(us[0], 1),
+                            "fused_us": round(us[1], 1), "smallest_us": round(us[2], 1)}
+                    if base is not None:
+                        slow = [w for w, v, bv in zip(("topk", "fused", "smallest"), us, base) if v > 3 * bv and v > 30]
+                        if slow:
+                            line["over_3x_normal"] = slow
+                    print(json.dumps(line), flush=True)
+        return
 
     c1 = synth.classifier_logits(1, 1000, synth.SEEDS["C1"])
     c2 = synth.classifier_logits(256, 1000, synth.SEEDS["C2"])

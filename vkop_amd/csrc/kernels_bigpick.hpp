@@ -6,17 +6,19 @@
 //   bigpick_gather_kernel   rows * G2 workgroups.  Every workgroup finds, from the
 //                           row's block maxima, a value that at least k+1 of them
 //                           reach (a 2048-bin LDS histogram of every fourth key over
-//                           the range the keys span, then a count over all of them),
+//                           the range the keys span, then a count over all of them;
+//                           after coarse bins a second round inside one bin),
 //                           lowers it by a margin
 //                           that keeps probability ties above it (softmax variant),
 //                           reads again those of ITS share of the blocks that reach
-//                           it and appends their elements at or above the value to
-//                           the row's candidate list in global memory -- for the
+//                           it and appends their elements to the row's candidate
+//                           lists in global memory: everything above the value, and
+//                           up to a quota of what lies at or just below it -- for the
 //                           softmax variant with the element's accurate term
 //                           exp(x - M), whose difference to the fast term the scan
 //                           added goes into the row's correction (an integer sum, so
 //                           that the order of arrival does not show in it);
-//   bigpick_rank_kernel     rows * 128 workgroups, 32 candidates each.  Every
+//   bigpick_rank_kernel     rows * 256 workgroups, 32 candidates each.  Every
 //                           workgroup takes the whole list into registers, a quarter
 //                           per wave (softmax: as probabilities, term / corrected
 //                           sum), counts for each of its own 32 how many of the list
@@ -24,12 +26,15 @@
 //                           vector compare and a population count per 64 pairs --
 //                           and stores those that rank below k at their place.
 //
-// Whatever this cannot hold or decide -- more candidates than the list's capacity
-// (rows full of equal values), fewer than k+1 (rows of mostly -inf), a sum that is
-// not a positive finite number, probabilities so small that the margin does not
-// separate them -- is left to the first workgroup of the row, which runs the exact
-// single-workgroup select over the whole row (select.hpp); every workgroup of the row
-// reaches the same verdict from the same numbers.
+// Rows whose cut falls into a crowd -- one value in thousands of places, rows of mostly
+// -inf, probabilities that underflow to 0 and tie -- exceed the quota: the lists then
+// hold everything that ranks ABOVE the threshold's own rank group, and the row's last
+// rank workgroup takes that group's first members from a walk over the row in index
+// order (first_members_by_vectors).  Rows of NaN probabilities are written directly.
+// What is left -- more elements above the threshold than the lists hold, a group too
+// small to fill the places -- goes to the first workgroup of the row, which runs the
+// exact single-workgroup select over the whole row (select.hpp); every workgroup of the
+// row reaches the same verdict from the same numbers.
 #pragma once
 
 #include "kernels_stream.hpp"
@@ -47,7 +52,7 @@ static __device__ unsigned long long g_bp_stamps[64];
 
 constexpr int kBigPickThreads = 256;
 constexpr int kBigPickWaves = kBigPickThreads / kWave;
-constexpr int kBigPickCap = 4096;       // candidates of a row that are ranked
+constexpr int kBigPickCap = 8192;       // candidates of a row that are ranked (block-clustered rows have about 2 (k+1))
 constexpr int kBigPickLists = 8;        // lists a row's candidates are appended to (gather workgroup p uses list p % 8:
                                         // eight counters instead of one that every workgroup of the row queues for)
 constexpr int kBigPickListCap = 2048;   // entries per list
@@ -375,8 +380,9 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
     // reach thr and all but one are such blocks; a row of one value: every block is), two
     // facts about the block minima make the candidates few again without a look at the
     // elements:
-    //  * m = ceil((k+1) / (16 * VEC)) block minima reach their m-th largest, so k+1 elements
-    //    reach it: a threshold as valid as thr and, on such rows, far higher;
+    //  * a block whose minimum reaches a value holds 16 * VEC elements that do, a block whose
+    //    maximum does holds one: the largest value for which these known elements come to k+1 is
+    //    a threshold as valid as thr and, on such rows, far higher;
     //  * in index order, let B be the first block at which the count "all of a block whose
     //    minimum reaches thr, one of a block whose maximum does" comes to k+1: k+1 elements
     //    at or above thr lie in blocks up to B, so an element at or below thr in a later
@@ -393,15 +399,19 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
         const uint32_t both = bigpick_count_sum(c2, cslots[flip]);
         const uint32_t nfull = both >> 16, nhit = both & 0xFFFFu;
         if (nfull * BE + (nhit - nfull) > static_cast<uint32_t>(kBigPickCap)) {  // (the same for every thread of every workgroup of the row)
-            const uint32_t m = (want + BE - 1) / BE;
+            // the largest value (its low ten bits aside) that k+1 elements are KNOWN to reach
             uint32_t tmin = 0;
             for (int bit = 31; bit >= 10; bit--) {
                 const uint32_t trial = tmin | (1u << bit);
                 uint32_t c = 0;
 #pragma unroll
-                for (int e = 0; e < GE; e++) c += static_cast<uint32_t>(__popcll(__ballot(gn[e] >= trial && gk[e] != 0u)));
+                for (int e = 0; e < GE; e++)
+                    c += (static_cast<uint32_t>(__popcll(__ballot(gn[e] >= trial && gk[e] != 0u))) << 16) +
+                         static_cast<uint32_t>(__popcll(__ballot(gk[e] >= trial)));
                 flip ^= 1u;
-                if (bigpick_count_sum(c, cslots[flip]) >= m) tmin = trial;
+                const uint32_t packed = bigpick_count_sum(c, cslots[flip]);
+                const uint32_t full = packed >> 16, reached = packed & 0xFFFFu;
+                if (full * BE + (reached - full) >= want) tmin = trial;
             }
             if (tmin > thr) {
                 thr = tmin;
@@ -652,7 +662,9 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_rank_kernel(const T *
     __shared__ double dscratch[NW];
     __shared__ uint32_t walk_slots[NW], walk_counts[2 * NW], walk_keys[2];
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t row = blockIdx.x / G3, g = blockIdx.x - row * G3;
+    // (workgroup g of every row before workgroup g + 1 of any: the few that have candidates are dispatched first)
+    const uint32_t rows = gridDim.x / G3;
+    const uint32_t g = blockIdx.x / rows, row = blockIdx.x - g * rows;
     const T *rowp = in + static_cast<size_t>(row) * n;
     T *ov = values + static_cast<size_t>(row) * k;
     int32_t *oi = indices + static_cast<size_t>(row) * k;
@@ -781,7 +793,7 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_rank_kernel(const T *
         const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
         uint32_t before = 0;  // lane j: the count for candidate j
         // (entries past the wave's share are 0 and count for nothing: the loop over them is
-        // compiled for 4, 8, 12 and 16 entries a lane, without a branch inside)
+        // compiled for 4, 8, 12, 16, 24 and 32 entries a lane, without a branch inside)
         auto count_all = [&](auto steps_tag) __attribute__((always_inline)) {
             constexpr int STEPS = decltype(steps_tag)::value;
             for (int j = 0; j < kBigPickMine; j++) {
@@ -796,7 +808,9 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_rank_kernel(const T *
         if (steps <= 4u) count_all(std::integral_constant<int, 4>{});
         else if (steps <= 8u) count_all(std::integral_constant<int, 8>{});
         else if (steps <= 12u) count_all(std::integral_constant<int, 12>{});
-        else count_all(std::integral_constant<int, 16>{});
+        else if (steps <= 16u) count_all(std::integral_constant<int, 16>{});
+        else if (steps <= 24u) count_all(std::integral_constant<int, 24>{});
+        else count_all(std::integral_constant<int, kBigRankPerLane>{});
         if (lane < static_cast<uint32_t>(kBigPickMine)) smem.part[wave][lane] = before;
         __syncthreads();
         BPS(19);
