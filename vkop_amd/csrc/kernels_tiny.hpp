@@ -188,21 +188,42 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             if (static_cast<uint32_t>(__popcll(__ballot(lmk >= trial))) >= want) tie = trial;
         }
         tie = max(tie, kKeyNegInf);
-        // the elements above T, as in step 4
-        uint32_t above = 0;  // wave-uniform
+        // the elements above T, as in step 4 (all threads call; returns their number)
+        auto gather_above = [&](uint32_t t) __attribute__((always_inline)) -> uint32_t {
+            uint32_t count = 0;  // wave-uniform
 #pragma unroll
-        for (int i = 0; i < V; i++) {
+            for (int i = 0; i < V; i++) {
 #pragma unroll
-            for (int c = 0; c < VEC; c++) {
-                const bool pass = key[i * VEC + c] > tie;
-                const uint64_t mask = __ballot(pass);
-                if (mask != 0ull) {
-                    const uint32_t at = above + lanes_below(mask);
-                    const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
-                    if (pass && at < static_cast<uint32_t>(kWave)) smem.cand[at] = composite(key[i * VEC + c], e);
-                    above += static_cast<uint32_t>(__popcll(mask));
+                for (int c = 0; c < VEC; c++) {
+                    const bool pass = key[i * VEC + c] > t;
+                    const uint64_t mask = __ballot(pass);
+                    if (mask != 0ull) {
+                        const uint32_t at = count + lanes_below(mask);
+                        const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
+                        if (pass && at < static_cast<uint32_t>(kWave)) smem.cand[at] = composite(key[i * VEC + c], e);
+                        count += static_cast<uint32_t>(__popcll(mask));
+                    }
                 }
             }
+            return count;
+        };
+        uint32_t above = gather_above(tie);
+        if (above >= want) {
+            // More than k elements above the (k+1)-th largest LANE maximum: the top of the row
+            // sits in few lanes (a sorted row: a lane's elements are neighbours).  The exact
+            // (k+1)-th largest ELEMENT then, by a descent over all of them; fewer than k+1
+            // elements lie above that.
+            uint32_t t2 = 0;
+            for (int bit = 31; bit >= 0; bit--) {
+                const uint32_t trial = t2 | (1u << bit);
+                uint32_t c = 0;
+#pragma unroll
+                for (int e = 0; e < ELEMS; e++) c += static_cast<uint32_t>(__popcll(__ballot(key[e] >= trial)));
+                if (c >= want) t2 = trial;
+            }
+            tie = max(t2, kKeyNegInf);
+            __syncthreads();  // (one wave: the list is written again)
+            above = gather_above(tie);
         }
         if (above < want) {
             // the first want - above elements equal to T: vector by vector, lane by lane, element by element
