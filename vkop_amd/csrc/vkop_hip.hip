@@ -362,10 +362,17 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype, bool for_size = false) 
         // exact select, 70 to 700 us measured; the multi-pass radix select takes 50 us
         // whatever the data.  (rows.path = 1 keeps these kernels on every shape they can do.)
         if (!for_size && k > kWideRowMinK && g_rows_path.load() != 1) return c;
+        // a row that one workgroup of 256 threads can hold: the smallest such shape (many short rows
+        // would otherwise get the largest workgroup, most of its threads without an element); else the
         // largest per-workgroup chunk that still leaves >= 1024 workgroups; if the
         // tensor is too small for that, the smallest shape that covers a row
         int pick = -1;
-        for (int i = 0; i < 6; i++) {
+        for (int i = 0; i < 4 && pick < 0; i++) {
+            const uint64_t span = static_cast<uint64_t>(shapes[i][0]) * shapes[i][1] * vec;
+            if (shapes[i][0] == 256 && span >= n && fits(shapes[i][0], shapes[i][1], 1)) pick = i;
+        }
+        const bool one_workgroup = pick >= 0;
+        for (int i = 0; i < 6 && !one_workgroup; i++) {
             const uint32_t span = static_cast<uint32_t>(shapes[i][0]) * shapes[i][1] * vec;
             const uint32_t g = (n + span - 1) / span;
             if (!fits(shapes[i][0], shapes[i][1], g)) continue;
