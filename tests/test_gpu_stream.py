@@ -197,7 +197,7 @@ def test_scan_with_spread_out_pick_for_large_k_equals_radix_select_and_oracle(op
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
 @pytest.mark.parametrize("n,k", [(1000, 5), (1000, 16), (33, 5), (5, 5), (1024, 1), (2048, 7), (777, 10), (256, 3), (64, 16),
-                                 (1001, 5), (130, 2)])
+                                 (1001, 5), (130, 2), (1000, 32), (2048, 24), (1500, 20), (40, 32)])
 def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k, dtype):
     """Short rows, small k (a classifier head): the one-wave-per-row kernel against the
     chunk kernel (rows.path = 1) and the oracle, on regular rows and on the ones it hands
@@ -207,7 +207,7 @@ def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
 @pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (1048576, 100, 2), (262144, 1024, 3), (300000, 600, 3), (1000, 5, 4),
-                                      (2048, 16, 4)])
+                                      (2048, 16, 4), (2048, 32, 4)])
 def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtype):
     """Rows that defeat a threshold taken from block or lane maxima -- one value everywhere
     (with a key that is not a round number), two values a float apart, rows sorted

@@ -29,7 +29,7 @@
 
 namespace vkop {
 
-constexpr int kTinyMaxK = 16;
+constexpr int kTinyMaxK = 32;  // (k + 1 candidates, one per lane, and room for a few more)
 
 template <typename T, int V, bool SOFTMAX, bool ALIGNED>
 __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ in, T *__restrict__ values,
