@@ -218,9 +218,11 @@ int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_ca
  * setting change between its workspace query and its launch is refused with
  * VKOP_HIP_ERR_WORKSPACE at worst, never runs out of bounds: *_workspace_bytes()
  * covers every setting).
- *   "rows.path": 0 (default) = long last-axis rows go through the scan + pick
- *       kernel pair where it applies (k up to 511; beyond that, scan + gather +
- *       rank); 1 = never (the chunk + merge kernels, the multi-pass radix select).
+ *   "rows.path": 0 (default) = short last-axis rows with k up to 32 go through
+ *       the one-wave-per-row kernel, rows too long for one workgroup through the
+ *       scan + pick kernel pair where it applies (k up to 511; beyond that, scan +
+ *       gather + rank); 1 = never (the chunk + merge kernels, the multi-pass radix
+ *       select).
  *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the
  *       chunk kernel (threads per workgroup, 128-bit loads per thread,
  *       workgroups per row); all three must be set, 0 = automatic (default).

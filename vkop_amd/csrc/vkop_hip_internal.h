@@ -18,9 +18,10 @@ extern "C" {
 int vkop_hip_measure_stages(int stages);
 
 /* Which streaming kernels a fused / top-k (largest) call on this tensor would run
- * with the current tuning settings: 2 = rows_scan_kernel + rows_pick_kernel, 1 =
- * rows_chunk_kernel (+ rows_merge_kernel when a row is split), 0 = other kernels,
- * -1 = bad arguments. */
+ * with the current tuning settings: 4 = rows_tiny_kernel (one wave per row), 2 =
+ * rows_scan_kernel + rows_pick_kernel, 3 = rows_scan_kernel + bigpick_gather_kernel +
+ * bigpick_rank_kernel, 1 = rows_chunk_kernel (+ rows_merge_kernel when a row is
+ * split), 0 = other kernels, -1 = bad arguments. */
 int vkop_hip_measure_path(int dtype, const int *shape, int ndim, int axis, int k);
 
 #ifdef __cplusplus
