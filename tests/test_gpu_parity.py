@@ -47,7 +47,8 @@ def assert_softmax_close(got, x, axis, what=""):
     if got.dtype == np.float16:
         assert half_ulp_diff(got, exp).max() <= 1, what
         g, e = got.astype(np.float32), exp.astype(np.float32)
-        ok = np.abs(g - e) <= 1e-3 * np.abs(e) + 6e-8
+        with np.errstate(invalid="ignore"):
+            ok = (np.abs(g - e) <= 1e-3 * np.abs(e) + 6e-8) | (np.isnan(g) & np.isnan(e))
         assert ok.all(), what
     else:
         d = ulp_diff(got, exp)
@@ -81,6 +82,22 @@ def test_softmax_ragged_lengths(ops, n):
     assert_softmax_close(host(ops.softmax(dev(x))), x, -1, "n=%d" % n)
     xh = x.astype(np.float16)
     assert_softmax_close(host(ops.softmax(dev(xh))), xh, -1, "n=%d half" % n)
+
+
+@pytest.mark.parametrize("shape", [(1001, 197), (7, 64), (4099, 33), (513, 512), (12, 5, 197, 197), (70000, 8)])
+def test_softmax_many_short_rows(ops, shape):
+    """Rows of up to 512 elements take a wave each, four rows a workgroup: row counts that
+    are not a multiple of four, rows that do not start on 16 bytes, an attention-shaped
+    tensor, rows shorter than a wave; a NaN row, a +inf row and a row of -inf among them."""
+    rng = np.random.default_rng(shape[0] + shape[-1])
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    flat = x.reshape(-1, shape[-1])
+    flat[1, shape[-1] // 2] = np.nan
+    flat[2, 0] = np.inf
+    flat[3, :] = -np.inf
+    assert_softmax_close(host(ops.softmax(dev(x))), x, -1, str(shape))
+    xh = x.astype(np.float16)
+    assert_softmax_close(host(ops.softmax(dev(xh))), xh, -1, str(shape) + " half")
 
 
 @pytest.mark.parametrize("shape,axis", [((5, 7, 9), 0), ((5, 7, 9), 1), ((5, 7, 9), 2), ((2, 3, 4, 5), 0), ((2, 3, 4, 5), 1),

@@ -10,6 +10,8 @@
 //                           writes exp(x - M) / S for its chunk.  The second
 //                           read of the input comes from the Infinity Cache for
 //                           tensors that fit it.
+//   softmax_wave_kernel     rows of up to 512 elements: one wave per row, four rows a
+//                           workgroup, no LDS.
 // Strided lines (another axis, short lines):
 //   softmax_strided_reg_kernel  one thread per line, threads along the
 //                           contiguous inner axis; the line's elements stay in
@@ -102,6 +104,50 @@ __global__ __launch_bounds__(NT) void softmax_row_kernel(const T *in, T *out, ui
         }
         if constexpr (ALIGNED)
             if (e0 < n) *reinterpret_cast<uint4 *>(orow + e0) = r.v;
+    }
+}
+
+// ---- short rows: one wave per row ---------------------------------------------------------
+// Rows of up to 64 * E elements (E <= 8): lane l holds elements l, l + 64, ...; every
+// load and store instruction of a wave covers 64 neighbouring elements whatever the row's
+// alignment; maximum and sum cross the lanes without LDS or a barrier.  Four rows a
+// workgroup.  (A workgroup of 256 threads per row leaves three quarters of them idle on a
+// 64-element row and takes two barriers: [65536,64] took 68 us.)
+constexpr int kSoftmaxWaveRows = 4;  // rows (waves) per workgroup
+template <typename T, int E>
+__global__ __launch_bounds__(kSoftmaxWaveRows *kWave) void softmax_wave_kernel(const T *__restrict__ in, T *__restrict__ out,
+                                                                                uint32_t rows, uint32_t n, int nan_where,
+                                                                                float nan_value) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t row = blockIdx.x * kSoftmaxWaveRows + threadIdx.x / kWave;
+    if (row >= rows) return;  // (the whole wave)
+    const T *rowp = in + static_cast<size_t>(row) * n;
+    T *orow = out + static_cast<size_t>(row) * n;
+    float x[E];
+#pragma unroll
+    for (int j = 0; j < E; j++) {
+        const uint32_t e = static_cast<uint32_t>(j) * kWave + lane;
+        x[j] = load_elem(rowp, e < n ? e : 0u);
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < E; j++)
+        if (static_cast<uint32_t>(j) * kWave + lane < n) m = fmaxf(m, x[j]);  // (drops NaN)
+    m = wave_max_f32_uniform(m);
+    float t[E];
+    double acc = 0.0;
+#pragma unroll
+    for (int j = 0; j < E; j++) {
+        t[j] = static_cast<uint32_t>(j) * kWave + lane < n ? softmax_term(x[j], m) : 0.f;
+        acc += static_cast<double>(t[j]);
+    }
+    const double rinv = 1.0 / wave_sum_f64_uniform(acc);
+#pragma unroll
+    for (int j = 0; j < E; j++) {
+        const uint32_t e = static_cast<uint32_t>(j) * kWave + lane;
+        float p = round_to_storage<T>(static_cast<float>(static_cast<double>(t[j]) * rinv));
+        if (nan_where && p != p) p = nan_value;
+        if (e < n) store_elem(orow, e, p);
     }
 }
 

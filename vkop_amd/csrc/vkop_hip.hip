@@ -152,7 +152,7 @@ const RowShape kShapesF32[] = {{256, 1}, {256, 2}, {256, 4}, {256, 8}, {512, 8},
 const RowShape kShapesF16[] = {{256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}, {1024, 4}};
 
 struct SoftmaxPlan {
-    enum Kind { kGeneralLines, kGeneralStrided, kRow, kChunked, kStridedRegs } kind = kGeneralLines;
+    enum Kind { kGeneralLines, kGeneralStrided, kRow, kWaveRow, kChunked, kStridedRegs } kind = kGeneralLines;
     RowShape shape{0, 0};
     uint32_t g = 1, per = 0;
     size_t workspace = 0;
@@ -189,6 +189,10 @@ SoftmaxPlan plan_softmax(const View &v, int dtype) {
     if (v.g.inner != 1) {
         if (n <= static_cast<uint32_t>(vkop::kStridedMaxN)) p.kind = SoftmaxPlan::kStridedRegs;
         else p.kind = n >= 2048 ? SoftmaxPlan::kGeneralLines : SoftmaxPlan::kGeneralStrided;
+        return p;
+    }
+    if (n <= 8u * vkop::kWave) {  // short rows: a wave each
+        p.kind = SoftmaxPlan::kWaveRow;
         return p;
     }
     const uint32_t biggest = static_cast<uint32_t>(shapes[5].nt) * shapes[5].v * vec;
@@ -245,6 +249,19 @@ int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, f
 #undef VKOP_ROW
         if (!done) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no softmax_row_kernel for %d x %d", p.shape.nt, p.shape.v);
         return launched("softmax_row_kernel");
+    }
+    case SoftmaxPlan::kWaveRow: {
+        const uint32_t blocks = (lines + vkop::kSoftmaxWaveRows - 1) / vkop::kSoftmaxWaveRows;
+        const uint32_t per_lane = (v.g.n + vkop::kWave - 1) / vkop::kWave;
+#define VKOP_WAVE_ROW(E)                                                                                    \
+    vkop::softmax_wave_kernel<T, E><<<blocks, vkop::kSoftmaxWaveRows * vkop::kWave, 0, st>>>(in, out, lines, v.g.n, \
+                                                                                              nan_where, nan_value)
+        if (per_lane <= 1) VKOP_WAVE_ROW(1);
+        else if (per_lane <= 2) VKOP_WAVE_ROW(2);
+        else if (per_lane <= 4) VKOP_WAVE_ROW(4);
+        else VKOP_WAVE_ROW(8);
+#undef VKOP_WAVE_ROW
+        return launched("softmax_wave_kernel");
     }
     case SoftmaxPlan::kChunked: {
         if (ws == nullptr || ws_bytes < p.workspace)
