@@ -101,11 +101,20 @@ def test_softmax_many_short_rows(ops, shape):
 
 
 @pytest.mark.parametrize("shape,axis", [((5, 7, 9), 0), ((5, 7, 9), 1), ((5, 7, 9), 2), ((2, 3, 4, 5), 0), ((2, 3, 4, 5), 1),
-                                        ((2, 3, 4, 5), -2), ((300,), 0), ((4, 2500, 3), 1), ((3, 70, 130), 1), ((2, 5, 64), 1)])
+                                        ((2, 3, 4, 5), -2), ((300,), 0), ((4, 2500, 3), 1), ((3, 70, 130), 1), ((2, 5, 64), 1),
+                                        ((2, 1000, 64), 1), ((1, 4096, 300), 1), ((2, 200, 7, 5), 1), ((3, 129, 2), 1),
+                                        ((2, 777, 65), 1), ((5000, 33), 0)])
 def test_softmax_axes(ops, shape, axis):
     rng = np.random.default_rng(5)
     x = (rng.standard_normal(shape) * 2).astype(np.float32)
+    if x.size > 4000:   # a NaN line, a +inf line, a line of -inf
+        xv = np.moveaxis(x, axis, -1)
+        xv[..., 0, 5] = np.nan
+        xv[..., 1, 3] = np.inf
+        xv[..., 2, :] = -np.inf
     assert_softmax_close(host(ops.softmax(dev(x), axis)), x, axis, str((shape, axis)))
+    xh = x.astype(np.float16)
+    assert_softmax_close(host(ops.softmax(dev(xh), axis)), xh, axis, str((shape, axis)) + " half")
 
 
 def test_softmax_special_values_and_nan_option(ops):

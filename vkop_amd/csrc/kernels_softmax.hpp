@@ -12,6 +12,9 @@
 //                           tensors that fit it.
 //   softmax_wave_kernel     rows of up to 512 elements: one wave per row, four rows a
 //                           workgroup, no LDS.
+// Strided lines (another axis, long lines):
+//   softmax_strided_tile_kernel  a tile of up to 64 neighbouring lines per workgroup of 16 waves,
+//                           rows dealt to the waves, three passes over the tile.
 // Strided lines (another axis, short lines):
 //   softmax_strided_reg_kernel  one thread per line, threads along the
 //                           contiguous inner axis; the line's elements stay in
@@ -249,6 +252,100 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
         }
         if constexpr (ALIGNED)
             if (e0 < c1) *reinterpret_cast<uint4 *>(orow + e0) = r.v;
+    }
+}
+
+// ---- long strided lines: a tile of neighbouring lines per workgroup -----------------------------
+// Lines along a non-last axis that the register kernel below does not hold (n above
+// kStridedMaxN).  A workgroup takes TI neighbouring lines (TI = the power of two at or
+// above min(inner, 64)); lane l of a wave looks at line l % TI of the tile and, with 64 / TI
+// rows per instruction, at row l / TI of the instruction's rows, so every load and store
+// covers contiguous pieces of TI elements; the workgroup's waves take the rows in turn.
+// Three passes over the tile (maximum, sum of terms, output; the second and third come
+// from the cache for tiles of a few hundred kilobytes), each reduced across a wave's row
+// groups by shuffles and across the waves through LDS.  One thread per line -- what this
+// replaces -- had 2048 threads on a [32,1000,64] tensor: 741 us for 16 MB.
+constexpr int kStridedTileThreads = 1024;
+template <typename T>
+__global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kernel(const T *__restrict__ in, T *__restrict__ out,
+                                                                                    LineGeom g, uint32_t ti_shift, int nan_where,
+                                                                                    float nan_value) {
+    constexpr int NT = kStridedTileThreads, NW = NT / kWave;
+    constexpr int U = 16;  // rows a lane has in flight (a pass is a chain of n / (16 waves * U) round trips)
+    __shared__ float fmax_lds[NW][kWave];
+    __shared__ double dsum_lds[NW][kWave];
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t TI = 1u << ti_shift, RPW = kWave >> ti_shift;  // lines a tile, rows per wave instruction
+    const uint32_t tiles = (g.inner + TI - 1) >> ti_shift;
+    const uint32_t o = blockIdx.x / tiles, tile = blockIdx.x - o * tiles;
+    const uint32_t col = (tile << ti_shift) + (lane & (TI - 1)), r = lane >> ti_shift;
+    const bool col_ok = col < g.inner;
+    const size_t base = static_cast<size_t>(o) * g.n * g.inner + (col_ok ? col : 0u);
+    const uint32_t step = NW * RPW;  // rows the workgroup covers per turn
+    // element of row j of this lane's line
+    auto at = [&](uint32_t j) { return base + static_cast<size_t>(j) * g.inner; };
+    // combine v over the lanes of a wave that look at the same line, then over the waves; all threads call
+    auto reduce_max = [&](float v) -> float {
+        for (uint32_t off = TI; off < static_cast<uint32_t>(kWave); off <<= 1) v = fmaxf(v, __shfl_xor(v, static_cast<int>(off), kWave));
+        fmax_lds[wave][lane] = v;
+        __syncthreads();
+        float m = fmax_lds[0][lane & (TI - 1)];
+#pragma unroll
+        for (int w = 1; w < NW; w++) m = fmaxf(m, fmax_lds[w][lane & (TI - 1)]);
+        return m;
+    };
+    auto reduce_sum = [&](double v) -> double {
+        for (uint32_t off = TI; off < static_cast<uint32_t>(kWave); off <<= 1) v += __shfl_xor(v, static_cast<int>(off), kWave);
+        dsum_lds[wave][lane] = v;
+        __syncthreads();
+        double sum = dsum_lds[0][lane & (TI - 1)];
+#pragma unroll
+        for (int w = 1; w < NW; w++) sum += dsum_lds[w][lane & (TI - 1)];  // fixed order: run-to-run stable
+        return sum;
+    };
+    // ---- 1. the lines' maxima
+    float m = -INFINITY;
+    for (uint32_t j0 = wave * RPW + r; j0 < g.n; j0 += step * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
+            x[u] = load_elem(in, at(j < g.n ? j : 0u));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (j0 + static_cast<uint32_t>(u) * step < g.n) m = fmaxf(m, x[u]);  // (drops NaN)
+    }
+    m = reduce_max(m);
+    // ---- 2. the sums of the terms
+    double acc = 0.0;
+    for (uint32_t j0 = wave * RPW + r; j0 < g.n; j0 += step * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
+            x[u] = load_elem(in, at(j < g.n ? j : 0u));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            if (j0 + static_cast<uint32_t>(u) * step < g.n) acc += static_cast<double>(softmax_term(x[u], m));
+    }
+    const LineStats st{m, 0.f, 1.0 / reduce_sum(acc)};
+    // ---- 3. the probabilities
+    for (uint32_t j0 = wave * RPW + r; j0 < g.n; j0 += step * U) {
+        float x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
+            x[u] = load_elem(in, at(j < g.n ? j : 0u));
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
+            float p = round_to_storage<T>(softmax_prob(x[u], st));
+            if (nan_where && p != p) p = nan_value;
+            if (j < g.n && col_ok) store_elem(out, at(j), p);
+        }
     }
 }
 

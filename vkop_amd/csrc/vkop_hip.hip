@@ -152,7 +152,7 @@ const RowShape kShapesF32[] = {{256, 1}, {256, 2}, {256, 4}, {256, 8}, {512, 8},
 const RowShape kShapesF16[] = {{256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}, {1024, 4}};
 
 struct SoftmaxPlan {
-    enum Kind { kGeneralLines, kGeneralStrided, kRow, kWaveRow, kChunked, kStridedRegs } kind = kGeneralLines;
+    enum Kind { kGeneralLines, kGeneralStrided, kRow, kWaveRow, kChunked, kStridedRegs, kStridedTile } kind = kGeneralLines;
     RowShape shape{0, 0};
     uint32_t g = 1, per = 0;
     size_t workspace = 0;
@@ -188,7 +188,7 @@ SoftmaxPlan plan_softmax(const View &v, int dtype) {
     const uint32_t n = v.g.n, rows = v.g.outer;
     if (v.g.inner != 1) {
         if (n <= static_cast<uint32_t>(vkop::kStridedMaxN)) p.kind = SoftmaxPlan::kStridedRegs;
-        else p.kind = n >= 2048 ? SoftmaxPlan::kGeneralLines : SoftmaxPlan::kGeneralStrided;
+        else p.kind = SoftmaxPlan::kStridedTile;
         return p;
     }
     if (n <= 8u * vkop::kWave) {  // short rows: a wave each
@@ -290,6 +290,14 @@ int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, f
     case SoftmaxPlan::kStridedRegs: {
         launch_strided_reg<T, false>(in, out, v, nan_where, nan_value, st);
         return launched("softmax_strided_reg_kernel");
+    }
+    case SoftmaxPlan::kStridedTile: {
+        uint32_t ti_shift = 0;  // lines a tile: the power of two at or above min(inner, 64)
+        while (ti_shift < 6 && (1u << ti_shift) < v.g.inner) ti_shift++;
+        const uint32_t tiles = (v.g.inner + (1u << ti_shift) - 1) >> ti_shift;
+        vkop::softmax_strided_tile_kernel<T><<<v.g.outer * tiles, vkop::kStridedTileThreads, 0, st>>>(in, out, v.g, ti_shift,
+                                                                                                       nan_where, nan_value);
+        return launched("softmax_strided_tile_kernel");
     }
     case SoftmaxPlan::kGeneralLines:
         vkop::softmax_lines_kernel<T, kLineThreads>
