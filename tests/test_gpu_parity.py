@@ -103,8 +103,12 @@ def test_softmax_many_short_rows(ops, shape):
 @pytest.mark.parametrize("shape,axis", [((5, 7, 9), 0), ((5, 7, 9), 1), ((5, 7, 9), 2), ((2, 3, 4, 5), 0), ((2, 3, 4, 5), 1),
                                         ((2, 3, 4, 5), -2), ((300,), 0), ((4, 2500, 3), 1), ((3, 70, 130), 1), ((2, 5, 64), 1),
                                         ((2, 1000, 64), 1), ((1, 4096, 300), 1), ((2, 200, 7, 5), 1), ((3, 129, 2), 1),
-                                        ((2, 777, 65), 1), ((5000, 33), 0)])
+                                        ((2, 777, 65), 1), ((5000, 33), 0), ((1, 8192, 3), 1), ((300, 200, 64), 1),
+                                        ((40, 1000, 16), 1), ((1, 4100, 130), -2)])
 def test_softmax_axes(ops, shape, axis):
+    """Every axis of small tensors; lines along a non-last axis short (held in registers) and
+    long (a tile of lines per workgroup, and -- with few tiles -- the tile's rows split over
+    several workgroups in two launches), with tiles and row chunks that end ragged."""
     rng = np.random.default_rng(5)
     x = (rng.standard_normal(shape) * 2).astype(np.float32)
     if x.size > 4000:   # a NaN line, a +inf line, a line of -inf
@@ -419,7 +423,9 @@ def test_detection_style_chain(ops, golden):
 
 @pytest.mark.parametrize("shape,axis,dtype", [((16, 80, 8400), 1, np.float32), ((3, 80, 1000), 1, np.float16),
                                               ((5, 7, 9), 0, np.float32), ((4, 300), 1, np.float32),
-                                              ((2, 200, 33), 1, np.float32), ((6, 5000), -1, np.float32)])
+                                              ((2, 200, 33), 1, np.float32), ((6, 5000), -1, np.float32),
+                                              ((2, 1000, 64), 1, np.float32), ((1, 4100, 130), 1, np.float16),
+                                              ((300, 200, 64), 1, np.float32)])
 def test_softmax_then_max_in_one_pass(ops, shape, axis, dtype):
     """The per-line maximum of the softmax equals, bit for bit, the max operator
     applied to the softmax operator's output; NaN and -inf lines included."""

@@ -3,6 +3,7 @@
 
   python -m vkop_amd.bench_ops [--steps K] [--warmup W] [--only NAME_SUBSTRING] [--eager]
   python -m vkop_amd.bench_ops --data-sweep [--only NAME_SUBSTRING]
+  python -m vkop_amd.bench_ops --softmax-sweep [--only NAME_SUBSTRING]
 
 bench.py at the repository root measures the headline (fused softmax -> top-k on
 [64,128256]); this script covers the rest: plain softmax, plain top-k, the fused
@@ -17,6 +18,10 @@ shapes x fourteen kinds of rows (sorted, constant, two values, a dozen levels, m
 NaN / +inf rows, one value with peaks, sorted runs, ...) in single and half precision and
 flags every case that takes more than three times the same shape's normal rows: the
 places where a selection kernel falls off a cliff.
+
+--softmax-sweep times the plain softmax on two dozen shapes (short rows by the ten
+thousand, attention-shaped tensors, the workloads' shapes, rows of a million, lines along
+a non-last axis short and long) in single and half precision against the bytes moved.
 """
 import argparse
 import json
@@ -34,6 +39,7 @@ def main():
     ap.add_argument("--only", default="")
     ap.add_argument("--data-sweep", action="store_true",
                     help="time top-k and the fused call on shapes x kinds of awkward rows instead of the workloads")
+    ap.add_argument("--softmax-sweep", action="store_true", help="time the plain softmax on a range of shapes and axes")
     ap.add_argument("--eager", action="store_true",
                     help="launch every call from the host instead of replaying a recording (for counter runs under "
                          "rocprofv3 --pmc; the timings of such a run mean nothing)")
@@ -123,6 +129,28 @@ def main():
                                        ptr, nb + 256, stream)
         us = timed(call, len(bufs))
         report(name, us, x.nbytes + rows * k * (x.itemsize + 4))
+
+    if args.softmax_sweep:
+        shapes = [((256, 1000), -1), ((4096, 32), -1), ((65536, 64), -1), ((16384, 128), -1), ((8192, 256), -1), ((4096, 1024), -1),
+                  ((2048, 2048), -1), ((1024, 4096), -1), ((256, 8192), -1), ((128, 16384), -1), ((64, 32768), -1), ((32, 50257), -1),
+                  ((64, 128256), -1), ((8, 262144), -1), ((4, 1048576), -1), ((128, 12, 197, 197), -1), ((16, 32, 1024, 1024), -1),
+                  ((16, 80, 8400), 1), ((64, 8, 4096), 1), ((8, 21, 512, 512), 1), ((32, 1000, 64), 1), ((8, 4096, 256), 1),
+                  ((1, 4096, 4096), 1)]
+        rng = np.random.default_rng(3)
+        for shape, axis in shapes:
+            for dt, tdt, dname in ((F32, torch.float32, "f32"), (F16, torch.float16, "f16")):
+                name = "softmax %s axis %d %s" % (list(shape), axis, dname)
+                if args.only not in name:
+                    continue
+                x = (rng.standard_normal(shape, dtype=np.float32) * np.float32(1.25))
+                nb = max(2, min(16, (300 << 20) // (x.nbytes if dt == F32 else x.nbytes // 2)))
+                bufs = [torch.from_numpy(x).cuda().to(tdt) for _ in range(nb)]
+                out = torch.empty_like(bufs[0])
+                wsb = capi.softmax_workspace_bytes(dt, shape, axis)
+                ws, ptr = workspace(wsb + 256)
+                us = timed(lambda b: capi.softmax(bufs[b].data_ptr(), out.data_ptr(), dt, shape, axis, 0, 0.0, ptr, wsb + 256, stream), nb)
+                report(name, us, 2 * bufs[0].numel() * bufs[0].element_size())
+        return
 
     if args.data_sweep:
         shapes = [(256, 1000, 5), (8192, 256, 8), (4096, 1024, 32), (1024, 4096, 64), (256, 8192, 100), (16, 8400, 300),

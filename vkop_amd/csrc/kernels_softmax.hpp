@@ -14,7 +14,8 @@
 //                           workgroup, no LDS.
 // Strided lines (another axis, long lines):
 //   softmax_strided_tile_kernel  a tile of up to 64 neighbouring lines per workgroup of 16 waves,
-//                           rows dealt to the waves, three passes over the tile.
+//                           rows dealt to the waves, three passes over the tile; with few
+//                           tiles, the tile's rows split over several workgroups (two launches).
 // Strided lines (another axis, short lines):
 //   softmax_strided_reg_kernel  one thread per line, threads along the
 //                           contiguous inner axis; the line's elements stay in
@@ -266,19 +267,32 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
 // groups by shuffles and across the waves through LDS.  One thread per line -- what this
 // replaces -- had 2048 threads on a [32,1000,64] tensor: 741 us for 16 MB.
 constexpr int kStridedTileThreads = 1024;
-template <typename T>
+// What a launch of the tile kernel does: the whole softmax of its tiles, or -- when the tensor
+// has too few tiles to fill the chip -- one of the two halves of a split over G row chunks a
+// tile: every chunk's maximum and sum (hardware-exp terms against the chunk's own maximum, as
+// in the chunked row kernels) into stats[(tile * G + chunk) * TI + line], then the
+// probabilities from the line's G results.  G * TI <= 1024.
+// The ...Max modes write, instead of the tensor, each line's largest probability to out[line]
+// (softmax followed by a max over the same axis): from the same statistics, so bit-equal to
+// the maximum of what the other modes write.
+enum { kTileWhole = 0, kTileStats = 1, kTileScale = 2, kTileWholeMax = 3, kTileFoldMax = 4 };
+template <typename T, int MODE>
 __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kernel(const T *__restrict__ in, T *__restrict__ out,
-                                                                                    LineGeom g, uint32_t ti_shift, int nan_where,
-                                                                                    float nan_value) {
+                                                                                    ChunkStat *__restrict__ stats, LineGeom g,
+                                                                                    uint32_t ti_shift, uint32_t G, uint32_t per,
+                                                                                    int nan_where, float nan_value) {
     constexpr int NT = kStridedTileThreads, NW = NT / kWave;
     constexpr int U = 16;  // rows a lane has in flight (a pass is a chain of n / (16 waves * U) round trips)
-    __shared__ float fmax_lds[NW][kWave];
-    __shared__ double dsum_lds[NW][kWave];
+    __shared__ float fmax_lds[NW * kWave];
+    __shared__ double dsum_lds[NW * kWave];
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t TI = 1u << ti_shift, RPW = kWave >> ti_shift;  // lines a tile, rows per wave instruction
     const uint32_t tiles = (g.inner + TI - 1) >> ti_shift;
-    const uint32_t o = blockIdx.x / tiles, tile = blockIdx.x - o * tiles;
-    const uint32_t col = (tile << ti_shift) + (lane & (TI - 1)), r = lane >> ti_shift;
+    const uint32_t tileid = blockIdx.x / G, chunk = blockIdx.x - tileid * G;
+    const uint32_t o = tileid / tiles, tile = tileid - o * tiles;
+    const uint32_t c0 = min(chunk * per, g.n), c1 = min(c0 + per, g.n);  // this workgroup's rows
+    const uint32_t mine = lane & (TI - 1);                               // this lane's line of the tile
+    const uint32_t col = (tile << ti_shift) + mine, r = lane >> ti_shift;
     const bool col_ok = col < g.inner;
     const size_t base = static_cast<size_t>(o) * g.n * g.inner + (col_ok ? col : 0u);
     const uint32_t step = NW * RPW;  // rows the workgroup covers per turn
@@ -287,66 +301,87 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
     // combine v over the lanes of a wave that look at the same line, then over the waves; all threads call
     auto reduce_max = [&](float v) -> float {
         for (uint32_t off = TI; off < static_cast<uint32_t>(kWave); off <<= 1) v = fmaxf(v, __shfl_xor(v, static_cast<int>(off), kWave));
-        fmax_lds[wave][lane] = v;
+        fmax_lds[tid] = v;
         __syncthreads();
-        float m = fmax_lds[0][lane & (TI - 1)];
+        float m = fmax_lds[mine];
 #pragma unroll
-        for (int w = 1; w < NW; w++) m = fmaxf(m, fmax_lds[w][lane & (TI - 1)]);
+        for (int w = 1; w < NW; w++) m = fmaxf(m, fmax_lds[w * kWave + mine]);
         return m;
     };
     auto reduce_sum = [&](double v) -> double {
         for (uint32_t off = TI; off < static_cast<uint32_t>(kWave); off <<= 1) v += __shfl_xor(v, static_cast<int>(off), kWave);
-        dsum_lds[wave][lane] = v;
+        dsum_lds[tid] = v;
         __syncthreads();
-        double sum = dsum_lds[0][lane & (TI - 1)];
+        double sum = dsum_lds[mine];
 #pragma unroll
-        for (int w = 1; w < NW; w++) sum += dsum_lds[w][lane & (TI - 1)];  // fixed order: run-to-run stable
+        for (int w = 1; w < NW; w++) sum += dsum_lds[w * kWave + mine];  // fixed order: run-to-run stable
         return sum;
     };
-    // ---- 1. the lines' maxima
-    float m = -INFINITY;
-    for (uint32_t j0 = wave * RPW + r; j0 < g.n; j0 += step * U) {
-        float x[U];
+    // one pass over the workgroup's rows: use(x, j) for every element of this lane's line
+    auto pass = [&](auto use) {
+        for (uint32_t j0 = c0 + wave * RPW + r; j0 < c1; j0 += step * U) {
+            float x[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
-            x[u] = load_elem(in, at(j < g.n ? j : 0u));
+            for (int u = 0; u < U; u++) {
+                const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
+                x[u] = load_elem(in, at(j < c1 ? j : c0));
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
+                if (j < c1) use(x[u], j);
+            }
         }
-#pragma unroll
-        for (int u = 0; u < U; u++)
-            if (j0 + static_cast<uint32_t>(u) * step < g.n) m = fmaxf(m, x[u]);  // (drops NaN)
-    }
-    m = reduce_max(m);
-    // ---- 2. the sums of the terms
-    double acc = 0.0;
-    for (uint32_t j0 = wave * RPW + r; j0 < g.n; j0 += step * U) {
-        float x[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
-            x[u] = load_elem(in, at(j < g.n ? j : 0u));
+    };
+    constexpr bool kFold = MODE == kTileScale || MODE == kTileFoldMax;
+    constexpr bool kMaxOnly = MODE == kTileWholeMax || MODE == kTileFoldMax;
+    if (MODE == kTileFoldMax && chunk != 0) return;  // (the whole workgroup: one writer a tile)
+    LineStats st{0.f, 0.f, 0.0};
+    if constexpr (!kFold) {
+        // ---- 1. the lines' maxima
+        float m = -INFINITY;
+        pass([&](float x, uint32_t) { m = fmaxf(m, x); });  // (drops NaN)
+        m = reduce_max(m);
+        // ---- 2. the sums of the terms
+        double acc = 0.0;
+        if constexpr (MODE != kTileStats) {
+            pass([&](float x, uint32_t) { acc += static_cast<double>(softmax_term(x, m)); });
+            st = LineStats{m, 0.f, 1.0 / reduce_sum(acc)};
+        } else {
+            // reference of the chunk's sum: its maximum, or 0 when that is not finite (then
+            // every term is 0, inf or NaN, and NaN / inf must reach the sum)
+            const float ref = (m > -INFINITY && m < INFINITY) ? m : 0.f;
+            pass([&](float x, uint32_t) { acc += static_cast<double>(fast_term_unbiased(x, ref)); });
+            const double sum = reduce_sum(acc);
+            if (tid < TI) stats[(static_cast<size_t>(tileid) * G + chunk) * TI + tid] = ChunkStat{sum, m, ref};
+            return;
         }
-#pragma unroll
-        for (int u = 0; u < U; u++)
-            if (j0 + static_cast<uint32_t>(u) * step < g.n) acc += static_cast<double>(softmax_term(x[u], m));
+    } else {
+        // thread c * TI + l fetches chunk c's result for line l; every lane then folds its line's G
+        const bool holds = tid < G * TI;
+        ChunkStat cs{0.0, -INFINITY, 0.f};
+        if (holds) cs = stats[(static_cast<size_t>(tileid) * G + (tid >> ti_shift)) * TI + mine];
+        fmax_lds[tid] = cs.m;
+        __syncthreads();
+        float M = fmax_lds[mine];
+        for (uint32_t c = 1; c < G; c++) M = fmaxf(M, fmax_lds[c * TI + mine]);
+        dsum_lds[tid] = (holds && cs.s != 0.0) ? cs.s * exp(static_cast<double>(cs.ref) - static_cast<double>(M)) : 0.0;
+        __syncthreads();
+        double sum = dsum_lds[mine];
+        for (uint32_t c = 1; c < G; c++) sum += dsum_lds[c * TI + mine];
+        st = LineStats{M, 0.f, 1.0 / sum};
     }
-    const LineStats st{m, 0.f, 1.0 / reduce_sum(acc)};
+    if constexpr (kMaxOnly) {
+        // the line's maximum has the term exp_accurate(0) = 1 (NaN statistics give NaN, as the tensor would)
+        if (tid < TI && col_ok) store_elem(out, static_cast<size_t>(o) * g.inner + col, softmax_prob(st.m, st));
+        return;
+    }
     // ---- 3. the probabilities
-    for (uint32_t j0 = wave * RPW + r; j0 < g.n; j0 += step * U) {
-        float x[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
-            x[u] = load_elem(in, at(j < g.n ? j : 0u));
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const uint32_t j = j0 + static_cast<uint32_t>(u) * step;
-            float p = round_to_storage<T>(softmax_prob(x[u], st));
-            if (nan_where && p != p) p = nan_value;
-            if (j < g.n && col_ok) store_elem(out, at(j), p);
-        }
-    }
+    pass([&](float x, uint32_t j) {
+        float p = round_to_storage<T>(softmax_prob(x, st));
+        if (nan_where && p != p) p = nan_value;
+        if (col_ok) store_elem(out, at(j), p);
+    });
 }
 
 // ---- short strided lines held in registers -------------------------------------------------

@@ -155,6 +155,7 @@ struct SoftmaxPlan {
     enum Kind { kGeneralLines, kGeneralStrided, kRow, kWaveRow, kChunked, kStridedRegs, kStridedTile } kind = kGeneralLines;
     RowShape shape{0, 0};
     uint32_t g = 1, per = 0;
+    uint32_t ti_shift = 0;  // kStridedTile: log2 of the lines a tile
     size_t workspace = 0;
 };
 
@@ -188,7 +189,28 @@ SoftmaxPlan plan_softmax(const View &v, int dtype) {
     const uint32_t n = v.g.n, rows = v.g.outer;
     if (v.g.inner != 1) {
         if (n <= static_cast<uint32_t>(vkop::kStridedMaxN)) p.kind = SoftmaxPlan::kStridedRegs;
-        else p.kind = SoftmaxPlan::kStridedTile;
+        else {
+            // a tile of TI lines (the power of two at or above min(inner, 64)) per workgroup; with too
+            // few tiles to fill the chip, every tile's rows are split over G workgroups (two launches)
+            p.kind = SoftmaxPlan::kStridedTile;
+            while (p.ti_shift < 6 && (1u << p.ti_shift) < v.g.inner) p.ti_shift++;
+            const uint32_t ti = 1u << p.ti_shift;
+            const uint64_t tiles = static_cast<uint64_t>(rows) * ((v.g.inner + ti - 1) >> p.ti_shift);
+            const uint32_t turn = (vkop::kStridedTileThreads / vkop::kWave) * (vkop::kWave >> p.ti_shift);  // rows per turn
+            p.g = 1;
+            p.per = n;
+            if (tiles < 256 && n >= 8 * turn) {
+                uint32_t want = static_cast<uint32_t>((512 + tiles - 1) / tiles);
+                want = std::min(want, static_cast<uint32_t>(vkop::kStridedTileThreads) >> p.ti_shift);
+                uint32_t per = (n + want - 1) / want;
+                per = std::max((per + turn - 1) / turn * turn, 4 * turn);
+                p.g = (n + per - 1) / per;
+                p.per = per;
+                if (p.g > 1)
+                    p.workspace = kTicketBytes + align_up(static_cast<size_t>(tiles) * p.g * ti * sizeof(vkop::ChunkStat));
+                else p.per = n;
+            }
+        }
         return p;
     }
     if (n <= 8u * vkop::kWave) {  // short rows: a wave each
@@ -292,12 +314,20 @@ int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, f
         return launched("softmax_strided_reg_kernel");
     }
     case SoftmaxPlan::kStridedTile: {
-        uint32_t ti_shift = 0;  // lines a tile: the power of two at or above min(inner, 64)
-        while (ti_shift < 6 && (1u << ti_shift) < v.g.inner) ti_shift++;
-        const uint32_t tiles = (v.g.inner + (1u << ti_shift) - 1) >> ti_shift;
-        vkop::softmax_strided_tile_kernel<T><<<v.g.outer * tiles, vkop::kStridedTileThreads, 0, st>>>(in, out, v.g, ti_shift,
-                                                                                                       nan_where, nan_value);
-        return launched("softmax_strided_tile_kernel");
+        const uint32_t tiles = v.g.outer * ((v.g.inner + (1u << p.ti_shift) - 1) >> p.ti_shift);
+        if (p.g == 1) {
+            vkop::softmax_strided_tile_kernel<T, vkop::kTileWhole>
+                <<<tiles, vkop::kStridedTileThreads, 0, st>>>(in, out, nullptr, v.g, p.ti_shift, 1, v.g.n, nan_where, nan_value);
+            return launched("softmax_strided_tile_kernel");
+        }
+        if (ws == nullptr || ws_bytes < p.workspace)
+            return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, p.workspace);
+        auto *stats = reinterpret_cast<vkop::ChunkStat *>(static_cast<unsigned char *>(ws) + kTicketBytes);
+        vkop::softmax_strided_tile_kernel<T, vkop::kTileStats>
+            <<<tiles * p.g, vkop::kStridedTileThreads, 0, st>>>(in, out, stats, v.g, p.ti_shift, p.g, p.per, nan_where, nan_value);
+        vkop::softmax_strided_tile_kernel<T, vkop::kTileScale>
+            <<<tiles * p.g, vkop::kStridedTileThreads, 0, st>>>(in, out, stats, v.g, p.ti_shift, p.g, p.per, nan_where, nan_value);
+        return launched("softmax_strided_tile_kernel (split)");
     }
     case SoftmaxPlan::kGeneralLines:
         vkop::softmax_lines_kernel<T, kLineThreads>
@@ -807,7 +837,25 @@ int softmax_reduce_max_impl(const T *in, T *out, const View &v, void *ws, size_t
         launch_strided_reg<T, true>(in, out, v, 0, 0.f, st);
         return launched("softmax_strided_reg_kernel");
     }
-    // longer lines: the line statistics, then exp_accurate(0) / S per line
+    if (v.g.inner != 1) {
+        // long lines along a non-last axis: the statistics of the tile kernel, as the softmax itself takes them
+        const SoftmaxPlan p = plan_softmax(v, sizeof(T) == 4 ? VKOP_HIP_F32 : VKOP_HIP_F16);
+        const uint32_t tiles = v.g.outer * ((v.g.inner + (1u << p.ti_shift) - 1) >> p.ti_shift);
+        if (p.g == 1) {
+            vkop::softmax_strided_tile_kernel<T, vkop::kTileWholeMax>
+                <<<tiles, vkop::kStridedTileThreads, 0, st>>>(in, out, nullptr, v.g, p.ti_shift, 1, v.g.n, 0, 0.f);
+            return launched("softmax_strided_tile_kernel (max)");
+        }
+        if (ws == nullptr || ws_bytes < p.workspace)
+            return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, p.workspace);
+        auto *cstats = reinterpret_cast<vkop::ChunkStat *>(static_cast<unsigned char *>(ws) + kTicketBytes);
+        vkop::softmax_strided_tile_kernel<T, vkop::kTileStats>
+            <<<tiles * p.g, vkop::kStridedTileThreads, 0, st>>>(in, out, cstats, v.g, p.ti_shift, p.g, p.per, 0, 0.f);
+        vkop::softmax_strided_tile_kernel<T, vkop::kTileFoldMax>
+            <<<tiles * p.g, vkop::kStridedTileThreads, 0, st>>>(in, out, cstats, v.g, p.ti_shift, p.g, p.per, 0, 0.f);
+        return launched("softmax_strided_tile_kernel (split, max)");
+    }
+    // long rows: the line statistics, then exp_accurate(0) / S per line
     const size_t need = kTicketBytes + align_up(static_cast<size_t>(lines) * sizeof(vkop::LineStats));
     if (ws == nullptr || ws_bytes < need)
         return fail(VKOP_HIP_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
@@ -1301,6 +1349,7 @@ size_t vkop_hip_softmax_reduce_max_workspace_bytes(int dtype, const int *shape, 
     View v;
     if (check_dtype(dtype) || make_view(shape, ndim, axis, &v)) return 0;
     if (v.g.n <= static_cast<uint32_t>(vkop::kStridedMaxN)) return 0;
+    if (v.g.inner != 1) return plan_softmax(v, dtype).workspace;
     return kTicketBytes + align_up(static_cast<size_t>(v.g.outer) * v.g.inner * sizeof(vkop::LineStats));
 }
 
