@@ -149,7 +149,7 @@ struct RowShape {
     int nt, v;
 };
 const RowShape kShapesF32[] = {{256, 1}, {256, 2}, {256, 4}, {256, 8}, {512, 8}, {1024, 8}};
-const RowShape kShapesF16[] = {{256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}, {1024, 4}};
+const RowShape kShapesF16[] = {{128, 1}, {256, 1}, {256, 2}, {256, 4}, {512, 4}, {1024, 4}};
 
 struct SoftmaxPlan {
     enum Kind { kGeneralLines, kGeneralStrided, kRow, kWaveRow, kChunked, kStridedRegs, kStridedTile } kind = kGeneralLines;
@@ -248,7 +248,8 @@ SoftmaxPlan plan_softmax(const View &v, int dtype) {
 
 #define VKOP_FOR_EACH_ROW_SHAPE(X, T) \
     X(256, 1) X(256, 2) X(256, 4) X(512, 4) X(1024, 4)                          \
-    if constexpr (sizeof(T) == 4) { X(256, 8) X(512, 8) X(1024, 8) }
+    if constexpr (sizeof(T) == 4) { X(256, 8) X(512, 8) X(1024, 8) }          \
+    if constexpr (sizeof(T) == 2) { X(128, 1) }
 
 template <typename T>
 int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, float nan_value, void *ws,
