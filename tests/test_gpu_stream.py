@@ -206,7 +206,7 @@ def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
-@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (1048576, 100, 2), (262144, 1024, 3), (300000, 600, 3), (1000, 5, 4),
+@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (1048576, 100, 2), (262144, 1024, 3), (300000, 600, 3), (131072, 800, 3), (1000, 5, 4),
                                       (2048, 16, 4), (2048, 32, 4)])
 def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtype):
     """Rows that defeat a threshold taken from block or lane maxima -- one value everywhere
@@ -217,14 +217,16 @@ def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtyp
     _compare_paths(ops, n, k, dtype, 4, TIE_KINDS, path)
 
 
-@pytest.mark.parametrize("n,k", [(262144, 1024), (262144, 2000), (524288, 2048), (300000, 600), (300001, 700)])
+@pytest.mark.parametrize("n,k", [(262144, 1024), (262144, 2000), (524288, 2048), (300000, 600), (300001, 700), (65536, 512),
+                                 (100000, 1200)])
 def test_large_k_rows_whose_cut_falls_into_a_crowd(ops, n, k):
     """The large-k kernels on rows where the threshold's own rank group is too large for the
     candidate lists (one value in half of the places, -inf nearly everywhere, probabilities
     that underflow to 0, -0 and +0, a dozen levels) -- its first members come from a walk over
     the row in index order, also on rows that do not start on 16 bytes -- on rows of NaN
     probabilities, on block maxima of both signs and on sorted rows at a k close to the
-    lists' capacity; against the radix select and the oracle."""
+    lists' capacity, and on rows with hardly more blocks than wanted places (1.3 a place:
+    most of the row is a candidate); against the radix select and the oracle."""
     _compare_paths(ops, n, k, np.float32, 4, WALK_KINDS, 3)
 
 

@@ -490,7 +490,8 @@ struct ScanCfg {
 
 // Long last-axis rows, largest first, k up to kFastMaxK: the scan + pick pair.  The
 // largest chunk that still leaves 512 workgroups (else the smallest); rows too short
-// to be split, or with fewer than 2 (k + 1) blocks (4 (k + 1) for k > 255), or with more blocks than the pick
+// to be split, or with fewer than 2 (k + 1) blocks (4 (k + 1) for k > 255; 1.25 (k + 1) for k > 511 on up to
+// 16 rows), or with more blocks than the pick
 // kernel takes in (16 per thread), are left to the other kernels.
 // (for_size: what a call could use whatever the tuning knobs say at that time)
 ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) {
@@ -508,8 +509,13 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
     // (the pick kernel's threshold is the (k+1)-th largest of its 512 threads' maxima: at or
     // above their median -- k + 1 <= 256, twice as many blocks -- few blocks and elements reach
     // it; closer to the smallest of them, more blocks have to stand behind every thread)
-    const uint32_t blocks_per_place = big ? 2u : (k + 1 <= 256 ? 2u : 4u);
-    if (blocks < blocks_per_place * (static_cast<uint32_t>(k) + 1u)) return c;
+    // The large-k kernels behind the scan get by with 1.25 blocks per wanted place on a few rows (they
+    // read most of the row again then, and still beat the radix select: [8,262144] f16 k = 1024, 2048
+    // blocks: 21.7 against 42.8 us; [2,65536] k = 512: 16.0 against 37.8 us); with many rows their
+    // ranking is what the time goes into ([64,100000] k = 1240: 125 against 64 us), and the pick kernel
+    // falls off a cliff on sorted rows below its ratio ([32,50257] f16 k = 200 sorted: 235 against 48 us).
+    const uint32_t quarters = big ? (rows <= 16 ? 5u : 8u) : (k + 1 <= 256 ? 8u : 16u);  // blocks per place, in quarters
+    if (4ull * blocks < static_cast<uint64_t>(quarters) * (static_cast<uint32_t>(k) + 1u)) return c;
     if (!big && !for_size) {
         // a row that ONE workgroup of the chunk kernel holds (up to 8192 elements for k <= 64, up to
         // 32768 beyond): one launch instead of two, measured 1.4 to 1.6 times faster on spread-out
