@@ -179,16 +179,19 @@ def _compare_paths(ops, n, k, dtype, rows, kinds, path):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
 @pytest.mark.parametrize("n,k", [(128256, 50), (128256, 1), (128256, 255), (40000, 7), (16385, 20), (13057, 50),
-                                 (262144, 64), (100003, 33), (500000, 100), (300000, 511)])
+                                 (262144, 64), (100003, 33), (500000, 100), (300000, 511), (50257, 300)])
 def test_scan_pick_pair_equals_chunk_merge_and_oracle(ops, n, k, dtype):
-    _compare_paths(ops, n, k, dtype, 6, KINDS, 2)
+    """(From k = 256 on the pair is the library's choice on more than 16 rows only, there also
+    with fewer than two blocks per wanted place.)"""
+    _compare_paths(ops, n, k, dtype, 20 if k >= 256 else 6, KINDS, 2)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
 @pytest.mark.parametrize("n,k", [(262144, 1024), (262144, 600), (524288, 2048), (200003, 700), (131072, 512),
-                                 (300000, 1500)])
+                                 (300000, 1500), (200000, 300), (50257, 200), (100000, 400)])
 def test_scan_with_spread_out_pick_for_large_k_equals_radix_select_and_oracle(ops, n, k, dtype):
-    """k beyond one workgroup's candidate list: scan, then the gather and rank kernels
+    """k beyond one workgroup's candidate list (and, on a few rows, from k = 256 on, or from
+    k = 160 where the row has too few blocks for the pick kernel): scan, then the gather and rank kernels
     that spread a row's candidates over many workgroups, against the multi-pass radix
     select (rows.path = 1) and the oracle -- the regular rows, and the ones the pair hands
     to its exact fallback (constant and masked rows, levels with thousands of equals)."""
@@ -206,7 +209,7 @@ def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
-@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (1048576, 100, 2), (262144, 1024, 3), (300000, 600, 3), (131072, 800, 3), (1000, 5, 4),
+@pytest.mark.parametrize("n,k,path", [(128256, 50, 2), (40000, 255, 2), (262144, 200, 2), (1048576, 100, 2), (262144, 1024, 3), (300000, 600, 3), (131072, 800, 3), (1000, 5, 4),
                                       (2048, 16, 4), (2048, 32, 4)])
 def test_rows_of_equal_and_clustered_values_on_every_route(ops, n, k, path, dtype):
     """Rows that defeat a threshold taken from block or lane maxima -- one value everywhere

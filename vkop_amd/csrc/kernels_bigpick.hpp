@@ -101,19 +101,9 @@ template <typename T, bool SOFTMAX> __device__ __forceinline__ uint32_t bigpick_
     return (t > -INFINITY) ? max(order_key(t), kKeyNegInf + 1u) : kKeyNegInf + 1u;
 }
 
-// hist[d] += 1 for every lane with `on`.  The lanes that share the first such lane's
-// digit add once between them: block maxima repeat (tied data, a dominant value), and
-// same-address LDS atomics of one instruction are carried out one after the other.
+// hist[d] += 1 for every lane with `on` (hist_add_grouped: lanes that share a digit add once).
 __device__ __forceinline__ void bigpick_hist_add(uint32_t *hist, bool on, uint32_t d) {
-    if (on) {
-        const uint32_t lead = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(d)));
-        const uint64_t same = __ballot(d == lead);
-        if (d == lead) {
-            if (lanes_below(same) == 0) atomicAdd(&hist[lead], static_cast<uint32_t>(__popcll(same)));
-        } else {
-            atomicAdd(&hist[d], 1u);
-        }
-    }
+    if (on) hist_add_grouped(hist, d);
 }
 
 // The digit d of hist[0..2048) with #(digits above d) < need <= #(digits >= d); all

@@ -451,6 +451,50 @@ __device__ __forceinline__ uint32_t first_members_by_scan(uint32_t *counts, cons
     return found;
 }
 
+// hist[d] += 1 for every lane that calls (lanes may call under divergence).  The lanes that
+// share the first such lane's digit add once between them: keys repeat (tied data, a dominant
+// value, the leading bits of a sorted row), and same-address LDS atomics of one instruction
+// are carried out one after the other.
+__device__ __forceinline__ void hist_add_grouped(uint32_t *hist, uint32_t d) {
+    const uint32_t lead = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(d)));
+    const uint64_t same = __ballot(d == lead);
+    if (d == lead) {
+        if (lanes_below(same) == 0) atomicAdd(&hist[lead], static_cast<uint32_t>(__popcll(same)));
+    } else {
+        atomicAdd(&hist[d], 1u);
+    }
+}
+
+// The digit d of hist[0..256) with #(entries of digits above d) < need <= #(entries of digits
+// >= d), and that first count; one whole wave calls (hist is complete and visible to it).
+// d = 256 when the histogram holds fewer than need entries.
+__device__ __forceinline__ uint2 hist256_resolve(const uint32_t *hist, uint32_t need) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint4 h4 = reinterpret_cast<const uint4 *>(hist)[lane];  // lane l owns digits 4 l .. 4 l + 3
+    const uint32_t h[4] = {h4.x, h4.y, h4.z, h4.w};
+    const uint32_t s = (h[0] + h[1]) + (h[2] + h[3]);
+    uint32_t incl = s;  // entries of this lane's digits and of the lanes above
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t t = __shfl_down(incl, o, kWave);
+        if (lane + static_cast<uint32_t>(o) < static_cast<uint32_t>(kWave)) incl += t;
+    }
+    uint32_t above = incl - s, d = 256u;
+    if (above < need && need <= incl) {
+#pragma unroll
+        for (int j = 3; j >= 0; j--) {
+            if (d == 256u) {
+                if (need <= above + h[j]) d = lane * 4u + static_cast<uint32_t>(j);
+                else above += h[j];
+            }
+        }
+    }
+    const uint64_t holder = __ballot(d != 256u);
+    const int src = holder != 0ull ? __ffsll(static_cast<unsigned long long>(holder)) - 1 : 0;
+    return make_uint2(static_cast<uint32_t>(__shfl(static_cast<int>(d), src, kWave)),
+                      static_cast<uint32_t>(__shfl(static_cast<int>(above), src, kWave)));
+}
+
 // The same for a row that starts on a 16-byte boundary and is walked far (members
 // may be sparse): a thread takes 16 consecutive elements a round (128-bit loads), the
 // next round's loads in flight while the current tile is counted, membership by

@@ -205,6 +205,11 @@ union PickSharedUnion {
 //      several loads per thread in flight; their elements at or above the value are
 //      the candidates (everything else in the row is below k+1 elements);
 //   E. finish_row: exact ranks, accurate terms, probabilities, ties, ordered store.
+// More candidates than the list holds: a second threshold a level down (the largest
+// element every thread saw), then -- if that left fewer but still too many: rows sorted
+// in runs -- the exact (k+1)-th largest of those blocks' elements by a radix select over
+// them, or -- if it left as many: equal values en masse -- the first elements equal to the
+// exact threshold from the row's start.
 // A probability tie across the k-th place that reaches below the value gathers again
 // with the tied interval's lower end (settle_tie); what that cannot hold (rows full of
 // equal values) goes to the scan from the row's start or, from D, to the exact radix
@@ -370,9 +375,15 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     uint32_t round = 0;
     // (always inlined: a call would put the block keys, captured by reference, into scratch memory)
     // dry_tag true: nothing is appended; dry_max becomes the largest key this thread saw in [lo, hi).
+    // dry_tag 2: nothing is appended; the keys in [lo, hi) that agree with digit_prefix above bit
+    // digit_shift + 8 are counted by their eight bits from digit_shift up, into digit_hist.
     uint32_t dry_max = 0;
+    uint32_t *digit_hist = reinterpret_cast<uint32_t *>(sh.cand);  // (the list is gathered anew afterwards)
+    uint32_t digit_prefix = 0;
+    int digit_shift = 24;
     auto gather = [&](uint32_t lo, uint64_t hi, auto dry_tag) __attribute__((always_inline)) -> bool {
-        constexpr bool DRY = decltype(dry_tag)::value;
+        constexpr int MODE = static_cast<int>(decltype(dry_tag)::value);
+        constexpr bool DRY = MODE == 1;
         uint32_t wave_n = 0;  // wave-uniform
 #pragma unroll
         for (int e = 0; e < GE; e++) wave_n += static_cast<uint32_t>(__popcll(__ballot(gk[e] >= lo)));
@@ -437,6 +448,9 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                         if (idx < cend[u] && key >= lo && static_cast<uint64_t>(key) < hi) {
                             if constexpr (DRY) {
                                 dry_max = max(dry_max, key);
+                            } else if constexpr (MODE == 2) {
+                                if ((static_cast<uint64_t>(key ^ digit_prefix) >> (digit_shift + 8)) == 0ull)
+                                    hist_add_grouped(digit_hist, (key >> digit_shift) & 255u);
                             } else {
                                 const uint32_t at = atomicAdd(&sh.count, 1u);
                                 if (at < static_cast<uint32_t>(kFastCap)) sh.cand[at] = composite(key, idx);
@@ -478,6 +492,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     }
     uint32_t C2 = sh.count;
     uint32_t level_max = lmk;  // the thread maxima the current threshold was taken from
+    bool fewer = false;        // the step below left fewer candidates than it found
     if (!many_groups && C2 > static_cast<uint32_t>(kFastCap)) {
         // More elements at or above thr than the list holds although only k+1 and a few
         // blocks reach it: those blocks' maxima are alike and so are their other elements
@@ -487,6 +502,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         // (k+1)-th largest of these thread maxima is a threshold as good as thr -- k+1
         // elements reach it, and whatever reaches it lies in a block whose maximum does --
         // and far tighter.
+        const uint32_t before = C2;
         dry_max = 0;
         gather(thr, 1ull << 32, std::true_type{});
         level_max = dry_max;
@@ -496,6 +512,51 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         thr = max(thr, tight);
         many_groups = gather(thr, 1ull << 32, std::false_type{});
         C2 = sh.count;
+        fewer = C2 < before;
+    }
+    bool thr_is_exact = false;  // thr is the key of the row's (k+1)-th largest element
+    if (!many_groups && C2 > static_cast<uint32_t>(kFastCap) && fewer) {
+        // Still more than the list holds, but fewer than before: the blocks that reach thr are
+        // full of elements that do (a row sorted in runs: k+1 blocks of 16 vectors whose every
+        // element lies above the next block's maximum; the step above ends at one element per
+        // vector at best -- 4 (k+1) of them, 8 (k+1) in half precision).  The (k+1)-th largest
+        // of those blocks' elements is the row's, and a radix select finds it whatever the
+        // values: four passes over the same blocks, eight bits of the key each, counted in LDS.
+        // (As many as before means equal values en masse: the step below, without these passes.)
+        uint32_t need = want;
+        digit_prefix = 0;
+        bool found = true;
+        for (digit_shift = 24; digit_shift >= 0 && found; digit_shift -= 8) {
+            __syncthreads();
+            if (tid < 256u) digit_hist[tid] = 0;
+            __syncthreads();
+            gather(thr, 1ull << 32, std::integral_constant<int, 2>{});  // (ends with a barrier)
+            if (wave == 0) {
+                const uint2 r = hist256_resolve(digit_hist, need);
+                if (lane == 0) {
+                    sh.wave_thr[0] = r.x;
+                    sh.wave_thr[1] = r.y;
+                }
+            }
+            __syncthreads();
+            const uint32_t d = sh.wave_thr[0];
+            found = d < 256u;  // (k+1 elements reach thr, so a digit is always found)
+            if (found) {
+                digit_prefix |= d << digit_shift;
+                need -= sh.wave_thr[1];
+            }
+        }
+        __syncthreads();
+        if (tid == 0) sh.count = 0;
+        __syncthreads();
+        if (found) {
+            thr = max(thr, digit_prefix);
+            thr_is_exact = true;
+            many_groups = gather(thr, 1ull << 32, std::false_type{});
+            C2 = sh.count;
+        } else {
+            many_groups = true;
+        }
     }
     // Still too many: equal values en masse AT the threshold (rows of few distinct
     // values, constant rows).  k+1 elements reach thr, so the row's k+1 largest are the
@@ -503,7 +564,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // the first elements equal to it, in index order: those are found by reading the row
     // from its start, where a value this frequent turns up at once.
     bool first_equals_only = false;  // the candidates hold only some of the elements equal to thr
-    if (many_groups || C2 > static_cast<uint32_t>(kFastCap)) {
+    if ((many_groups || C2 > static_cast<uint32_t>(kFastCap)) && !thr_is_exact) {
         // (thr so far is a value rounded down; this needs the key of an element: the exact
         // (k+1)-th largest of the thread maxima it came from)
         __syncthreads();

@@ -488,35 +488,51 @@ struct ScanCfg {
     uint32_t g2 = 0;  // k beyond the pick kernel's list: workgroups a row of the gather kernel (kernels_bigpick.hpp)
 };
 
-// Long last-axis rows, largest first, k up to kFastMaxK: the scan + pick pair.  The
-// largest chunk that still leaves 512 workgroups (else the smallest); rows too short
-// to be split, or with fewer than 2 (k + 1) blocks (4 (k + 1) for k > 255; 1.25 (k + 1) for k > 511 on up to
-// 16 rows), or with more blocks than the pick
-// kernel takes in (16 per thread), are left to the other kernels.
+// Long last-axis rows, largest first: the scan kernel followed by the pick kernel (k up to
+// kFastMaxK) or by the large-k pair (g2 != 0: beyond that k, and on up to 16 rows from k = 256,
+// or from k = 160 where the pick kernel has too few blocks).  The largest chunk that still
+// leaves 512 workgroups (else the smallest); rows too short to be split, or with too few
+// blocks per wanted place (below), or with more blocks than the kernel behind the scan takes
+// in, are left to the other kernels.
 // (for_size: what a call could use whatever the tuning knobs say at that time)
 ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) {
     ScanCfg c;
     if (v.g.inner != 1 || k > vkop::kMaxK || v.g.n == 0 || v.g.outer == 0) return c;
-    const bool big = k > vkop::kFastMaxK;
+    const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
+    const uint32_t n = v.g.n, rows = v.g.outer;
+    // The pick kernel ranks a row in one workgroup, the large-k pair spreads it over many: on up to 16
+    // rows that pair is the faster one from k = 256 on ([8,262144] k = 256: 17.7 against 23.1 us;
+    // [4,100000] k = 500: 15.6 against 44 us), with more rows the pick kernel stays ahead up to its
+    // limit ([64,128256] k = 500 fused: 50 against 52 us; [128,65536] k = 256: 24 against 39 us).
+    const bool few_rows = rows <= 16;
+    bool big = k > vkop::kFastMaxK || (few_rows && k >= 256);
     if (!for_size) {
         if (g_rows_path.load() == 1) return c;
         // a forced shape of the other streaming kernels
         if (g_rows_threads.load() > 0 && g_rows_loads.load() > 0 && g_rows_chunks.load() > 0) return c;
     }
-    const uint32_t vec = dtype == VKOP_HIP_F32 ? 4u : 8u;
-    const uint32_t n = v.g.n, rows = v.g.outer;
     const uint32_t blocks = (n + vkop::kBlockLanes * vec - 1) / (vkop::kBlockLanes * vec);
-    // (the pick kernel's threshold is the (k+1)-th largest of its 512 threads' maxima: at or
-    // above their median -- k + 1 <= 256, twice as many blocks -- few blocks and elements reach
-    // it; closer to the smallest of them, more blocks have to stand behind every thread)
-    // The large-k kernels behind the scan get by with 1.25 blocks per wanted place on a few rows (they
+    // Blocks per wanted place, in quarters.  The pick kernel's threshold is the (k+1)-th largest of its
+    // 512 threads' maxima: at or above their median -- k + 1 <= 256, twice as many blocks -- few blocks
+    // and elements reach it; closer to the smallest of them, more blocks have to stand behind every
+    // thread -- which costs one workgroup per row less when other rows keep the chip busy: with more
+    // than 16 rows, 1.75 blocks a place are enough at every k ([64,128256] f16 k = 300, 3.3 a place:
+    // 28.9 us, fused 34.5, against 49 / 132 us of the radix select; [32,50257] f16 k = 200, 1.95 a
+    // place: 24.4 against 46.8 us).  The large-k kernels get by with 1.25 a place on a few rows (they
     // read most of the row again then, and still beat the radix select: [8,262144] f16 k = 1024, 2048
     // blocks: 21.7 against 42.8 us; [2,65536] k = 512: 16.0 against 37.8 us); with many rows their
-    // ranking is what the time goes into ([64,100000] k = 1240: 125 against 64 us), and the pick kernel
-    // falls off a cliff on sorted rows below its ratio ([32,50257] f16 k = 200 sorted: 235 against 48 us).
-    const uint32_t quarters = big ? (rows <= 16 ? 5u : 8u) : (k + 1 <= 256 ? 8u : 16u);  // blocks per place, in quarters
-    if (4ull * blocks < static_cast<uint64_t>(quarters) * (static_cast<uint32_t>(k) + 1u)) return c;
-    if (!big && !for_size) {
+    // ranking is what the time goes into ([64,100000] k = 1240: 125 against 64 us).
+    const uint64_t places = static_cast<uint64_t>(k) + 1u;
+    uint32_t quarters = big ? (few_rows ? 5u : 8u) : (!few_rows ? 7u : (places <= 256 ? 8u : 16u));
+    if (!big && few_rows && k >= 160 && 4ull * blocks < quarters * places) {
+        // too few blocks for the pick kernel on a few rows: the large-k pair again, from k = 160 on (below,
+        // rows sorted in runs cost it several times the radix select: [16,128256] k = 128: 422 us)
+        // ([8,50257] f16 k = 200: 16.8 against 44.5 us of the radix select; [16,100000] f16 k = 400: 21.0 against 38.9)
+        big = true;
+        quarters = 5u;
+    }
+    if (4ull * blocks < quarters * places) return c;
+    if (k <= vkop::kFastMaxK && !for_size) {
         // a row that ONE workgroup of the chunk kernel holds (up to 8192 elements for k <= 64, up to
         // 32768 beyond): one launch instead of two, measured 1.4 to 1.6 times faster on spread-out
         // rows ([1024,4096] k = 16: 9.0 against 14.5 us; [64,32768] k = 200: 12.5 against 20.3 us)
