@@ -371,13 +371,14 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
 
     // ---- D. the elements with keys in [lo, hi) of the blocks whose maximum reaches lo -> sh.cand ----
     // All threads call; ends with a barrier.  Returns true (in every thread) when more
-    // than kPickHitCap blocks reach lo: nothing was gathered then.
+    // than hit_cap blocks reach lo: nothing was gathered then.
     uint32_t round = 0;
     // (always inlined: a call would put the block keys, captured by reference, into scratch memory)
     // dry_tag true: nothing is appended; dry_max becomes the largest key this thread saw in [lo, hi).
     // dry_tag 2: nothing is appended; the keys in [lo, hi) that agree with digit_prefix above bit
     // digit_shift + 8 are counted by their eight bits from digit_shift up, into digit_hist.
     uint32_t dry_max = 0;
+    uint32_t hit_cap = kPickHitCap;  // more blocks than this are not read: gather returns true
     uint32_t *digit_hist = reinterpret_cast<uint32_t *>(sh.cand);  // (the list is gathered anew afterwards)
     uint32_t digit_prefix = 0;
     int digit_shift = 24;
@@ -398,7 +399,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             pos += (static_cast<uint32_t>(w) < wave) ? c : 0u;
             H += c;
         }
-        if (H > static_cast<uint32_t>(kPickHitCap)) return true;
+        if (H > hit_cap) return true;
 #pragma unroll
         for (int e = 0; e < GE; e++) {
             const bool pass = gk[e] >= lo;
@@ -463,6 +464,13 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         __syncthreads();
         return false;
     };
+    // The first value is reached by k+1 blocks and a few (about 2.5 (k+1) on spread-out rows at
+    // k = 50, fewer at larger k).  Three times k+1 and more are a row whose block maxima are equal en
+    // masse (a constant row, a few levels) or whose threads' shares are not alike (below): reading
+    // all of them again -- the whole row, for a constant one -- settles nothing.
+    // (The same when EVERY block reaches it and the row has a quarter more blocks than places.)
+    hit_cap = min(static_cast<uint32_t>(kPickHitCap), 3u * want + 64u);
+    if (blocks > want + want / 4u) hit_cap = min(hit_cap, blocks - 1u);
     bool many_groups = gather(thr, 1ull << 32, std::false_type{});
     if (many_groups) {
         // More than kPickHitCap blocks reach thr: the threads' shares of the block maxima are
@@ -490,6 +498,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             many_groups = gather(thr, 1ull << 32, std::false_type{});
         }
     }
+    hit_cap = kPickHitCap;  // (from here on: whatever the list of blocks holds)
     uint32_t C2 = sh.count;
     uint32_t level_max = lmk;  // the thread maxima the current threshold was taken from
     bool fewer = false;        // the step below left fewer candidates than it found
