@@ -222,6 +222,42 @@ def test_topk_nan_inf(ops):
         assert np.array_equal(np.isnan(host(v)), np.isnan(ev))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("n,k", [(1000, 5), (256, 8), (1024, 32), (777, 20), (64, 16), (33, 33), (2048, 1)])
+def test_topk_smallest_on_short_rows(ops, n, k, dtype):
+    """The k smallest of rows that a wave holds (the one-wave kernel with its order keys turned
+    round): spread-out rows, ties, constant rows, -0 and +0, rows of mostly +inf (the floor of
+    that direction), -inf entries (its summit), NaN entries -- still the largest values, so they
+    come last, also where the k smallest reach into them -- and sorted rows; against the oracle,
+    in both directions."""
+    rng = np.random.default_rng(n * 7 + k)
+    rows = 12
+    x = (rng.standard_normal((rows, n)) * 3).astype(np.float32)
+    x[1] = np.round(x[1])                          # ties
+    x[2] = 1.5                                     # constant
+    x[3, ::2] = -0.0
+    x[3, 1::2] = 0.0
+    x[4, :] = np.inf
+    x[4, rng.integers(0, n, max(1, k // 2))] = rng.standard_normal(max(1, k // 2))   # fewer numbers than k
+    x[5, rng.integers(0, n, 5)] = -np.inf
+    x[6, rng.integers(0, n, 7)] = np.nan
+    x[7, :] = np.nan
+    x[7, rng.integers(0, n, max(1, k - 2))] = rng.standard_normal(max(1, k - 2))     # the k smallest reach into the NaNs
+    x[8] = np.sort(x[8])
+    x[9] = np.sort(x[9])[::-1]
+    x[10, :] = np.inf
+    x[10, 3 % n] = np.nan                          # +inf, then the NaN
+    x = x.astype(dtype)
+    for largest in (False, True):
+        v, ix = ops.topk(dev(x), k, -1, largest)
+        ev, eix = oracle.topk(x.astype(np.float32), k, -1, largest)
+        v, ix = host(v).astype(np.float32), host(ix)
+        assert np.array_equal(ix, eix), (n, k, largest, np.argwhere(ix != eix)[:4])
+        assert np.array_equal(np.isnan(v), np.isnan(ev))
+        ok = ~np.isnan(ev)
+        assert np.array_equal(v[ok].view(np.uint32), ev[ok].astype(np.float32).view(np.uint32))   # (bit copies: signs of zeros too)
+
+
 def test_topk_workloads(ops, golden):
     x4 = synth.grid_values(8, 262144, synth.SEEDS["C4"])
     v, ix = assert_topk_exact(ops, x4, 1024)

@@ -20,6 +20,7 @@
 // element of the row that has that probability.  What is left -- a sum that is not a
 // positive finite number, more than k distinct larger values crowded into few lanes --
 // goes to the exact single-workgroup select over the row (select.hpp) in the same kernel.
+// The plain top-k also runs smallest first: the same steps on order keys turned round.
 #pragma once
 
 #include "kernels_general.hpp"
@@ -33,9 +34,23 @@ constexpr int kTinyMaxK = 32;  // (k + 1 candidates, one per lane, and room for 
 
 template <typename T, int V, bool SOFTMAX, bool ALIGNED>
 __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ in, T *__restrict__ values,
-                                                          int32_t *__restrict__ indices, uint32_t n, uint32_t k) {
+                                                          int32_t *__restrict__ indices, uint32_t n, uint32_t k,
+                                                          uint32_t smallest = 0) {
     constexpr int VEC = Vec128<T>::N;
     constexpr int ELEMS = V * VEC;
+    // smallest (plain top-k only): the k smallest, in increasing order.  Everything below works
+    // on order keys, so the keys are turned round where they are made: the complement for a
+    // number or an infinity (+inf takes -inf's key, the floor that never becomes a candidate),
+    // 1 for a NaN -- still the largest value, hence last, below every other element's key; a
+    // row whose k smallest reach into its NaNs ends in the exact select like any row the
+    // candidates do not settle.
+    auto key_of_value = [&](float x) -> uint32_t {
+        const uint32_t kx = order_key(x);
+        if constexpr (!SOFTMAX) {
+            if (smallest) return (x != x) ? 1u : ~kx;
+        }
+        return kx;
+    };
     __shared__ union U {
         uint64_t cand[kWave];
         SelectShared exact;
@@ -74,7 +89,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
             const float x = q[i].get(c);
             const bool live = e < n && !(SOFTMAX && x != x);
-            key[i * VEC + c] = live ? order_key(x) : 0u;
+            key[i * VEC + c] = live ? key_of_value(x) : 0u;
             lmk = max(lmk, key[i * VEC + c]);
             if (e < n) m = fmaxf(m, x);  // (drops NaN)
         }
@@ -352,7 +367,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             oi[r] = static_cast<int32_t>(idx);
         }
     } else {
-        select_topk_line<kWave>(ex, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
+        select_topk_line<kWave>(ex, n, kk, [&](uint32_t j) { return key_of_value(load_elem(rowp, j)); });
         for (uint32_t r = lane; r < kk; r += kWave) {
             const uint32_t idx = composite_index(ex.sel[r]);
             ov[r] = rowp[idx];

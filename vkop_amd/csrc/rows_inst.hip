@@ -148,10 +148,12 @@ template <typename T, bool SOFTMAX> bool launch_rows_tiny(const TinyLaunch &a) {
     if (a.v == V) {                                                                                    \
         if (a.aligned)                                                                                 \
             rows_tiny_kernel<T, V, SOFTMAX, true><<<a.rows, kWave, 0, a.stream>>>(                     \
-                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k);        \
+                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k,         \
+                a.smallest ? 1u : 0u);                                                                 \
         else                                                                                           \
             rows_tiny_kernel<T, V, SOFTMAX, false><<<a.rows, kWave, 0, a.stream>>>(                    \
-                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k);        \
+                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k,         \
+                a.smallest ? 1u : 0u);                                                                 \
         return true;                                                                                   \
     }
     VKOP_TINY_CASE(1)

@@ -60,6 +60,7 @@ struct TinyLaunch {
     int32_t *indices;
     uint32_t rows, n, k, v;
     bool aligned;
+    bool smallest = false;  // plain top-k: the k smallest, increasing
     hipStream_t stream;
 };
 template <typename T, bool SOFTMAX> bool launch_rows_tiny(const TinyLaunch &a);

@@ -464,7 +464,8 @@ int choose_tiny_loads(const View &v, int k, int dtype) {
 }
 
 template <typename T, bool SOFTMAX>
-int launch_tiny(const T *in, T *values, int32_t *indices, const View &v, int k, int loads, hipStream_t st) {
+int launch_tiny(const T *in, T *values, int32_t *indices, const View &v, int k, int loads, hipStream_t st,
+                bool smallest = false) {
     vkop::TinyLaunch a;
     a.in = in;
     a.values = values;
@@ -474,6 +475,7 @@ int launch_tiny(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.k = static_cast<uint32_t>(k);
     a.v = static_cast<uint32_t>(loads);
     a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % (16 / sizeof(T)) == 0);
+    a.smallest = smallest;
     a.stream = st;
     if (!vkop::launch_rows_tiny<T, SOFTMAX>(a)) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_tiny_kernel for %d loads", loads);
     return launched("rows_tiny_kernel");
@@ -782,7 +784,8 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
 template <typename T>
 int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int dtype, void *ws,
               size_t ws_bytes, hipStream_t st) {
-    if (const int tiny = largest ? choose_tiny_loads(v, k, dtype) : 0) return launch_tiny<T, false>(in, values, indices, v, k, tiny, st);
+    // (the one-wave kernel serves both directions: it turns its order keys round)
+    if (const int tiny = choose_tiny_loads(v, k, dtype)) return launch_tiny<T, false>(in, values, indices, v, k, tiny, st, !largest);
     const ScanCfg sc = largest ? choose_scan_cfg(v, k, dtype) : ScanCfg{};
     const RowsCfg c = (largest && !sc.ok) ? choose_rows_cfg(v, k, dtype) : RowsCfg{};
     const BigKCfg b = (c.ok || sc.ok) ? BigKCfg{} : choose_bigk_cfg(v, k, dtype);
