@@ -65,6 +65,26 @@ __device__ __forceinline__ uint32_t composite_index(uint64_t c) {
     return 0xFFFFFFFFu - static_cast<uint32_t>(c);
 }
 
+// Number of lanes below the caller among those set in `mask`.
+__device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+// hist[d] += 1 for every lane that calls (lanes may call under divergence).  The lanes that
+// share the first such lane's digit add once between them: keys repeat (tied data, a dominant
+// value, the leading bits of a sorted row), and same-address LDS atomics of one instruction
+// are carried out one after the other.
+__device__ __forceinline__ void hist_add_grouped(uint32_t *hist, uint32_t d) {
+    const uint32_t lead = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(d)));
+    const uint64_t same = __ballot(d == lead);
+    if (d == lead) {
+        if (lanes_below(same) == 0) atomicAdd(&hist[lead], static_cast<uint32_t>(__popcll(same)));
+    } else {
+        atomicAdd(&hist[d], 1u);
+    }
+}
+
 // ------------------------------------------------------- block order ----
 // Workgroups are handed to the chip's 8 XCDs in turn (workgroup b runs on XCD b mod 8),
 // and each XCD has an L2 of its own: two workgroups with neighbouring blockIdx never

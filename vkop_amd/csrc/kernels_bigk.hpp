@@ -186,11 +186,12 @@ __global__ __launch_bounds__(kBigThreads) void bigk_hist_kernel(const T *__restr
         for (int c = 0; c < VEC; c++) {
             if (e0 + c < c1) {
                 const uint32_t key = bigk_key<T, SOFTMAX>(q[i].get(c), st, flip);
-                if constexpr (PASS == 0) atomicAdd(&lh[key >> 21], 1u);
+                // (lanes that share a digit add once between them: rows of equal values)
+                if constexpr (PASS == 0) hist_add_grouped(lh, key >> 21);
                 else if constexpr (PASS == 1) {
-                    if ((key >> 21) == want_hi) atomicAdd(&lh[(key >> 10) & 2047u], 1u);
+                    if ((key >> 21) == want_hi) hist_add_grouped(lh, (key >> 10) & 2047u);
                 } else {
-                    if ((key >> 10) == want_hi) atomicAdd(&lh[key & 1023u], 1u);
+                    if ((key >> 10) == want_hi) hist_add_grouped(lh, key & 1023u);
                 }
             }
         }

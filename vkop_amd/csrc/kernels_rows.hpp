@@ -121,12 +121,6 @@ __device__ __forceinline__ float wave_max_f32_uniform(float v) {
 
 constexpr uint32_t kKeyNegInf = 0x007FFFFFu;  // order key of -inf, the smallest key of a real element
 
-// Number of lanes below the caller among those set in `mask`.
-__device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
-    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
-                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
-}
-
 // Float threshold equivalent to an order-key threshold: x passes iff
 // !(x < thr_f).  Keys at or below the key of -inf mean "everything passes".
 __device__ __forceinline__ float key_threshold_to_float(uint32_t thr) {
@@ -449,20 +443,6 @@ __device__ __forceinline__ uint32_t first_members_by_scan(uint32_t *counts, cons
         found += in_tile;
     }
     return found;
-}
-
-// hist[d] += 1 for every lane that calls (lanes may call under divergence).  The lanes that
-// share the first such lane's digit add once between them: keys repeat (tied data, a dominant
-// value, the leading bits of a sorted row), and same-address LDS atomics of one instruction
-// are carried out one after the other.
-__device__ __forceinline__ void hist_add_grouped(uint32_t *hist, uint32_t d) {
-    const uint32_t lead = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(d)));
-    const uint64_t same = __ballot(d == lead);
-    if (d == lead) {
-        if (lanes_below(same) == 0) atomicAdd(&hist[lead], static_cast<uint32_t>(__popcll(same)));
-    } else {
-        atomicAdd(&hist[d], 1u);
-    }
 }
 
 // The digit d of hist[0..256) with #(entries of digits above d) < need <= #(entries of digits

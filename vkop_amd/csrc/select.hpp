@@ -64,7 +64,7 @@ __device__ __forceinline__ void select_topk_line(SelectShared &sh, uint32_t n, u
         for (uint32_t j = tid; j < n; j += NT) {
             const uint64_t c = composite(keyfn(j), j);
             if (bits == 0 || (c >> (64 - bits)) == prefix)
-                atomicAdd(&sh.hist[static_cast<uint32_t>(c >> shift) & 0xFFu], 1u);
+                hist_add_grouped(sh.hist, static_cast<uint32_t>(c >> shift) & 0xFFu);
         }
         __syncthreads();
         // Wave 0 locates the digit d with  #(digit > d) < need <= #(digit >= d).
