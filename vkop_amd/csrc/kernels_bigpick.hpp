@@ -43,12 +43,6 @@ namespace vkop {
 
 // In-kernel time stamps of the first workgroup's phases, for tuning: compiled in only
 // with -DVKOP_STAMPS=<name of the C function that reads them out> (rows_inst.hip).
-#ifdef VKOP_STAMPS
-static __device__ unsigned long long g_bp_stamps[64];
-#define BPS(i) do { if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[i] = wall_clock64(); } while (0)
-#else
-#define BPS(i) do { } while (0)
-#endif
 
 constexpr int kBigPickThreads = 256;
 constexpr int kBigPickWaves = kBigPickThreads / kWave;

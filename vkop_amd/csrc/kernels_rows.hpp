@@ -47,6 +47,15 @@
 
 namespace vkop {
 
+// Debug builds only (-DVKOP_STAMPS=<name of the C function that reads them out>, rows_inst.hip):
+// clock stamps of workgroup 0's first thread.
+#ifdef VKOP_STAMPS
+static __device__ unsigned long long g_bp_stamps[64];
+#define BPS(i) do { if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[i] = wall_clock64(); } while (0)
+#else
+#define BPS(i) do { } while (0)
+#endif
+
 constexpr int kFastCap = 1024;       // LDS slots for elements above the merge threshold
 constexpr int kFastMaxK = 511;       // k + 1 <= 512 ranks are kept in LDS (the merging workgroup has a thread per rank:
                                      // k <= 255 for rows_merge_kernel, more only where one larger workgroup holds the row)
@@ -1114,6 +1123,9 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     }
 
     // ---- exact path: radix select over the whole row ----------------------------
+#ifdef VKOP_STAMPS
+    if (threadIdx.x == 0) atomicAdd(&g_bp_stamps[61], 1ull);
+#endif
     __syncthreads();  // LDS changes owner
     if constexpr (SOFTMAX) {
         // redo the statistics the way the general kernels define them
@@ -1164,6 +1176,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
     __shared__ float fscratch[FUSED ? NW : 1];
     __shared__ double dscratch[FUSED ? NW : 1];
     __shared__ uint64_t local_ws[LOCAL ? kLocalCap + 3 * NW : 1];  // candidate list, then the wave records
+#ifdef VKOP_STAMPS
+    const unsigned long long dbg_t0 = wall_clock64();
+#endif
     __shared__ uint32_t s_last;
     ChunkShared<NT> *csp;
     if constexpr (FUSED) csp = &smem.chunk;
@@ -1407,7 +1422,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             return over ? 0xFFFFFFFFu : wcount;
         };
         uint32_t staged = 0;
+        BPS(48);
         uint32_t wave_candidates = compact(thr, staged, std::false_type{}, 0u);
+        BPS(49);
 
         // ---- the wave's partial sum (here, so that none of it is live across what follows) ------
         if constexpr (SOFTMAX) {
@@ -1463,16 +1480,33 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             }
             wk = wave_max_u32(wk);
             if (lane == 0) cs.wave_thr[wave] = wk;
-            if (tid < 32) cs.refine[tid] = 0;
+            if (tid < 34) cs.refine[tid] = tid == 32 ? 0xFFFFFFFFu : 0u;
             __syncthreads();
             uint32_t hi = cs.wave_thr[0];
 #pragma unroll
             for (int w = 1; w < NW; w++) hi = max(hi, cs.wave_thr[w]);
             // count(trial): elements of this wave at or above trial (wave-uniform)
-            auto exact_threshold = [&](auto count) -> uint32_t {
+            // floor_at(t): the smallest key at or above t among this lane's elements (all ones if none)
+            auto exact_threshold = [&](auto count, auto floor_at) -> uint32_t {
                 if (thr >= hi) return thr;
-                const int d = 31 - __clz(static_cast<int>(thr ^ hi));  // highest bit in which they differ
-                uint32_t t = hi & ~((2u << d) - 1u);                    // their common prefix
+                // Equal values en masse first (a row of few distinct values): the smallest key at or
+                // above the bound is then the answer -- k+1 elements reach it, fewer exceed it -- and
+                // costs two passes over the elements instead of one per bit.
+                uint32_t lb = thr;
+                const uint32_t wmin = ~wave_max_u32(~floor_at(thr));
+                if (lane == 0) atomicMin(&cs.refine[32], wmin);
+                __syncthreads();
+                const uint32_t t0 = cs.refine[32];
+                if (t0 < hi) {  // (the same in every thread; t0 >= thr)
+                    const uint32_t c = count(t0 + 1u);
+                    if (lane == 0 && c) atomicAdd(&cs.refine[33], c);
+                    __syncthreads();
+                    if (cs.refine[33] < want) return t0;
+                    lb = t0 + 1u;  // k+1 elements reach it
+                }
+                if (lb >= hi) return lb;
+                const int d = 31 - __clz(static_cast<int>(lb ^ hi));  // highest bit in which they differ
+                uint32_t t = hi & ~((2u << d) - 1u);                   // their common prefix
                 for (int bit = d; bit >= 0; bit--) {
                     const uint32_t trial = t | (1u << bit);
                     const uint32_t c = count(trial);
@@ -1480,8 +1514,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     __syncthreads();
                     if (cs.refine[bit] >= want) t = trial;
                 }
-                return max(t, thr);
+                return max(t, lb);
             };
+            BPS(55);
             if (from_stage) {
                 uint32_t keys[PASSES];
 #pragma unroll
@@ -1498,18 +1533,74 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
 #pragma unroll
                     for (int p = 0; p < PASSES; p++) c += static_cast<uint32_t>(__popcll(__ballot(keys[p] >= trial)));
                     return c;
+                }, [&](uint32_t t) {
+                    uint32_t f = 0xFFFFFFFFu;
+#pragma unroll
+                    for (int p = 0; p < PASSES; p++) f = keys[p] >= t ? min(f, keys[p]) : f;
+                    return f;
                 });
-            } else {
-                thr = exact_threshold([&](uint32_t trial) {
-                    uint32_t c = 0;
+            } else if (thr < hi) {
+                // Every element held in registers: a radix select over the keys, eight bits a
+                // pass, counted in LDS (lanes that share a digit add once) -- four passes whatever
+                // the values, where a descent over the bits in which bound and maximum differ
+                // takes up to two dozen (a pass costs the same either way: the keys are derived
+                // from the loaded vectors again).  Rows of few distinct values first: the
+                // smallest key at or above the bound is their answer -- k+1 elements reach it,
+                // fewer exceed it.
+                static_assert(sizeof(cs.stage_v) >= 256 * sizeof(uint32_t), "the digit counts take 256 words");
+                uint32_t *hist = reinterpret_cast<uint32_t *>(cs.stage_v);  // (the stage is filled anew afterwards)
+                uint32_t f = 0xFFFFFFFFu, above = 0;
 #pragma unroll
-                    for (int i = 0; i < V; i++) {
+                for (int i = 0; i < V; i++) {
 #pragma unroll
-                        for (int cc = 0; cc < VEC; cc++) c += static_cast<uint32_t>(__popcll(__ballot(key_of(i, cc) >= trial)));
+                    for (int cc = 0; cc < VEC; cc++) {
+                        const uint32_t kx = key_of(i, cc);
+                        f = kx >= thr ? min(f, kx) : f;
                     }
-                    return c;
-                });
+                }
+                f = ~wave_max_u32(~f);
+                if (lane == 0) atomicMin(&cs.refine[32], f);
+                __syncthreads();
+                const uint32_t t0 = cs.refine[32];  // (>= thr: the same in every thread)
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+#pragma unroll
+                    for (int cc = 0; cc < VEC; cc++) above += static_cast<uint32_t>(__popcll(__ballot(key_of(i, cc) > t0)));
+                }
+                if (lane == 0 && above) atomicAdd(&cs.refine[33], above);
+                __syncthreads();
+                if (cs.refine[33] < want) {
+                    thr = t0;
+                } else {
+                    uint32_t prefix = 0, need = want;
+                    for (int shift = 24; shift >= 0; shift -= 8) {
+                        __syncthreads();  // (the last pass's answer has been read)
+                        if (tid < 256u) hist[tid] = 0;
+                        __syncthreads();
+#pragma unroll
+                        for (int i = 0; i < V; i++) {
+#pragma unroll
+                            for (int cc = 0; cc < VEC; cc++) {
+                                const uint32_t kx = key_of(i, cc);  // (0 past the chunk's end: the lowest digit, below every element)
+                                if ((static_cast<uint64_t>(kx ^ prefix) >> (shift + 8)) == 0ull) hist_add_grouped(hist, (kx >> shift) & 255u);
+                            }
+                        }
+                        __syncthreads();
+                        if (wave == 0) {
+                            const uint2 r = hist256_resolve(hist, need);
+                            if (lane == 0) {
+                                cs.refine[32] = r.x;
+                                cs.refine[33] = r.y;
+                            }
+                        }
+                        __syncthreads();
+                        prefix |= (cs.refine[32] & 255u) << shift;  // (a digit is always found: the chunk holds k+1 elements at or above thr)
+                        need -= cs.refine[33];
+                    }
+                    thr = max(thr, prefix);
+                }
             }
+            BPS(50);
             // Index of the last equal element to list: elements are in index order by
             // (vector, wave, lane, position in the vector).
 #pragma unroll
@@ -1553,8 +1644,57 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 }
             }
             __syncthreads();
-            wave_candidates = compact(thr, staged, std::true_type{}, cs.thr);
+            BPS(51);
+            // The list, straight from the registers: at most 2 k + 1 entries (fewer than k+1 above the
+            // value, the first k+1 equal to it), each at a place of its own from counts per (vector,
+            // wave) -- not through the waves' stages of 64 vectors, which a sorted row, whose
+            // candidates all sit in one wave's elements, would overflow again.
+            {
+                const uint32_t idx_limit = cs.thr;
+                uint32_t *counts = cs.lane_key + V * NW;  // (behind the table of ties: 2 V NW <= NT words)
+                auto listed = [&](uint32_t kx, uint32_t idx) { return kx > thr || (kx == thr && idx <= idx_limit); };
+                uint32_t wave_total = 0;  // wave-uniform
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+                    uint32_t cnt = 0;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) cnt += static_cast<uint32_t>(__popcll(__ballot(listed(key_of(i, c), e0 + c))));
+                    if (lane == 0) counts[i * NW + wave] = cnt;
+                    wave_total += cnt;
+                }
+                __syncthreads();
+                uint32_t before_mine = 0;
+                if (tid < static_cast<uint32_t>(V * NW)) {
+#pragma unroll 1
+                    for (uint32_t j = 0; j < tid; j++) before_mine += counts[j];
+                }
+                __syncthreads();
+                if (tid < static_cast<uint32_t>(V * NW)) {
+                    if (tid == static_cast<uint32_t>(V * NW) - 1u) cs.total = before_mine + counts[tid];
+                    counts[tid] = before_mine;
+                }
+                __syncthreads();
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+                    uint32_t pos = counts[i * NW + wave];
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        const uint32_t kx = key_of(i, c);
+                        const bool pass = listed(kx, e0 + c);
+                        const uint64_t mask = __ballot(pass);
+                        if (mask != 0ull) {
+                            const uint32_t at = pos + lanes_below(mask);
+                            if (pass && at < ws.cap) publish(cand_out + at, composite(kx, e0 + c));
+                            pos += static_cast<uint32_t>(__popcll(mask));
+                        }
+                    }
+                }
+                wave_candidates = wave_total;
+            }
             __syncthreads();  // (cs.total is final)
+            BPS(52);
         }
         // the unused entries of the list read as "no element": the merge tells live
         // candidates from stale ones by that alone
@@ -1587,9 +1727,17 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
     }
     if constexpr (LOCAL) {
         __syncthreads();  // the list and the records are in LDS; so is what the merge builds, in other arrays
+        BPS(53);
         merge_row<T, NT, SOFTMAX, kLocalCap, true>(smem.fast, smem.exact, fscratch, dscratch, rowp,
                                              values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k, n, k,
                                              1u, per, NT, local_ws + kLocalCap, local_ws, ws.cap_shift);
+        BPS(54);
+#ifdef VKOP_STAMPS
+        if (threadIdx.x == 0) {
+            atomicMax(&g_bp_stamps[60], wall_clock64() - dbg_t0);
+            atomicAdd(&g_bp_stamps[62], 1ull);
+        }
+#endif
         (void)s_last;
     } else if constexpr (FUSED) {
         __syncthreads();

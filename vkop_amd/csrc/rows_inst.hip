@@ -175,6 +175,9 @@ template void launch_rows_merge<VKOP_ROWS_T, VKOP_ROWS_SOFTMAX>(const RowsLaunch
 
 #ifdef VKOP_STAMPS
 extern "C" int VKOP_STAMPS(unsigned long long *out) {
-    return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(vkop::g_bp_stamps), 64 * sizeof(unsigned long long)));
+    const int rc = static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(vkop::g_bp_stamps), 64 * sizeof(unsigned long long)));
+    static const unsigned long long zeros[64] = {};
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(vkop::g_bp_stamps), zeros, sizeof(zeros));  // (each readout starts the next interval)
+    return rc;
 }
 #endif
