@@ -1329,8 +1329,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
 
         // ---- 4. the elements at or above the threshold go to the chunk's candidate list --------
         // Returns the wave's count (all ones if the wave had more than 64 vectors to stage;
-        // staged_vectors = how many it staged).  With the truncation tag, of the elements
-        // equal to the threshold only those up to index idx_limit are listed.
+        // staged_vectors = how many it staged).
         uint64_t *cand_out;
         if constexpr (LOCAL) cand_out = local_ws;
         else cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
@@ -1339,8 +1338,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         else record = ws.sums + 3 * static_cast<size_t>(went);
         uint4 *stv = cs.stage_v + wave * kWave;
         uint32_t *ste = cs.stage_e + wave * kWave;
-        auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors, auto trunc_tag, uint32_t idx_limit) -> uint32_t {
-            constexpr bool TRUNC = decltype(trunc_tag)::value;
+        auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors) -> uint32_t {
             const float thr_f = ordered_to_float(thr_key);
             // 4a. the wave's vectors holding such an element -> LDS
             uint32_t nv = 0;  // wave-uniform
@@ -1348,22 +1346,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             for (int i = 0; i < V; i++) {
                 const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
                 bool hit;
-                if constexpr (!TRUNC) {
-                    if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
-                    else hit = vkey[i] >= thr_key && in_range(e0);
-                } else {
-                    // (the vector's largest key again from the vector itself: nothing the
-                    // first pass used stays live for the sake of this one)
-                    uint32_t vk = 0u;
-#pragma unroll
-                    for (int c = 0; c < VEC; c++) {
-                        float x = q[i].get(c);
-                        asm volatile("" : "+v"(x));
-                        const uint32_t key = (SOFTMAX && x != x) ? 0u : order_key(x);
-                        vk = max(vk, in_range(ALIGNED ? e0 : e0 + c) ? key : 0u);
-                    }
-                    hit = vk >= thr_key && in_range(e0) && (vk > thr_key || e0 <= idx_limit);
-                }
+                if constexpr (SOFTMAX) hit = !(vmax[i] < thr_f) && in_range(e0);
+                else hit = vkey[i] >= thr_key && in_range(e0);
                 const uint64_t mask = __ballot(hit);
                 if (mask != 0ull) {
                     if (hit) {
@@ -1397,8 +1381,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
                     const float x = r.get(static_cast<int>(lane % VEC));
                     const uint32_t key = order_key(x);
-                    bool pass = live && idx < c1 && key >= thr_key;
-                    if constexpr (TRUNC) pass = pass && (key > thr_key || idx <= idx_limit);
+                    const bool pass = live && idx < c1 && key >= thr_key;
                     const uint64_t mask = __ballot(pass);
                     if (pass) {
                         mine[p] = composite(key, idx);
@@ -1423,7 +1406,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         };
         uint32_t staged = 0;
         BPS(48);
-        uint32_t wave_candidates = compact(thr, staged, std::false_type{}, 0u);
+        uint32_t wave_candidates = compact(thr, staged);
         BPS(49);
 
         // ---- the wave's partial sum (here, so that none of it is live across what follows) ------
