@@ -204,8 +204,9 @@ def test_scan_with_spread_out_pick_for_large_k_equals_radix_select_and_oracle(op
 def test_one_wave_kernel_for_short_rows_equals_chunk_kernel_and_oracle(ops, n, k, dtype):
     """Short rows, small k (a classifier head): the one-wave-per-row kernel against the
     chunk kernel (rows.path = 1) and the oracle, on regular rows and on the ones it hands
-    to its exact fallback (ties en masse, masked rows, constant rows)."""
-    _compare_paths(ops, n, k, dtype, 6, KINDS, 4)
+    to its exact fallback (ties en masse, masked rows, constant rows), and on rows whose
+    probabilities underflow to 0 for all but a few elements (a tie at 0 that runs to the row's end)."""
+    _compare_paths(ops, n, k, dtype, 6, KINDS + ["huge", "masked90"], 4)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])

@@ -121,6 +121,38 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             return;
         }
     }
+    // Places g0 .. k-1 of the result go to the first elements, in index order, whose keys lie in
+    // [lo_key, hi_key] -- a group of equal probability pc; all of the row is in this wave's registers.
+    auto fill_group = [&](uint32_t g0, uint32_t lo_key, uint32_t hi_key, float pc) {
+        const uint32_t places = kk - g0;
+        uint32_t filled = 0;  // wave-uniform
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            if (filled < places) {
+                uint32_t mine_in = 0;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) mine_in += (key[i * VEC + c] >= lo_key && key[i * VEC + c] <= hi_key) ? 1u : 0u;
+                uint32_t incl = mine_in;
+#pragma unroll
+                for (int o = 1; o < kWave; o <<= 1) {
+                    const uint32_t t = __shfl_up(incl, o, kWave);
+                    if (lane >= static_cast<uint32_t>(o)) incl += t;
+                }
+                uint32_t pos = filled + incl - mine_in;
+#pragma unroll
+                for (int c = 0; c < VEC; c++) {
+                    if (key[i * VEC + c] >= lo_key && key[i * VEC + c] <= hi_key) {
+                        if (pos < places) {
+                            store_elem(ov, g0 + pos, pc);
+                            oi[g0 + pos] = static_cast<int32_t>((static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c));
+                        }
+                        pos++;
+                    }
+                }
+                filled += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
+            }
+        }
+    };
     // Steps 3 to 6, at most three times: with k+1 lane maxima, then with twice and four
     // times as many when a probability tie runs off the end of the candidates.
     bool exact = bad;
@@ -152,6 +184,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
         if (C > static_cast<uint32_t>(kWave) || C < min(want, n)) break;
         const bool have = lane < C;
         uint64_t mine = have ? smem.cand[lane] : 0ull;
+        const uint32_t xkey = static_cast<uint32_t>(mine >> 32);  // the candidate's logit
         __syncthreads();  // (the list may be written again)
         if constexpr (SOFTMAX) {
             // ---- 5. accurate terms for the candidates, the corrected sum, probabilities
@@ -177,6 +210,21 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
                 const uint32_t p_cut = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), __builtin_ctzll(at_cut)));
                 const uint32_t p_end = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), __builtin_ctzll(at_end)));
                 if (p_cut == p_end) {
+                    if (p_cut == order_key(0.f)) {
+                        // A tie at probability 0: the underflowed tail of the row, which runs to the
+                        // row's end -- the candidates of probability 0 and everything below the
+                        // candidates.  Its places go to its first elements in index order.
+                        const uint32_t g0 = static_cast<uint32_t>(__popcll(__ballot(have && mine_hi > p_cut)));
+                        uint32_t hi_key = (have && mine_hi == p_cut) ? xkey : 0u;
+#pragma unroll
+                        for (int o = 32; o > 0; o >>= 1) hi_key = max(hi_key, static_cast<uint32_t>(__shfl_xor(static_cast<int>(hi_key), o, kWave)));
+                        fill_group(g0, 1u, hi_key, 0.f);
+                        if (have && before < g0) {
+                            store_elem(ov, before, ordered_to_float(mine_hi));
+                            oi[before] = static_cast<int32_t>(composite_index(mine));
+                        }
+                        return;
+                    }
                     if (lanes_wanted >= static_cast<uint32_t>(kWave)) break;
                     continue;  // more candidates
                 }
@@ -312,34 +360,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
 #pragma unroll
                             for (int o = 32; o > 0; o >>= 1) hi_key = max(hi_key, static_cast<uint32_t>(__shfl_xor(static_cast<int>(hi_key), o, kWave)));
                             const uint32_t lo_key = pc > 0.f ? lowest_key_of_probability(hi_key, pc, prob_of_key) : 1u;
-                            const uint32_t places = kk - g0;
-                            uint32_t filled = 0;  // wave-uniform
-#pragma unroll
-                            for (int i = 0; i < V; i++) {
-                                if (filled < places) {
-                                    uint32_t mine_in = 0;
-#pragma unroll
-                                    for (int c = 0; c < VEC; c++) mine_in += (key[i * VEC + c] >= lo_key && key[i * VEC + c] <= hi_key) ? 1u : 0u;
-                                    uint32_t incl = mine_in;
-#pragma unroll
-                                    for (int o = 1; o < kWave; o <<= 1) {
-                                        const uint32_t t = __shfl_up(incl, o, kWave);
-                                        if (lane >= static_cast<uint32_t>(o)) incl += t;
-                                    }
-                                    uint32_t pos = filled + incl - mine_in;
-#pragma unroll
-                                    for (int c = 0; c < VEC; c++) {
-                                        if (key[i * VEC + c] >= lo_key && key[i * VEC + c] <= hi_key) {
-                                            if (pos < places) {
-                                                store_elem(ov, g0 + pos, pc);
-                                                oi[g0 + pos] = static_cast<int32_t>((static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c));
-                                            }
-                                            pos++;
-                                        }
-                                    }
-                                    filled += static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
-                                }
-                            }
+                            fill_group(g0, lo_key, hi_key, pc);
                         }
                     }
                 }
