@@ -277,12 +277,29 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             // (k+1)-th largest ELEMENT then, by a descent over all of them; fewer than k+1
             // elements lie above that.
             uint32_t t2 = 0;
-            for (int bit = 31; bit >= 0; bit--) {
-                const uint32_t trial = t2 | (1u << bit);
-                uint32_t c = 0;
+            if (above <= static_cast<uint32_t>(kWave)) {
+                // (up to 64 of them: each is in the list, a lane each counts the ones that rank
+                // before its own, and the one with k before it is the element looked for)
+                __syncthreads();  // (one wave: the list is written)
+                const bool listed = lane < above;
+                const uint64_t own = listed ? smem.cand[lane] : 0ull;
+                const uint32_t own_lo = static_cast<uint32_t>(own), own_hi = static_cast<uint32_t>(own >> 32);
+                uint32_t ahead = 0;
+                for (uint32_t c = 0; c < above; c++) {
+                    const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_hi), static_cast<int>(c)))) << 32) |
+                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_lo), static_cast<int>(c)));
+                    ahead += (other > own) ? 1u : 0u;
+                }
+                const uint64_t holder = __ballot(listed && ahead == want - 1u);  // (exactly one lane: composites differ)
+                t2 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_hi), __builtin_ctzll(holder)));
+            } else {
+                for (int bit = 31; bit >= 0; bit--) {
+                    const uint32_t trial = t2 | (1u << bit);
+                    uint32_t c = 0;
 #pragma unroll
-                for (int e = 0; e < ELEMS; e++) c += static_cast<uint32_t>(__popcll(__ballot(key[e] >= trial)));
-                if (c >= want) t2 = trial;
+                    for (int e = 0; e < ELEMS; e++) c += static_cast<uint32_t>(__popcll(__ballot(key[e] >= trial)));
+                    if (c >= want) t2 = trial;
+                }
             }
             tie = max(t2, kKeyNegInf);
             __syncthreads();  // (one wave: the list is written again)
