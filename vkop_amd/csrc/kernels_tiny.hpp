@@ -121,6 +121,24 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             return;
         }
     }
+    // How many of the C composites that the lanes 0 .. C-1 hold (0 in the other lanes) rank before
+    // this lane's: the composites go through LDS, where every lane reads all of them -- one
+    // address per load for the whole wave, eight loads in flight (lane-to-lane reads through
+    // scalar registers took 36 ns a candidate).  All lanes call; the list in LDS is overwritten.
+    auto rank_among = [&](uint64_t own, uint32_t C) -> uint32_t {
+        __syncthreads();  // (one wave: whoever still reads the list is done)
+        smem.cand[lane] = own;
+        __syncthreads();
+        uint32_t ahead = 0;
+        for (uint32_t c0 = 0; c0 < C; c0 += 8) {
+            uint64_t other[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) other[j] = smem.cand[c0 + static_cast<uint32_t>(j)];  // (C <= 64 entries; past C: 0, never ahead)
+#pragma unroll
+            for (int j = 0; j < 8; j++) ahead += (other[j] > own) ? 1u : 0u;
+        }
+        return ahead;
+    };
     // Places g0 .. k-1 of the result go to the first elements, in index order, whose keys lie in
     // [lo_key, hi_key] -- a group of equal probability pc; all of the row is in this wave's registers.
     auto fill_group = [&](uint32_t g0, uint32_t lo_key, uint32_t hi_key, float pc) {
@@ -155,6 +173,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
     };
     // Steps 3 to 6, at most three times: with k+1 lane maxima, then with twice and four
     // times as many when a probability tie runs off the end of the candidates.
+    BPS(21);
     bool exact = bad;
     for (uint32_t lanes_wanted = want; !exact; lanes_wanted = 2u * lanes_wanted + 2u) {
         // ---- 3. the lanes_wanted-th largest lane maximum, to 16 bits (-inf never becomes a candidate)
@@ -196,13 +215,8 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             mine = have ? ((static_cast<uint64_t>(order_key(p)) << 32) | (mine & 0xFFFFFFFFull)) : 0ull;
         }
         // ---- 6. ranks among the candidates
-        const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
-        uint32_t before = 0;
-        for (uint32_t c = 0; c < C; c++) {
-            const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), static_cast<int>(c)))) << 32) |
-                                   static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_lo), static_cast<int>(c)));
-            before += (other > mine) ? 1u : 0u;
-        }
+        const uint32_t mine_hi = static_cast<uint32_t>(mine >> 32);
+        const uint32_t before = rank_among(mine, C);
         if constexpr (SOFTMAX) {
             // a probability shared by the k-th place and the last candidate may go on below the candidates
             if (C < n && C > kk) {
@@ -244,6 +258,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
     // first elements equal to T in index order.  A probability that the k-th place shares
     // with the place behind it (equal values do, and different values can) is settled over
     // every element of the row that has it.
+    BPS(22);
     if (!bad) {
         uint32_t tie = 0;
         for (int bit = 31; bit >= 0; bit--) {
@@ -270,7 +285,12 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             }
             return count;
         };
+        BPS(23);
         uint32_t above = gather_above(tie);
+        BPS(24);
+#ifdef VKOP_STAMPS
+        if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[29] = above;
+#endif
         if (above >= want) {
             // More than k elements above the (k+1)-th largest LANE maximum: the top of the row
             // sits in few lanes (a sorted row: a lane's elements are neighbours).  The exact
@@ -278,20 +298,13 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             // elements lie above that.
             uint32_t t2 = 0;
             if (above <= static_cast<uint32_t>(kWave)) {
-                // (up to 64 of them: each is in the list, a lane each counts the ones that rank
-                // before its own, and the one with k before it is the element looked for)
+                // (up to 64 of them: each is in the list, a lane each, and the descent is over one key a lane)
                 __syncthreads();  // (one wave: the list is written)
-                const bool listed = lane < above;
-                const uint64_t own = listed ? smem.cand[lane] : 0ull;
-                const uint32_t own_lo = static_cast<uint32_t>(own), own_hi = static_cast<uint32_t>(own >> 32);
-                uint32_t ahead = 0;
-                for (uint32_t c = 0; c < above; c++) {
-                    const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_hi), static_cast<int>(c)))) << 32) |
-                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_lo), static_cast<int>(c)));
-                    ahead += (other > own) ? 1u : 0u;
+                const uint32_t own = lane < above ? static_cast<uint32_t>(smem.cand[lane] >> 32) : 0u;
+                for (int bit = 31; bit >= 0; bit--) {
+                    const uint32_t trial = t2 | (1u << bit);
+                    if (static_cast<uint32_t>(__popcll(__ballot(own >= trial))) >= want) t2 = trial;
                 }
-                const uint64_t holder = __ballot(listed && ahead == want - 1u);  // (exactly one lane: composites differ)
-                t2 = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(own_hi), __builtin_ctzll(holder)));
             } else {
                 for (int bit = 31; bit >= 0; bit--) {
                     const uint32_t trial = t2 | (1u << bit);
@@ -302,8 +315,10 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
                 }
             }
             tie = max(t2, kKeyNegInf);
+            BPS(25);
             __syncthreads();  // (one wave: the list is written again)
             above = gather_above(tie);
+            BPS(26);
         }
         if (above < want) {
             // the first want - above elements equal to T: vector by vector, lane by lane, element by element
@@ -352,13 +367,8 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
                     const float p = round_to_storage<T>(static_cast<float>(static_cast<double>(term) * rinv));
                     mine = have ? ((static_cast<uint64_t>(order_key(p)) << 32) | (mine & 0xFFFFFFFFull)) : 0ull;
                 }
-                const uint32_t mine_lo = static_cast<uint32_t>(mine), mine_hi = static_cast<uint32_t>(mine >> 32);
-                uint32_t before = 0;
-                for (uint32_t c = 0; c < C; c++) {
-                    const uint64_t other = (static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_hi), static_cast<int>(c)))) << 32) |
-                                           static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mine_lo), static_cast<int>(c)));
-                    before += (other > mine) ? 1u : 0u;
-                }
+                const uint32_t mine_hi = static_cast<uint32_t>(mine >> 32);
+                const uint32_t before = rank_among(mine, C);
                 uint32_t g0 = kk;  // ranks from here on are filled as one group of equal probability
                 if constexpr (SOFTMAX) {
                     if (C > kk) {
@@ -392,6 +402,10 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
         }
     }
     // ---- the exact select over the whole row -----------------------------------------------
+#ifdef VKOP_STAMPS
+    if (threadIdx.x == 0) atomicAdd(&g_bp_stamps[30], 1ull);
+#endif
+    BPS(27);
     __syncthreads();  // LDS changes owner
     SelectShared &ex = smem.exact;
     if constexpr (SOFTMAX) {
