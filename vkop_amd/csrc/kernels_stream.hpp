@@ -240,6 +240,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     const uint32_t want = k + 1;
     const uint32_t kk = min(k, n);
     const uint32_t waves = G * kScanWaves;
+    BPS(14);
     // ---- A. everything the kernel reads first, in one round trip --------------------
     // (never a branch around a load: out-of-range threads re-read entry 0)
     const uint64_t *recs = ws.recs + 2 * static_cast<size_t>(row) * waves;
@@ -259,6 +260,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     }
 
     // ---- B. the row's maximum and sum from the wave partials --------------------------
+    BPS(8);
     for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;  // for block_rank, barriers away
     if (tid == 0) sh.count = 0;
     if constexpr (SOFTMAX) {
@@ -304,6 +306,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     }
 
     // ---- C. a value that k+1 block maxima reach ---------------------------------------------
+    BPS(9);
     uint32_t lmk = 0;
 #pragma unroll
     for (int e = 0; e < GE; e++) {
@@ -347,6 +350,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         return t;
     };
     uint32_t thr = threshold_of_thread_maxima(lmk, true);
+    BPS(10);
     float M = 0.f;
     double s_base = 0.0;
     if constexpr (SOFTMAX) {
@@ -472,6 +476,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     hit_cap = min(static_cast<uint32_t>(kPickHitCap), 3u * want + 64u);
     if (blocks > want + want / 4u) hit_cap = min(hit_cap, blocks - 1u);
     bool many_groups = gather(thr, 1ull << 32, std::false_type{});
+    BPS(11);
     if (many_groups) {
         // More than kPickHitCap blocks reach thr: the threads' shares of the block maxima are
         // not alike (rows sorted in runs as long as the stride between a thread's blocks put
@@ -632,8 +637,10 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             const uint32_t b = idx / per, off = idx - b * per;
             return b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;
         };
+        BPS(12);
         finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing, scale,
                                    counts != nullptr ? counts + row : nullptr, top_p);
+        BPS(13);
         return;
     }
 
