@@ -234,6 +234,29 @@ def test_large_k_rows_whose_cut_falls_into_a_crowd(ops, n, k):
     _compare_paths(ops, n, k, np.float32, 4, WALK_KINDS, 3)
 
 
+@pytest.mark.parametrize("rows,n,k", [(16, 131072, 1), (32, 50000, 3), (4, 262144, 1024), (8, 100000, 600), (64, 8192, 3),
+                                      (256, 1000, 5), (7, 128255, 50)])
+def test_rows_of_one_repeated_value_and_a_few_peaks(ops, rows, n, k):
+    """One value everywhere but in three places: the row's sum is that value's term times its
+    count, and the term is, by definition, the correctly rounded float exponential of the
+    ROUNDED difference to the maximum -- off the exact exponential of the exact difference by up
+    to 3e-7, the same for every copy.  A streaming pass that sums against a reference of its
+    own has to say so exactly (the scan kernel records a wave of equal elements as a count and
+    the value), or the probabilities drift by several ulp; every route, the plain softmax too."""
+    rng = np.random.default_rng(rows + n + k)
+    for rep in range(2):
+        x = np.zeros((rows, n), np.float32) + (rng.standard_normal((rows, 1)) * 2).astype(np.float32)
+        for r in range(rows):
+            x[r, rng.choice(n, 3, replace=False)] = x[r, 0] + (rng.random(3) * 8 + 1).astype(np.float32)
+        v, ix = ops.softmax_topk(dev(x), k)
+        v, ix = host(v), host(ix)
+        ov, oix = oracle.softmax_topk(x, k)
+        assert ulp_diff(v, ov).max() <= 2, (rows, n, k, int(ulp_diff(v, ov).max()))
+        assert np.array_equal(ix, oix), (rows, n, k)
+        y = host(ops.softmax(dev(x)))
+        assert ulp_diff(y, oracle.softmax(x)).max() <= 2, (rows, n, k)
+
+
 @pytest.mark.parametrize("n", [16388, 40002, 128255])
 def test_scan_pick_pair_on_rows_that_do_not_start_on_16_bytes(ops, n):
     """n not a multiple of the vector width (rows after the first are unaligned), and a

@@ -535,7 +535,8 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
             // what the element should contribute, exp(fl(x - M)), minus what its wave
             // added for it, fast_term(x, ref) * exp(ref - M)
             const double cr = static_cast<double>(term) -
-                              static_cast<double>(fast_term(xv, ref)) * exp_rescale(static_cast<double>(ref) - static_cast<double>(M));
+                              static_cast<double>(fast_term(xv, ref)) *
+                                  sum_rescale(__longlong_as_double(static_cast<long long>(recs[2 * sp])), ref, M);
             if (cr > -1.0 && cr < 1.0) fix += static_cast<long long>(cr * kBigPickFixUnit);  // (anything else: the row's sum is not finite)
             lterm[t] = term;
         }
@@ -588,7 +589,7 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
             for (uint32_t w = tid; w < waves; w += NT) {
                 const double sv = __longlong_as_double(static_cast<long long>(recs[2 * w]));
                 const float ref = __uint_as_float(static_cast<uint32_t>(recs[2 * w + 1]));
-                if (sv != 0.0) acc += sv * exp_rescale(static_cast<double>(ref) - static_cast<double>(M));
+                if (sv != 0.0) acc += sv * sum_rescale(sv, ref, M);
             }
             const double s_base = block_sum_fast<NT>(acc, dscratch);
             if (tid == 0) {

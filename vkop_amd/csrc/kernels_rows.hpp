@@ -209,6 +209,17 @@ __device__ __forceinline__ double exp_rescale(double x) {
     return ldexp(p, static_cast<int>(n));
 }
 
+// The factor that carries a partial sum of terms exp(x - ref) over to the row's maximum M.
+// A sum that is a whole number comes from terms that were all exactly 1 (or 0): a flat stretch
+// of the row, every element equal to the reference (or -inf).  Each of them counts
+// exp_accurate(fl(ref - M)) in the sum as defined (kernels_general.hpp) -- a float, off the exact
+// exponential of the exact difference by up to 3e-7 relative, the same for every copy -- so that
+// is the factor then: rows that are one repeated value and a few peaks stay within the bar.
+__device__ __forceinline__ double sum_rescale(double s, float ref, float M) {
+    if (s == rint(s)) return static_cast<double>(softmax_term(ref, M));
+    return exp_rescale(static_cast<double>(ref) - static_cast<double>(M));
+}
+
 // ---- memory shared between workgroups ------------------------------------------
 // Everything one workgroup writes for another to read goes through device-scope
 // atomic stores and loads (relaxed): such a store is written through to memory
@@ -908,7 +919,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
             const float m = wave_max_f32_uniform(p0.m);
             double acc = 0.0;
             if (tid < waves) {
-                const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+                const double sc = sum_rescale(p0.s, p0.ref, m);
                 sh.scale[tid] = sc;
                 if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
             }
@@ -922,7 +933,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         const float m = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.ref is published)
         double acc = 0.0;
         if (tid < waves) {
-            const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+            const double sc = sum_rescale(p0.s, p0.ref, m);
             sh.scale[tid] = sc;
             if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
         }

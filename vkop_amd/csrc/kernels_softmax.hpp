@@ -236,7 +236,7 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
     if (tid < G) st = stats[static_cast<size_t>(row) * G + tid];
     const float M = block_max<NT>(st.m, fscratch);
     double part = 0.0;
-    if (tid < G && st.s != 0.0) part = st.s * exp(static_cast<double>(st.ref) - static_cast<double>(M));
+    if (tid < G && st.s != 0.0) part = st.s * sum_rescale(st.s, st.ref, M);
     const LineStats ls{M, 0.f, 1.0 / block_sum<NT>(part, dscratch)};
     T *orow = out + row0;
 #pragma unroll
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
         __syncthreads();
         float M = fmax_lds[mine];
         for (uint32_t c = 1; c < G; c++) M = fmaxf(M, fmax_lds[c * TI + mine]);
-        dsum_lds[tid] = (holds && cs.s != 0.0) ? cs.s * exp(static_cast<double>(cs.ref) - static_cast<double>(M)) : 0.0;
+        dsum_lds[tid] = (holds && cs.s != 0.0) ? cs.s * sum_rescale(cs.s, cs.ref, M) : 0.0;
         __syncthreads();
         double sum = dsum_lds[mine];
         for (uint32_t c = 1; c < G; c++) sum += dsum_lds[c * TI + mine];

@@ -86,6 +86,7 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
             return in_range(ALIGNED ? e0 : e0 + static_cast<uint32_t>(c)) ? x : -INFINITY;
         };
         float ref = 0.f;
+        float wm0 = -INFINITY;  // the maximum of the wave's first vectors
         double acc = 0.0;  // every term is added in double: a dominant term must not swallow what follows it
         static_for<0, V>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                     // reference of the wave's partial sum: kRefLift above the maximum of its
                     // first vectors; 0 if they hold no finite element (terms are then 0, or
                     // NaN, which must survive -- never -inf - -inf)
-                    const float wm0 = wave_max_f32_uniform(vm);
+                    wm0 = wave_max_f32_uniform(vm);
                     ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
                 }
 #pragma unroll
@@ -170,6 +171,27 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                     for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(elem(i_tag, c), ref));
                 });
                 wsum = wave_sum_f64_uniform(acc);
+            } else if (wm == wm0 && wm0 > -INFINITY) {
+                // A wave of equal elements (a flat stretch of the row): every lane's sum is its
+                // number of elements times the one term -- terms never exceed the maximum's, so
+                // nothing else adds up to that.  Its record says so exactly: the count as the sum,
+                // the value itself as the reference.  Whoever combines the records counts
+                // exp_accurate(fl(value - M)) for each of them, as the sum is defined, instead of
+                // a hardware exponential of value - reference times an exponential of
+                // reference - M, whose error -- the same for every copy -- a row made of one
+                // repeated value and a few peaks carried into its probabilities (up to 7 ulp).
+                uint32_t mine_n = 0;
+                static_for<0, V>([&](auto i_tag) {
+                    constexpr int i = decltype(i_tag)::value;
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) mine_n += (FULL || in_range(ALIGNED ? e0 : e0 + static_cast<uint32_t>(c))) ? 1u : 0u;
+                });
+                const bool flat = acc == static_cast<double>(mine_n) * static_cast<double>(fast_term(wm0, ref));
+                if (__ballot(!flat) == 0ull) {
+                    wsum = FULL ? static_cast<double>(kWave * V * VEC) : wave_sum_f64_uniform(static_cast<double>(mine_n));
+                    ref = wm0;
+                }
             }
             if (lane == 0) {
                 uint64_t *record = ws.recs + 2 * (static_cast<size_t>(row * G + chunk) * NW + wave);
@@ -279,7 +301,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                 const float m = wave_max_f32_uniform(p0.m);
                 double acc = 0.0;
                 if (tid < waves) {
-                    const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+                    const double sc = sum_rescale(p0.s, p0.ref, m);
                     sh.scale[tid] = sc;
                     if (p0.s != 0.0) acc = p0.s * sc;
                 }
@@ -293,7 +315,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             const float m = block_max_fast<NT>(p0.m, fscratch);  // (barrier: sh.ref is published)
             double acc = 0.0;
             if (tid < waves) {
-                const double sc = exp_rescale(static_cast<double>(p0.ref) - static_cast<double>(m));
+                const double sc = sum_rescale(p0.s, p0.ref, m);
                 sh.scale[tid] = sc;
                 if (p0.s != 0.0) acc = p0.s * sc;
             }
