@@ -121,6 +121,23 @@ def test_softmax_axes(ops, shape, axis):
     assert_softmax_close(host(ops.softmax(dev(xh), axis)), xh, axis, str((shape, axis)) + " half")
 
 
+@pytest.mark.parametrize("shape,axis", [((128, 33000), -1), ((16, 131072), -1), ((64, 40000), -1), ((8, 4096, 256), 1),
+                                        ((32, 1000, 64), 1), ((300, 200, 64), 1), ((4096, 1024), -1)])
+def test_softmax_of_one_repeated_value_and_a_few_peaks(ops, shape, axis):
+    """Lines that are one value but for a peak in five thousand elements: the sum is that value's
+    term times its count, the term being the float exponential of the ROUNDED difference to the
+    maximum; the kernels that sum chunks against their own maxima count the copies of each
+    chunk's smallest value apart, so that they enter the sum as defined (4 ulp otherwise)."""
+    rng = np.random.default_rng(len(shape) + shape[-1])
+    x = np.full(shape, 0.25, np.float32)
+    x.ravel()[rng.integers(0, x.size, max(1, x.size // 5000))] = 6.0
+    x.ravel()[rng.integers(0, x.size, 3)] = -np.inf
+    assert_softmax_close(host(ops.softmax(dev(x), axis)), x, axis, str(shape))
+    y = (x * np.float32(-1.0)).astype(np.float32)      # the repeated value on top, the rest far below
+    y[np.isinf(y)] = -np.inf
+    assert_softmax_close(host(ops.softmax(dev(y), axis)), y, axis, str(shape) + " flipped")
+
+
 def test_softmax_special_values_and_nan_option(ops):
     x = np.zeros((5, 130), np.float32)
     x[0, 7] = np.nan

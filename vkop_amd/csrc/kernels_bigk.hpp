@@ -392,8 +392,11 @@ __global__ __launch_bounds__(kWave) void bigk_row_stats_kernel(const ChunkStat *
     for (uint32_t g = lane; g < G; g += kWave) m = fmaxf(m, c[g].m);
     m = wave_max(m);
     double s = 0.0;
-    for (uint32_t g = lane; g < G; g += kWave)
-        if (c[g].s != 0.0) s += c[g].s * exp(static_cast<double>(c[g].ref) - static_cast<double>(m));
+    for (uint32_t g = lane; g < G; g += kWave) {
+        if (c[g].s != 0.0) s += c[g].s * sum_rescale(c[g].s, c[g].ref, m);
+        // (the copies of the chunk's minimum, which its sum leaves out)
+        if (c[g].nmin != 0u) s += static_cast<double>(c[g].nmin) * static_cast<double>(softmax_term(c[g].vmin, m));
+    }
     s = wave_sum(s);
     if (lane == 0) stats[row] = LineStats{m, 0.f, 1.0 / s};
 }

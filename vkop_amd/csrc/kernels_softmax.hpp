@@ -42,9 +42,11 @@ __device__ __forceinline__ float fast_term_unbiased(float x, float m) {
 }
 
 struct ChunkStat {
-    double s;   // sum of exp(x - ref) over the chunk
-    float m;    // maximum of the chunk (NaN ignored; -inf for an empty chunk)
-    float ref;  // reference of the sum: m, or 0 when m is not finite
+    double s;       // sum of exp(x - ref) over the chunk (softmax_stats_kernel: without the copies of its minimum)
+    float m;        // maximum of the chunk (NaN ignored; -inf for an empty chunk)
+    float ref;      // reference of the sum: m, or 0 when m is not finite
+    float vmin;     // softmax_stats_kernel: the chunk's minimum ...
+    uint32_t nmin;  // ... and how many elements equal it (0: none set apart)
 };
 
 // ---- a whole row per workgroup ------------------------------------------------------
@@ -165,6 +167,8 @@ __global__ __launch_bounds__(NT) void softmax_stats_kernel(const T *__restrict__
     constexpr int NW = NT / kWave;
     __shared__ float fscratch[NW];
     __shared__ double dscratch[NW];
+    __shared__ float fscratch2[NW];
+    __shared__ uint32_t uscratch[NW];
     const uint32_t tid = threadIdx.x;
     const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
     const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
@@ -181,28 +185,73 @@ __global__ __launch_bounds__(NT) void softmax_stats_kernel(const T *__restrict__
             for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < c1 ? e0 + c : 0u));
         }
     }
-    float m = -INFINITY;
+    // The copies of the chunk's smallest value are set apart and counted: a value that fills most
+    // of a row (padding, a floor, zeros) is usually its smallest, every copy of it has the same
+    // term, and that term's error would go into the sum thousands of times over -- the row's sum
+    // is DEFINED with exp_accurate(fl(x - M)) for each, which only the kernel that knows M can
+    // count (4 ulp on rows of one value and a few peaks otherwise).  Maximum and minimum in one
+    // pass and one reduction.
+    float m = -INFINITY, mn = INFINITY;
 #pragma unroll
     for (int i = 0; i < V; i++) {
         const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
 #pragma unroll
-        for (int c = 0; c < VEC; c++)
-            if (e0 + c < c1) m = fmaxf(m, q[i].get(c));
+        for (int c = 0; c < VEC; c++) {
+            if (e0 + c < c1) {
+                m = fmaxf(m, q[i].get(c));   // (drops NaN)
+                mn = fminf(mn, q[i].get(c));
+            }
+        }
     }
-    m = block_max<NT>(m, fscratch);
+    m = wave_max(m);
+    mn = -wave_max(-mn);
+    if constexpr (NW > 1) {
+        if ((tid & (kWave - 1)) == 0) {
+            fscratch[tid / kWave] = m;
+            fscratch2[tid / kWave] = mn;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            m = fmaxf(m, fscratch[w]);
+            mn = fminf(mn, fscratch2[w]);
+        }
+    }
     // reference of the chunk's sum: its maximum, or 0 when that is not finite
     // (then every term is 0, inf or NaN, and NaN / inf must reach the sum)
     const float ref = (m > -INFINITY && m < INFINITY) ? m : 0.f;
+    const bool apart = mn > -INFINITY && mn < INFINITY;  // (copies of -inf count for nothing either way)
     double acc = 0.0;
+    uint32_t copies = 0;
 #pragma unroll
     for (int i = 0; i < V; i++) {
         const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
 #pragma unroll
-        for (int c = 0; c < VEC; c++)
-            if (e0 + c < c1) acc += static_cast<double>(fast_term_unbiased(q[i].get(c), ref));
+        for (int c = 0; c < VEC; c++) {
+            const float x = q[i].get(c);
+            const bool live = e0 + c < c1;
+            const bool copy = live && apart && x == mn;
+            copies += copy ? 1u : 0u;
+            acc += (live && !copy) ? static_cast<double>(fast_term_unbiased(x, ref)) : 0.0;
+        }
     }
-    const double s = block_sum<NT>(acc, dscratch);
-    if (tid == 0) stats[blockIdx.x] = ChunkStat{s, m, ref};
+    acc = wave_sum(acc);
+    copies = wave_sum(copies);
+    if constexpr (NW > 1) {
+        if ((tid & (kWave - 1)) == 0) {
+            dscratch[tid / kWave] = acc;
+            uscratch[tid / kWave] = copies;
+        }
+        __syncthreads();
+        acc = dscratch[0];
+        copies = uscratch[0];
+#pragma unroll
+        for (int w = 1; w < NW; w++) {  // fixed order: run-to-run stable
+            acc += dscratch[w];
+            copies += uscratch[w];
+        }
+    }
+    if (tid == 0) stats[blockIdx.x] = ChunkStat{acc, m, ref, mn, copies};
 }
 
 // ---- chunked rows: exp(x - M) / S -----------------------------------------------------
@@ -232,11 +281,12 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
         }
     }
     // the row's maximum and sum from its G chunk results (G <= NT)
-    ChunkStat st{0.0, -INFINITY, 0.f};
+    ChunkStat st{0.0, -INFINITY, 0.f, 0.f, 0u};
     if (tid < G) st = stats[static_cast<size_t>(row) * G + tid];
     const float M = block_max<NT>(st.m, fscratch);
     double part = 0.0;
     if (tid < G && st.s != 0.0) part = st.s * sum_rescale(st.s, st.ref, M);
+    if (tid < G && st.nmin != 0u) part += static_cast<double>(st.nmin) * static_cast<double>(softmax_term(st.vmin, M));
     const LineStats ls{M, 0.f, 1.0 / block_sum<NT>(part, dscratch)};
     T *orow = out + row0;
 #pragma unroll
@@ -339,8 +389,11 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
     LineStats st{0.f, 0.f, 0.0};
     if constexpr (!kFold) {
         // ---- 1. the lines' maxima
-        float m = -INFINITY;
-        pass([&](float x, uint32_t) { m = fmaxf(m, x); });  // (drops NaN)
+        float m = -INFINITY, mn_own = INFINITY;
+        pass([&](float x, uint32_t) {
+            m = fmaxf(m, x);  // (drops NaN)
+            if constexpr (MODE == kTileStats) mn_own = fminf(mn_own, x);
+        });
         m = reduce_max(m);
         // ---- 2. the sums of the terms
         double acc = 0.0;
@@ -351,21 +404,33 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
             // reference of the chunk's sum: its maximum, or 0 when that is not finite (then
             // every term is 0, inf or NaN, and NaN / inf must reach the sum)
             const float ref = (m > -INFINITY && m < INFINITY) ? m : 0.f;
-            pass([&](float x, uint32_t) { acc += static_cast<double>(fast_term_unbiased(x, ref)); });
+            // (the copies of the chunk's minimum are counted apart, as in softmax_stats_kernel)
+            __syncthreads();  // (fmax_lds is read by every thread of the first reduction)
+            const float mn = -reduce_max(-mn_own);
+            const bool apart = mn > -INFINITY && mn < INFINITY;
+            double copies = 0.0;
+            pass([&](float x, uint32_t) {
+                if (apart && x == mn) copies += 1.0;
+                else acc += static_cast<double>(fast_term_unbiased(x, ref));
+            });
             const double sum = reduce_sum(acc);
-            if (tid < TI) stats[(static_cast<size_t>(tileid) * G + chunk) * TI + tid] = ChunkStat{sum, m, ref};
+            __syncthreads();  // (dsum_lds likewise)
+            const double nmin = reduce_sum(copies);
+            if (tid < TI)
+                stats[(static_cast<size_t>(tileid) * G + chunk) * TI + tid] = ChunkStat{sum, m, ref, mn, static_cast<uint32_t>(nmin)};
             return;
         }
     } else {
         // thread c * TI + l fetches chunk c's result for line l; every lane then folds its line's G
         const bool holds = tid < G * TI;
-        ChunkStat cs{0.0, -INFINITY, 0.f};
+        ChunkStat cs{0.0, -INFINITY, 0.f, 0.f, 0u};
         if (holds) cs = stats[(static_cast<size_t>(tileid) * G + (tid >> ti_shift)) * TI + mine];
         fmax_lds[tid] = cs.m;
         __syncthreads();
         float M = fmax_lds[mine];
         for (uint32_t c = 1; c < G; c++) M = fmaxf(M, fmax_lds[c * TI + mine]);
-        dsum_lds[tid] = (holds && cs.s != 0.0) ? cs.s * sum_rescale(cs.s, cs.ref, M) : 0.0;
+        dsum_lds[tid] = ((holds && cs.s != 0.0) ? cs.s * sum_rescale(cs.s, cs.ref, M) : 0.0) +
+                        ((holds && cs.nmin != 0u) ? static_cast<double>(cs.nmin) * static_cast<double>(softmax_term(cs.vmin, M)) : 0.0);
         __syncthreads();
         double sum = dsum_lds[mine];
         for (uint32_t c = 1; c < G; c++) sum += dsum_lds[c * TI + mine];
