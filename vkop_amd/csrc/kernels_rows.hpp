@@ -216,7 +216,7 @@ __device__ __forceinline__ double exp_rescale(double x) {
 // exponential of the exact difference by up to 3e-7 relative, the same for every copy -- so that
 // is the factor then: rows that are one repeated value and a few peaks stay within the bar.
 __device__ __forceinline__ double sum_rescale(double s, float ref, float M) {
-    if (s == rint(s)) return static_cast<double>(softmax_term(ref, M));
+    if (s != 0.0 && s == rint(s)) return static_cast<double>(softmax_term(ref, M));  // (0: an idle lane's, or nothing to carry)
     return exp_rescale(static_cast<double>(ref) - static_cast<double>(M));
 }
 

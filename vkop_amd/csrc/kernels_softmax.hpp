@@ -228,13 +228,16 @@ __global__ __launch_bounds__(NT) void softmax_stats_kernel(const T *__restrict__
         const uint32_t e0 = c0 + (static_cast<uint32_t>(i) * NT + tid) * VEC;
 #pragma unroll
         for (int c = 0; c < VEC; c++) {
-            const float x = q[i].get(c);
-            const bool live = e0 + c < c1;
-            const bool copy = live && apart && x == mn;
-            copies += copy ? 1u : 0u;
-            acc += (live && !copy) ? static_cast<double>(fast_term_unbiased(x, ref)) : 0.0;
+            if (e0 + c < c1) {
+                const float x = q[i].get(c);
+                copies += (x == mn) ? 1u : 0u;
+                acc += static_cast<double>(fast_term_unbiased(x, ref));
+            }
         }
     }
+    // (every copy added the same float: taking them out again is exact to the sum's own rounding)
+    if (apart) acc -= static_cast<double>(copies) * static_cast<double>(fast_term_unbiased(mn, ref));
+    else copies = 0;
     acc = wave_sum(acc);
     copies = wave_sum(copies);
     if constexpr (NW > 1) {
