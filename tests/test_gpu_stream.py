@@ -263,12 +263,14 @@ def test_random_shapes_k_and_row_kinds_on_whatever_route_they_take(ops, seed):
     comparison of the library's own choice of kernels with the kernels rows.path = 1 selects and
     with the oracle: the shapes between the ones the other tests name (this is how the rows of
     one repeated value and three peaks, and a row that overflowed a wave's stage twice, were found).
-    The kind "flat_with_peaks" is not drawn here: with dozens of peaks per thousand copies most
-    waves of the scan kernel hold a peak beside the copies, the copies' terms are then approximate
-    ones with one common error, and single rows of that kind measure 3 ulp against the oracle
-    ([n = 20001, k = 16] under seed 23) -- the one known excess over the 2-ulp bar; the kind is
-    tested at the shapes of test_rows_of_equal_and_clustered_values_on_every_route and with few
-    peaks in test_rows_of_one_repeated_value_and_a_few_peaks."""
+    The kind "flat_with_peaks" is not drawn here: a flat row with dozens of peaks per thousand
+    copies ([n = 20001, k = 16] under seed 23) measured 3 ulp until the scan kernel counted the
+    copies of its waves' smallest value apart -- 1 ulp since on the library's own route -- and
+    still measures 3 ulp on the chunk + merge kernels over several chunks, which this comparison
+    forces with rows.path = 1 (their wave records have no room for the count): the one known
+    excess over the 2-ulp bar.  The kind is tested on the library's routes in
+    test_rows_of_equal_and_clustered_values_on_every_route and
+    test_rows_of_one_repeated_value_and_a_few_peaks."""
     from vkop_amd import capi
     rng = np.random.default_rng(seed)
     kinds_all = [t for t in dict.fromkeys(KINDS + TIE_KINDS + WALK_KINDS) if t != "flat_with_peaks"]

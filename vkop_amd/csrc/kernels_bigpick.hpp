@@ -531,12 +531,15 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
             const uint32_t b = idx / per, off = idx - b * per;
             const uint32_t sp = b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;  // the scan wave that summed it
             const float ref = __uint_as_float(static_cast<uint32_t>(recs[2 * sp + 1]));
+            const uint64_t apart = ws.recs2[static_cast<size_t>(row) * waves + sp];  // the value that wave counted apart
+            const bool copy = static_cast<uint32_t>(apart) != 0u && xv == __uint_as_float(static_cast<uint32_t>(apart >> 32));
             const float term = softmax_term(xv, M);
             // what the element should contribute, exp(fl(x - M)), minus what its wave
-            // added for it, fast_term(x, ref) * exp(ref - M)
-            const double cr = static_cast<double>(term) -
-                              static_cast<double>(fast_term(xv, ref)) *
-                                  sum_rescale(__longlong_as_double(static_cast<long long>(recs[2 * sp])), ref, M);
+            // added for it, fast_term(x, ref) * exp(ref - M) (a copy went in with this very term)
+            const double cr = copy ? 0.0
+                                   : static_cast<double>(term) -
+                                         static_cast<double>(fast_term(xv, ref)) *
+                                             sum_rescale(__longlong_as_double(static_cast<long long>(recs[2 * sp])), ref, M);
             if (cr > -1.0 && cr < 1.0) fix += static_cast<long long>(cr * kBigPickFixUnit);  // (anything else: the row's sum is not finite)
             lterm[t] = term;
         }
@@ -590,6 +593,10 @@ __global__ __launch_bounds__(kBigPickThreads) void bigpick_gather_kernel(const T
                 const double sv = __longlong_as_double(static_cast<long long>(recs[2 * w]));
                 const float ref = __uint_as_float(static_cast<uint32_t>(recs[2 * w + 1]));
                 if (sv != 0.0) acc += sv * sum_rescale(sv, ref, M);
+                const uint64_t apart = ws.recs2[static_cast<size_t>(row) * waves + w];
+                if (static_cast<uint32_t>(apart) != 0u)
+                    acc += static_cast<double>(static_cast<uint32_t>(apart)) *
+                           static_cast<double>(softmax_term(__uint_as_float(static_cast<uint32_t>(apart >> 32)), M));
             }
             const double s_base = block_sum_fast<NT>(acc, dscratch);
             if (tid == 0) {

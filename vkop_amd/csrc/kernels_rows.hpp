@@ -273,6 +273,7 @@ struct RowsShared {  // merge phase
     double corr[kFastMaxK + 1];
     double scale[kMergeWavesMax];  // exp(ref - M) per wave partial
     float ref[kMergeWavesMax];
+    float x0[kMergeWavesMax];        // the value whose copies the wave's sum leaves out (counted apart); NaN: none
     uint32_t cnt[kMergeChunksMax];   // live candidates per chunk
     uint32_t cthr[kMergeChunksMax];  // threshold per chunk: the chunk's elements at or above it are candidates
     uint32_t pkey[kFastMaxK + 1];    // order key of the logit, by rank
@@ -744,8 +745,10 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
                 const float xv = ordered_to_float(key);
                 // what the element should contribute, exp(fl(x - M)), minus what
                 // its wave added for it, fast_term(x, ref) * exp(ref - M)
+                // (a copy of the value its wave counted apart went in with this very term)
                 term = softmax_term(xv, M);
-                cr = static_cast<double>(term) - static_cast<double>(fast_term_as<REDUCED>(xv, sh.ref[sp])) * sh.scale[sp];
+                cr = (xv == sh.x0[sp]) ? 0.0
+                                       : static_cast<double>(term) - static_cast<double>(fast_term_as<REDUCED>(xv, sh.ref[sp])) * sh.scale[sp];
             }
             sh.prob[r] = term;  // scaled to a probability below
             sh.corr[r] = cr;
@@ -905,6 +908,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         p0.ref = __uint_as_float(static_cast<uint32_t>(rm_bits));
         p0.m = __uint_as_float(static_cast<uint32_t>(rm_bits >> 32));
         sh.ref[tid] = p0.ref;
+        sh.x0[tid] = __uint_as_float(0x7FC00000u);  // (the chunk kernel's sums leave nothing out)
     }
     if (tid < G) {
         sh.cnt[tid] = static_cast<uint32_t>(cm < cap ? cm : cap);

@@ -28,6 +28,8 @@ struct ScanWorkspace {
                        // ones if the block holds a NaN); block b = elements b * 16 * vector width ... of the row
     uint64_t *recs;    // [rows][G][kScanWaves][2]: sum of exp(x - ref) over the wave's elements (double bits); ref
                        // (low half) and the wave's maximum (high half) as float bits
+    uint64_t *recs2;   // [rows][G][kScanWaves]: the value whose copies the wave counted apart (float bits, high half)
+                       // and how many it found (low half; 0: none): its sum leaves them out
     uint32_t blocks;   // blocks per row: ceil(n / (16 * vector width))
     uint32_t *bmin;    // null, or (WITH_MIN) [rows][blocks]: order key of the block's minimum (NaN dropped; the key
                        // of -inf for a block that reaches past the row's end or holds -inf)
@@ -87,6 +89,14 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
         };
         float ref = 0.f;
         float wm0 = -INFINITY;  // the maximum of the wave's first vectors
+        // The copies of one value -- the smallest finite element of the wave's first vectors: a
+        // value that fills a row is usually its floor and turns up at once -- are counted and left
+        // out of the sum: every copy has the same term, so its error (the hardware exponential's, and
+        // the rounding of x - M that the definition asks for and a pass that does not know M cannot
+        // make) would enter the sum once per copy; the kernel that knows M adds
+        // exp_accurate(fl(x0 - M)) for each of them instead.
+        float x0 = __uint_as_float(0x7FC00000u);  // (NaN: equal to nothing)
+        uint32_t ncopy = 0;
         double acc = 0.0;  // every term is added in double: a dominant term must not swallow what follows it
         static_for<0, V>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
@@ -110,9 +120,17 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                     // NaN, which must survive -- never -inf - -inf)
                     wm0 = wave_max_f32_uniform(vm);
                     ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
+                    float lowest = INFINITY;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) lowest = (xv[c] > -INFINITY) ? fminf(lowest, xv[c]) : lowest;
+                    lowest = -wave_max_f32_uniform(-lowest);
+                    if (lowest < INFINITY) x0 = lowest;
                 }
 #pragma unroll
-                for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(xv[c], ref));
+                for (int c = 0; c < VEC; c++) {
+                    acc += static_cast<double>(fast_term(xv[c], ref));
+                    ncopy += (xv[c] == x0) ? 1u : 0u;
+                }
                 // the sum so far exists HERE, under the loads still in flight (or the
                 // compiler moves all of it behind the last load)
                 asm volatile("" : "+v"(acc));
@@ -160,6 +178,8 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
         // ---- the wave's record ---------------------------------------------------------------
         if constexpr (SOFTMAX) {
             const float wm = wave_max_f32_uniform(bm);
+            // (every copy added the same float: taking them out again is exact to the sum's own rounding)
+            if (ncopy != 0u) acc -= static_cast<double>(ncopy) * static_cast<double>(fast_term(x0, ref));
             double wsum = wave_sum_f64_uniform(acc);
             if (wm - ref > kTermSwitch) {  // wave-uniform
                 // an element well above the reference: its fast term is poor (or has
@@ -170,29 +190,12 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
 #pragma unroll
                     for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(elem(i_tag, c), ref));
                 });
+                if (ncopy != 0u) acc -= static_cast<double>(ncopy) * static_cast<double>(fast_term(x0, ref));
                 wsum = wave_sum_f64_uniform(acc);
-            } else if (wm == wm0 && wm0 > -INFINITY) {
-                // A wave of equal elements (a flat stretch of the row): every lane's sum is its
-                // number of elements times the one term -- terms never exceed the maximum's, so
-                // nothing else adds up to that.  Its record says so exactly: the count as the sum,
-                // the value itself as the reference.  Whoever combines the records counts
-                // exp_accurate(fl(value - M)) for each of them, as the sum is defined, instead of
-                // a hardware exponential of value - reference times an exponential of
-                // reference - M, whose error -- the same for every copy -- a row made of one
-                // repeated value and a few peaks carried into its probabilities (up to 7 ulp).
-                uint32_t mine_n = 0;
-                static_for<0, V>([&](auto i_tag) {
-                    constexpr int i = decltype(i_tag)::value;
-                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-#pragma unroll
-                    for (int c = 0; c < VEC; c++) mine_n += (FULL || in_range(ALIGNED ? e0 : e0 + static_cast<uint32_t>(c))) ? 1u : 0u;
-                });
-                const bool flat = acc == static_cast<double>(mine_n) * static_cast<double>(fast_term(wm0, ref));
-                if (__ballot(!flat) == 0ull) {
-                    wsum = FULL ? static_cast<double>(kWave * V * VEC) : wave_sum_f64_uniform(static_cast<double>(mine_n));
-                    ref = wm0;
-                }
             }
+            const uint32_t copies = static_cast<uint32_t>(wave_sum_f64_uniform(static_cast<double>(ncopy)));
+            if (lane == 0)
+                ws.recs2[static_cast<size_t>(row * G + chunk) * NW + wave] = (static_cast<uint64_t>(__float_as_uint(x0)) << 32) | copies;
             if (lane == 0) {
                 uint64_t *record = ws.recs + 2 * (static_cast<size_t>(row * G + chunk) * NW + wave);
                 record[0] = static_cast<uint64_t>(__double_as_longlong(wsum));
@@ -267,10 +270,11 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // (never a branch around a load: out-of-range threads re-read entry 0)
     const uint64_t *recs = ws.recs + 2 * static_cast<size_t>(row) * waves;
     const uint32_t wq = tid < waves ? tid : 0u;
-    uint64_t s_bits = 0, rm_bits = 0;
+    uint64_t s_bits = 0, rm_bits = 0, c_bits = 0;
     if constexpr (SOFTMAX) {
         s_bits = recs[2 * wq];
         rm_bits = recs[2 * wq + 1];
+        c_bits = ws.recs2[static_cast<size_t>(row) * waves + wq];
     }
     const uint32_t blocks = ws.blocks;
     const uint32_t *bmax = ws.bmax + static_cast<size_t>(row) * blocks;
@@ -292,7 +296,13 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             p0.ref = __uint_as_float(static_cast<uint32_t>(rm_bits));
             p0.m = __uint_as_float(static_cast<uint32_t>(rm_bits >> 32));
             sh.ref[tid] = p0.ref;
+            sh.x0[tid] = static_cast<uint32_t>(c_bits) != 0u ? __uint_as_float(static_cast<uint32_t>(c_bits >> 32)) : __uint_as_float(0x7FC00000u);
         }
+        // the copies the wave counted apart: each counts exp_accurate(fl(x0 - M)), as the sum is defined
+        auto copies_term = [&](float m) -> double {
+            const uint32_t cn = tid < waves ? static_cast<uint32_t>(c_bits) : 0u;
+            return cn != 0u ? static_cast<double>(cn) * static_cast<double>(softmax_term(__uint_as_float(static_cast<uint32_t>(c_bits >> 32)), m)) : 0.0;
+        };
         // With at most 64 wave records (one per lane of wave 0) that wave alone combines
         // them, by cross-lane steps, while the others go on to the threshold; the
         // results are published by the barrier there.
@@ -305,6 +315,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                     sh.scale[tid] = sc;
                     if (p0.s != 0.0) acc = p0.s * sc;
                 }
+                acc += copies_term(m);
                 const double total = wave_sum_f64_uniform(acc);
                 if (lane == 0) {
                     sh.row_max = m;
@@ -319,6 +330,7 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                 sh.scale[tid] = sc;
                 if (p0.s != 0.0) acc = p0.s * sc;
             }
+            acc += copies_term(m);
             const double total = block_sum_fast<NT>(acc, dscratch);  // (barrier: sh.scale is published)
             if (tid == 0) {
                 sh.row_max = m;

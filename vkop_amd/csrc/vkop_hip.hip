@@ -615,7 +615,7 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
         l.bmax = off;
         off += align_up(lines * sc.blocks * sizeof(uint32_t));
         l.recs = off;
-        off += align_up(lines * sc.g * vkop::kScanWaves * 2 * sizeof(uint64_t));
+        off += align_up(lines * sc.g * vkop::kScanWaves * 3 * sizeof(uint64_t));  // (two words a wave, then the waves' third words)
         if (sc.g2 != 0) {
             l.bmin = off;
             off += align_up(lines * sc.blocks * sizeof(uint32_t));
@@ -715,6 +715,7 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.top_p = top_p;
     a.ws.bmax = reinterpret_cast<uint32_t *>(base + l.bmax);
     a.ws.recs = reinterpret_cast<uint64_t *>(base + l.recs);
+    a.ws.recs2 = a.ws.recs + 2 * static_cast<size_t>(v.g.outer) * c.g * vkop::kScanWaves;
     a.ws.blocks = c.blocks;
     a.ws.bmin = nullptr;
     a.ws.zero = nullptr;
