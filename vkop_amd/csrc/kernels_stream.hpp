@@ -89,14 +89,15 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
         };
         float ref = 0.f;
         float wm0 = -INFINITY;  // the maximum of the wave's first vectors
-        // The copies of one value -- the smallest finite element of the wave's first vectors: a
-        // value that fills a row is usually its floor and turns up at once -- are counted and left
+        // The copies of one value -- the wave's first element, where half of the lanes' first
+        // elements equal it: a value that fills a row turns up at once -- are counted and left
         // out of the sum: every copy has the same term, so its error (the hardware exponential's, and
         // the rounding of x - M that the definition asks for and a pass that does not know M cannot
         // make) would enter the sum once per copy; the kernel that knows M adds
         // exp_accurate(fl(x0 - M)) for each of them instead.
         float x0 = __uint_as_float(0x7FC00000u);  // (NaN: equal to nothing)
         uint32_t ncopy = 0;
+        bool counting = false;
         double acc = 0.0;  // every term is added in double: a dominant term must not swallow what follows it
         static_for<0, V>([&](auto i_tag) {
             constexpr int i = decltype(i_tag)::value;
@@ -120,17 +121,15 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                     // NaN, which must survive -- never -inf - -inf)
                     wm0 = wave_max_f32_uniform(vm);
                     ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
-                    float lowest = INFINITY;
-#pragma unroll
-                    for (int c = 0; c < VEC; c++) lowest = (xv[c] > -INFINITY) ? fminf(lowest, xv[c]) : lowest;
-                    lowest = -wave_max_f32_uniform(-lowest);
-                    if (lowest < INFINITY) x0 = lowest;
+                    // (the wave's very first element, if most lanes' first elements equal it: on
+                    // spread-out rows none does, and nothing below is done for it)
+                    const float first = __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(__float_as_uint(xv[0])))));
+                    const bool mine = xv[0] == first && first > -INFINITY && first < INFINITY;
+                    x0 = first;
+                    counting = __popcll(__ballot(mine)) >= kWave / 2;
                 }
 #pragma unroll
-                for (int c = 0; c < VEC; c++) {
-                    acc += static_cast<double>(fast_term(xv[c], ref));
-                    ncopy += (xv[c] == x0) ? 1u : 0u;
-                }
+                for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term(xv[c], ref));
                 // the sum so far exists HERE, under the loads still in flight (or the
                 // compiler moves all of it behind the last load)
                 asm volatile("" : "+v"(acc));
@@ -178,6 +177,12 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
         // ---- the wave's record ---------------------------------------------------------------
         if constexpr (SOFTMAX) {
             const float wm = wave_max_f32_uniform(bm);
+            if (counting) {  // (wave-uniform; everything is still in registers)
+                static_for<0, V>([&](auto i_tag) {
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) ncopy += (elem(i_tag, c) == x0) ? 1u : 0u;
+                });
+            }
             // (every copy added the same float: taking them out again is exact to the sum's own rounding)
             if (ncopy != 0u) acc -= static_cast<double>(ncopy) * static_cast<double>(fast_term(x0, ref));
             double wsum = wave_sum_f64_uniform(acc);
@@ -193,7 +198,7 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                 if (ncopy != 0u) acc -= static_cast<double>(ncopy) * static_cast<double>(fast_term(x0, ref));
                 wsum = wave_sum_f64_uniform(acc);
             }
-            const uint32_t copies = static_cast<uint32_t>(wave_sum_f64_uniform(static_cast<double>(ncopy)));
+            const uint32_t copies = counting ? static_cast<uint32_t>(wave_sum_f64_uniform(static_cast<double>(ncopy))) : 0u;
             if (lane == 0)
                 ws.recs2[static_cast<size_t>(row * G + chunk) * NW + wave] = (static_cast<uint64_t>(__float_as_uint(x0)) << 32) | copies;
             if (lane == 0) {
