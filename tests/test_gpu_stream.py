@@ -265,7 +265,7 @@ def test_random_shapes_k_and_row_kinds_on_whatever_route_they_take(ops, seed):
     one repeated value and three peaks, and a row that overflowed a wave's stage twice, were found).
     The kind "flat_with_peaks" is not drawn here: a flat row with dozens of peaks per thousand
     copies ([n = 20001, k = 16] under seed 23) measured 3 ulp until the scan kernel counted the
-    copies of its waves' smallest value apart -- 1 ulp since on the library's own route -- and
+    copies of a value that fills its waves apart -- 1 ulp since on the library's own route -- and
     still measures 3 ulp on the chunk + merge kernels over several chunks, which this comparison
     forces with rows.path = 1 (their wave records have no room for the count): the one known
     excess over the 2-ulp bar.  The kind is tested on the library's routes in
