@@ -114,6 +114,20 @@ __device__ __forceinline__ double wave_sum_f64_uniform(double v) {
     };
     return (row(0) + row(16)) + (row(32) + row(48));
 }
+// Inclusive prefix sum over the wave's lanes: four shifts inside each row of 16 lanes, then the
+// last lane of row 0 (rows 0 and 1) broadcast into the rows above (lanes without a source add 0).
+__device__ __forceinline__ uint32_t wave_inclusive_sum_u32(uint32_t v) {
+#define VKOP_DPP_ADD(ctrl, rows) \
+    v += static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), ctrl, rows, 0xF, false))
+    VKOP_DPP_ADD(0x111, 0xF);  // row_shr:1
+    VKOP_DPP_ADD(0x112, 0xF);  // row_shr:2
+    VKOP_DPP_ADD(0x114, 0xF);  // row_shr:4
+    VKOP_DPP_ADD(0x118, 0xF);  // row_shr:8
+    VKOP_DPP_ADD(0x142, 0xA);  // row_bcast:15 into rows 1 and 3
+    VKOP_DPP_ADD(0x143, 0xC);  // row_bcast:31 into rows 2 and 3
+#undef VKOP_DPP_ADD
+    return v;
+}
 #undef VKOP_DPP_U32
 
 // Bijective order-preserving float <-> uint32 (no NaN / -0 canonicalisation).
@@ -286,6 +300,7 @@ struct RowsShared {  // merge phase
     uint32_t thr;
     uint32_t count;
     uint32_t flag;
+    uint32_t wave_overflow;          // pick kernel: a wave found more blocks to read again than its share of the list holds
     double total;
 };
 
@@ -351,22 +366,25 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
     const uint32_t tid = threadIdx.x;
     if (C == 0) return;
     if (C <= NT) {
-        const uint32_t parts = NT / C;                  // >= 1
-        const uint32_t span = (C + parts - 1) / parts;  // entries per part
-        const uint32_t part = tid / C, i = tid - part * C;
-        if (part < parts) {
+        // the threads form NT / P groups (P: the power of two at or above C), each candidate has a
+        // thread in every group, and a group takes one part of the list (shifts only: a division
+        // by a number known at run time is three dozen dependent instructions)
+        const uint32_t pshift = C > 1u ? 32u - static_cast<uint32_t>(__clz(C - 1u)) : 0u;
+        const uint32_t parts = static_cast<uint32_t>(NT) >> pshift;                   // >= 1, a power of two
+        const uint32_t span = (C + parts - 1u) >> (31u - static_cast<uint32_t>(__clz(parts)));  // entries per part
+        const uint32_t part = tid >> pshift, i = tid & ((1u << pshift) - 1u);
+        if (i < C) {
             const uint64_t mine = sh.cand[i];
             const uint32_t j0 = part * span, j1 = min(j0 + span, C);
             uint32_t cnt = 0;
             uint32_t j = j0;
-            for (; j + 8 <= j1; j += 8) {  // eight independent reads in flight
+            for (; j < j1; j += 8) {  // eight independent reads in flight (past the part's end: entry 0, not counted)
                 uint64_t o[8];
 #pragma unroll
-                for (int u = 0; u < 8; u++) o[u] = sh.cand[j + u];
+                for (int u = 0; u < 8; u++) o[u] = sh.cand[j + u < j1 ? j + u : 0u];
 #pragma unroll
-                for (int u = 0; u < 8; u++) cnt += (o[u] > mine) ? 1u : 0u;
+                for (int u = 0; u < 8; u++) cnt += (j + u < j1 && o[u] > mine) ? 1u : 0u;
             }
-            for (; j < j1; j++) cnt += (sh.cand[j] > mine) ? 1u : 0u;
             if (parts > 1) {
                 if (cnt) atomicAdd(&sh.rank[i], cnt);
             } else {
@@ -381,6 +399,31 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
             sh.rank[i] = cnt;
         }
     }
+    __syncthreads();
+}
+
+// The same for a list that is followed by zeros up to the power of two P at or above C (a
+// zero ranks behind every candidate), 64 <= P <= NT, sh.rank[0..P) zero: every thread takes
+// P * P / NT entries, two per LDS read, without a test per entry.  Ends with a barrier.
+template <int NT> __device__ __forceinline__ void block_rank_padded(RowsShared &sh, uint32_t C) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t pshift = 32u - static_cast<uint32_t>(__clz(C - 1u));  // (C > 32)
+    const uint32_t span = (1u << pshift << pshift) / static_cast<uint32_t>(NT);  // entries per thread: 8, 32, 128, 512
+    const uint32_t i = tid & ((1u << pshift) - 1u);
+    const uint64_t mine = sh.cand[i];
+    const uint4 *src = reinterpret_cast<const uint4 *>(sh.cand + (tid >> pshift) * span);
+    uint32_t cnt = 0;
+    for (uint32_t j = 0; j < span / 2; j += 4) {  // four reads of two entries in flight
+        uint4 o[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) o[u] = src[j + u];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            cnt += (((static_cast<uint64_t>(o[u].y) << 32) | o[u].x) > mine) ? 1u : 0u;
+            cnt += (((static_cast<uint64_t>(o[u].w) << 32) | o[u].z) > mine) ? 1u : 0u;
+        }
+    }
+    if (cnt) atomicAdd(&sh.rank[i], cnt);
     __syncthreads();
 }
 
@@ -725,7 +768,9 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1);
     uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
     // ---- E. exact ranks; accurate terms for the ranked elements ----------------
+    BPS(30);
     block_rank<NT>(sh, C2);
+    BPS(31);
     // only the k+1 largest are used from here on: which other candidates
     // passed the threshold depends on the order the chunks stored theirs in,
     // and nothing that reaches the output may
@@ -755,6 +800,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
         }
     }
     __syncthreads();
+    BPS(32);
     // every wave adds up the corrections itself (same values, same tree, same
     // result, run after run), which saves a trip through LDS and a barrier
     double csum = 0.0;
@@ -766,6 +812,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
         if (tid <= kk && tid < ranked)
             sh.prob[tid] = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[tid]) * rinv));
         __syncthreads();
+        BPS(33);
         // Probabilities are non-increasing along the rank order, so equal
         // ones are neighbours.  A tie that reaches past the k-th place is
         // settled by index over every element of the row with that
@@ -789,6 +836,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
         fill_group_by_scan<T, NT, false>(sh.scan_counts, rowp, ov, oi, n, C2, kk, kKeyNegInf, kKeyNegInf, 0.f);
     }
 
+    BPS(34);
     const uint32_t plain = min(kk, tie_g0);  // ranks at or after tie_g0 were written by settle_tie
     for (uint32_t r = tid; r < plain; r += NT) {
         const uint32_t idx = sh.pidx[r];

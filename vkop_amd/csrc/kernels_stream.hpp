@@ -19,6 +19,33 @@
 
 namespace vkop {
 
+// Debug builds only (-DVKOP_STAMPS): a log of (kernel, workspace, workgroup, entry and exit clock) records,
+// appended by some workgroups as they leave, for a timeline of calls that overlap.
+#ifdef VKOP_STAMPS
+struct TimelineRec {
+    unsigned long long tag, t0, t1;
+};
+constexpr unsigned kTimelineCap = 1u << 20;
+static __device__ TimelineRec g_timeline[kTimelineCap];
+static __device__ unsigned g_timeline_n;
+#define VKOP_TL_BEGIN() const unsigned long long tl_t0 = wall_clock64()
+#define VKOP_TL_END(kind, wsptr, logged)                                                                            \
+    do {                                                                                                            \
+        if (threadIdx.x == 0 && (logged)) {                                                                         \
+            const unsigned long long tl_t1 = wall_clock64();                                                        \
+            const unsigned tl_i = atomicAdd(&g_timeline_n, 1u);                                                     \
+            if (tl_i < kTimelineCap)                                                                                \
+                g_timeline[tl_i] = TimelineRec{(static_cast<unsigned long long>(kind) << 63) |                      \
+                                                   (static_cast<unsigned long long>(blockIdx.x & 0xFFFFu) << 40) |   \
+                                                   ((reinterpret_cast<unsigned long long>(wsptr) >> 8) & 0xFFFFFFFFFFull), \
+                                               tl_t0, tl_t1};                                                       \
+        }                                                                                                           \
+    } while (0)
+#else
+#define VKOP_TL_BEGIN() do { } while (0)
+#define VKOP_TL_END(kind, wsptr, logged) do { } while (0)
+#endif
+
 constexpr int kScanThreads = 256;
 constexpr int kScanWaves = kScanThreads / kWave;
 constexpr int kBlockLanes = 16;  // lanes (vectors) per block: one row of a wave's cross-lane network
@@ -46,6 +73,7 @@ struct ScanWorkspace {
 template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED = false, bool WITH_MIN = false>
 __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__restrict__ in, uint32_t n, uint32_t G,
                                                                  ScanWorkspace ws, float scale = 1.f) {
+    VKOP_TL_BEGIN();
     constexpr int NT = kScanThreads, NW = kScanWaves;
     constexpr int VEC = Vec128<T>::N;
     constexpr uint32_t per = static_cast<uint32_t>(NT) * V * VEC;
@@ -63,8 +91,8 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
     // all loads in flight (never a branch around a load: out-of-chunk lanes read the
     // row's first element(s) instead and are masked where the data is used)
     Vec128<T> q[V];
-#pragma unroll
-    for (int i = 0; i < V; i++) {
+    auto issue_load = [&](auto i_tag) __attribute__((always_inline)) {
+        constexpr int i = decltype(i_tag)::value;
         const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
         q[i].v = make_uint4(0, 0, 0, 0);
         if constexpr (ALIGNED) {
@@ -73,7 +101,8 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
 #pragma unroll
             for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < c1 ? e0 + c : 0u));
         }
-    }
+    };
+    static_for<0, V>(issue_load);
 
     // The rest exists twice: for a chunk that fills every lane of every vector (no
     // masking anywhere) and for a ragged one.
@@ -210,13 +239,17 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
     };
     if (c1 - c0 == per) body(std::true_type{});
     else body(std::false_type{});
+    VKOP_TL_END(0, ws.bmax, blockIdx.x % 16u == 0u || blockIdx.x + 48u >= gridDim.x);
 }
 
 constexpr int kPickHitCap = 1024;  // blocks one gather reads again
 
+constexpr int kPickThreads = 512;
 struct PickShared {
     RowsShared fast;
-    uint32_t hits[kPickHitCap];  // the blocks to read again
+    uint32_t hits[kPickHitCap];  // the blocks to read again (the first gather: a part per wave)
+    uint4 stage_v[kPickThreads / kWave][kWave];     // per wave: the vectors that hold an element at or above the threshold ...
+    uint32_t stage_e[kPickThreads / kWave][kWave];  // ... and the index of their first element
 };
 union PickSharedUnion {
     PickShared pick;
@@ -244,11 +277,10 @@ union PickSharedUnion {
 // with the tied interval's lower end (settle_tie); what that cannot hold (rows full of
 // equal values) goes to the scan from the row's start or, from D, to the exact radix
 // select over the whole row.
-constexpr int kPickThreads = 512;
-
 // scale: as in the scan kernel (1 when that ran unscaled); counts (softmax variant,
 // may be null): per row the nucleus cut of its result for top_p (finish_row).
-template <typename T, bool SOFTMAX, bool ALIGNED, int GE, int NT = kPickThreads>
+// SCALED false: scale is 1, and the common case does without the multiplications.
+template <typename T, bool SOFTMAX, bool ALIGNED, int GE, bool SCALED = true, int NT = kPickThreads>
 __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                        int32_t *__restrict__ indices, uint32_t n, uint32_t k, uint32_t G,
                                                        uint32_t per, ScanWorkspace ws, float scale = 1.f,
@@ -270,7 +302,14 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     const uint32_t want = k + 1;
     const uint32_t kk = min(k, n);
     const uint32_t waves = G * kScanWaves;
+    // (a short chain of dependent steps per row, often beside the streaming kernel of another call on the same
+    // CU, whose waves issue all the time: this kernel's waves go first)
+    __builtin_amdgcn_s_setprio(3);
+    VKOP_TL_BEGIN();
     BPS(14);
+#ifdef VKOP_STAMPS
+    if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[60] = clock64();
+#endif
     // ---- A. everything the kernel reads first, in one round trip --------------------
     // (never a branch around a load: out-of-range threads re-read entry 0)
     const uint64_t *recs = ws.recs + 2 * static_cast<size_t>(row) * waves;
@@ -291,10 +330,20 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     }
 
     // ---- B. the row's maximum and sum from the wave partials --------------------------
+    // (runs while the blocks that are read again are on their way: nothing before the ranking needs it)
     BPS(8);
     for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;  // for block_rank, barriers away
-    if (tid == 0) sh.count = 0;
-    if constexpr (SOFTMAX) {
+    sh.cand[tid] = 0;  // (the list the waves make below ends in zeros: block_rank_padded)
+    auto times_scale = [&](float x) {
+        if constexpr (SCALED) return scaled(x, scale);
+        else return x;
+    };
+    if (tid == 0) {
+        sh.count = 0;
+        sh.wave_overflow = 0;
+    }
+    auto combine_records = [&]() __attribute__((always_inline)) {
+      if constexpr (SOFTMAX) {
         SumPartial p0{0.0, 0.f, -INFINITY};
         if (tid < waves) {
             p0.s = __longlong_as_double(static_cast<long long>(s_bits));
@@ -342,7 +391,8 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                 sh.total = total;
             }
         }
-    }
+      }
+    };
 
     // ---- C. a value that k+1 block maxima reach ---------------------------------------------
     BPS(9);
@@ -367,9 +417,13 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         const uint32_t quota = (want + NW - 1) / NW;
         uint32_t mine_q = 0;
         if (by_quota && quota <= 32u) {
-            for (int bit = 31; bit > 13; bit--) {
-                const uint32_t trial = mine_q | (1u << bit);
-                if (static_cast<uint32_t>(__popcll(__ballot(mine_max >= trial))) >= quota) mine_q = trial;
+            // two bits a step (three trial values counted side by side): the steps depend on each other
+            for (int bit = 30; bit > 13; bit -= 2) {
+                const uint32_t t1 = mine_q | (1u << bit), t2 = mine_q | (2u << bit), t3 = mine_q | (3u << bit);
+                const uint32_t c1 = static_cast<uint32_t>(__popcll(__ballot(mine_max >= t1)));
+                const uint32_t c2 = static_cast<uint32_t>(__popcll(__ballot(mine_max >= t2)));
+                const uint32_t c3 = static_cast<uint32_t>(__popcll(__ballot(mine_max >= t3)));
+                mine_q = c3 >= quota ? t3 : c2 >= quota ? t2 : c1 >= quota ? t1 : mine_q;
             }
         }
         sh.lane_key[tid] = mine_max;
@@ -390,15 +444,252 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     };
     uint32_t thr = threshold_of_thread_maxima(lmk, true);
     BPS(10);
+    // -inf never becomes a candidate: a row with k+1 larger elements does not need it,
+    // and finish_row fills any other row's last places from the row itself
+    thr = max(thr, kKeyNegInf + 1u);
+
+    // ---- D1. the first gather, wave by wave ------------------------------------------------
+    // Every wave reads again ITS threads' blocks that reach thr (a list of its own in LDS: no
+    // workgroup barrier between the threshold and the loads), 16 lanes a block, 2 U loads per
+    // lane in flight (the second U only in a wave with more than 16 such blocks); phase B runs
+    // under them.  A vector that holds an element at or above thr (one in 16 of those read) goes
+    // to the wave's stage in LDS, and one lane per staged vector lists its elements in sh.cand:
+    // a prefix sum over the lanes and one LDS atomic per wave give the places.
+    // A wave with more blocks or vectors than its lists hold only raises sh.wave_overflow: the
+    // workgroup then gathers the general way (below).
+    constexpr uint32_t kWaveHitCap = 2 * U * (kWave / kBlockLanes);  // blocks a wave reads again in one go
+    static_assert(NW * kWaveHitCap <= kPickHitCap, "every wave's list of blocks fits");
+    static_assert(NW <= kPickThreads / kWave, "a stage per wave");
+    {
+        uint32_t wave_n = 0;  // wave-uniform
+#pragma unroll
+        for (int e = 0; e < GE; e++) wave_n += static_cast<uint32_t>(__popcll(__ballot(gk[e] >= thr)));
+        const bool wave_ok = wave_n <= kWaveHitCap;
+        uint32_t *whits = hits + wave * kWaveHitCap;
+        if (wave_ok) {
+            uint32_t pos = 0;
+#pragma unroll
+            for (int e = 0; e < GE; e++) {
+                const bool pass = gk[e] >= thr;
+                const uint64_t mask = __ballot(pass);
+                if (pass) whits[pos + lanes_below(mask)] = static_cast<uint32_t>(e) * NT + tid;
+                pos += static_cast<uint32_t>(__popcll(mask));
+            }
+        }
+        __builtin_amdgcn_wave_barrier();  // (the wave reads its own list: LDS keeps a wave's accesses in order)
+        const uint32_t items = wave_ok ? wave_n * kBlockLanes : 0u;  // one per vector of a block that is read again
+        const float lo_f = ordered_to_float(thr);
+        Vec128<T> r[2 * U];
+        uint32_t e0[2 * U];
+        auto issue = [&](auto u_tag) __attribute__((always_inline)) {
+            constexpr int u = decltype(u_tag)::value;
+            const uint32_t j = static_cast<uint32_t>(u) * kWave + lane;
+            const uint32_t b = whits[j < items ? j / kBlockLanes : 0u];
+            // (a slot past the wave's items reads the row's start and is marked by an index past the row's end)
+            e0[u] = j < items ? b * BE + (j % kBlockLanes) * VEC : 0xFFFFFFFFu;
+            r[u].v = make_uint4(0, 0, 0, 0);
+            if constexpr (ALIGNED) {
+                r[u].load(rowp + (e0[u] < n ? e0[u] : 0u));
+            } else {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) r[u].set(c, load_elem(rowp, e0[u] < n && e0[u] + c < n ? e0[u] + c : 0u));
+            }
+        };
+        static_for<0, U>(issue);
+        const bool second_half = items > static_cast<uint32_t>(U) * kWave;  // wave-uniform
+        if (second_half) static_for<U, 2 * U>(issue);
+        combine_records();
+        // vectors with an element at or above thr -> the wave's stage
+        uint4 *stage_v = smem.pick.stage_v[wave];
+        uint32_t *stage_e = smem.pick.stage_e[wave];
+        uint32_t nv = 0;  // wave-uniform
+        auto sift = [&](auto u_tag) __attribute__((always_inline)) {
+            constexpr int u = decltype(u_tag)::value;
+            float vm = -INFINITY;
+            bool any_nan = false;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const float x = times_scale(r[u].get(c));
+                vm = fmaxf(vm, x);
+                if constexpr (!SOFTMAX) any_nan = any_nan || x != x;
+            }
+            const bool pv = e0[u] < n && (!(vm < lo_f) || any_nan);
+            const uint64_t mask = __ballot(pv);
+            if (mask != 0ull) {
+                const uint32_t slot = nv + lanes_below(mask);
+                if (pv && slot < static_cast<uint32_t>(kWave)) {
+                    stage_v[slot] = r[u].v;
+                    stage_e[slot] = e0[u];
+                }
+                nv += static_cast<uint32_t>(__popcll(mask));
+            }
+        };
+        static_for<0, U>(sift);
+        if (second_half) static_for<U, 2 * U>(sift);
+        __builtin_amdgcn_wave_barrier();
+        if (!wave_ok || nv > static_cast<uint32_t>(kWave)) {
+            if (lane == 0) sh.wave_overflow = 1;
+        } else if (nv != 0u) {
+            // lane l lists the elements of staged vector l
+            Vec128<T> sv;
+            sv.v = stage_v[lane < nv ? lane : 0u];
+            const uint32_t eb = stage_e[lane < nv ? lane : 0u];
+            uint32_t pbits = 0;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                const float x = times_scale(sv.get(c));
+                // (softmax: a NaN never passes, and thr is the key of a number, so the floats compare as the keys do)
+                bool pass;
+                if constexpr (SOFTMAX) pass = x >= lo_f;
+                else pass = order_key(x) >= thr;
+                pass = pass && lane < nv && (ALIGNED || eb + static_cast<uint32_t>(c) < n);
+                pbits |= pass ? (1u << c) : 0u;
+            }
+            const uint32_t mine_n = static_cast<uint32_t>(__popc(pbits));
+            const uint32_t incl = wave_inclusive_sum_u32(mine_n);
+            const uint32_t wave_total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
+            uint32_t base = 0;
+            if (lane == 0) base = atomicAdd(&sh.count, wave_total);
+            base = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(base)));
+            uint32_t at = base + incl - mine_n;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                if (pbits & (1u << c)) {
+                    const float x = times_scale(sv.get(c));
+                    if (at < static_cast<uint32_t>(kFastCap)) sh.cand[at] = composite(order_key(x), eb + static_cast<uint32_t>(c));
+                    at++;
+                }
+            }
+        }
+    }
+    BPS(44);
+    __syncthreads();  // the candidates and phase B's results
+    BPS(11);
     float M = 0.f;
     double s_base = 0.0;
     if constexpr (SOFTMAX) {
         M = sh.row_max;
         s_base = sh.total;
     }
-    // -inf never becomes a candidate: a row with k+1 larger elements does not need it,
-    // and finish_row fills any other row's last places from the row itself
-    thr = max(thr, kKeyNegInf + 1u);
+    const uint32_t per_shift = 31u - static_cast<uint32_t>(__clz(per));
+    // the scan-kernel wave that summed element idx (per = 256 * V vectors: a power of two)
+    auto wave_of = [&](uint32_t idx) {
+        const uint32_t b = idx >> per_shift, off = idx & (per - 1u);
+        return b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;
+    };
+
+    // ---- E1. the common case to its end ---------------------------------------------------------
+    // Every wave listed its candidates, they are at least k+1 and a thread can take one each, and
+    // the row's sum is a positive number: ranks, accurate terms for the k+1 first, probabilities.
+    // Equal probabilities among the k+1 (in order by index, and across the k-th place a matter of
+    // the whole row) leave it to the general code below, as does everything else.
+    {
+        const uint32_t C2 = sh.count;
+        bool common = sh.wave_overflow == 0u && C2 >= want && C2 <= static_cast<uint32_t>(NT) && kk == k;
+        if constexpr (SOFTMAX) common = common && s_base > 0.0 && s_base < static_cast<double>(INFINITY) && M > -INFINITY && M < INFINITY;
+        if (__builtin_expect(common, 1)) {
+            // the candidate's own part first (its wave's record, its accurate term), then its share of the ranking
+            uint64_t mine = 0;
+            float term = 0.f;
+            double cr = 0.0;
+            if (tid < C2) {
+                mine = sh.cand[tid];
+                if constexpr (SOFTMAX) {
+                    const uint32_t key = static_cast<uint32_t>(mine >> 32);
+                    const uint32_t sp = wave_of(composite_index(mine));
+                    const float xv = ordered_to_float(key);
+                    // what the element should contribute, exp(fl(x - M)), minus what its wave added for it,
+                    // fast_term(x, ref) * exp(ref - M) (a copy of the value its wave counted apart went in with this very term)
+                    term = softmax_term(xv, M);
+                    cr = (xv == sh.x0[sp]) ? 0.0 : static_cast<double>(term) - static_cast<double>(fast_term(xv, sh.ref[sp])) * sh.scale[sp];
+                }
+            }
+            BPS(30);
+            if (C2 > 32u) block_rank_padded<NT>(sh, C2);  // (both end with a barrier)
+            else block_rank<NT>(sh, C2);
+            BPS(31);
+            if (tid < C2) {
+                const uint32_t rk = sh.rank[tid];
+                if (rk < want) {
+                    sh.pidx[rk] = composite_index(mine);
+                    sh.pkey[rk] = static_cast<uint32_t>(mine >> 32);
+                    sh.prob[rk] = term;
+                    sh.corr[rk] = cr;
+                }
+            }
+            __syncthreads();
+            BPS(32);
+            // every wave works the rest out for itself: the same values in the same order, so every
+            // wave decides alike whether the row is done, and no barrier is needed for that
+            bool tie = false;
+            if constexpr (SOFTMAX) {
+                double csum = 0.0;
+                for (uint32_t r = lane; r < want; r += kWave) csum += sh.corr[r];
+                const double rinv = 1.0 / (s_base + wave_sum_f64_uniform(csum));
+                float p_first = 0.f;  // lane l of the first 64 ranks: its probability
+                for (uint32_t base = 0; base < k; base += kWave) {
+                    const uint32_t r = base + lane;  // ranks r and r + 1 <= k
+                    const float p0 = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r : 0u]) * rinv));
+                    const float p1 = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r + 1u : 0u]) * rinv));
+                    tie = tie || (r < k && p0 == p1);
+                    if (base == 0) p_first = p0;
+                }
+                tie = __ballot(tie) != 0ull;
+                if (!tie) {
+                    // (the waves take the ranks 64 at a time, in turn)
+                    for (uint32_t base = wave * kWave; base < k; base += NW * kWave) {
+                        const uint32_t r = base + lane;
+                        const float p0 = base == 0 ? p_first
+                                                   : round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r : 0u]) * rinv));
+                        if (r < k) {
+                            store_elem(ov, r, p0);
+                            oi[r] = static_cast<int32_t>(sh.pidx[r]);
+                        }
+                    }
+                }
+                if (!tie && counts != nullptr && wave == 0) {
+                    // the nucleus cut: the stored values walked in order through the lanes, as topp_count_kernel does
+                    float sum = 0.f;
+                    uint32_t count = k;
+                    for (uint32_t base = 0; base < k && count == k; base += kWave) {
+                        const uint32_t r = base + lane;
+                        const float v = base == 0 ? p_first
+                                                  : round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r : 0u]) * rinv));
+                        const uint32_t m = min(static_cast<uint32_t>(kWave), k - base);
+                        for (uint32_t j = 0; j < m; j++) {
+                            sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(
+                                                     __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
+                            if (sum >= top_p) {
+                                count = base + j + 1;
+                                break;
+                            }
+                        }
+                    }
+                    if (lane == 0) counts[row] = static_cast<int32_t>(count);
+                }
+            } else {
+                // values are bit copies of the elements: the key gives the bits back, except for a zero (either sign) and a NaN
+                for (uint32_t r = tid; r < k; r += NT) {
+                    const uint32_t key = sh.pkey[r], idx = sh.pidx[r];
+                    if (key == 0x80000000u || key == 0xFFFFFFFFu) ov[r] = rowp[idx];
+                    else store_elem(ov, r, ordered_to_float(key));
+                    oi[r] = static_cast<int32_t>(idx);
+                }
+            }
+            BPS(13);
+#ifdef VKOP_STAMPS
+            if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[61] = clock64();
+#endif
+            VKOP_TL_END(1, ws.bmax, true);
+            if (__builtin_expect(!tie, 1)) return;
+            // (equal probabilities: what was stored is written again below, in its final order)
+        }
+        // the general code starts from an empty list
+        __syncthreads();
+        for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;
+        if (tid == 0) sh.count = 0;
+        __syncthreads();
+    }
     if constexpr (SOFTMAX) {
         if (!(s_base > 0.0 && s_base < static_cast<double>(INFINITY)) || !(M > -INFINITY && M < INFINITY)) {
             // a NaN or +inf element, or nothing above -inf: every probability of the
@@ -515,7 +806,6 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     hit_cap = min(static_cast<uint32_t>(kPickHitCap), 3u * want + 64u);
     if (blocks > want + want / 4u) hit_cap = min(hit_cap, blocks - 1u);
     bool many_groups = gather(thr, 1ull << 32, std::false_type{});
-    BPS(11);
     if (many_groups) {
         // More than kPickHitCap blocks reach thr: the threads' shares of the block maxima are
         // not alike (rows sorted in runs as long as the stride between a thread's blocks put
@@ -671,15 +961,13 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             }
             return true;
         };
-        // the scan-kernel wave that summed element idx
-        auto wave_of = [&](uint32_t idx) {
-            const uint32_t b = idx / per, off = idx - b * per;
-            return b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;
-        };
         BPS(12);
         finish_row<T, NT, SOFTMAX>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing, scale,
                                    counts != nullptr ? counts + row : nullptr, top_p);
         BPS(13);
+#ifdef VKOP_STAMPS
+        if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[61] = clock64();
+#endif
         return;
     }
 
