@@ -70,19 +70,20 @@ struct ScanWorkspace {
 // in single precision before anything else sees it.
 // WITH_MIN: the blocks' minima as well (for the large-k kernels behind it: a block whose
 // minimum reaches a value holds 16 * vector width elements that do).
-template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED = false, bool WITH_MIN = false>
-__global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__restrict__ in, uint32_t n, uint32_t G,
-                                                                 ScanWorkspace ws, float scale = 1.f) {
-    VKOP_TL_BEGIN();
+// One chunk of one row by kScanThreads threads (tid: 0 .. kScanThreads - 1; block: row * G + chunk).
+// No barrier inside, so several chunks can share a workgroup.  vm_lds: [kScanWaves][V][kWave] floats
+// (per wave: the maximum of every lane's vector i), vmin_lds the same for WITH_MIN.
+template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED, bool WITH_MIN>
+__device__ __forceinline__ void scan_chunk(const T *__restrict__ in, uint32_t n, uint32_t G, const ScanWorkspace &ws,
+                                           float scale, uint32_t block, uint32_t tid, float (*vm_lds)[V][kWave],
+                                           float (*vmin_lds)[V][kWave]) {
     constexpr int NT = kScanThreads, NW = kScanWaves;
     constexpr int VEC = Vec128<T>::N;
     constexpr uint32_t per = static_cast<uint32_t>(NT) * V * VEC;
     constexpr int WB = V * (kWave / kBlockLanes);  // blocks a wave covers: V vectors x 4 rows of 16 lanes
     static_assert(WB <= kWave, "a lane per block of the wave");
-    __shared__ float vm_lds[NW][V][kWave];  // per wave: the maximum of every lane's vector i
-    __shared__ float vmin_lds[WITH_MIN ? NW : 1][WITH_MIN ? V : 1][kWave];
-    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t row = blockIdx.x / G, chunk = blockIdx.x - row * G;
+    const uint32_t lane = tid & (kWave - 1), wave = tid / kWave;
+    const uint32_t row = block / G, chunk = block - row * G;
     const uint32_t c0 = min(chunk * per, n), c1 = min(c0 + per, n);
     const T *rowp = in + static_cast<size_t>(row) * n;
     const uint32_t e_first = c0 + tid * VEC;  // this lane's first element; vector i starts NT * VEC * i later
@@ -228,9 +229,8 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
                 wsum = wave_sum_f64_uniform(acc);
             }
             const uint32_t copies = counting ? static_cast<uint32_t>(wave_sum_f64_uniform(static_cast<double>(ncopy))) : 0u;
-            if (lane == 0)
-                ws.recs2[static_cast<size_t>(row * G + chunk) * NW + wave] = (static_cast<uint64_t>(__float_as_uint(x0)) << 32) | copies;
             if (lane == 0) {
+                ws.recs2[static_cast<size_t>(row * G + chunk) * NW + wave] = (static_cast<uint64_t>(__float_as_uint(x0)) << 32) | copies;
                 uint64_t *record = ws.recs + 2 * (static_cast<size_t>(row * G + chunk) * NW + wave);
                 record[0] = static_cast<uint64_t>(__double_as_longlong(wsum));
                 record[1] = (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref);
@@ -239,6 +239,20 @@ __global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__rest
     };
     if (c1 - c0 == per) body(std::true_type{});
     else body(std::false_type{});
+}
+
+// Launch: rows * G workgroups of kScanThreads, a chunk each.
+template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED = false, bool WITH_MIN = false>
+__global__ __launch_bounds__(kScanThreads) void rows_scan_kernel(const T *__restrict__ in, uint32_t n, uint32_t G,
+                                                                 ScanWorkspace ws, float scale = 1.f) {
+    VKOP_TL_BEGIN();
+    __shared__ float vm_lds[kScanWaves][V][kWave];
+    if constexpr (WITH_MIN) {
+        __shared__ float vmin_lds[kScanWaves][V][kWave];
+        scan_chunk<T, V, SOFTMAX, ALIGNED, SCALED, true>(in, n, G, ws, scale, blockIdx.x, threadIdx.x, vm_lds, vmin_lds);
+    } else {
+        scan_chunk<T, V, SOFTMAX, ALIGNED, SCALED, false>(in, n, G, ws, scale, blockIdx.x, threadIdx.x, vm_lds, nullptr);
+    }
     VKOP_TL_END(0, ws.bmax, blockIdx.x % 16u == 0u || blockIdx.x + 48u >= gridDim.x);
 }
 
@@ -250,6 +264,7 @@ struct PickShared {
     uint32_t hits[kPickHitCap];  // the blocks to read again (the first gather: a part per wave)
     uint4 stage_v[kPickThreads / kWave][kWave];     // per wave: the vectors that hold an element at or above the threshold ...
     uint32_t stage_e[kPickThreads / kWave][kWave];  // ... and the index of their first element
+    uint32_t trial_cnt[kPickThreads / kWave][kPickThreads / kWave];  // [wave][trial]: the wave's thread maxima that reach another wave's bound
 };
 union PickSharedUnion {
     PickShared pick;
@@ -280,22 +295,19 @@ union PickSharedUnion {
 // scale: as in the scan kernel (1 when that ran unscaled); counts (softmax variant,
 // may be null): per row the nucleus cut of its result for top_p (finish_row).
 // SCALED false: scale is 1, and the common case does without the multiplications.
-template <typename T, bool SOFTMAX, bool ALIGNED, int GE, bool SCALED = true, int NT = kPickThreads>
-__global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in, T *__restrict__ values,
-                                                       int32_t *__restrict__ indices, uint32_t n, uint32_t k, uint32_t G,
-                                                       uint32_t per, ScanWorkspace ws, float scale = 1.f,
-                                                       int32_t *__restrict__ counts = nullptr, float top_p = 0.f) {
+// pick_row: one row by all NT threads of a workgroup (smem, fscratch, dscratch: its LDS).
+template <typename T, bool SOFTMAX, bool ALIGNED, int GE, bool SCALED, int NT>
+__device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch, double *dscratch, uint32_t row,
+                                         const T *__restrict__ in, T *__restrict__ values, int32_t *__restrict__ indices,
+                                         uint32_t n, uint32_t k, uint32_t G, uint32_t per, const ScanWorkspace &ws,
+                                         float scale, int32_t *__restrict__ counts, float top_p) {
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
     constexpr int U = NT >= 1024 ? 2 : NT >= 512 ? 4 : 8;  // loads per thread in flight while blocks are read again (128 blocks a round)
     constexpr uint32_t BE = kBlockLanes * VEC;  // elements per block
-    __shared__ PickSharedUnion smem;
-    __shared__ float fscratch[NW];
-    __shared__ double dscratch[NW];
     RowsShared &sh = smem.pick.fast;
     uint32_t *hits = smem.pick.hits;
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t row = blockIdx.x;
     const T *rowp = in + static_cast<size_t>(row) * n;
     T *ov = values + static_cast<size_t>(row) * k;
     int32_t *oi = indices + static_cast<size_t>(row) * k;
@@ -305,7 +317,6 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
     // (a short chain of dependent steps per row, often beside the streaming kernel of another call on the same
     // CU, whose waves issue all the time: this kernel's waves go first)
     __builtin_amdgcn_s_setprio(3);
-    VKOP_TL_BEGIN();
     BPS(14);
 #ifdef VKOP_STAMPS
     if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[60] = clock64();
@@ -429,9 +440,34 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         sh.lane_key[tid] = mine_max;
         if (lane == 0) sh.wave_thr[wave] = mine_q;
         __syncthreads();
-        uint32_t t = sh.wave_thr[0];
+        uint32_t bound[NW];
+        uint32_t t = 0xFFFFFFFFu;
 #pragma unroll
-        for (int w = 1; w < NW; w++) t = min(t, sh.wave_thr[w]);
+        for (int w = 0; w < NW; w++) {
+            bound[w] = sh.wave_thr[w];
+            t = min(t, bound[w]);
+        }
+        if (by_quota && t > 1u) {
+            // The smallest of the waves' bounds is reached by k+1 thread maxima but is lower than it need be
+            // (about 1.8 (k+1) blocks reach it at k = 50).  Every wave counts its thread maxima that reach
+            // each of the NW bounds; the largest bound that k+1 maxima in all reach is the threshold (1.15 (k+1)
+            // blocks): a barrier more, fewer blocks to read again, half as many candidates to rank.
+            uint32_t mine_c = 0;
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                const uint32_t c = static_cast<uint32_t>(__popcll(__ballot(mine_max >= bound[w])));
+                mine_c = lane == static_cast<uint32_t>(w) ? c : mine_c;
+            }
+            if (lane < static_cast<uint32_t>(NW)) smem.pick.trial_cnt[wave][lane] = mine_c;
+            __syncthreads();
+            uint32_t reach = 0, mine_b = 0;
+            if (lane < static_cast<uint32_t>(NW)) {
+#pragma unroll
+                for (int w = 0; w < NW; w++) reach += smem.pick.trial_cnt[w][lane];
+                mine_b = sh.wave_thr[lane];
+            }
+            return wave_max_u32(reach >= want ? mine_b : t);  // (the smallest bound always qualifies)
+        }
         if (t <= 1u) {  // (the same for every thread)
             if (wave == 0) {
                 const uint32_t f = block_kth_largest_floor<NW>(sh.lane_key, want, bits);
@@ -588,7 +624,13 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
         bool common = sh.wave_overflow == 0u && C2 >= want && C2 <= static_cast<uint32_t>(NT) && kk == k;
         if constexpr (SOFTMAX) common = common && s_base > 0.0 && s_base < static_cast<double>(INFINITY) && M > -INFINITY && M < INFINITY;
         if (__builtin_expect(common, 1)) {
-            // the candidate's own part first (its wave's record, its accurate term), then its share of the ranking
+            // A candidate's own part (its wave's record, its accurate term) and the ranking are two chains of
+            // a hundred instructions and more: where the candidates fill at most half of the workgroup's waves
+            // (P, the power of two at or above their number, up to NT / 2), those waves take the terms and the
+            // others the ranking -- NT / P - 1 groups of P threads, a group a part of the list, which ends in zeros.
+            static_assert(NT == 512, "the table of parts below");
+            const uint32_t pshift = C2 > 64u ? 32u - static_cast<uint32_t>(__clz(C2 - 1u)) : 6u;  // P >= 64
+            const bool apart = pshift <= 8u;
             uint64_t mine = 0;
             float term = 0.f;
             double cr = 0.0;
@@ -605,8 +647,31 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
                 }
             }
             BPS(30);
-            if (C2 > 32u) block_rank_padded<NT>(sh, C2);  // (both end with a barrier)
-            else block_rank<NT>(sh, C2);
+            if (apart) {
+                if (tid >= (1u << pshift)) {
+                    // 7 groups of 64 take 10 entries each, 3 groups of 128 take 44, 1 group of 256 all of them (even numbers: two per read)
+                    const uint32_t span = pshift == 6u ? 10u : pshift == 7u ? 44u : 256u;
+                    const uint32_t i = tid & ((1u << pshift) - 1u);
+                    const uint64_t cmp = sh.cand[i];
+                    const uint4 *src = reinterpret_cast<const uint4 *>(sh.cand + ((tid >> pshift) - 1u) * span);
+                    uint32_t cnt = 0;
+                    for (uint32_t j = 0; j < span / 2; j += 4) {  // four reads of two entries in flight (past the span: counted by the next group too -- never: zeros or skipped)
+                        uint4 o[4];
+#pragma unroll
+                        for (int u = 0; u < 4; u++) o[u] = src[j + u < span / 2 ? j + u : 0u];
+#pragma unroll
+                        for (int u = 0; u < 4; u++) {
+                            const bool in = j + u < span / 2;
+                            cnt += (in && ((static_cast<uint64_t>(o[u].y) << 32) | o[u].x) > cmp) ? 1u : 0u;
+                            cnt += (in && ((static_cast<uint64_t>(o[u].w) << 32) | o[u].z) > cmp) ? 1u : 0u;
+                        }
+                    }
+                    if (cnt) atomicAdd(&sh.rank[i], cnt);
+                }
+                __syncthreads();
+            } else {
+                block_rank_padded<NT>(sh, C2);  // (ends with a barrier)
+            }
             BPS(31);
             if (tid < C2) {
                 const uint32_t rk = sh.rank[tid];
@@ -680,7 +745,6 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
 #ifdef VKOP_STAMPS
             if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[61] = clock64();
 #endif
-            VKOP_TL_END(1, ws.bmax, true);
             if (__builtin_expect(!tie, 1)) return;
             // (equal probabilities: what was stored is written again below, in its final order)
         }
@@ -1015,6 +1079,21 @@ __global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in,
             oi[r] = static_cast<int32_t>(idx);
         }
     }
+}
+
+// Launch: one workgroup of NT threads per row, after rows_scan_kernel on the same stream.
+template <typename T, bool SOFTMAX, bool ALIGNED, int GE, bool SCALED = true, int NT = kPickThreads>
+__global__ __launch_bounds__(NT) void rows_pick_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                       int32_t *__restrict__ indices, uint32_t n, uint32_t k, uint32_t G,
+                                                       uint32_t per, ScanWorkspace ws, float scale = 1.f,
+                                                       int32_t *__restrict__ counts = nullptr, float top_p = 0.f) {
+    __shared__ PickSharedUnion smem;
+    __shared__ float fscratch[NT / kWave];
+    __shared__ double dscratch[NT / kWave];
+    VKOP_TL_BEGIN();
+    pick_row<T, SOFTMAX, ALIGNED, GE, SCALED, NT>(smem, fscratch, dscratch, blockIdx.x, in, values, indices, n, k, G, per,
+                                                         ws, scale, counts, top_p);
+    VKOP_TL_END(1, ws.bmax, true);
 }
 
 }  // namespace vkop
