@@ -121,13 +121,44 @@ def test_softmax_axes(ops, shape, axis):
     assert_softmax_close(host(ops.softmax(dev(xh), axis)), xh, axis, str((shape, axis)) + " half")
 
 
+@pytest.mark.parametrize("shape,axis", [((4096, 64), -1), ((4096, 1024), -1), ((8192, 512), -1), ((300, 2048), -1), ((64, 40000), -1),
+                                        ((16, 80, 840), 1), ((2, 1000, 64), 1), ((8, 4096, 64), 1)])
+def test_softmax_half_near_rounding_boundaries(ops, shape, axis):
+    """Half tensors take their terms from the single-precision exponential (about 2^-22 relative
+    before the rounding to 11 bits) and scale them in single precision.  Where the exact
+    probability -- worked out here in float64 -- lies within 2^-14 relative of the boundary
+    between two halves, either neighbour is a result within the bar (one unit of a half against
+    the oracle); away from the boundaries the result must be the oracle's own, on every kernel
+    that writes half tensors (a wave a row, a wave a row with 128-bit loads, a workgroup a row,
+    chunked rows, strided lines in registers and in tiles, tiles split over workgroups)."""
+    rng = np.random.default_rng(shape[0] * 7 + shape[-1])
+    x = (rng.standard_normal(shape) * 2.5).astype(np.float16)
+    got = host(ops.softmax(dev(x), axis))
+    exp = oracle.softmax(x, axis)
+    x64 = np.moveaxis(x.astype(np.float64), axis, -1)
+    e64 = np.exp(x64 - x64.max(-1, keepdims=True))
+    p64 = np.moveaxis(e64 / e64.sum(-1, keepdims=True), -1, axis)
+    # distance of the exact probability to the nearest boundary between two halves, in units of its own size
+    lo = p64.astype(np.float16)
+    lo = np.where(lo.astype(np.float64) > p64, np.nextafter(lo, np.float16(0)), lo)     # the half at or below
+    hi = np.nextafter(lo, np.float16(1))
+    mid = (lo.astype(np.float64) + hi.astype(np.float64)) / 2
+    near = np.abs(p64 - mid) <= p64 * 2.0 ** -14
+    d = half_ulp_diff(got, exp)
+    assert d.max() <= 1, "%s: %d units of a half" % (shape, d.max())
+    assert near.sum() > 50, "the case holds no probability near a boundary"
+    assert np.all(d[~near] == 0), "%s: %d results away from every boundary differ from the oracle" % (shape, int((d[~near] != 0).sum()))
+    assert (d != 0).mean() < 0.01
+
+
 @pytest.mark.parametrize("shape,axis", [((128, 33000), -1), ((16, 131072), -1), ((64, 40000), -1), ((8, 4096, 256), 1),
                                         ((32, 1000, 64), 1), ((300, 200, 64), 1), ((4096, 1024), -1)])
 def test_softmax_of_one_repeated_value_and_a_few_peaks(ops, shape, axis):
     """Lines that are one value but for a peak in five thousand elements: the sum is that value's
     term times its count, the term being the float exponential of the ROUNDED difference to the
-    maximum; the kernels that sum chunks against their own maxima count the copies of each
-    chunk's smallest value apart, so that they enter the sum as defined (4 ulp otherwise)."""
+    maximum; the kernels that sum chunks against their own maxima count the copies of one value
+    apart (the chunk's smallest; for strided tiles the line's first element in the chunk, where
+    the second equals it), so that they enter the sum as defined (4 ulp otherwise)."""
     rng = np.random.default_rng(len(shape) + shape[-1])
     x = np.full(shape, 0.25, np.float32)
     x.ravel()[rng.integers(0, x.size, max(1, x.size // 5000))] = 6.0

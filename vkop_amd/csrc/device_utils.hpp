@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace vkop {
 
 constexpr int kWave = 64;
@@ -180,5 +182,40 @@ __device__ __forceinline__ float exp_accurate(float d) {
 
 // One softmax term: exp of the single-precision difference x - m.
 __device__ __forceinline__ float softmax_term(float x, float m) { return exp_accurate(x - m); }
+
+// exp(d) in single precision throughout, good to about two units in the last place of a float: the
+// hardware exponential of a = fl(d log2 e), and what that rounding and the low part of log2 e left
+// out as a first-order factor (2^(a + l) = 2^a (1 + l ln 2), |l| < 1e-6).  For results that are
+// stored in half precision: 2^-22 relative before a rounding to 11 bits moves one result in two
+// thousand by one unit of a half, and costs a third of exp_accurate.  Results below 2^-126 are 0.
+__device__ __forceinline__ float exp_half_grade(float d) {
+    constexpr float kHi = 1.44269502162933349609375f;  // float(log2 e)
+    constexpr float kLo = 1.925963033500011e-8f;       // log2 e - kHi
+    const float a = d * kHi;
+    const float l = fmaf(d, kLo, fmaf(d, kHi, -a));  // (d = -inf: NaN, and so is the product below)
+    const float e = __builtin_amdgcn_exp2f(a);
+    const float t = fmaf(e, l * 0.693147180559945309f, e);
+    return e > 0.f && e < INFINITY ? t : e;  // (0, inf and NaN as the hardware unit gives them)
+}
+
+// The term as the element type asks for it: float tensors get the correctly rounded exponential,
+// half tensors (uint16_t) the single-precision one.  Every kernel that writes a softmax TENSOR
+// takes its terms from here, so the results of one element type agree between them.
+template <typename T> __device__ __forceinline__ float softmax_term_as(float x, float m) {
+    if constexpr (sizeof(T) == 2) return exp_half_grade(x - m);
+    else return exp_accurate(x - m);
+}
+
+// What a thread adds its own few terms up in, and how a term becomes a probability, in the same
+// kernels: double for float tensors (the sum and the quotient as the definition rounds them), float
+// for half tensors (a few dozen terms a thread: 2^-19 relative at worst, against 2^-11 of a half;
+// the threads' sums are then added in double like everyone's).  Conversions to and from double are
+// a quarter-rate instruction each, four of them an element: half tensors ran at the speed of float
+// tensors of the same shape, for half the bytes.
+template <typename T> using TermSum = std::conditional_t<sizeof(T) == 2, float, double>;
+template <typename T> __device__ __forceinline__ float scale_term(float e, double rinv) {
+    if constexpr (sizeof(T) == 2) return e * static_cast<float>(rinv);
+    else return static_cast<float>(static_cast<double>(e) * rinv);
+}
 
 }  // namespace vkop

@@ -53,6 +53,9 @@ __device__ __forceinline__ LineStats line_stats(const T *x, size_t base, uint32_
 __device__ __forceinline__ float softmax_prob(float x, LineStats st) {
     return static_cast<float>(static_cast<double>(softmax_term(x, st.m)) * st.rinv);
 }
+template <typename T> __device__ __forceinline__ float softmax_prob_as(float x, LineStats st) {
+    return scale_term<T>(softmax_term_as<T>(x, st.m), st.rinv);
+}
 
 // ---- softmax, one workgroup per line ---------------------------------------
 template <typename T, int NT>

@@ -45,71 +45,152 @@ struct ChunkStat {
     double s;       // sum of exp(x - ref) over the chunk (softmax_stats_kernel: without the copies of its minimum)
     float m;        // maximum of the chunk (NaN ignored; -inf for an empty chunk)
     float ref;      // reference of the sum: m, or 0 when m is not finite
-    float vmin;     // softmax_stats_kernel: the chunk's minimum ...
+    float vmin;     // the value whose copies the sum leaves out (softmax_stats_kernel: the chunk's minimum; the
+                    // strided tiles: the line's first element in the chunk) ...
     uint32_t nmin;  // ... and how many elements equal it (0: none set apart)
 };
 
 // ---- a whole row per workgroup ------------------------------------------------------
+// A workgroup takes the rows blockIdx.x, blockIdx.x + gridDim.x, ... (the launch caps the grid:
+// half a million workgroups of one short row each are handed out at about 2 ns apiece, which
+// bounded [16,32,1024,1024] in both precisions); the next row's loads are issued before the
+// current row's arithmetic.
+constexpr uint32_t kSoftmaxRowGridMax = 16384;
 template <typename T, int NT, int V, bool ALIGNED>
-__global__ __launch_bounds__(NT) void softmax_row_kernel(const T *in, T *out, uint32_t n, int nan_where,
+__global__ __launch_bounds__(NT) void softmax_row_kernel(const T *in, T *out, uint32_t rows, uint32_t n, int nan_where,
                                                          float nan_value) {
     constexpr int VEC = Vec128<T>::N;
     constexpr int NW = NT / kWave;
     __shared__ float fscratch[NW];
     __shared__ double dscratch[NW];
     const uint32_t tid = threadIdx.x;
-    const size_t row0 = static_cast<size_t>(blockIdx.x) * n;
-    const T *rowp = in + row0;
-    Vec128<T> q[V];
+    auto load_row = [&](Vec128<T> (&q)[V], uint32_t row) __attribute__((always_inline)) {
+        const T *rowp = in + static_cast<size_t>(row) * n;
 #pragma unroll
-    for (int i = 0; i < V; i++) {
-        const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
-        q[i].v = make_uint4(0, 0, 0, 0);
-        if constexpr (ALIGNED) {
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
+            q[i].v = make_uint4(0, 0, 0, 0);
+            if constexpr (ALIGNED) {
+                q[i].load(rowp + (e0 < n ? e0 : 0u));
+            } else {
+#pragma unroll
+                for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < n ? e0 + c : 0u));
+            }
+        }
+    };
+    Vec128<T> q[V], qn[V];
+    load_row(q, blockIdx.x);
+    for (uint32_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const uint32_t next = row + gridDim.x;
+        if (next < rows) load_row(qn, next);  // (the same in every thread)
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
+#pragma unroll
+            for (int c = 0; c < VEC; c++)
+                if (e0 + c < n) m = fmaxf(m, q[i].get(c));
+        }
+        m = block_max<NT>(m, fscratch);
+        // the terms replace the inputs in the registers (a term is a float; for half
+        // tensors it is kept in a float array instead)
+        float e[V][VEC];
+        TermSum<T> acc = 0;
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                e[i][c] = e0 + c < n ? softmax_term_as<T>(q[i].get(c), m) : 0.f;
+                acc += static_cast<TermSum<T>>(e[i][c]);
+            }
+        }
+        const double rinv = 1.0 / block_sum<NT>(static_cast<double>(acc), dscratch);
+        T *orow = out + static_cast<size_t>(row) * n;
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
+            Vec128<T> r;
+            r.v = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                float p = round_to_storage<T>(scale_term<T>(e[i][c], rinv));
+                if (nan_where && p != p) p = nan_value;
+                if constexpr (ALIGNED) r.set(c, p);
+                else if (e0 + c < n) store_elem(orow, e0 + c, p);
+            }
+            if constexpr (ALIGNED)
+                if (e0 < n) *reinterpret_cast<uint4 *>(orow + e0) = r.v;
+        }
+#pragma unroll
+        for (int i = 0; i < V; i++) q[i] = qn[i];
+    }
+}
+
+// ---- rows of a few hundred to two thousand elements, many of them: a wave per row, 128-bit loads ----
+// Rows of up to 64 * V vectors that start on 16 bytes (n a multiple of the vector width): lane l
+// holds vectors l, l + 64, ...; maximum and sum cross the lanes without LDS or a barrier (a
+// workgroup per row pays four barriers a row for two waves' work), four rows a workgroup, each
+// wave on to its next row (grid-stride) with that row's loads issued before this row's arithmetic.
+constexpr int kSoftmaxVecRows = 4;  // rows (waves) per workgroup
+template <typename T, int V>
+__global__ __launch_bounds__(kSoftmaxVecRows *kWave) void softmax_wave_vec_kernel(const T *__restrict__ in, T *__restrict__ out,
+                                                                                  uint32_t rows, uint32_t n, int nan_where,
+                                                                                  float nan_value) {
+    constexpr int VEC = Vec128<T>::N;
+    const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const uint32_t step = gridDim.x * kSoftmaxVecRows;
+    auto load_row = [&](Vec128<T> (&q)[V], uint32_t row) __attribute__((always_inline)) {
+        const T *rowp = in + static_cast<size_t>(row) * n;
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = (static_cast<uint32_t>(i) * kWave + lane) * VEC;
             q[i].load(rowp + (e0 < n ? e0 : 0u));
-        } else {
-#pragma unroll
-            for (int c = 0; c < VEC; c++) q[i].set(c, load_elem(rowp, e0 + c < n ? e0 + c : 0u));
         }
-    }
-    float m = -INFINITY;
+    };
+    uint32_t row = blockIdx.x * kSoftmaxVecRows + wave;
+    if (row >= rows) return;  // (a whole wave)
+    Vec128<T> q[V], qn[V];
+    load_row(q, row);
+    for (; row < rows; row += step) {
+        if (row + step < rows) load_row(qn, row + step);  // (wave-uniform)
+        float m = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < V; i++) {
-        const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
+        for (int i = 0; i < V; i++) {
+            const bool live = (static_cast<uint32_t>(i) * kWave + lane) * VEC < n;
 #pragma unroll
-        for (int c = 0; c < VEC; c++)
-            if (e0 + c < n) m = fmaxf(m, q[i].get(c));
-    }
-    m = block_max<NT>(m, fscratch);
-    // the terms replace the inputs in the registers (a term is a float; for half
-    // tensors it is kept in a float array instead)
-    float e[V][VEC];
-    double acc = 0.0;
-#pragma unroll
-    for (int i = 0; i < V; i++) {
-        const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
-#pragma unroll
-        for (int c = 0; c < VEC; c++) {
-            e[i][c] = e0 + c < n ? softmax_term(q[i].get(c), m) : 0.f;
-            acc += static_cast<double>(e[i][c]);
+            for (int c = 0; c < VEC; c++)
+                if (live) m = fmaxf(m, q[i].get(c));
         }
-    }
-    const double rinv = 1.0 / block_sum<NT>(acc, dscratch);
-    T *orow = out + row0;
+        m = wave_max_f32_uniform(m);
+        float e[V][VEC];
+        TermSum<T> acc = 0;
 #pragma unroll
-    for (int i = 0; i < V; i++) {
-        const uint32_t e0 = (static_cast<uint32_t>(i) * NT + tid) * VEC;
-        Vec128<T> r;
-        r.v = make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < V; i++) {
+            const bool live = (static_cast<uint32_t>(i) * kWave + lane) * VEC < n;
 #pragma unroll
-        for (int c = 0; c < VEC; c++) {
-            float p = round_to_storage<T>(static_cast<float>(static_cast<double>(e[i][c]) * rinv));
-            if (nan_where && p != p) p = nan_value;
-            if constexpr (ALIGNED) r.set(c, p);
-            else if (e0 + c < n) store_elem(orow, e0 + c, p);
+            for (int c = 0; c < VEC; c++) {
+                e[i][c] = live ? softmax_term_as<T>(q[i].get(c), m) : 0.f;
+                acc += static_cast<TermSum<T>>(e[i][c]);
+            }
         }
-        if constexpr (ALIGNED)
+        const double rinv = 1.0 / wave_sum_f64_uniform(static_cast<double>(acc));
+        T *orow = out + static_cast<size_t>(row) * n;
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const uint32_t e0 = (static_cast<uint32_t>(i) * kWave + lane) * VEC;
+            Vec128<T> r;
+            r.v = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int c = 0; c < VEC; c++) {
+                float p = round_to_storage<T>(scale_term<T>(e[i][c], rinv));
+                if (nan_where && p != p) p = nan_value;
+                r.set(c, p);
+            }
             if (e0 < n) *reinterpret_cast<uint4 *>(orow + e0) = r.v;
+        }
+#pragma unroll
+        for (int i = 0; i < V; i++) q[i] = qn[i];
     }
 }
 
@@ -141,17 +222,17 @@ __global__ __launch_bounds__(kSoftmaxWaveRows *kWave) void softmax_wave_kernel(c
         if (static_cast<uint32_t>(j) * kWave + lane < n) m = fmaxf(m, x[j]);  // (drops NaN)
     m = wave_max_f32_uniform(m);
     float t[E];
-    double acc = 0.0;
+    TermSum<T> acc = 0;
 #pragma unroll
     for (int j = 0; j < E; j++) {
-        t[j] = static_cast<uint32_t>(j) * kWave + lane < n ? softmax_term(x[j], m) : 0.f;
-        acc += static_cast<double>(t[j]);
+        t[j] = static_cast<uint32_t>(j) * kWave + lane < n ? softmax_term_as<T>(x[j], m) : 0.f;
+        acc += static_cast<TermSum<T>>(t[j]);
     }
-    const double rinv = 1.0 / wave_sum_f64_uniform(acc);
+    const double rinv = 1.0 / wave_sum_f64_uniform(static_cast<double>(acc));
 #pragma unroll
     for (int j = 0; j < E; j++) {
         const uint32_t e = static_cast<uint32_t>(j) * kWave + lane;
-        float p = round_to_storage<T>(static_cast<float>(static_cast<double>(t[j]) * rinv));
+        float p = round_to_storage<T>(scale_term<T>(t[j], rinv));
         if (nan_where && p != p) p = nan_value;
         if (e < n) store_elem(orow, e, p);
     }
@@ -289,7 +370,7 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
     const float M = block_max<NT>(st.m, fscratch);
     double part = 0.0;
     if (tid < G && st.s != 0.0) part = st.s * sum_rescale(st.s, st.ref, M);
-    if (tid < G && st.nmin != 0u) part += static_cast<double>(st.nmin) * static_cast<double>(softmax_term(st.vmin, M));
+    if (tid < G && st.nmin != 0u) part += static_cast<double>(st.nmin) * static_cast<double>(softmax_term_as<T>(st.vmin, M));
     const LineStats ls{M, 0.f, 1.0 / block_sum<NT>(part, dscratch)};
     T *orow = out + row0;
 #pragma unroll
@@ -299,7 +380,7 @@ __global__ __launch_bounds__(NT) void softmax_scale_kernel(const T *in, T *out, 
         r.v = make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int c = 0; c < VEC; c++) {
-            float p = round_to_storage<T>(softmax_prob(q[i].get(c), ls));
+            float p = round_to_storage<T>(softmax_prob_as<T>(q[i].get(c), ls));
             if (nan_where && p != p) p = nan_value;
             if constexpr (ALIGNED) r.set(c, p);
             else if (e0 + c < c1) store_elem(orow, e0 + c, p);
@@ -338,6 +419,7 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
     constexpr int U = 16;  // rows a lane has in flight (a pass is a chain of n / (16 waves * U) round trips)
     __shared__ float fmax_lds[NW * kWave];
     __shared__ double dsum_lds[NW * kWave];
+    __shared__ uint32_t ucnt_lds[MODE == kTileStats ? NW * kWave : 1];
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const uint32_t TI = 1u << ti_shift, RPW = kWave >> ti_shift;  // lines a tile, rows per wave instruction
     const uint32_t tiles = (g.inner + TI - 1) >> ti_shift;
@@ -392,35 +474,48 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
     LineStats st{0.f, 0.f, 0.0};
     if constexpr (!kFold) {
         // ---- 1. the lines' maxima
-        float m = -INFINITY, mn_own = INFINITY;
-        pass([&](float x, uint32_t) {
-            m = fmaxf(m, x);  // (drops NaN)
-            if constexpr (MODE == kTileStats) mn_own = fminf(mn_own, x);
-        });
+        float m = -INFINITY;
+        pass([&](float x, uint32_t) { m = fmaxf(m, x); });  // (drops NaN)
         m = reduce_max(m);
         // ---- 2. the sums of the terms
         double acc = 0.0;
         if constexpr (MODE != kTileStats) {
-            pass([&](float x, uint32_t) { acc += static_cast<double>(softmax_term(x, m)); });
+            pass([&](float x, uint32_t) { acc += static_cast<double>(softmax_term_as<T>(x, m)); });
             st = LineStats{m, 0.f, 1.0 / reduce_sum(acc)};
         } else {
             // reference of the chunk's sum: its maximum, or 0 when that is not finite (then
             // every term is 0, inf or NaN, and NaN / inf must reach the sum)
             const float ref = (m > -INFINITY && m < INFINITY) ? m : 0.f;
-            // (the copies of the chunk's minimum are counted apart, as in softmax_stats_kernel)
-            __syncthreads();  // (fmax_lds is read by every thread of the first reduction)
-            const float mn = -reduce_max(-mn_own);
-            const bool apart = mn > -INFINITY && mn < INFINITY;
-            double copies = 0.0;
+            // The copies of ONE value are counted apart (as in softmax_stats_kernel: the kernel that knows
+            // the line's maximum adds the accurate term for each): the line's first element in this chunk,
+            // where the second equals it -- a value that fills a line turns up at once, every lane of the
+            // line reads the same two elements (from the cache) and decides alike, and a line of spread-out
+            // values pays a comparison per element and nothing else.
+            const float x0 = load_elem(in, at(c0 < c1 ? c0 : 0u)), x1 = load_elem(in, at(c0 + 1u < c1 ? c0 + 1u : 0u));
+            const bool apart = c0 + 1u < c1 && x0 == x1 && x0 > -INFINITY && x0 < INFINITY;
+            uint32_t copies = 0;
             pass([&](float x, uint32_t) {
-                if (apart && x == mn) copies += 1.0;
+                if (apart && x == x0) copies += 1u;
                 else acc += static_cast<double>(fast_term_unbiased(x, ref));
             });
-            const double sum = reduce_sum(acc);
-            __syncthreads();  // (dsum_lds likewise)
-            const double nmin = reduce_sum(copies);
-            if (tid < TI)
-                stats[(static_cast<size_t>(tileid) * G + chunk) * TI + tid] = ChunkStat{sum, m, ref, mn, static_cast<uint32_t>(nmin)};
+            // (both sums in one round: over the lanes of a wave that look at the same line, then over the waves)
+            for (uint32_t off = TI; off < static_cast<uint32_t>(kWave); off <<= 1) {
+                acc += __shfl_xor(acc, static_cast<int>(off), kWave);
+                copies += __shfl_xor(copies, static_cast<int>(off), kWave);
+            }
+            dsum_lds[tid] = acc;
+            ucnt_lds[tid] = copies;
+            __syncthreads();
+            if (tid < TI) {
+                double sum = dsum_lds[tid];
+                uint32_t nx0 = ucnt_lds[tid];
+#pragma unroll
+                for (int w = 1; w < NW; w++) {  // fixed order: run-to-run stable
+                    sum += dsum_lds[w * kWave + tid];
+                    nx0 += ucnt_lds[w * kWave + tid];
+                }
+                stats[(static_cast<size_t>(tileid) * G + chunk) * TI + tid] = ChunkStat{sum, m, ref, x0, nx0};
+            }
             return;
         }
     } else {
@@ -433,7 +528,7 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
         float M = fmax_lds[mine];
         for (uint32_t c = 1; c < G; c++) M = fmaxf(M, fmax_lds[c * TI + mine]);
         dsum_lds[tid] = ((holds && cs.s != 0.0) ? cs.s * sum_rescale(cs.s, cs.ref, M) : 0.0) +
-                        ((holds && cs.nmin != 0u) ? static_cast<double>(cs.nmin) * static_cast<double>(softmax_term(cs.vmin, M)) : 0.0);
+                        ((holds && cs.nmin != 0u) ? static_cast<double>(cs.nmin) * static_cast<double>(softmax_term_as<T>(cs.vmin, M)) : 0.0);
         __syncthreads();
         double sum = dsum_lds[mine];
         for (uint32_t c = 1; c < G; c++) sum += dsum_lds[c * TI + mine];
@@ -441,12 +536,12 @@ __global__ __launch_bounds__(kStridedTileThreads) void softmax_strided_tile_kern
     }
     if constexpr (kMaxOnly) {
         // the line's maximum has the term exp_accurate(0) = 1 (NaN statistics give NaN, as the tensor would)
-        if (tid < TI && col_ok) store_elem(out, static_cast<size_t>(o) * g.inner + col, softmax_prob(st.m, st));
+        if (tid < TI && col_ok) store_elem(out, static_cast<size_t>(o) * g.inner + col, softmax_prob_as<T>(st.m, st));
         return;
     }
     // ---- 3. the probabilities
     pass([&](float x, uint32_t j) {
-        float p = round_to_storage<T>(softmax_prob(x, st));
+        float p = round_to_storage<T>(softmax_prob_as<T>(x, st));
         if (nan_where && p != p) p = nan_value;
         if (col_ok) store_elem(out, at(j), p);
     });
@@ -497,14 +592,15 @@ __global__ __launch_bounds__(kStridedThreads) void softmax_strided_reg_kernel(co
 #pragma unroll
     for (int o = LPW; o < kWave; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, kWave));
     // terms replace the elements; the parts' sums are added in a fixed order
-    double s = 0.0;
+    TermSum<T> s_own = 0;
 #pragma unroll
     for (int i = 0; i < NPER; i++) {
         if (static_cast<uint32_t>(i) * P + part < n) {
-            x[i] = softmax_term(x[i], m);
-            s += static_cast<double>(x[i]);
+            x[i] = softmax_term_as<T>(x[i], m);
+            s_own += static_cast<TermSum<T>>(x[i]);
         }
     }
+    double s = static_cast<double>(s_own);
 #pragma unroll
     for (int o = LPW; o < kWave; o <<= 1) s += __shfl_xor(s, o, kWave);
     const double rinv = 1.0 / s;
@@ -523,7 +619,7 @@ __global__ __launch_bounds__(kStridedThreads) void softmax_strided_reg_kernel(co
             const float other = __shfl_xor(top, o, kWave);
             top = (other != other) ? other : ((top != top) ? top : fmaxf(top, other));
         }
-        float p = round_to_storage<T>(static_cast<float>(static_cast<double>(top) * rinv));
+        float p = round_to_storage<T>(scale_term<T>(top, rinv));
         if (nan_where && p != p) p = nan_value;
         if (live && part == 0) store_elem(out, line, p);
         return;
@@ -532,7 +628,7 @@ __global__ __launch_bounds__(kStridedThreads) void softmax_strided_reg_kernel(co
     for (int i = 0; i < NPER; i++) {
         const uint32_t j = static_cast<uint32_t>(i) * P + part;
         if (live && j < n) {
-            float p = round_to_storage<T>(static_cast<float>(static_cast<double>(x[i]) * rinv));
+            float p = round_to_storage<T>(scale_term<T>(x[i], rinv));
             if (nan_where && p != p) p = nan_value;
             store_elem(out, base + static_cast<size_t>(j) * g.inner, p);
         }

@@ -262,10 +262,23 @@ int softmax_impl(const T *in, T *out, const View &v, int dtype, int nan_where, f
     switch (p.kind) {
     case SoftmaxPlan::kRow: {
         bool done = false;
+        const uint32_t row_grid = std::min(lines, vkop::kSoftmaxRowGridMax);
+        // thousands of rows that a wave holds in a few 128-bit loads a lane: a wave per row, no barrier
+        const uint32_t vectors = (v.g.n + vec - 1) / vec;
+        if (aligned && lines >= 4096 && vectors <= 4 * vkop::kWave) {
+            const uint32_t wgs = std::min((lines + vkop::kSoftmaxVecRows - 1) / vkop::kSoftmaxVecRows, 8192u);
+#define VKOP_VEC_ROW(V)                                                                                                          \
+    vkop::softmax_wave_vec_kernel<T, V><<<wgs, vkop::kSoftmaxVecRows * vkop::kWave, 0, st>>>(in, out, lines, v.g.n, nan_where, nan_value)
+            if (vectors <= vkop::kWave) VKOP_VEC_ROW(1);
+            else if (vectors <= 2 * vkop::kWave) VKOP_VEC_ROW(2);
+            else VKOP_VEC_ROW(4);
+#undef VKOP_VEC_ROW
+            return launched("softmax_wave_vec_kernel");
+        }
 #define VKOP_ROW(NT, V)                                                                                        \
     if (!done && p.shape.nt == NT && p.shape.v == V) {                                                         \
-        if (aligned) vkop::softmax_row_kernel<T, NT, V, true><<<lines, NT, 0, st>>>(in, out, v.g.n, nan_where, nan_value); \
-        else vkop::softmax_row_kernel<T, NT, V, false><<<lines, NT, 0, st>>>(in, out, v.g.n, nan_where, nan_value);        \
+        if (aligned) vkop::softmax_row_kernel<T, NT, V, true><<<row_grid, NT, 0, st>>>(in, out, lines, v.g.n, nan_where, nan_value); \
+        else vkop::softmax_row_kernel<T, NT, V, false><<<row_grid, NT, 0, st>>>(in, out, lines, v.g.n, nan_where, nan_value);        \
         done = true;                                                                                           \
     }
         VKOP_FOR_EACH_ROW_SHAPE(VKOP_ROW, T)
