@@ -14,7 +14,7 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
     const uint32_t per = kScanThreads * a.v * VEC;
     const uint32_t ge = (a.ws.blocks + kPickThreads - 1) / kPickThreads;
     const uint32_t ge_big = (a.ws.blocks + kBigPickThreads - 1) / kBigPickThreads;
-    if (a.g2 == 0 ? ge > 16 : ge_big > 32) return false;
+    if (a.g2 == 0 ? ge > 32 : ge_big > 32) return false;
     bool scanned = (a.stages & 1) == 0;
     const bool scaled = SOFTMAX && a.scale != 1.f;
 #define VKOP_SCAN_LAUNCH(V, AL, SC) \
@@ -85,6 +85,7 @@ template <typename T, bool SOFTMAX> bool launch_rows_scan(const ScanLaunch &a) {
     VKOP_PICK_CASE(4)
     VKOP_PICK_CASE(8)
     VKOP_PICK_CASE(16)
+    VKOP_PICK_CASE(32)
 #undef VKOP_PICK_CASE
 #undef VKOP_PICK_LAUNCH
     return false;

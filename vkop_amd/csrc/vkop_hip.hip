@@ -440,6 +440,12 @@ RowsCfg choose_rows_cfg(const View &v, int k, int dtype, bool for_size = false) 
             const uint64_t span = static_cast<uint64_t>(shapes[i][0]) * shapes[i][1] * vec;
             if (shapes[i][0] == 256 && span >= n && fits(shapes[i][0], shapes[i][1], 1)) pick = i;
         }
+        // a row just past those shapes that has too few blocks for the scan kernels (8193 to 8320 elements at
+        // k = 64): the wider workgroup that holds it, rather than several chunks and a merge
+        const uint32_t blocks = (n + vkop::kBlockLanes * vec - 1) / (vkop::kBlockLanes * vec);
+        if (pick < 0 && wide >= 0 && !forced_nt && g_rows_path.load() != 1 &&
+            4ull * blocks < (rows <= 16 ? 8ull : 7ull) * (static_cast<uint64_t>(k) + 1u))
+            pick = wide;
         const bool one_workgroup = pick >= 0;
         for (int i = 0; i < 6 && !one_workgroup; i++) {
             const uint32_t span = static_cast<uint32_t>(shapes[i][0]) * shapes[i][1] * vec;
@@ -554,7 +560,7 @@ ScanCfg choose_scan_cfg(const View &v, int k, int dtype, bool for_size = false) 
         const RowsCfg one = choose_rows_cfg(v, k, dtype);
         if (one.ok && one.g == 1 && one.nt >= 256) return c;
     }
-    if (!big && (blocks + vkop::kPickThreads - 1) / vkop::kPickThreads > 16u) return c;
+    if (!big && (blocks + vkop::kPickThreads - 1) / vkop::kPickThreads > 32u) return c;
     if (big && (blocks + vkop::kBigPickThreads - 1) / vkop::kBigPickThreads > 32u) return c;
     if (big && static_cast<uint64_t>(rows) * (vkop::kBigPickCap / vkop::kBigPickMine) >= (1ull << 31)) return c;
     const uint32_t waves_max = big ? static_cast<uint32_t>(vkop::kBigPickRecsMax) : static_cast<uint32_t>(vkop::kMergeWavesMax);
