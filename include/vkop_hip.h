@@ -211,8 +211,14 @@ int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_ca
                  void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---- Tuning knobs (no counterpart in the reference, whose shaders fix their
- * workgroup shapes at compile time).  Results are identical for every setting;
- * only the kernels and launch shapes chosen differ.  The settings are
+ * workgroup shapes at compile time).  Only the kernels and launch shapes chosen
+ * differ.  What is identical for every setting: the softmax operator's output,
+ * plain top-k values and indices, and the indices of the fused call wherever the
+ * k+1 largest probabilities of a row differ by more than the kernels' sums do.
+ * What is equal to within the bar (2 ulp of float against the CPU definition, one
+ * unit of a half): the fused call's probabilities -- each route adds a row's
+ * terms up in its own order, and two routes may round a row's sum one ulp apart.
+ * The settings are
  * process-wide and read when a call is made: set them before the threads that
  * call the operators start, not while calls are being made (a call that sees a
  * setting change between its workspace query and its launch is refused with
@@ -222,7 +228,8 @@ int vkop_hip_nms(const void *boxes, const void *scores, int32_t *out, int out_ca
  *       the one-wave-per-row kernel, rows too long for one workgroup through the
  *       scan + pick kernel pair where it applies (k up to 511; beyond that, scan +
  *       gather + rank); 1 = never (the chunk + merge kernels, the multi-pass radix
- *       select).
+ *       select: with the default, rows of several chunks never take chunk + merge,
+ *       which the tests compare every other route with).
  *   "rows.threads", "rows.loads", "rows.chunks": force the launch shape of the
  *       chunk kernel (threads per workgroup, 128-bit loads per thread,
  *       workgroups per row); all three must be set, 0 = automatic (default).

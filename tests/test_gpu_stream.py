@@ -263,17 +263,13 @@ def test_random_shapes_k_and_row_kinds_on_whatever_route_they_take(ops, seed):
     comparison of the library's own choice of kernels with the kernels rows.path = 1 selects and
     with the oracle: the shapes between the ones the other tests name (this is how the rows of
     one repeated value and three peaks, and a row that overflowed a wave's stage twice, were found).
-    The kind "flat_with_peaks" is not drawn here: a flat row with dozens of peaks per thousand
-    copies ([n = 20001, k = 16] under seed 23) measured 3 ulp until the scan kernel counted the
-    copies of a value that fills its waves apart -- 1 ulp since on the library's own route -- and
-    still measures 3 ulp on the chunk + merge kernels over several chunks, which this comparison
-    forces with rows.path = 1 (their wave records have no room for the count): the one known
-    excess over the 2-ulp bar.  The kind is tested on the library's routes in
-    test_rows_of_equal_and_clustered_values_on_every_route and
-    test_rows_of_one_repeated_value_and_a_few_peaks."""
+    A flat row with dozens of peaks per thousand copies ([n = 20001, k = 16] under seed 23) measured
+    3 ulp on every streaming route until their waves counted the copies of a value that fills them
+    apart (a record word of its own: the scan kernel's, then the chunk kernel's): the kind
+    "flat_with_peaks" is drawn like any other."""
     from vkop_amd import capi
     rng = np.random.default_rng(seed)
-    kinds_all = [t for t in dict.fromkeys(KINDS + TIE_KINDS + WALK_KINDS) if t != "flat_with_peaks"]
+    kinds_all = list(dict.fromkeys(KINDS + TIE_KINDS + WALK_KINDS))
     ns = [33, 64, 100, 255, 256, 257, 777, 1000, 1024, 2047, 2048, 4096, 5000, 8191, 8192, 8400, 12000, 16384, 20001, 32768, 40000,
           50257, 65536, 100000, 128256, 200003]
     ks = [1, 2, 5, 8, 16, 31, 32, 33, 50, 64, 65, 100, 128, 159, 160, 200, 255, 256, 257, 300, 408, 409, 500, 511, 512, 600, 1024, 2000, 2048]
@@ -286,6 +282,33 @@ def test_random_shapes_k_and_row_kinds_on_whatever_route_they_take(ops, seed):
         capi.tune("rows.path", 0)
         path = capi.measure_path(capi.F32 if dtype == np.float32 else capi.F16, (rows, n), -1, k)
         _compare_paths(ops, n, k, dtype, rows, kinds, path)
+
+
+@pytest.mark.parametrize("rows,n,k", [(17, 20001, 16), (8, 20001, 16), (24, 50000, 40), (5, 131072, 64), (16, 16385, 5)])
+def test_flat_rows_with_dozens_of_peaks_on_the_chunk_and_merge_kernels(ops, rows, n, k):
+    """The chunk + merge kernels over several chunks (rows.path = 1: no shape takes them by itself any
+    more) on rows that are one value and dozens of peaks: most waves hold a larger element beside the
+    copies, all of them sum against references of their own, and the copies' common term error came to
+    3 ulp of the probabilities (n = 20001, k = 16) until the chunk kernel's waves counted the copies
+    apart, in a record word of their own, for the merge to add them as the sum is defined."""
+    from vkop_amd import capi
+    rng = np.random.default_rng(rows * 1000 + k)
+    x = np.full((rows, n), np.float32(-0.3))
+    for r in range(rows):
+        at = rng.choice(n, size=20 + 13 * r, replace=False)
+        x[r, at] = np.float32(2.0) + rng.random(at.size).astype(np.float32)
+    ov, oix = oracle.softmax_topk(x, k)
+    try:
+        capi.tune("rows.path", 1)
+        assert capi.measure_path(capi.F32, (rows, n), -1, k) == 1 and capi.rows_plan(capi.F32, (rows, n), -1, k)[2] > 1
+        v, ix = ops.softmax_topk(dev(x), k)
+        v, ix = host(v), host(ix)
+    finally:
+        capi.tune("rows.path", 0)
+    assert np.array_equal(ix, oix), (rows, n, k)
+    assert ulp_diff(v, ov).max() <= 2, (rows, n, k, int(ulp_diff(v, ov).max()))
+    v0, ix0 = ops.softmax_topk(dev(x), k)
+    assert np.array_equal(host(ix0), oix) and ulp_diff(host(v0), ov).max() <= 2, (rows, n, k)
 
 
 @pytest.mark.parametrize("n", [16388, 40002, 128255])

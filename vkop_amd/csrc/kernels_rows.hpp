@@ -253,12 +253,15 @@ __device__ __forceinline__ void drain_stores() {
     __builtin_amdgcn_s_waitcnt(0);                          // vmcnt(0) expcnt(0) lgkmcnt(0)
 }
 
+constexpr int kRecWords = 4;  // 64-bit words of a chunk-kernel wave's record
 struct RowsWorkspace {
     uint32_t *tickets;  // [rows]: chunks of the row that have published; 0 between calls
-    uint64_t *sums;     // [rows][G * waves per chunk][3]: the wave's sum of exp(x - ref) as double bits; ref (low
+    uint64_t *sums;     // [rows][G * waves per chunk][kRecWords]: the wave's sum of exp(x - ref) as double bits; ref (low
                         // half) and the wave's maximum (high half) as float bits; the candidates the wave
                         // contributed to its chunk's list (low half; all ones: it could not stage them all)
-                        // and the chunk's threshold as an order key (high half)
+                        // and the chunk's threshold as an order key (high half); the value whose copies the
+                        // wave counted apart (float bits, high half) and how many it found (low half; 0: none):
+                        // its sum leaves them out
     uint64_t *cand;     // [rows][G][cap]: composites (order key, ~index) of the elements at or above the chunk threshold
     uint32_t cap;       // candidate slots per chunk (power of two)
     uint32_t cap_shift;
@@ -911,8 +914,9 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     // ---- A. everything the merge reads, in one round trip ---------------------------
     // (never a branch around a load: out-of-range threads re-read entry 0)
     const uint32_t wq = tid < waves ? tid : 0u;
-    const uint64_t s_bits = fetch(sums + 3 * wq);
-    const uint64_t rm_bits = fetch(sums + 3 * wq + 1);
+    const uint64_t s_bits = fetch(sums + kRecWords * wq);
+    const uint64_t rm_bits = fetch(sums + kRecWords * wq + 1);
+    const uint64_t c_bits = fetch(sums + kRecWords * wq + 3);
     // thread b < G adds up the candidate counts of chunk b's waves
     // (four loads in flight at a time; a chunk workgroup has 4, 8 or 16 waves)
     uint64_t cm = 0;       // the chunk's candidates, all ones if any of its waves overflowed
@@ -921,7 +925,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         uint64_t c[4];
 #pragma unroll
         for (int u = 0; u < 4; u++)  // (a one-wave workgroup has a single record: it is read four times, counted once)
-            c[u] = fetch(sums + 3 * ((tid < G ? tid : 0u) * src_nw + (w0 + u < src_nw ? w0 + u : 0u)) + 2);
+            c[u] = fetch(sums + kRecWords * ((tid < G ? tid : 0u) * src_nw + (w0 + u < src_nw ? w0 + u : 0u)) + 2);
 #pragma unroll
         for (int u = 0; u < 4; u++) {
             const uint32_t cnt = w0 + u < src_nw ? static_cast<uint32_t>(c[u]) : 0u;
@@ -956,13 +960,18 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         p0.ref = __uint_as_float(static_cast<uint32_t>(rm_bits));
         p0.m = __uint_as_float(static_cast<uint32_t>(rm_bits >> 32));
         sh.ref[tid] = p0.ref;
-        sh.x0[tid] = __uint_as_float(0x7FC00000u);  // (the chunk kernel's sums leave nothing out)
+        sh.x0[tid] = static_cast<uint32_t>(c_bits) != 0u ? __uint_as_float(static_cast<uint32_t>(c_bits >> 32)) : __uint_as_float(0x7FC00000u);
     }
     if (tid < G) {
         sh.cnt[tid] = static_cast<uint32_t>(cm < cap ? cm : cap);
         sh.cthr[tid] = cthr;
         bad = cm > cap;
     }
+    // the copies the wave counted apart: each counts exp_accurate(fl(x0 - M)), as the sum is defined
+    auto copies_term = [&](float m) -> double {
+        const uint32_t cn = (SOFTMAX && tid < waves) ? static_cast<uint32_t>(c_bits) : 0u;
+        return cn != 0u ? static_cast<double>(cn) * static_cast<double>(softmax_term(__uint_as_float(static_cast<uint32_t>(c_bits >> 32)), m)) : 0.0;
+    };
     // With at most 64 wave records (one per lane of wave 0) that wave alone combines
     // them, by cross-lane steps, while the others go on to the threshold; the
     // results are published by the barrier there.
@@ -975,6 +984,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                 sh.scale[tid] = sc;
                 if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
             }
+            acc += copies_term(m);
             const double total = wave_sum_f64_uniform(acc);
             if (lane == 0) {
                 sh.row_max = m;
@@ -989,6 +999,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
             sh.scale[tid] = sc;
             if (SOFTMAX && p0.s != 0.0) acc = p0.s * sc;
         }
+        acc += copies_term(m);
         const double total = block_sum_fast<NT>(acc, dscratch);  // (barrier: sh.scale is published)
         if (tid == 0) {
             sh.row_max = m;
@@ -1238,7 +1249,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
     __shared__ std::conditional_t<FUSED, RowsSharedUnion<NT>, ChunkShared<NT>> smem;
     __shared__ float fscratch[FUSED ? NW : 1];
     __shared__ double dscratch[FUSED ? NW : 1];
-    __shared__ uint64_t local_ws[LOCAL ? kLocalCap + 3 * NW : 1];  // candidate list, then the wave records
+    __shared__ uint64_t local_ws[LOCAL ? kLocalCap + kRecWords * NW : 1];  // candidate list, then the wave records
 #ifdef VKOP_STAMPS
     const unsigned long long dbg_t0 = wall_clock64();
 #endif
@@ -1293,6 +1304,9 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         float lmax = -INFINITY, ref = 0.f;
         double acc = 0.0;
         uint32_t lkey = 0u;
+        float x0 = __uint_as_float(0x7FC00000u);  // the value whose copies the wave counts apart (NaN: equal to nothing)
+        bool counting = false;
+        uint32_t counted = 0;  // this lane's copies
         if constexpr (SOFTMAX && LOCAL) {
             // A row in one workgroup is summed by a few waves, and against the ROW's maximum:
             // fl(x - ref) is then the subtraction the softmax definition itself rounds.  (Against
@@ -1333,6 +1347,15 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     // NaN, which must survive -- never -inf - -inf)
                     const float wm0 = wave_max_f32_uniform(vm);
                     ref = (wm0 > -INFINITY) ? wm0 + kRefLift : 0.f;
+                    // The copies of one value -- the wave's first element, where half of the lanes' first
+                    // elements equal it: a value that fills a row turns up at once -- are counted after the
+                    // loop and left out of the sum: every copy has the same term, so its error would enter
+                    // the sum once per copy; the merge, which knows the row's maximum, adds
+                    // exp_accurate(fl(x0 - M)) for each of them instead.
+                    const float first = __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(__float_as_uint(xv[0])))));
+                    const bool mine = xv[0] == first && first > -INFINITY && first < INFINITY;
+                    x0 = first;
+                    counting = __popcll(__ballot(mine)) >= kWave / 2;
                 }
 #pragma unroll
                 for (int c = 0; c < VEC; c++) acc += static_cast<double>(fast_term_as<LOCAL>(xv[c], ref));  // (a row in one workgroup: few waves)
@@ -1397,8 +1420,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         if constexpr (LOCAL) cand_out = local_ws;
         else cand_out = ws.cand + (static_cast<size_t>(row * G + chunk) << ws.cap_shift);
         uint64_t *record;  // this wave's
-        if constexpr (LOCAL) record = local_ws + kLocalCap + 3 * wave;
-        else record = ws.sums + 3 * static_cast<size_t>(went);
+        if constexpr (LOCAL) record = local_ws + kLocalCap + kRecWords * wave;
+        else record = ws.sums + kRecWords * static_cast<size_t>(went);
         uint4 *stv = cs.stage_v + wave * kWave;
         uint32_t *ste = cs.stage_e + wave * kWave;
         auto compact = [&](uint32_t thr_key, uint32_t &staged_vectors) -> uint32_t {
@@ -1473,6 +1496,23 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         BPS(49);
 
         // ---- the wave's partial sum (here, so that none of it is live across what follows) ------
+        uint32_t copies = 0;  // wave-uniform: the copies of x0 the sum leaves out
+        if constexpr (SOFTMAX && !LOCAL) {
+            if (counting) {  // (wave-uniform; everything is still in registers)
+                uint32_t ncopy = 0;
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) ncopy += (in_range(ALIGNED ? e0 : e0 + c) && q[i].get(c) == x0) ? 1u : 0u;
+                }
+                // (every copy added the same float: taking them out again is exact to the sum's own rounding)
+                if (ncopy != 0u) acc -= static_cast<double>(ncopy) * static_cast<double>(fast_term(x0, ref));
+                wsum = wave_sum_f64_uniform(acc);
+                copies = static_cast<uint32_t>(wave_sum_f64_uniform(static_cast<double>(ncopy)));
+                counted = ncopy;
+            }
+        }
         if constexpr (SOFTMAX) {
             if (wm - ref > kTermSwitch) {  // wave-uniform
                 // an element well above the reference: its fast term is poor (or has
@@ -1488,12 +1528,14 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                         acc += static_cast<double>(fast_term_as<LOCAL>(x, ref));
                     }
                 }
+                if (counted != 0u) acc -= static_cast<double>(counted) * static_cast<double>(fast_term(x0, ref));
                 wsum = wave_sum_f64_uniform(acc);
             }
         }
         if (lane == 0) {
             publish(record, static_cast<uint64_t>(__double_as_longlong(wsum)));
             publish(record + 1, (static_cast<uint64_t>(__float_as_uint(wm)) << 32) | __float_as_uint(ref));
+            publish(record + 3, (static_cast<uint64_t>(__float_as_uint(x0)) << 32) | copies);
         }
         __syncthreads();
         if (__builtin_expect(cs.total > ws.cap || cs.over != 0u, 0)) {
@@ -1790,7 +1832,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         if (s_last == 0u) return;
         merge_row<T, NT, SOFTMAX>(smem.fast, smem.exact, fscratch, dscratch, rowp, values + static_cast<size_t>(row) * k,
                                   indices + static_cast<size_t>(row) * k, n, k, G, per, NT,
-                                  ws.sums + 3 * static_cast<size_t>(row) * G * NW,
+                                  ws.sums + kRecWords * static_cast<size_t>(row) * G * NW,
                                   ws.cand + (static_cast<size_t>(row) * G << ws.cap_shift), ws.cap_shift);
     } else {
         (void)values;
@@ -1821,7 +1863,7 @@ __global__ __launch_bounds__(kMergeThreads) void rows_merge_kernel(const T *__re
     merge_row<T, kMergeThreads, SOFTMAX, RECS>(smem.fast, smem.exact, fscratch, dscratch, in + static_cast<size_t>(row) * n,
                                          values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k,
                                          n, k, G, per, src_nt,
-                                         ws.sums + 3 * static_cast<size_t>(row) * G * (src_nt / kWave),
+                                         ws.sums + kRecWords * static_cast<size_t>(row) * G * (src_nt / kWave),
                                          ws.cand + (static_cast<size_t>(row) * G << ws.cap_shift), ws.cap_shift);
 }
 

@@ -650,7 +650,7 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
     } else if (c.ok) {
         const size_t chunks = lines * c.g;
         l.sums = off;
-        off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * 3 * sizeof(uint64_t));
+        off += align_up(chunks * (static_cast<size_t>(c.nt) / 64) * vkop::kRecWords * sizeof(uint64_t));
         l.cand = off;
         off += align_up(chunks * c.cap * sizeof(uint64_t));
     } else if (b.ok) {
