@@ -88,6 +88,32 @@ def traffic_from_profiles(workload, kernel):
     return int(m.group(3)) if m else None
 
 
+def runtime_api_leg(runs=200):
+    """The headline tensor through the operator interface a user of the reference has: the C++
+    program's benchmark mode registers SOFTMAX + TOPK as post-processing of a [64,128256] output and
+    calls Runtime::Run() in a loop, as benchmark/main.cpp:112-137 does, reporting the mean of the
+    wall-clock milliseconds Run() returns.  Run as a child process, before this process touches the
+    GPU."""
+    import subprocess
+    exe = os.path.join(ROOT, "vkop_amd", "host", "build", "test_ops")
+    if not os.path.exists(exe):
+        return {"error": "vkop_amd/host/build/test_ops is not built (make -C vkop_amd/host)"}
+    try:
+        r = subprocess.run([exe, "--bench-runtime", str(runs)], capture_output=True, text=True, timeout=300,
+                           cwd=os.path.join(ROOT, "vkop_amd", "host"))
+        legs = [json.loads(line) for line in r.stdout.splitlines() if line.startswith("{")]
+        if r.returncode != 0 or not legs:
+            return {"error": "test_ops --bench-runtime failed (%d): %s" % (r.returncode, (r.stderr or r.stdout)[-300:])}
+        out = {"what": legs[0]["what"], "shape": legs[0]["shape"], "k": legs[0]["k"], "runs": legs[0]["runs"],
+               "calls_in_flight": 1, "queues": "the runtime's own two (core/Runtime.hpp kInflight), one operator chain"}
+        for leg in legs:
+            out["fused" if leg["fused"] else "two_operators"] = {"mean_ms": leg["mean_ms"], "min_ms": leg["min_ms"],
+                                                                 "operators": leg["operators"]}
+        return out
+    except Exception as exc:  # the figure is informative only
+        return {"error": str(exc)}
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -181,6 +207,12 @@ def main():
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-host", action="store_true", help="skip the host-buffer (PCIe) round-trip leg")
+    ap.add_argument("--no-runtime-api", action="store_true", help="skip the Runtime::Run() leg (the C++ program as a child process)")
+    ap.add_argument("--kernel-legs", action="store_true",
+                    help="run only the legs that time each kernel of the step by itself and print them as one JSON line: "
+                         "they need the benchmark build of the library (libvkop_hip_bench.so, whose measurement hook can "
+                         "leave a kernel out of a call), so bench.py runs them in a child process of this form while its own "
+                         "figures come from the library that ships")
     ap.add_argument("--hw-queues", type=int, default=DEFAULT_HW_QUEUES,
                     help="hardware queues this process may use (GPU_MAX_HW_QUEUES); 0 = leave the environment as it is")
     ap.add_argument("--inflight", type=int, default=0,
@@ -208,12 +240,29 @@ def main():
               "(rows are independent: shard the batch and run one process per GPU)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
+    # (child processes, before this one initialises the GPU)
+    runtime_api = None if (args.kernel_legs or args.no_runtime_api or args.workload != "C3") else runtime_api_leg()
+    kernel_legs = None
+    if not args.kernel_legs and not args.eager:
+        import subprocess
+        cmd = [sys.executable, os.path.abspath(__file__), "--kernel-legs", "--steps", str(args.steps), "--warmup", str(args.warmup),
+               "--workload", args.workload, "--hw-queues", str(args.hw_queues), "--inflight", str(args.inflight),
+               "--rows-path", str(args.rows_path)] + (["--no-gate"] if args.no_gate else [])
+        try:
+            r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+            lines = [line for line in r.stdout.splitlines() if line.startswith("{")]
+            kernel_legs = json.loads(lines[-1]) if r.returncode == 0 and lines else {"error": (r.stderr or r.stdout)[-300:]}
+        except Exception as exc:
+            kernel_legs = {"error": str(exc)}
+
     import numpy as np
     import torch
 
     import oracle
     from vkop_amd import capi, synth
 
+    if args.kernel_legs:
+        capi.use_bench_library()
     capi.lib()
     capi.init(0)
     capi.tune("rows.path", args.rows_path)
@@ -343,14 +392,20 @@ def main():
     MIN_TIMED = 400
     replays = max(1, -(-MIN_TIMED // args.steps))
 
+    def set_stages(stages):
+        if args.kernel_legs:
+            capi.measure_stages(stages)
+        elif stages != 3:
+            raise RuntimeError("one kernel by itself: only with --kernel-legs (the benchmark build of the library)")
+
     def timed(stages, nlanes, nb=nbuf, prime=False):
         """(device ms per step, host wall ms per step of ungated replays) after W warm-up steps."""
-        capi.measure_stages(3)
+        set_stages(3)
         if prime:   # leave in every lane's workspace what a whole call on the (single) buffer leaves
             for ln in lanes[:nlanes]:
                 call(bufs[0], ln)
                 capi.stream_sync(ln["stream"])
-        capi.measure_stages(stages)
+        set_stages(stages)
         graphs = []
         if args.warmup > 0:
             gw = record(args.warmup, 0, nlanes, nb)
@@ -392,7 +447,7 @@ def main():
         if not args.eager:
             for g in graphs:
                 capi.graph_destroy(g)
-        capi.measure_stages(3)
+        set_stages(3)
         n = replays * args.steps
         return max(capi.event_elapsed_ms(e0, e1), 0.0) / n, wall / n
 
@@ -404,16 +459,23 @@ def main():
     path = capi.measure_path(capi.F32, shape, -1, k)
     names = PATH_KERNELS.get(path)
     two_kernels = names is not None and plan[2] > 1
-    serial_ms = timed(3, 1)[0]
-    if two_kernels:
+    if args.kernel_legs:
         # one call in flight.  The second kernel by itself reads the workspace an earlier whole call
         # left; the pick kernel also reads the input again, so it is timed on one buffer with
         # that buffer's workspace (its few re-reads then come from the cache)
-        stage_ms[names[0]] = timed(1, 1)[0]
-        stage_ms[names[1]] = timed(2, 1, 1, True)[0] if path == 2 else timed(2, 1)[0]
-        if len(lanes) > 1:
-            stage_overlapped = {names[0]: timed(1, len(lanes))[0] * 1e3,
-                                names[1]: (timed(2, len(lanes), 1, True)[0] if path == 2 else timed(2, len(lanes))[0]) * 1e3}
+        if two_kernels:
+            stage_ms[names[0]] = timed(1, 1)[0]
+            stage_ms[names[1]] = timed(2, 1, 1, True)[0] if path == 2 else timed(2, 1)[0]
+            if len(lanes) > 1:
+                stage_overlapped = {names[0]: timed(1, len(lanes))[0] * 1e3,
+                                    names[1]: (timed(2, len(lanes), 1, True)[0] if path == 2 else timed(2, len(lanes))[0]) * 1e3}
+        print(json.dumps({"stage_ms": stage_ms, "stage_overlapped": stage_overlapped,
+                          "library": os.path.basename(capi.LIB_PATH)}))
+        return
+    if kernel_legs is not None and "stage_ms" in kernel_legs:
+        stage_ms = kernel_legs["stage_ms"]
+        stage_overlapped = kernel_legs["stage_overlapped"]
+    serial_ms = timed(3, 1)[0]
     ms_per_step, wall_per_step = timed(3, len(lanes))
     resident_ms = timed(3, len(lanes), 1)[0]
     # the kernel that moves the bytes (the first of the pair; the second reads a few kilobytes per row)
@@ -455,7 +517,10 @@ def main():
                      "whole_step_us_one_in_flight": serial_ms * 1e3,
                      "whole_step_frac_one_in_flight": algo_bytes / (serial_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "timing": "HIP events on the launch stream around %d back-to-back launches of that kernel alone, one "
-                               "call in flight (recorded submissions); includes the gap between launches" % (replays * args.steps)},
+                               "call in flight (recorded submissions); includes the gap between launches; measured in a child "
+                               "process on libvkop_hip_bench.so, the library's build with the hook that leaves the other kernel "
+                               "out (every other figure: libvkop_hip.so)" % (replays * args.steps),
+                     "kernel_legs_error": (kernel_legs or {}).get("error")},
         "parity": parity,
     }
     # For a caller whose logits sit in host memory: upload over PCIe from pinned
@@ -488,6 +553,8 @@ def main():
                                        "blocking copies, one call at a time (host clock)"}
     except Exception as exc:  # the figure is informative only
         out["host_buffers"] = {"error": str(exc)}
+    if runtime_api is not None:
+        out["runtime_api"] = runtime_api
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(host_inputs[0], k)
     capi.event_destroy(e0)

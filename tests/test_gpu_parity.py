@@ -348,7 +348,11 @@ def test_topk_long_rows_nan_inf(ops):
 
 # -------------------------------------------------------------------- fused --
 
-def assert_fused(ops, x, k, axis=-1, largest=True):
+def assert_fused(ops, x, k, axis=-1, largest=True, rows_may_differ=0):
+    """rows_may_differ: how many rows of step (3) may come out in another order than the tensor
+    route's -- by a probability tie that the two routes' row sums, an ulp apart, open or close; the
+    ceiling a test passes is what its seeded inputs measure (0 on every case so far), so that a
+    change that moves it shows."""
     v, ix, p = ops.softmax_topk(dev(x), k, axis, largest, return_probs=True)
     v, ix, p = host(v), host(ix), host(p)
     # (1) exactly the top-k of the softmax tensor the same call wrote
@@ -379,9 +383,8 @@ def assert_fused(ops, x, k, axis=-1, largest=True):
             if not np.array_equal(i2[r], i1[r]):
                 tolerant += 1
                 assert sorted(pm[r][i2[r]].tolist()) == sorted(pm[r][i1[r]].tolist()), r
-        print("assert_fused %s k=%d: %d of %d rows differ from the tensor route by a tie the row sum opened or closed"
-              % (x.shape, k, tolerant, pm.shape[0]))
-        assert tolerant <= max(1, pm.shape[0] // 5), (tolerant, pm.shape[0])
+        assert tolerant <= rows_may_differ, "%s k=%d: %d of %d rows differ from the tensor route by a tie the row sum opened or closed (ceiling %d)" % (
+            x.shape, k, tolerant, pm.shape[0], rows_may_differ)
     if largest:
         # whichever way such a tie went, the result is ranked by (probability, then lower
         # index) of a monotone function of the logits: checked on the logits themselves
@@ -808,9 +811,9 @@ def test_awkward_rows_against_the_oracle(ops, n, k):
             d = half_ulp_diff(v[r], ev[r]) if dtype == np.float16 else ulp_diff(v[r], ev[r])
             assert d.max() <= 1, (r, n, k)
             assert len(set(ix[r].tolist())) == k
-        print("awkward rows n=%d k=%d %s: %d of %d rows differ from the tensor route by a tie the row sum opened or closed"
-              % (n, k, np.dtype(dtype).name, int((~rows_equal).sum()), len(rows_equal)))
-        assert rows_equal.mean() > 0.8
+        # (how many: 0 of 24 on every case here; the ceiling is that measurement, so that a change which moves it shows)
+        assert int((~rows_equal).sum()) <= 0, "n=%d k=%d %s: %d of %d rows differ from the tensor route by a tie the row sum opened or closed" % (
+            n, k, np.dtype(dtype).name, int((~rows_equal).sum()), len(rows_equal))
         # every row, tolerant branch or not: ranked by (probability, then lower index) of a
         # monotone function of the logits; and exactly the oracle's indices wherever its
         # probabilities around the cut are well apart (or tie through equal logits)

@@ -12,6 +12,10 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(_HERE)
 LIB_PATH = os.path.join(_HERE, "libvkop_hip.so")
+# the same library built with the benchmark's hook (vkop_hip_measure_stages): bench.py's per-kernel legs load
+# this one instead, in a process of their own (use_bench_library() before the first lib())
+BENCH_LIB_PATH = os.path.join(_HERE, "libvkop_hip_bench.so")
+BENCH_ONLY = ("vkop_hip_measure_stages",)
 HEADER_PATH = os.path.join(ROOT, "include", "vkop_hip.h")
 
 OK, ERR_INVALID, ERR_DEVICE, ERR_WORKSPACE, ERR_UNSUPPORTED = 0, 1, 2, 3, 4
@@ -38,8 +42,17 @@ def declared_symbols():
     return sorted(set(re.findall(r"\b(vkop_hip_[a-z0-9_]+)\s*\(", text)))
 
 
+def use_bench_library():
+    """Load libvkop_hip_bench.so instead of libvkop_hip.so (only before the first lib())."""
+    global LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("the library is loaded already")
+    LIB_PATH = BENCH_LIB_PATH
+
+
 def internal_symbols():
-    """Names of the measurement hooks vkop_amd/csrc/vkop_hip_internal.h declares (not part of the public interface)."""
+    """Names of the measurement hooks vkop_amd/csrc/vkop_hip_internal.h declares (not part of the public interface;
+    those in BENCH_ONLY exist in libvkop_hip_bench.so alone)."""
     text = open(os.path.join(_HERE, "csrc", "vkop_hip_internal.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(vkop_hip_[a-z0-9_]+)\s*\(", text)))
@@ -103,6 +116,9 @@ def lib():
         "vkop_hip_measure_path": (i, [i, ip, i, i, i]),
         "vkop_hip_rows_plan": (i, [i, ip, i, i, i, ip, ip, ip]),
     }
+    for name in BENCH_ONLY:
+        if not hasattr(L, name):
+            del sig[name]
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
         fn.restype = res
@@ -275,7 +291,10 @@ def tune(name, value):
 
 def measure_stages(stages):
     """Benchmarks only (vkop_amd/csrc/vkop_hip_internal.h): launch only the first (1) or second (2) kernel of a
-    two-kernel streaming call, or both (3, the normal state).  Results are not valid with 1 or 2."""
+    two-kernel streaming call, or both (3, the normal state).  Results are not valid with 1 or 2.
+    libvkop_hip_bench.so only (use_bench_library())."""
+    if not hasattr(lib(), "vkop_hip_measure_stages"):
+        raise RuntimeError("vkop_hip_measure_stages exists only in libvkop_hip_bench.so: call capi.use_bench_library() first")
     check(lib().vkop_hip_measure_stages(int(stages)))
 
 

@@ -127,8 +127,16 @@ int resolve_static_scratch(void **ptr, int *device) {
 }
 
 // vkop_hip_tune state
-std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_stages{3}, g_rows_fused{0}, g_rows_path{0},
+std::atomic<int> g_rows_threads{0}, g_rows_loads{0}, g_rows_chunks{0}, g_rows_fused{0}, g_rows_path{0},
     g_nms_threads{0};
+// Which kernels of a two-kernel streaming call are launched: both, except in the benchmark build of the
+// library (-DVKOP_BENCH_HOOKS, libvkop_hip_bench.so), where vkop_hip_measure_stages can leave one out.
+#ifdef VKOP_BENCH_HOOKS
+std::atomic<int> g_rows_stages{3};
+inline int measured_stages() { return g_rows_stages.load(); }
+#else
+inline int measured_stages() { return 3; }
+#endif
 
 // The per-row arrival counters of the one-kernel top-k variant sit at a fixed
 // place, the first kTicketRows words of every workspace, whatever the operator
@@ -728,7 +736,7 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.v = static_cast<uint32_t>(c.v);
     a.g = c.g;
     a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % vec == 0);
-    a.stages = g_rows_stages.load();
+    a.stages = measured_stages();
     a.scale = scale;
     a.counts = counts;
     a.top_p = top_p;
@@ -787,7 +795,7 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
                                                                                 : vkop::kMergeSplit;
     a.ws = w;
     a.stream = st;
-    const int stages = a.merge != vkop::kMergeSplit ? 1 : g_rows_stages.load();
+    const int stages = a.merge != vkop::kMergeSplit ? 1 : measured_stages();
     if (stages & 1) {
         if (!vkop::launch_rows_chunk<T, SOFTMAX>(a))
             return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_chunk_kernel for %d threads x %d loads", c.nt, c.v);
@@ -1360,11 +1368,13 @@ int vkop_hip_measure_path(int dtype, const int *shape, int ndim, int axis, int k
     return 0;
 }
 
+#ifdef VKOP_BENCH_HOOKS
 int vkop_hip_measure_stages(int stages) {
     if (stages < 1 || stages > 3) return fail(VKOP_HIP_ERR_INVALID, "stages must be 1, 2 or 3");
     g_rows_stages = stages;
     return VKOP_HIP_OK;
 }
+#endif
 
 int vkop_hip_rows_plan(int dtype, const int *shape, int ndim, int axis, int k, int *threads, int *loads,
                        int *chunks) {

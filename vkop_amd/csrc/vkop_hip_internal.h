@@ -1,6 +1,10 @@
 /*
- * Measurement hooks of libvkop_hip.so that are NOT part of its public interface
- * (include/vkop_hip.h): exported for this repository's benchmarks only.
+ * Measurement hooks that are NOT part of the public interface (include/vkop_hip.h):
+ * for this repository's benchmarks and tests only.  vkop_hip_measure_path is a pure
+ * query and part of libvkop_hip.so; vkop_hip_measure_stages changes what a call
+ * launches and exists only in the benchmark build of the library
+ * (libvkop_hip_bench.so: the same objects, the C ABI source compiled with
+ * -DVKOP_BENCH_HOOKS).
  */
 #ifndef VKOP_HIP_INTERNAL_H_
 #define VKOP_HIP_INTERNAL_H_
@@ -14,8 +18,11 @@ extern "C" {
  * first, 2 = only the second (it reads the workspace an earlier whole call left).
  * With 1 or 2 the top-k and fused entry points do NOT produce valid results: the
  * settings exist so that a benchmark can time each kernel by itself with the
- * launches a real call makes.  Not thread-safe; set it back to 3. */
+ * launches a real call makes.  Not thread-safe; set it back to 3.
+ * libvkop_hip_bench.so only. */
+#ifdef VKOP_BENCH_HOOKS
 int vkop_hip_measure_stages(int stages);
+#endif
 
 /* Which streaming kernels a fused / top-k (largest) call on this tensor would run
  * with the current tuning settings: 4 = rows_tiny_kernel (one wave per row), 2 =

@@ -999,7 +999,48 @@ static void model_file_mutation_tests() {
     EXPECT(other == 0 && refused > 1000 && parsed > 1000);
 }
 
+// `--bench-runtime [runs]`: the benchmark's loop (benchmark/main.cpp:112-137) on the headline
+// tensor -- SOFTMAX and TOPK registered as post-processing of a [64,128256] float output,
+// Runtime::Run() called `runs` times after 20 untimed calls -- and the mean of what Run() returns
+// (host wall clock around record + submit + wait), once with the pair fused and once as two
+// operators.  Prints one line of JSON per arrangement, nothing else.
+static int bench_runtime(int runs) {
+    TestEnv::initialize();
+    auto dev = TestEnv::dev;
+    auto pool = TestEnv::pool;
+    const std::vector<int> shape{64, 128256};
+    const int k = 50;
+    torch::manual_seed(11);
+    auto x = torch::randn({shape[0], shape[1]}) * 1.25;
+    for (int fuse = 1; fuse >= 0; fuse--) {
+        auto rt = std::make_shared<vkop::core::Runtime>(pool, "", 0);
+        rt->set_postprocess_fusion(fuse == 1);
+        auto cls = std::make_shared<Tensor<float>>(shape);
+        fill_from_torch(cls, x);
+        cls->as_storage_buffer(dev);
+        cls->copyToGPU(pool);
+        rt->SetOutput(cls);
+        auto sf = std::make_shared<Tensor<float>>(shape, true);
+        rt->RegisterPostProcess(ops::OpType::SOFTMAX, {{"axis", "-1"}}, {cls}, {sf});
+        auto indexs = std::make_shared<Tensor<int>>(shape, true);
+        auto values = std::make_shared<Tensor<float>>(shape, true);
+        rt->RegisterPostProcess(ops::OpType::TOPK, {{"k", std::to_string(k)}}, {sf}, {values, indexs});
+        for (int i = 0; i < 20; i++) rt->Run();
+        double sum = 0, best = 1e30;
+        for (int i = 0; i < runs; i++) {
+            const double ms = rt->Run();
+            sum += ms;
+            best = std::min(best, ms);
+        }
+        std::printf("{\"what\": \"Runtime::Run() of the registered SOFTMAX + TOPK post-processing, host wall clock per run\", "
+                    "\"shape\": [%d, %d], \"k\": %d, \"operators\": %zu, \"fused\": %s, \"runs\": %d, \"mean_ms\": %.6f, \"min_ms\": %.6f}\n",
+                    shape[0], shape[1], k, rt->num_nodes(), fuse ? "true" : "false", runs, sum / runs, best);
+    }
+    return 0;
+}
+
 int main(int argc, char **argv) {
+    if (argc > 1 && std::strcmp(argv[1], "--bench-runtime") == 0) return bench_runtime(argc > 2 ? std::max(1, std::atoi(argv[2])) : 200);
     const bool no_gpu = argc > 1 && std::strcmp(argv[1], "--no-gpu") == 0;
     g_golden = (std::filesystem::path(argv[0]).parent_path() / ".." / ".." / ".." / "tests" / "golden").string();
     host_logic_tests();
