@@ -208,6 +208,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-host", action="store_true", help="skip the host-buffer (PCIe) round-trip leg")
     ap.add_argument("--no-runtime-api", action="store_true", help="skip the Runtime::Run() leg (the C++ program as a child process)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="time only the whole step with the given --hw-queues / --inflight and print a short JSON line (bench.py "
+                         "runs itself this way, as a child process, for the figure with the environment's own number of "
+                         "hardware queues)")
     ap.add_argument("--kernel-legs", action="store_true",
                     help="run only the legs that time each kernel of the step by itself and print them as one JSON line: "
                          "they need the benchmark build of the library (libvkop_hip_bench.so, whose measurement hook can "
@@ -227,6 +231,7 @@ def main():
                     help="run only a plain device copy of known size (the yardstick for the FETCH_SIZE / "
                          "WRITE_SIZE counters) and print its size")
     args = ap.parse_args()
+    env_as_started = dict(os.environ)
     if args.hw_queues > 0:
         os.environ["GPU_MAX_HW_QUEUES"] = str(min(args.hw_queues, 32))
     hw_queues = int(os.environ.get("GPU_MAX_HW_QUEUES", "4"))
@@ -241,9 +246,27 @@ def main():
         sys.exit(2)
 
     # (child processes, before this one initialises the GPU)
-    runtime_api = None if (args.kernel_legs or args.no_runtime_api or args.workload != "C3") else runtime_api_leg()
+    child = args.kernel_legs or args.headline_only
+    runtime_api = None if (child or args.no_runtime_api or args.workload != "C3") else runtime_api_leg()
     kernel_legs = None
-    if not args.kernel_legs and not args.eager:
+    default_queues = None
+    if not child and not args.eager and args.hw_queues > 0:
+        # the same step in the environment this process was started in (GPU_MAX_HW_QUEUES as it is: HIP's default
+        # is 4, one of which the default stream takes): what a caller who changes nothing sees
+        import subprocess
+        legs = {}
+        for name, inflight in (("same_calls_in_flight", max(1, args.inflight if args.inflight > 0 else 4)), ("calls_in_flight_3", 3)):
+            cmd = [sys.executable, os.path.abspath(__file__), "--headline-only", "--hw-queues", "0", "--inflight", str(inflight),
+                   "--steps", str(args.steps), "--warmup", str(args.warmup), "--workload", args.workload,
+                   "--rows-path", str(args.rows_path)] + (["--no-gate"] if args.no_gate else [])
+            try:
+                r = subprocess.run(cmd, capture_output=True, text=True, timeout=600, env=env_as_started)
+                lines = [line for line in r.stdout.splitlines() if line.startswith("{")]
+                legs[name] = json.loads(lines[-1]) if r.returncode == 0 and lines else {"error": (r.stderr or r.stdout)[-300:]}
+            except Exception as exc:
+                legs[name] = {"error": str(exc)}
+        default_queues = legs
+    if not child and not args.eager:
         import subprocess
         cmd = [sys.executable, os.path.abspath(__file__), "--kernel-legs", "--steps", str(args.steps), "--warmup", str(args.warmup),
                "--workload", args.workload, "--hw-queues", str(args.hw_queues), "--inflight", str(args.inflight),
@@ -472,6 +495,12 @@ def main():
         print(json.dumps({"stage_ms": stage_ms, "stage_overlapped": stage_overlapped,
                           "library": os.path.basename(capi.LIB_PATH)}))
         return
+    if args.headline_only:
+        ms, wall = timed(3, len(lanes))
+        print(json.dumps({"ms_per_step": ms, "rows_per_s": rows / (ms * 1e-3), "host_wall_ms_per_step": wall,
+                          "calls_in_flight": len(lanes), "hw_queues": hw_queues,
+                          "GPU_MAX_HW_QUEUES": os.environ.get("GPU_MAX_HW_QUEUES", "unset (HIP's default: 4)")}))
+        return
     if kernel_legs is not None and "stage_ms" in kernel_legs:
         stage_ms = kernel_legs["stage_ms"]
         stage_overlapped = kernel_legs["stage_overlapped"]
@@ -553,6 +582,8 @@ def main():
                                        "blocking copies, one call at a time (host clock)"}
     except Exception as exc:  # the figure is informative only
         out["host_buffers"] = {"error": str(exc)}
+    if default_queues is not None:
+        out["with_the_environments_hw_queues"] = default_queues
     if runtime_api is not None:
         out["runtime_api"] = runtime_api
     if not args.no_cpu:

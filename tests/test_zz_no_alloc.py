@@ -33,25 +33,31 @@ def _dev(a):
     return torch.from_numpy(a).cuda()
 
 
-def _with_workspace(capi, xd, k):
+def _out_shape(shape, axis, k):
+    out = list(shape)
+    out[axis] = k
+    return out
+
+
+def _with_workspace(capi, xd, k, axis=-1, largest=1):
     dt = capi.F32 if xd.dtype == torch.float32 else capi.F16
     shape = list(xd.shape)
-    need = capi.softmax_topk_workspace_bytes(dt, shape, -1, k)
+    need = capi.softmax_topk_workspace_bytes(dt, shape, axis, k)
     ws = torch.zeros(max(need, 4) // 4 + 64, dtype=torch.int32, device="cuda")
     ptr = (ws.data_ptr() + 255) // 256 * 256
-    vals = torch.empty(shape[:-1] + [k], dtype=xd.dtype, device="cuda")
-    idx = torch.empty(shape[:-1] + [k], dtype=torch.int32, device="cuda")
-    capi.softmax_topk(xd.data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), dt, shape, -1, k, 1, ptr, need, 0)
+    vals = torch.empty(_out_shape(shape, axis, k), dtype=xd.dtype, device="cuda")
+    idx = torch.empty(_out_shape(shape, axis, k), dtype=torch.int32, device="cuda")
+    capi.softmax_topk(xd.data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), dt, shape, axis, k, largest, ptr, need, 0)
     torch.cuda.synchronize()
     return vals.cpu().numpy(), idx.cpu().numpy(), need
 
 
-def _static(capi, xd, k):
+def _static(capi, xd, k, axis=-1, largest=1):
     dt = capi.F32 if xd.dtype == torch.float32 else capi.F16
     shape = list(xd.shape)
-    vals = torch.full(shape[:-1] + [k], -1.0, dtype=xd.dtype, device="cuda")
-    idx = torch.full(shape[:-1] + [k], -1, dtype=torch.int32, device="cuda")
-    capi.softmax_topk_static(xd.data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, shape, -1, k, 1, 0)
+    vals = torch.full(_out_shape(shape, axis, k), -1.0, dtype=xd.dtype, device="cuda")
+    idx = torch.full(_out_shape(shape, axis, k), -1, dtype=torch.int32, device="cuda")
+    capi.softmax_topk_static(xd.data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, shape, axis, k, largest, 0)
     torch.cuda.synchronize()
     return vals.cpu().numpy(), idx.cpu().numpy()
 
@@ -60,11 +66,11 @@ def _bits(a):
     return a.view(np.uint32) if a.dtype == np.float32 else a.view(np.uint16)
 
 
-def _same(capi, x, k, what):
+def _same(capi, x, k, what, axis=-1, largest=1):
     xd = _dev(x)
-    ev, ei, need = _with_workspace(capi, xd, k)
+    ev, ei, need = _with_workspace(capi, xd, k, axis, largest)
     assert need <= capi.STATIC_SCRATCH_BYTES, what
-    gv, gi = _static(capi, xd, k)
+    gv, gi = _static(capi, xd, k, axis, largest)
     assert np.array_equal(gi, ei), what + ": indices differ"
     assert np.array_equal(_bits(gv), _bits(ev)), what + ": values differ"
 
@@ -87,6 +93,32 @@ def test_static_scratch_large_k_route_and_ties(capi):
     x = synth.grid_values(2, 65536, seed=45)
     _same(capi, x, 600, "grid [2,65536] k=600")
     _same(capi, x[:1, :20000], 300, "grid [1,20000] k=300")
+
+
+def test_static_scratch_on_the_other_routes_each_after_a_call_of_a_different_one(capi):
+    """The array is never cleared between calls: every route has to cope with what another one left.
+    The multi-pass radix select (its histograms, state and counts), the chunk + merge kernels over
+    several chunks (rows.path = 1), lines along a non-last axis (the general kernels' line statistics)
+    and the smallest-first direction, each right after a call that used the same bytes otherwise."""
+    rng = np.random.default_rng(47)
+    scan = synth.llm_logits(8, 65536, seed=48)
+    _same(capi, scan, 40, "scan + pick first")
+    # half-precision rows with too few blocks for the scan kernels at this k: the radix select
+    x = (rng.standard_normal((64, 60000)) * 2).astype(np.float16)
+    assert capi.measure_path(capi.F16, [64, 60000], -1, 300) == 0
+    _same(capi, x, 300, "radix select after scan + pick")
+    _same(capi, scan, 40, "scan + pick after the radix select")
+    try:
+        capi.tune("rows.path", 1)
+        assert capi.measure_path(capi.F32, [6, 40000], -1, 16) == 1 and capi.rows_plan(capi.F32, [6, 40000], -1, 16)[2] > 1
+        _same(capi, synth.llm_logits(6, 40000, seed=49), 16, "chunk + merge over several chunks after scan + pick")
+    finally:
+        capi.tune("rows.path", 0)
+    y = (rng.standard_normal((3, 700, 40)) * 2).astype(np.float32)
+    _same(capi, y, 9, "lines along axis 1 after chunk + merge", axis=1)
+    _same(capi, scan, 25, "smallest first after the line kernels", largest=0)
+    _same(capi, x, 100, "half precision, smallest first", largest=0)
+    _same(capi, scan, 40, "and scan + pick once more")
 
 
 def test_static_scratch_refuses_what_it_cannot_hold(capi):

@@ -855,11 +855,15 @@ FusedPlan plan_fused(const View &v, int k, int dtype, int largest, bool want_pro
 
 template <typename T>
 int fused_impl(const T *in, T *probs, T *values, int32_t *indices, const View &v, int k, int largest, int dtype,
-               void *ws, hipStream_t st) {
+               void *ws, hipStream_t st, size_t ws_limit = ~static_cast<size_t>(0)) {
     if (const int tiny = (largest && probs == nullptr) ? choose_tiny_loads(v, k, dtype) : 0)
         return launch_tiny<T, true>(in, values, indices, v, k, tiny, st);
     const FusedPlan p = plan_fused(v, k, dtype, largest, probs != nullptr);
     const RowsLayout l = rows_layout(v, p.rows, p.big, p.scan);
+    // (the layout the kernels are given is the one checked here: a tuning change between a caller's
+    // size query and this call cannot put it past the end of what the caller holds)
+    if (l.total > ws_limit)
+        return fail(VKOP_HIP_ERR_WORKSPACE, "this call's scratch layout takes %zu bytes, %zu are there", l.total, ws_limit);
     if (p.scan.ok) return launch_scan<T, true>(in, values, indices, v, k, p.scan, ws, l, st);
     if (p.rows.ok) return launch_rows<T, true>(in, values, indices, v, k, p.rows, ws, l, st);
     if (p.big.ok) return launch_bigk<T, true>(in, values, indices, v, k, largest, p.big, ws, l, st);
@@ -1218,10 +1222,10 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values, int
     if (dtype == VKOP_HIP_F32)
         return fused_impl(static_cast<const float *>(in), static_cast<float *>(out_probs),
                           static_cast<float *>(out_values), out_indices, v, k, largest, dtype, workspace,
-                          as_stream(stream));
+                          as_stream(stream), workspace_bytes);
     return fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_probs),
                       static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, workspace,
-                      as_stream(stream));
+                      as_stream(stream), workspace_bytes);
 }
 
 int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *out_indices, int32_t *out_counts, int dtype,
@@ -1288,6 +1292,25 @@ int vkop_hip_softmax_topk_static(const void *in, void *out_values, int32_t *out_
                     need, static_cast<size_t>(VKOP_HIP_STATIC_SCRATCH_BYTES));
     void *sp = nullptr;
     int dev = 0;
+    {
+        // the stream belongs to the current device (each device has its own copy of the array), and the
+        // array's address is looked up outside a recording (vkop_hip_init does it)
+        int cur = 0;
+        VKOP_HIP_TRY(hipGetDevice(&cur));
+        if (stream != nullptr) {
+            int sdev = cur;
+            VKOP_HIP_TRY(hipStreamGetDevice(as_stream(stream), &sdev));
+            if (sdev != cur)
+                return fail(VKOP_HIP_ERR_INVALID, "the stream belongs to device %d, the current device is %d", sdev, cur);
+        }
+        if (cur >= 0 && cur < kMaxDevices && g_scratch_ptr[cur].load(std::memory_order_acquire) == nullptr) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            VKOP_HIP_TRY(hipStreamIsCapturing(as_stream(stream), &cs));
+            if (cs != hipStreamCaptureStatusNone)
+                return fail(VKOP_HIP_ERR_INVALID, "the static scratch of device %d is not resolved yet and the stream is recording: "
+                                                  "call vkop_hip_init(%d) before recording", cur, cur);
+        }
+    }
     if (int rc = resolve_static_scratch(&sp, &dev)) return rc;
     // The array keeps what the last call left.  All a call needs to find at zero
     // are the per-row arrival counters, which every call that completes returns
@@ -1305,10 +1328,11 @@ int vkop_hip_softmax_topk_static(const void *in, void *out_values, int32_t *out_
     int rc;
     if (dtype == VKOP_HIP_F32)
         rc = fused_impl(static_cast<const float *>(in), static_cast<float *>(nullptr), static_cast<float *>(out_values),
-                        out_indices, v, k, largest, dtype, sp, as_stream(stream));
+                        out_indices, v, k, largest, dtype, sp, as_stream(stream), static_cast<size_t>(VKOP_HIP_STATIC_SCRATCH_BYTES));
     else
         rc = fused_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(nullptr),
-                        static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, sp, as_stream(stream));
+                        static_cast<uint16_t *>(out_values), out_indices, v, k, largest, dtype, sp, as_stream(stream),
+                        static_cast<size_t>(VKOP_HIP_STATIC_SCRATCH_BYTES));
     if (rc != VKOP_HIP_OK) g_scratch_dirty[dev].store(1);
     return rc;
 }
