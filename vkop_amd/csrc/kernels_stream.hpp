@@ -72,7 +72,10 @@ struct ScanWorkspace {
 // minimum reaches a value holds 16 * vector width elements that do).
 // One chunk of one row by kScanThreads threads (tid: 0 .. kScanThreads - 1; block: row * G + chunk).
 // No barrier inside, so several chunks can share a workgroup.  vm_lds: [kScanWaves][V][kWave] floats
-// (per wave: the maximum of every lane's vector i), vmin_lds the same for WITH_MIN.
+// (per wave: the maximum of every lane's vector i), vmin_lds the same for WITH_MIN.  Lane l of vector i
+// writes to place l ^ 4 (i mod 4): the lane that later reads a block's 16 maxima as four 128-bit words
+// finds them in another order (a maximum does not care), and lanes 64 bytes apart no longer meet in the
+// same banks -- half of the LDS cycles of this kernel were bank conflicts of those reads.
 template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SCALED, bool WITH_MIN>
 __device__ __forceinline__ void scan_chunk(const T *__restrict__ in, uint32_t n, uint32_t G, const ScanWorkspace &ws,
                                            float scale, uint32_t block, uint32_t tid, float (*vm_lds)[V][kWave],
@@ -142,7 +145,7 @@ __device__ __forceinline__ void scan_chunk(const T *__restrict__ in, uint32_t n,
                 float vn = INFINITY;
 #pragma unroll
                 for (int c = 0; c < VEC; c++) vn = fminf(vn, xv[c]);  // (an element past the chunk's end counts as -inf)
-                vmin_lds[wave][i][lane] = vn;
+                vmin_lds[wave][i][lane ^ ((i & 3) << 2)] = vn;
             }
             if constexpr (SOFTMAX) {
                 if constexpr (i == 0) {
@@ -170,7 +173,7 @@ __device__ __forceinline__ void scan_chunk(const T *__restrict__ in, uint32_t n,
                 for (int c = 0; c < VEC; c += 2) has_nan = has_nan || __builtin_isunordered(xv[c], xv[c + 1]);
                 vm = has_nan ? __uint_as_float(0x7FC00000u) : vm;
             }
-            vm_lds[wave][i][lane] = vm;
+            vm_lds[wave][i][lane ^ ((i & 3) << 2)] = vm;
         });
         // ---- block maxima: lane L of the wave takes block L of the wave's WB blocks -----
         // (block (vector i, lanes 16 r .. 16 r + 15) is the wave's block 4 i + r, and its 16
@@ -182,7 +185,7 @@ __device__ __forceinline__ void scan_chunk(const T *__restrict__ in, uint32_t n,
             const float4 *src = reinterpret_cast<const float4 *>(&vm_lds[wave][0][0] + lane * kBlockLanes);
 #pragma unroll
             for (int j = 0; j < kBlockLanes / 4; j++) {
-                const float4 v4 = src[j];
+                const float4 v4 = src[j ^ ((lane >> 2) & 3)];  // (the block of vector lane / 4: its words are in the order 0..3 ^ that vector's number mod 4)
                 bm = fmaxf(fmaxf(bm, fmaxf(v4.x, v4.y)), fmaxf(v4.z, v4.w));
                 if constexpr (!SOFTMAX) b_nan = b_nan || __builtin_isunordered(v4.x, v4.y) || __builtin_isunordered(v4.z, v4.w);
             }
@@ -197,7 +200,7 @@ __device__ __forceinline__ void scan_chunk(const T *__restrict__ in, uint32_t n,
                     float bn = INFINITY;
 #pragma unroll
                     for (int j = 0; j < kBlockLanes / 4; j++) {
-                        const float4 v4 = srcn[j];
+                        const float4 v4 = srcn[j ^ ((lane >> 2) & 3)];
                         bn = fminf(fminf(bn, fminf(v4.x, v4.y)), fminf(v4.z, v4.w));
                     }
                     ws.bmin[static_cast<size_t>(row) * ws.blocks + e_block / (kBlockLanes * VEC)] = order_key(bn);
