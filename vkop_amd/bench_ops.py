@@ -130,6 +130,21 @@ def main():
         us = timed(call, len(bufs))
         report(name, us, x.nbytes + rows * k * (x.itemsize + 4))
 
+    def sampling_case(name, x, k, scale, top_p):
+        """vkop_hip_softmax_topk_sampling: temperature and nucleus count inside the call."""
+        if args.only not in name:
+            return
+        bufs = buffers(x)
+        rows = int(np.prod(x.shape[:-1]))
+        vals = torch.empty((rows, k), dtype=bufs[0].dtype, device="cuda")
+        idx = torch.empty((rows, k), dtype=torch.int32, device="cuda")
+        counts = torch.empty((rows,), dtype=torch.int32, device="cuda")
+        nb = capi.softmax_topk_workspace_bytes(F32, x.shape, -1, k)
+        ws, ptr = workspace(nb + 256)
+        us = timed(lambda b: capi.softmax_topk_sampling(bufs[b].data_ptr(), vals.data_ptr(), idx.data_ptr(), counts.data_ptr(), F32,
+                                                        x.shape, -1, k, scale, top_p, ptr, nb + 256, stream), len(bufs))
+        report(name, us, x.nbytes + rows * (k * (x.itemsize + 4) + 4))
+
     if args.softmax_sweep:
         shapes = [((256, 1000), -1), ((4096, 32), -1), ((65536, 64), -1), ((16384, 128), -1), ((8192, 256), -1), ((4096, 1024), -1),
                   ((2048, 2048), -1), ((1024, 4096), -1), ((256, 8192), -1), ((128, 16384), -1), ((64, 32768), -1), ((32, 50257), -1),
@@ -227,6 +242,10 @@ def main():
     c3i = np.ascontiguousarray(np.clip(np.round(c3 * 16), -128, 127).astype(np.float32) * np.float32(0.125))
     select_case("C3 int8-valued softmax+topk k=50 [64,128256] f32", c3i, 50, True)
     select_case("C3 int8-valued topk k=50 [64,128256] f32", c3i, 50, False)
+    # the sampling entry point: temperature 0.8 and the nucleus count for top_p = 0.9 in the same call
+    sampling_case("C3 sampling softmax+topk k=50 [64,128256] f32, scale 1.25, top_p 0.9", c3, 50, 1.25, 0.9)
+    sampling_case("C2 sampling softmax+topk k=5 [256,1000] f32, scale 1.25, top_p 0.9", c2, 5, 1.25, 0.9)
+    sampling_case("sampling softmax+topk k=40 [64,8192] f32, scale 1.25, top_p 0.9", np.ascontiguousarray(c3[:, :8192]), 40, 1.25, 0.9)
     softmax_case("C4 softmax [8,262144] f32", c4, -1)
     select_case("C4 topk k=1024 [8,262144] f32 (ties)", c4, 1024, False)
     select_case("C4 softmax+topk k=1024 [8,262144] f32", c4, 1024, True)

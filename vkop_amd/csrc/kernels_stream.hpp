@@ -617,11 +617,14 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
         return b * kScanWaves + ((off / VEC) % kScanThreads) / kWave;
     };
 
+    bool have_list = false;
     // ---- E1. the common case to its end ---------------------------------------------------------
     // Every wave listed its candidates, they are at least k+1 and a thread can take one each, and
     // the row's sum is a positive number: ranks, accurate terms for the k+1 first, probabilities.
-    // Equal probabilities among the k+1 (in order by index, and across the k-th place a matter of
-    // the whole row) leave it to the general code below, as does everything else.
+    // Equal probabilities of DIFFERENT logits among the k+1 (to be put in order by index; across the k-th
+    // place a matter of the whole row) leave it to the general code below, as does everything else.  Equal
+    // logits are no such case -- the ranking has them in index order already, and every element with the
+    // logit of rank k is in the list -- which is what logits that went through bfloat16 or int8 are full of.
     {
         const uint32_t C2 = sh.count;
         bool common = sh.wave_overflow == 0u && C2 >= want && C2 <= static_cast<uint32_t>(NT) && kk == k;
@@ -699,7 +702,7 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
                     const uint32_t r = base + lane;  // ranks r and r + 1 <= k
                     const float p0 = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r : 0u]) * rinv));
                     const float p1 = round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r + 1u : 0u]) * rinv));
-                    tie = tie || (r < k && p0 == p1);
+                    tie = tie || (r < k && p0 == p1 && sh.pkey[r] != sh.pkey[r < k ? r + 1u : 0u]);
                     if (base == 0) p_first = p0;
                 }
                 tie = __ballot(tie) != 0ull;
@@ -751,10 +754,13 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
             if (__builtin_expect(!tie, 1)) return;
             // (equal probabilities: what was stored is written again below, in its final order)
         }
-        // the general code starts from an empty list
+        // The general code: with the list the waves made, if every wave could list all of its blocks
+        // (the list may still hold fewer than k+1 entries, or have dropped what came after its capacity:
+        // sh.count says how many there were), else from an empty one.
+        have_list = sh.wave_overflow == 0u;
         __syncthreads();
         for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;
-        if (tid == 0) sh.count = 0;
+        if (!have_list && tid == 0) sh.count = 0;
         __syncthreads();
     }
     if constexpr (SOFTMAX) {
@@ -872,7 +878,7 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
     // (The same when EVERY block reaches it and the row has a quarter more blocks than places.)
     hit_cap = min(static_cast<uint32_t>(kPickHitCap), 3u * want + 64u);
     if (blocks > want + want / 4u) hit_cap = min(hit_cap, blocks - 1u);
-    bool many_groups = gather(thr, 1ull << 32, std::false_type{});
+    bool many_groups = have_list ? false : gather(thr, 1ull << 32, std::false_type{});
     if (many_groups) {
         // More than kPickHitCap blocks reach thr: the threads' shares of the block maxima are
         // not alike (rows sorted in runs as long as the stride between a thread's blocks put
