@@ -218,4 +218,34 @@ template <typename T> __device__ __forceinline__ float scale_term(float e, doubl
     else return static_cast<float>(static_cast<double>(e) * rinv);
 }
 
+// The nucleus cut of a sorted result, by all 64 lanes of one wave: the number of leading values whose
+// running sum -- added in order, in float, sum = fl(sum + v) -- first reaches p, or k if it never does
+// (a NaN reaches nothing).  value(r) gives rank r < k.  The running sums move through the lanes: every lane
+// keeps adding its own value to what its left neighbour holds (one instruction across the wave; lane 0
+// holds fl(carry + v0) and adds 0 to itself), and after t steps lanes 0..t hold their final sums -- the
+// additions of the walk one value at a time, in the same order, each a wave-wide instruction instead of
+// a read of one lane, an addition, a comparison and a branch.
+template <typename F> __device__ __forceinline__ uint32_t nucleus_count_wave(uint32_t k, float p, F &&value) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    float carry = 0.f;
+    for (uint32_t base = 0; base < k; base += kWave) {
+        const uint32_t m = min(static_cast<uint32_t>(kWave), k - base);
+        const float v = base + lane < k ? value(base + lane) : 0.f;
+        float s = lane == 0 ? __fadd_rn(carry, v) : v;
+        const float own = lane == 0 ? 0.f : v;
+        for (uint32_t t = 1; t < m; t += 4) {  // (steps past m - 1 change nothing below lane m)
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                // wave_shr:1 -- lane l reads lane l - 1, lane 0 (no source) keeps its own
+                const float left = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(s), __float_as_int(s), 0x138, 0xF, 0xF, false));
+                s = __fadd_rn(own, left);
+            }
+        }
+        const unsigned long long reached = __ballot(lane < m && s >= p);
+        if (reached != 0ull) return base + static_cast<uint32_t>(__builtin_ctzll(reached)) + 1u;
+        carry = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s), static_cast<int>(m - 1u)));
+    }
+    return k;
+}
+
 }  // namespace vkop

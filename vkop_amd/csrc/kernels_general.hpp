@@ -163,22 +163,9 @@ __global__ __launch_bounds__(NT) void reduce_max_lines_kernel(const T *__restric
 template <typename T>
 __global__ __launch_bounds__(kWave) void topp_count_kernel(const T *__restrict__ values, int32_t *__restrict__ counts, uint32_t k,
                                                             size_t row_stride, float p) {
-    const uint32_t lane = threadIdx.x;
     const T *row = values + static_cast<size_t>(blockIdx.x) * row_stride;
-    float sum = 0.f;
-    uint32_t count = k;
-    for (uint32_t base = 0; base < k && count == k; base += kWave) {
-        const float v = base + lane < k ? load_elem(row, base + lane) : 0.f;
-        const uint32_t n = min(static_cast<uint32_t>(kWave), k - base);
-        for (uint32_t j = 0; j < n; j++) {
-            sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
-            if (sum >= p) {
-                count = base + j + 1;
-                break;
-            }
-        }
-    }
-    if (lane == 0) counts[blockIdx.x] = static_cast<int32_t>(count);
+    const uint32_t count = nucleus_count_wave(k, p, [&](uint32_t r) { return load_elem(row, r); });
+    if (threadIdx.x == 0) counts[blockIdx.x] = static_cast<int32_t>(count);
 }
 
 // ---- top-k, one workgroup per line -----------------------------------------

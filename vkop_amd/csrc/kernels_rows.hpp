@@ -867,21 +867,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
             // place holds the tied group's probability (0 when the row ran out of elements
             // above -inf).  Walked through the lanes in order, as topp_count_kernel does.
             const float tail = (!partial && kk < C2) ? sh.prob[kk] : 0.f;
-            float sum = 0.f;
-            uint32_t count = kk;
-            for (uint32_t base = 0; base < kk && count == kk; base += kWave) {
-                const uint32_t r = base + lane;
-                const float v = r < kk ? (r < plain ? sh.prob[r] : tail) : 0.f;
-                const uint32_t m = min(static_cast<uint32_t>(kWave), kk - base);
-                for (uint32_t j = 0; j < m; j++) {
-                    sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(
-                                             __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
-                    if (sum >= top_p) {
-                        count = base + j + 1;
-                        break;
-                    }
-                }
-            }
+            const uint32_t count = nucleus_count_wave(kk, top_p, [&](uint32_t r) { return r < plain ? sh.prob[r] : tail; });
             if (lane == 0) *count_out = static_cast<int32_t>(count);
         }
     }

@@ -720,22 +720,9 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
                 }
                 if (!tie && counts != nullptr && wave == 0) {
                     // the nucleus cut: the stored values walked in order through the lanes, as topp_count_kernel does
-                    float sum = 0.f;
-                    uint32_t count = k;
-                    for (uint32_t base = 0; base < k && count == k; base += kWave) {
-                        const uint32_t r = base + lane;
-                        const float v = base == 0 ? p_first
-                                                  : round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r < k ? r : 0u]) * rinv));
-                        const uint32_t m = min(static_cast<uint32_t>(kWave), k - base);
-                        for (uint32_t j = 0; j < m; j++) {
-                            sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(
-                                                     __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
-                            if (sum >= top_p) {
-                                count = base + j + 1;
-                                break;
-                            }
-                        }
-                    }
+                    const uint32_t count = nucleus_count_wave(k, top_p, [&](uint32_t r) {
+                        return r < static_cast<uint32_t>(kWave) ? p_first : round_to_storage<T>(static_cast<float>(static_cast<double>(sh.prob[r]) * rinv));
+                    });
                     if (lane == 0) counts[row] = static_cast<int32_t>(count);
                 }
             } else {
@@ -1062,21 +1049,9 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
             // (rare path: the stored values are read back by the first wave, walked in order)
             __syncthreads();
             if (tid < static_cast<uint32_t>(kWave)) {
-                float sum = 0.f;
-                uint32_t count = kk;
-                for (uint32_t base = 0; base < kk && count == kk; base += kWave) {
-                    const uint32_t r = base + lane;
-                    const float v = r < kk ? round_to_storage<T>(softmax_prob(scaled(load_elem(rowp, composite_index(exact.sel[r < kk ? r : 0u])), scale), st)) : 0.f;
-                    const uint32_t m = min(static_cast<uint32_t>(kWave), kk - base);
-                    for (uint32_t j = 0; j < m; j++) {
-                        sum = __fadd_rn(sum, __uint_as_float(static_cast<uint32_t>(
-                                                 __builtin_amdgcn_readlane(static_cast<int>(__float_as_uint(v)), static_cast<int>(j)))));
-                        if (sum >= top_p) {
-                            count = base + j + 1;
-                            break;
-                        }
-                    }
-                }
+                const uint32_t count = nucleus_count_wave(kk, top_p, [&](uint32_t r) {
+                    return round_to_storage<T>(softmax_prob(scaled(load_elem(rowp, composite_index(exact.sel[r])), scale), st));
+                });
                 if (lane == 0) counts[row] = static_cast<int32_t>(count);
             }
         }
