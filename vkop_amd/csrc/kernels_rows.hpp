@@ -369,19 +369,39 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
     const uint32_t tid = threadIdx.x;
     if (C == 0) return;
     if (C <= NT) {
-        // the threads form NT / P groups (P: the power of two at or above C), each candidate has a
-        // thread in every group, and a group takes one part of the list (shifts only: a division
-        // by a number known at run time is three dozen dependent instructions)
-        const uint32_t pshift = C > 1u ? 32u - static_cast<uint32_t>(__clz(C - 1u)) : 0u;
-        const uint32_t parts = static_cast<uint32_t>(NT) >> pshift;                   // >= 1, a power of two
-        const uint32_t span = (C + parts - 1u) >> (31u - static_cast<uint32_t>(__clz(parts)));  // entries per part
-        const uint32_t part = tid >> pshift, i = tid & ((1u << pshift) - 1u);
-        if (i < C) {
+        // Every candidate has a thread in each of `parts` groups, and a group takes one part of the list.
+        // Short lists: groups of P threads, P the power of two at or above C -- shifts only, since a division by
+        // a number known at run time is three dozen dependent instructions, as much as the counting itself.
+        // Longer lists: groups of exactly C threads (NT = 1024, C = 300: three parts of 100 instead of two of 150).
+        uint32_t parts, span, part, i;
+        bool live;
+        if (C <= 128u) {
+            const uint32_t pshift = C > 1u ? 32u - static_cast<uint32_t>(__clz(C - 1u)) : 0u;
+            parts = static_cast<uint32_t>(NT) >> pshift;                               // >= 1, a power of two
+            span = (C + parts - 1u) >> (31u - static_cast<uint32_t>(__clz(parts)));  // entries per part
+            part = tid >> pshift;
+            i = tid & ((1u << pshift) - 1u);
+            live = i < C;
+        } else {
+            parts = static_cast<uint32_t>(NT) / C;
+            span = (C + parts - 1u) / parts;
+            part = tid / C;
+            i = tid - part * C;
+            live = part < parts;
+        }
+        if (live) {
             const uint64_t mine = sh.cand[i];
             const uint32_t j0 = part * span, j1 = min(j0 + span, C);
             uint32_t cnt = 0;
             uint32_t j = j0;
-            for (; j < j1; j += 8) {  // eight independent reads in flight (past the part's end: entry 0, not counted)
+            for (; j + 8 <= j1; j += 8) {  // eight independent reads in flight
+                uint64_t o[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) o[u] = sh.cand[j + u];
+#pragma unroll
+                for (int u = 0; u < 8; u++) cnt += (o[u] > mine) ? 1u : 0u;
+            }
+            if (j < j1) {  // the last few, again all at once (past the part's end: entry 0, not counted)
                 uint64_t o[8];
 #pragma unroll
                 for (int u = 0; u < 8; u++) o[u] = sh.cand[j + u < j1 ? j + u : 0u];

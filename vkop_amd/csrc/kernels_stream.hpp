@@ -499,7 +499,11 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
     constexpr uint32_t kWaveHitCap = 2 * U * (kWave / kBlockLanes);  // blocks a wave reads again in one go
     static_assert(NW * kWaveHitCap <= kPickHitCap, "every wave's list of blocks fits");
     static_assert(NW <= kPickThreads / kWave, "a stage per wave");
-    {
+    // About 1.15 (k+1) blocks reach thr, a wave's share of them has to fit its list, and the shares are not alike:
+    // from five eighths of the lists' total on, some wave of most rows has too many, and what the waves did is
+    // thrown away (an unaligned row pays a load per element for it).  Such rows go the general way at once.
+    const bool wave_lists = want <= NW * kWaveHitCap * 5u / 8u;
+    if (wave_lists) {
         uint32_t wave_n = 0;  // wave-uniform
 #pragma unroll
         for (int e = 0; e < GE; e++) wave_n += static_cast<uint32_t>(__popcll(__ballot(gk[e] >= thr)));
@@ -600,6 +604,8 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
                 }
             }
         }
+    } else {
+        combine_records();
     }
     BPS(44);
     __syncthreads();  // the candidates and phase B's results
@@ -627,7 +633,7 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
     // logit of rank k is in the list -- which is what logits that went through bfloat16 or int8 are full of.
     {
         const uint32_t C2 = sh.count;
-        bool common = sh.wave_overflow == 0u && C2 >= want && C2 <= static_cast<uint32_t>(NT) && kk == k;
+        bool common = wave_lists && sh.wave_overflow == 0u && C2 >= want && C2 <= static_cast<uint32_t>(NT) && kk == k;
         if constexpr (SOFTMAX) common = common && s_base > 0.0 && s_base < static_cast<double>(INFINITY) && M > -INFINITY && M < INFINITY;
         if (__builtin_expect(common, 1)) {
             // A candidate's own part (its wave's record, its accurate term) and the ranking are two chains of
@@ -744,7 +750,7 @@ __device__ __forceinline__ void pick_row(PickSharedUnion &smem, float *fscratch,
         // The general code: with the list the waves made, if every wave could list all of its blocks
         // (the list may still hold fewer than k+1 entries, or have dropped what came after its capacity:
         // sh.count says how many there were), else from an empty one.
-        have_list = sh.wave_overflow == 0u;
+        have_list = wave_lists && sh.wave_overflow == 0u;
         __syncthreads();
         for (uint32_t t = tid; t < static_cast<uint32_t>(kFastCap); t += NT) sh.rank[t] = 0;
         if (!have_list && tid == 0) sh.count = 0;
