@@ -856,6 +856,23 @@ def test_large_k_on_rows_one_workgroup_holds(ops, dtype, n, k):
     assert_fused(ops, x * 8, k)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("rows,n,k", [(16, 8400, 300), (48, 8192, 100), (40, 4096, 64), (24, 8190, 100), (12, 20000, 120)])
+@pytest.mark.parametrize("kind", ["runs", "levels", "ascending", "descending", "two_values"])
+def test_rows_in_order_and_rows_of_levels_on_the_one_workgroup_route(ops, kind, rows, n, k, dtype):
+    """Rows one workgroup holds whose first list of candidates overflows: values in order (the bound
+    from the lane maxima is far too low; the vector minima give a second one, and the list is made
+    straight from the registers) and values equal en masse (the cut is looked for among the next few
+    distinct values before any radix pass).  Shapes with vectors no thread holds (8400 elements in a
+    workgroup shaped for 32768), a row of an odd length, and one of 20000 elements."""
+    x = np.ascontiguousarray(synth.awkward_rows(kind, rows, n, seed=n + k).astype(dtype))
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    t, j = ops.topk(dev(x), k)
+    et, ej = oracle.topk(x, k)
+    assert np.array_equal(host(j), ej) and np.array_equal(host(t).view(bits), et.view(bits)), (kind, rows, n, k)
+    assert_fused(ops, x, k)
+
+
 # ---- non-maximum suppression ------------------------------------------------------------------------
 
 def _nms_boxes(rng, B, N, spread=1.3):

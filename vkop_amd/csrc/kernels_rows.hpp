@@ -48,10 +48,11 @@
 namespace vkop {
 
 // Debug builds only (-DVKOP_STAMPS=<name of the C function that reads them out>, rows_inst.hip):
-// clock stamps of workgroup 0's first thread.
+// clock stamps of one workgroup's first thread (workgroup 0 unless g_bp_block is set).
 #ifdef VKOP_STAMPS
 static __device__ unsigned long long g_bp_stamps[64];
-#define BPS(i) do { if (threadIdx.x == 0 && blockIdx.x == 0) g_bp_stamps[i] = wall_clock64(); } while (0)
+static __device__ unsigned int g_bp_block;
+#define BPS(i) do { if (threadIdx.x == 0 && blockIdx.x == g_bp_block) g_bp_stamps[i] = wall_clock64(); } while (0)
 #else
 #define BPS(i) do { } while (0)
 #endif
@@ -278,7 +279,8 @@ template <int NT> struct ChunkShared {  // chunk phase
     uint4 stage_v[NT];     // per wave: up to 64 vectors holding an element at or above the threshold ...
     uint32_t stage_e[NT];  // ... and the index of their first element
     uint32_t wave_thr[16];
-    uint32_t refine[34];  // element counts per bit of the exact threshold search; reaching / exceeding the result
+    uint32_t refine[40];  // element counts per bit of the exact threshold search; [32], [33]: smallest key at or above a bound / elements
+                          // above that key, and the same in [34] ... [39] for the next two distinct values up
     uint32_t thr, total, over;
 };
 
@@ -418,7 +420,15 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
         for (uint32_t i = tid; i < C; i += NT) {
             const uint64_t mine = sh.cand[i];
             uint32_t cnt = 0;
-            for (uint32_t j = 0; j < C; j++) cnt += (sh.cand[j] > mine) ? 1u : 0u;
+            uint32_t j = 0;
+            for (; j + 8 <= C; j += 8) {  // eight independent reads in flight
+                uint64_t o[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) o[u] = sh.cand[j + u];
+#pragma unroll
+                for (int u = 0; u < 8; u++) cnt += (o[u] > mine) ? 1u : 0u;
+            }
+            for (; j < C; j++) cnt += (sh.cand[j] > mine) ? 1u : 0u;
             sh.rank[i] = cnt;
         }
     }
@@ -866,12 +876,49 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
         if constexpr (SOFTMAX) {
             const float p = sh.prob[r];
             // final place inside a run of equal probabilities: by index
+            // (rows of few distinct values have runs of hundreds: the run's ends are looked for eight
+            // entries a step, not one dependent LDS read after the other; equal logits are in index order
+            // already, so a run of one logit -- the usual kind -- needs no count)
             uint32_t lo = r, hi = r, pos = r;
-            while (lo > 0 && sh.prob[lo - 1] == p) lo--;
-            while (hi + 1 < plain && sh.prob[hi + 1] == p) hi++;
-            if (hi > lo) {
+            if (lo > 0 && sh.prob[lo - 1] == p) {
+                bool more = true;
+                while (more && lo > 0) {
+                    float v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) v[u] = sh.prob[lo > static_cast<uint32_t>(u) ? lo - 1u - u : 0u];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const bool same = more && lo > 0 && v[u] == p;  // (v[u] was read for the lo of the step's start)
+                        more = same;
+                        lo -= same ? 1u : 0u;
+                    }
+                }
+            }
+            if (hi + 1 < plain && sh.prob[hi + 1] == p) {
+                bool more = true;
+                while (more && hi + 1 < plain) {
+                    float v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) v[u] = sh.prob[hi + 1u + u < plain ? hi + 1u + u : plain - 1u];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) {
+                        const bool same = more && hi + 1 < plain && v[u] == p;
+                        more = same;
+                        hi += same ? 1u : 0u;
+                    }
+                }
+            }
+            if (hi > lo && (sh.pkey[lo] != sh.pkey[hi])) {
                 pos = lo;
-                for (uint32_t q = lo; q <= hi; q++) pos += (sh.pidx[q] < idx) ? 1u : 0u;
+                uint32_t q = lo;
+                for (; q + 8 <= hi + 1; q += 8) {
+                    uint32_t o[8];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) o[u] = sh.pidx[q + u];
+#pragma unroll
+                    for (int u = 0; u < 8; u++) pos += (o[u] < idx) ? 1u : 0u;
+                }
+                for (; q <= hi; q++) pos += (sh.pidx[q] < idx) ? 1u : 0u;
             }
             store_elem(ov, pos, p);
             oi[pos] = static_cast<int32_t>(idx);
@@ -1054,7 +1101,21 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
         __syncthreads();
         thr = sh.thr;
     }
-    if (G == 1) thr = 1u;
+    if (G == 1) {
+        // One chunk: its list is cut at its own threshold, and as a rule everything in it is taken.  Where the
+        // list is half as long again as k+1 and more (values equal en masse just below the cut: the chunk's
+        // threshold comes from lane maxima), ranking all of it costs more than a threshold among the
+        // candidates themselves: the (k+1)-th largest thread maximum, by one wave.
+        thr = 1u;
+        if (sh.cnt[0] > want + (want >> 1) + 32u) {  // (the same for every thread)
+            if (wave == 0) {
+                const uint32_t t = block_kth_largest_floor<NW>(sh.lane_key, want, 20);
+                if (lane == 0) sh.thr = t > 1u ? t : 1u;
+            }
+            __syncthreads();
+            thr = sh.thr;
+        }
+    }
     uint32_t merge_thr = thr;  // candidates with keys at or above it are in sh.cand (of equal keys maybe only the first)
     const bool slow = sh.flag != 0u;
     if constexpr (SOFTMAX) {
@@ -1544,7 +1605,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             publish(record + 3, (static_cast<uint64_t>(__float_as_uint(x0)) << 32) | copies);
         }
         __syncthreads();
-        if (__builtin_expect(cs.total > ws.cap || cs.over != 0u, 0)) {
+        const bool too_many = cs.total > ws.cap || cs.over != 0u;  // (the same in every thread)
+        if (__builtin_expect(too_many, 0)) {
             // Too many.  The lane maxima give a loose bound when values in order or in
             // clusters put many large elements into few lanes, or when many are equal.
             // The list is made once more, with the exact (k+1)-th largest element of
@@ -1566,15 +1628,66 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 return in_range(ALIGNED ? e0 : e0 + c) ? order_key(x) : 0u;
             };
             const bool from_stage = cs.over == 0u;
+            // (a short row in a workgroup shaped for longer ones -- 8400 elements, 1024 threads, V = 8 -- has
+            // vectors no thread holds anything of: the passes below leave them out, the same in every thread)
+            const int v_used = static_cast<int>(min(static_cast<uint32_t>(V), (c1 - c0 + NT * VEC - 1u) / (NT * VEC)));
+            // Values in order (a sorted row, a row sorted in runs) put many large elements into few lanes, and
+            // the bound from the lane maxima is then far too low.  On such a row the elements of a VECTOR are
+            // alike, and every element of a vector reaches the vector's minimum: with q = ceil((k+1) / width)
+            // lanes that hold a vector whose minimum reaches T, k+1 elements reach T.  The q-th largest of the
+            // lanes' largest vector minima is such a T (its leading 24 bits: lower, so still reached) -- close
+            // under the cut on a row in order, useless, and then not used, on any other.  Where it beats the
+            // bound, everything at or above it is listed straight away if that fits (first turn of the loop
+            // below), and only otherwise the exact cut is looked for (second turn).
+            bool tight = false;
+            if (tid < 40) cs.refine[tid] = (tid >= 32 && (tid & 1u) == 0u) ? 0xFFFFFFFFu : 0u;
+            {
+                uint32_t a = 0;
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    if (i >= v_used) continue;
+                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
+                    float vm = INFINITY;  // (a NaN is dropped: it ranks above everything, the others' minimum still holds)
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) {
+                        float x = q[i].get(c);
+                        asm volatile("" : "+v"(x));
+                        vm = fminf(vm, in_range(ALIGNED ? e0 : e0 + c) ? x : -INFINITY);
+                    }
+                    a = max(a, vm == vm ? order_key(vm) : 0u);
+                }
+                cs.lane_key[tid] = a;
+                const uint32_t qn = (want + VEC - 1u) / VEC;
+                __syncthreads();
+                // (q lanes must beat the bound for T to: counted first, which is all a row not in order pays)
+                const uint32_t beat = static_cast<uint32_t>(__popcll(__ballot(a > thr)));
+                if (lane == 0 && beat) atomicAdd(&cs.refine[39], beat);
+                __syncthreads();
+                if (cs.refine[39] >= qn) {  // (the same in every thread)
+                    if (wave == 0) {
+                        const uint32_t t = block_kth_largest_floor<NW>(cs.lane_key, qn, 24);
+                        if (lane == 0) cs.thr = t;
+                    }
+                    __syncthreads();
+                    const uint32_t tmin = cs.thr;
+                    tight = tmin > thr;
+                    if (tight) thr = tmin;
+                    __syncthreads();  // (cs.thr and cs.lane_key are free again)
+                }
+            }
+#pragma unroll 1
+            for (int turn = tight ? 0 : 1; turn < 2; turn++) {
+            const bool exact = turn == 1;
+            if (exact) {
             uint32_t wk = 0;
 #pragma unroll
             for (int i = 0; i < V; i++) {
+                if (i >= v_used) continue;
 #pragma unroll
                 for (int c = 0; c < VEC; c++) wk = max(wk, key_of(i, c));
             }
             wk = wave_max_u32(wk);
             if (lane == 0) cs.wave_thr[wave] = wk;
-            if (tid < 34) cs.refine[tid] = tid == 32 ? 0xFFFFFFFFu : 0u;
             __syncthreads();
             uint32_t hi = cs.wave_thr[0];
 #pragma unroll
@@ -1643,29 +1756,49 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 // fewer exceed it.
                 static_assert(sizeof(cs.stage_v) >= 256 * sizeof(uint32_t), "the digit counts take 256 words");
                 uint32_t *hist = reinterpret_cast<uint32_t *>(cs.stage_v);  // (the stage is filled anew afterwards)
-                uint32_t f = 0xFFFFFFFFu, above = 0;
+                // (up to three distinct values from the bound up: the lane maxima of a row of a dozen levels
+                // put the bound a level or two under the cut, and a step costs two passes where the radix
+                // select costs eight)
+                uint32_t lb = thr;
+                bool settled = false, levels = true;
+                uint32_t reach = cs.total;  // elements at or above lb (at least: a wave whose stage overflowed counted short)
+#pragma unroll 1
+                for (uint32_t step = 0; step < 3u && !settled && levels; step++) {
+                    uint32_t f = 0xFFFFFFFFu, above = 0;
 #pragma unroll
-                for (int i = 0; i < V; i++) {
+                    for (int i = 0; i < V; i++) {
+                        if (i >= v_used) continue;
 #pragma unroll
-                    for (int cc = 0; cc < VEC; cc++) {
-                        const uint32_t kx = key_of(i, cc);
-                        f = kx >= thr ? min(f, kx) : f;
+                        for (int cc = 0; cc < VEC; cc++) {
+                            const uint32_t kx = key_of(i, cc);
+                            f = kx >= lb ? min(f, kx) : f;
+                        }
+                    }
+                    f = ~wave_max_u32(~f);
+                    if (lane == 0) atomicMin(&cs.refine[32 + 2 * step], f);
+                    __syncthreads();
+                    const uint32_t t0 = cs.refine[32 + 2 * step];  // (>= lb: the same in every thread)
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        if (i >= v_used) continue;
+#pragma unroll
+                        for (int cc = 0; cc < VEC; cc++) above += static_cast<uint32_t>(__popcll(__ballot(key_of(i, cc) > t0)));
+                    }
+                    if (lane == 0 && above) atomicAdd(&cs.refine[33 + 2 * step], above);
+                    __syncthreads();
+                    if (cs.refine[33 + 2 * step] < want) {
+                        thr = t0;  // k+1 elements reach it, fewer exceed it
+                        settled = true;
+                    } else {
+                        lb = t0 + 1u;  // (t0 < the row's maximum: k+1 elements exceed it)
+                        // a value that few elements have: not a row of levels, the next value up will not be the cut either
+                        const uint32_t exceed = cs.refine[33 + 2 * step];
+                        levels = reach >= exceed + 8u;
+                        reach = exceed;
                     }
                 }
-                f = ~wave_max_u32(~f);
-                if (lane == 0) atomicMin(&cs.refine[32], f);
-                __syncthreads();
-                const uint32_t t0 = cs.refine[32];  // (>= thr: the same in every thread)
-#pragma unroll
-                for (int i = 0; i < V; i++) {
-#pragma unroll
-                    for (int cc = 0; cc < VEC; cc++) above += static_cast<uint32_t>(__popcll(__ballot(key_of(i, cc) > t0)));
-                }
-                if (lane == 0 && above) atomicAdd(&cs.refine[33], above);
-                __syncthreads();
-                if (cs.refine[33] < want) {
-                    thr = t0;
-                } else {
+                if (!settled) {
+                    thr = lb;  // k+1 elements reach it
                     uint32_t prefix = 0, need = want;
                     for (int shift = 24; shift >= 0; shift -= 8) {
                         __syncthreads();  // (the last pass's answer has been read)
@@ -1673,6 +1806,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                         __syncthreads();
 #pragma unroll
                         for (int i = 0; i < V; i++) {
+                            if (i >= v_used) continue;
 #pragma unroll
                             for (int cc = 0; cc < VEC; cc++) {
                                 const uint32_t kx = key_of(i, cc);  // (0 past the chunk's end: the lowest digit, below every element)
@@ -1700,19 +1834,26 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
 #pragma unroll
             for (int i = 0; i < V; i++) {
                 uint32_t ties = 0;
+                if (i < v_used) {
 #pragma unroll
-                for (int c = 0; c < VEC; c++) ties += static_cast<uint32_t>(__popcll(__ballot(key_of(i, c) == thr)));
+                    for (int c = 0; c < VEC; c++) ties += static_cast<uint32_t>(__popcll(__ballot(key_of(i, c) == thr)));
+                }
                 if (lane == 0) cs.lane_key[i * NW + wave] = ties;
             }
             drain_stores();  // the first attempt's stores have landed before the same slots are written again
             __syncthreads();  // (and every wave is done with its stage)
-            // exclusive prefix over the (vector, wave) table, one entry per thread
+            // exclusive prefix over the (vector, wave) table, one entry per thread: a scan over the lanes of
+            // each of its (at most two) waves, the second adding the first one's total
+            static_assert(V * NW <= 2 * kWave, "the table takes at most two waves");
             uint32_t mine_before = 0;
-            if (tid < static_cast<uint32_t>(V * NW)) {
-#pragma unroll 1
-                for (uint32_t j = 0; j < tid; j++) mine_before += cs.lane_key[j];
+            {
+                const uint32_t val = tid < static_cast<uint32_t>(V * NW) ? cs.lane_key[tid] : 0u;
+                const uint32_t incl = wave_inclusive_sum_u32(val);
+                mine_before = incl - val;
+                if (tid == static_cast<uint32_t>(kWave) - 1u) cs.refine[32] = incl;
             }
             __syncthreads();
+            if (tid >= static_cast<uint32_t>(kWave)) mine_before += cs.refine[32];
             if (tid < static_cast<uint32_t>(V * NW)) cs.lane_key[tid] = mine_before;
             if (tid == 0) {
                 cs.total = 0;
@@ -1722,6 +1863,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             __syncthreads();
 #pragma unroll
             for (int i = 0; i < V; i++) {
+                if (i >= v_used) continue;
                 uint32_t pos = cs.lane_key[i * NW + wave];  // equal elements before this wave's vector i
                 bool tie[VEC];
 #pragma unroll
@@ -1739,12 +1881,16 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             }
             __syncthreads();
             BPS(51);
+            } else {
+                drain_stores();  // the first attempt's stores have landed before the same slots are written again
+                __syncthreads();
+            }
             // The list, straight from the registers: at most 2 k + 1 entries (fewer than k+1 above the
             // value, the first k+1 equal to it), each at a place of its own from counts per (vector,
             // wave) -- not through the waves' stages of 64 vectors, which a sorted row, whose
             // candidates all sit in one wave's elements, would overflow again.
             {
-                const uint32_t idx_limit = cs.thr;
+                const uint32_t idx_limit = exact ? cs.thr : 0xFFFFFFFFu;
                 uint32_t *counts = cs.lane_key + V * NW;  // (behind the table of ties: 2 V NW <= NT words)
                 auto listed = [&](uint32_t kx, uint32_t idx) { return kx > thr || (kx == thr && idx <= idx_limit); };
                 uint32_t wave_total = 0;  // wave-uniform
@@ -1752,25 +1898,35 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 for (int i = 0; i < V; i++) {
                     const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
                     uint32_t cnt = 0;
+                    if (i < v_used) {
 #pragma unroll
-                    for (int c = 0; c < VEC; c++) cnt += static_cast<uint32_t>(__popcll(__ballot(listed(key_of(i, c), e0 + c))));
+                        for (int c = 0; c < VEC; c++) cnt += static_cast<uint32_t>(__popcll(__ballot(listed(key_of(i, c), e0 + c))));
+                    }
                     if (lane == 0) counts[i * NW + wave] = cnt;
                     wave_total += cnt;
                 }
                 __syncthreads();
-                uint32_t before_mine = 0;
-                if (tid < static_cast<uint32_t>(V * NW)) {
-#pragma unroll 1
-                    for (uint32_t j = 0; j < tid; j++) before_mine += counts[j];
+                uint32_t before_mine = 0, mine_cnt = 0;
+                {
+                    mine_cnt = tid < static_cast<uint32_t>(V * NW) ? counts[tid] : 0u;
+                    const uint32_t incl = wave_inclusive_sum_u32(mine_cnt);
+                    before_mine = incl - mine_cnt;
+                    if (tid == static_cast<uint32_t>(kWave) - 1u) cs.refine[32] = incl;
                 }
                 __syncthreads();
+                if (tid >= static_cast<uint32_t>(kWave)) before_mine += cs.refine[32];
                 if (tid < static_cast<uint32_t>(V * NW)) {
-                    if (tid == static_cast<uint32_t>(V * NW) - 1u) cs.total = before_mine + counts[tid];
+                    if (tid == static_cast<uint32_t>(V * NW) - 1u) cs.total = before_mine + mine_cnt;
                     counts[tid] = before_mine;
                 }
                 __syncthreads();
+                if (!exact && cs.total > ws.cap) {  // (the same in every thread: on to the exact cut)
+                    __syncthreads();
+                    continue;
+                }
 #pragma unroll
                 for (int i = 0; i < V; i++) {
+                    if (i >= v_used) continue;
                     const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
                     uint32_t pos = counts[i * NW + wave];
 #pragma unroll
@@ -1786,6 +1942,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     }
                 }
                 wave_candidates = wave_total;
+            }
+            break;
             }
             __syncthreads();  // (cs.total is final)
             BPS(52);

@@ -102,4 +102,9 @@ extern "C" int VKOP_STAMPS(unsigned long long *out) {
     (void)hipMemcpyToSymbol(HIP_SYMBOL(vkop::g_bp_stamps), zeros, sizeof(zeros));  // (each readout starts the next interval)
     return rc;
 }
+#define VKOP_STAMPS_CAT2(a, b) a##b
+#define VKOP_STAMPS_CAT(a, b) VKOP_STAMPS_CAT2(a, b)
+extern "C" int VKOP_STAMPS_CAT(VKOP_STAMPS, _block)(unsigned int block) {
+    return static_cast<int>(hipMemcpyToSymbol(HIP_SYMBOL(vkop::g_bp_block), &block, sizeof(block)));
+}
 #endif

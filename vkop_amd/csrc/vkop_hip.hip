@@ -793,6 +793,13 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.merge = (c.g == 1 && c.cap <= static_cast<uint32_t>(vkop::kLocalCap)) ? vkop::kMergeLocal
               : (c.g == 1 || by_ticket)                                         ? vkop::kMergeByTicket
                                                                                 : vkop::kMergeSplit;
+    if (a.merge == vkop::kMergeLocal) {
+        // the list is in LDS, where the kernel reserves kLocalCap entries whatever k is: all of them are the
+        // list (an overflow -- values equal en masse at the cut -- makes the workgroup list a second time)
+        w.cap = static_cast<uint32_t>(vkop::kLocalCap);
+        w.cap_shift = 0;
+        while ((1u << w.cap_shift) < w.cap) w.cap_shift++;
+    }
     a.ws = w;
     a.stream = st;
     const int stages = a.merge != vkop::kMergeSplit ? 1 : measured_stages();
