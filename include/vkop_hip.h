@@ -105,10 +105,15 @@ int vkop_hip_softmax(const void *in, void *out, int dtype, const int *shape,
 
 /* ---- TopK: ops/Topk.hpp:95-218 over shaders/topk.comp:110-262.
  * out_values: dtype of in, out_indices: int32 positions along `axis`; both have
- * the shape of in with [axis] = k.  Always sorted (descending for largest != 0,
- * ascending otherwise); ties: lower index first; NaN ranks above +inf.
- * `sorted` is accepted for signature parity (the reference parses and ignores
- * it, ops/Topk.hpp:73-75).  1 <= k <= min(extent of axis, VKOP_HIP_MAX_K). */
+ * the shape of in with [axis] = k.  With sorted != 0: descending for
+ * largest != 0, ascending otherwise; ties: lower index first; NaN ranks above
+ * +inf.  With sorted == 0 (the reference parses the attribute and ignores it,
+ * ops/Topk.hpp:73-75; ONNX leaves the order open then) the same k elements
+ * come in an order the library chooses, the same from run to run: on the
+ * multi-pass radix select (smallest first on long rows, and rows no other
+ * route takes) as that select lists them, which saves its last step; on
+ * every other route in sorted order, which costs nothing there.
+ * 1 <= k <= min(extent of axis, VKOP_HIP_MAX_K). */
 size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k);
 int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices,
                   int dtype, const int *shape, int ndim, int axis, int k,

@@ -873,6 +873,37 @@ def test_rows_in_order_and_rows_of_levels_on_the_one_workgroup_route(ops, kind, 
     assert_fused(ops, x, k)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_topk_without_an_order(ops, dtype):
+    """sorted = 0 (the reference parses the attribute and ignores it, ops/Topk.hpp:73-75): the same k
+    elements in an order of the library's choosing, the same on every call.  On the multi-pass radix
+    select -- smallest first on long rows -- that is the order the select lists them in (its ranking
+    step is left out); on the other routes the sorted result."""
+    rng = np.random.default_rng(21)
+    bits = np.uint16 if dtype == np.float16 else np.uint32
+    cases = [((6, 100000), 300, False), ((3, 70000), 2048, False), ((5, 40000), 64, False), ((64, 9000), 7, True), ((8, 1000), 5, True),
+             ((4, 60000), 100, True)]
+    took_the_select = 0
+    for shape, k, largest in cases:
+        x = (np.round(rng.standard_normal(shape) * 64) / 64).astype(np.float32)     # ties at the cut in most rows
+        x[0, :5] = np.nan
+        x = np.ascontiguousarray(x.astype(dtype))
+        et, ej = oracle.topk(x, k, -1, largest)
+        t, j = ops.topk(dev(x), k, -1, largest, sorted=False)
+        t, j = host(t), host(j)
+        t2, j2 = ops.topk(dev(x), k, -1, largest, sorted=False)
+        assert np.array_equal(j, host(j2)) and np.array_equal(t.view(bits), host(t2).view(bits)), (shape, k, largest)
+        for r in range(shape[0]):
+            order = np.argsort(j[r], kind="stable")
+            want = np.argsort(ej[r], kind="stable")
+            assert np.array_equal(j[r][order], ej[r][want]), (shape, k, largest, r)          # the same elements (ties: lowest indices)
+            assert np.array_equal(t[r][order].view(bits), et[r][want].view(bits)), (shape, k, largest, r)
+        if not np.array_equal(j, ej):
+            took_the_select += 1
+            assert not largest, (shape, k)          # (largest first, these shapes take routes whose result is in order anyway)
+    assert took_the_select >= 2        # (the long smallest-first rows: their unordered result differs from the ordered one)
+
+
 # ---- non-maximum suppression ------------------------------------------------------------------------
 
 def _nms_boxes(rng, B, N, spread=1.3):

@@ -111,7 +111,7 @@ def main():
                                           stream), len(bufs))
         report(name, us, 2 * x.nbytes)
 
-    def select_case(name, x, k, fused):
+    def select_case(name, x, k, fused, largest=1, sorted_=1):
         if args.only not in name:
             return
         dt = F16 if x.dtype == np.float16 else F32
@@ -125,7 +125,7 @@ def main():
             call = lambda b: capi.softmax_topk(bufs[b].data_ptr(), 0, vals.data_ptr(), idx.data_ptr(), dt, x.shape, -1, k,
                                                1, ptr, nb + 256, stream)
         else:
-            call = lambda b: capi.topk(bufs[b].data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, x.shape, -1, k, 1, 1,
+            call = lambda b: capi.topk(bufs[b].data_ptr(), vals.data_ptr(), idx.data_ptr(), dt, x.shape, -1, k, largest, sorted_,
                                        ptr, nb + 256, stream)
         us = timed(call, len(bufs))
         report(name, us, x.nbytes + rows * k * (x.itemsize + 4))
@@ -249,6 +249,8 @@ def main():
     softmax_case("C4 softmax [8,262144] f32", c4, -1)
     select_case("C4 topk k=1024 [8,262144] f32 (ties)", c4, 1024, False)
     select_case("C4 softmax+topk k=1024 [8,262144] f32", c4, 1024, True)
+    select_case("C4 topk smallest k=1024 [8,262144] f32, sorted", c4, 1024, False, largest=0, sorted_=1)
+    select_case("C4 topk smallest k=1024 [8,262144] f32, sorted = 0", c4, 1024, False, largest=0, sorted_=0)
     softmax_case("C5 softmax axis 1 [16,80,8400] f32", c5, 1)
     if args.only in "C5 chain softmax axis 1 -> max -> topk k=300":
         # the detection-style chain: softmax over classes, per-anchor class maximum, top-k anchors

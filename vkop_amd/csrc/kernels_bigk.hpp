@@ -345,12 +345,31 @@ constexpr int kBigSortSlice = kBigSortThreads / 4;
 template <typename T, bool SOFTMAX>
 __global__ __launch_bounds__(kBigSortThreads) void bigk_sort_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                                     int32_t *__restrict__ indices, uint32_t n,
-                                                                    uint32_t k, uint32_t slices, BigKWorkspace ws) {
+                                                                    uint32_t k, uint32_t slices, BigKWorkspace ws,
+                                                                    uint32_t in_order) {
     __shared__ uint64_t sel[kMaxK];
     __shared__ uint32_t rank[kBigSortSlice];
     const uint32_t tid = threadIdx.x;
     const uint32_t row = blockIdx.x / slices, slice = blockIdx.x - row * slices;
     const uint64_t *src = ws.sel + static_cast<size_t>(row) * ws.kpad;
+    if (in_order == 0u) {
+        // the caller did not ask for an order (sorted = 0): the k elements as the select listed them -- those
+        // above the k-th element's value, then those equal to it, each group by position in the row -- without
+        // the ranking
+        const uint32_t t = slice * kBigSortSlice + tid;
+        if (tid < static_cast<uint32_t>(kBigSortSlice) && t < k) {
+            const uint32_t idx = composite_index(src[t]);
+            const T *rowp = in + static_cast<size_t>(row) * n;
+            if constexpr (SOFTMAX) {
+                const LineStats st = ws.stats[row];
+                store_elem(values, static_cast<size_t>(row) * k + t, softmax_prob(load_elem(rowp, idx), st));
+            } else {
+                values[static_cast<size_t>(row) * k + t] = rowp[idx];  // bit copy
+            }
+            indices[static_cast<size_t>(row) * k + t] = static_cast<int32_t>(idx);
+        }
+        return;
+    }
     const uint32_t k16 = (k + 15u) & ~15u;  // four quarters of whole groups of four
     for (uint32_t t = tid; t < k16; t += kBigSortThreads) sel[t] = t < k ? src[t] : 0ull;  // 0: below every composite
     if (tid < kBigSortSlice) rank[tid] = 0;

@@ -681,7 +681,7 @@ RowsLayout rows_layout(const View &v, const RowsCfg &c, const BigKCfg &b = BigKC
 
 template <typename T, bool SOFTMAX>
 int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, const BigKCfg &c, void *ws,
-                const RowsLayout &l, hipStream_t st) {
+                const RowsLayout &l, hipStream_t st, bool in_order = true) {
     auto *base = static_cast<unsigned char *>(ws);
     vkop::BigKWorkspace w;
     w.hist = reinterpret_cast<uint32_t *>(base + l.hist);
@@ -717,7 +717,7 @@ int launch_bigk(const T *in, T *values, int32_t *indices, const View &v, int k, 
     else run(std::false_type{});
     const uint32_t slices = (uk + vkop::kBigSortSlice - 1) / vkop::kBigSortSlice;
     vkop::bigk_sort_kernel<T, SOFTMAX>
-        <<<rows * slices, vkop::kBigSortThreads, 0, st>>>(in, values, indices, n, uk, slices, w);
+        <<<rows * slices, vkop::kBigSortThreads, 0, st>>>(in, values, indices, n, uk, slices, w, in_order ? 1u : 0u);
     return launched("multi-workgroup radix select");
 }
 
@@ -817,7 +817,7 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
 
 // ------------------------------------------------------------------ top-k ----
 template <typename T>
-int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int dtype, void *ws,
+int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, int largest, int sorted, int dtype, void *ws,
               size_t ws_bytes, hipStream_t st) {
     // (the one-wave kernel serves both directions: it turns its order keys round)
     if (const int tiny = choose_tiny_loads(v, k, dtype)) return launch_tiny<T, false>(in, values, indices, v, k, tiny, st, !largest);
@@ -832,7 +832,9 @@ int topk_impl(const T *in, T *values, int32_t *indices, const View &v, int k, in
             return fail(VKOP_HIP_ERR_WORKSPACE, "workspace must be %zu-byte aligned", kAlign);
         if (sc.ok) return launch_scan<T, false>(in, values, indices, v, k, sc, ws, l, st);
         if (c.ok) return launch_rows<T, false>(in, values, indices, v, k, c, ws, l, st);
-        return launch_bigk<T, false>(in, values, indices, v, k, largest, b, ws, l, st);
+        // (sorted == 0: the one route where an order costs a step of its own leaves it out; every other route's
+        // result is in order by construction, which satisfies "any order" too)
+        return launch_bigk<T, false>(in, values, indices, v, k, largest, b, ws, l, st, sorted != 0);
     }
     const uint32_t lines = v.g.outer * v.g.inner;
     // one workgroup per line: a big one when the line is long and lines are few
@@ -1187,7 +1189,6 @@ size_t vkop_hip_topk_workspace_bytes(int dtype, const int *shape, int ndim, int 
 
 int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dtype, const int *shape, int ndim,
                   int axis, int k, int largest, int sorted, void *workspace, size_t workspace_bytes, void *stream) {
-    (void)sorted;  // results are always sorted, which satisfies sorted == 0 too
     View v;
     if (int rc = check_dtype(dtype)) return rc;
     if (int rc = make_view(shape, ndim, axis, &v)) return rc;
@@ -1198,9 +1199,9 @@ int vkop_hip_topk(const void *in, void *out_values, int32_t *out_indices, int dt
         return fail(VKOP_HIP_ERR_INVALID, "null tensor pointer");
     if (dtype == VKOP_HIP_F32)
         return topk_impl(static_cast<const float *>(in), static_cast<float *>(out_values), out_indices, v, k, largest,
-                         dtype, workspace, workspace_bytes, as_stream(stream));
+                         sorted, dtype, workspace, workspace_bytes, as_stream(stream));
     return topk_impl(static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out_values), out_indices, v, k,
-                     largest, dtype, workspace, workspace_bytes, as_stream(stream));
+                     largest, sorted, dtype, workspace, workspace_bytes, as_stream(stream));
 }
 
 size_t vkop_hip_softmax_topk_workspace_bytes(int dtype, const int *shape, int ndim, int axis, int k) {
