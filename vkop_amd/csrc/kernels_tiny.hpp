@@ -65,6 +65,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
     int32_t *oi = indices + static_cast<size_t>(row) * k;
     const uint32_t want = k + 1, kk = min(k, n);
 
+    BPS(20);
     // ---- 1. the row: element c of vector i of this lane is element (i * 64 + lane) * VEC + c
     Vec128<T> q[V];
 #pragma unroll
@@ -97,6 +98,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
     float M = 0.f, ref = 0.f;
     double s_fast = 0.0;
     bool bad = false;
+    BPS(29);
     if constexpr (SOFTMAX) {
         M = wave_max_f32_uniform(m);
         ref = (M > -INFINITY && M < INFINITY) ? M : 0.f;
@@ -205,15 +207,18 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
         uint64_t mine = have ? smem.cand[lane] : 0ull;
         const uint32_t xkey = static_cast<uint32_t>(mine >> 32);  // the candidate's logit
         __syncthreads();  // (the list may be written again)
+        double rinv = 0.0;  // 1 / the corrected sum
         if constexpr (SOFTMAX) {
             // ---- 5. accurate terms for the candidates, the corrected sum, probabilities
             const float xv = ordered_to_float(static_cast<uint32_t>(mine >> 32));
             const float term = have ? softmax_term(xv, M) : 0.f;
             const double cr = have ? static_cast<double>(term) - static_cast<double>(fast_term_reduced(xv, ref)) : 0.0;
             const double total = s_fast + wave_sum_f64_uniform(cr);
-            const float p = round_to_storage<T>(static_cast<float>(static_cast<double>(term) * (1.0 / total)));
+            rinv = 1.0 / total;
+            const float p = round_to_storage<T>(static_cast<float>(static_cast<double>(term) * rinv));
             mine = have ? ((static_cast<uint64_t>(order_key(p)) << 32) | (mine & 0xFFFFFFFFull)) : 0ull;
         }
+        BPS(28);
         // ---- 6. ranks among the candidates
         const uint32_t mine_hi = static_cast<uint32_t>(mine >> 32);
         const uint32_t before = rank_among(mine, C);
@@ -239,8 +244,28 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
                         }
                         return;
                     }
+                    // The tie reaches the last candidate; whether it goes on below the candidates is a
+                    // question about ONE element, the largest that is not a candidate (every element from thr up
+                    // is one): with a probability below p_cut the group ends inside the candidates, and the
+                    // ranking just made stands.  Equal half-precision logits at the cut -- a few rows in a
+                    // hundred on a classifier's output -- are this case; going round again for them cost the
+                    // whole call the slowest wave's second turn.
+                    uint32_t below = 0;
+#pragma unroll
+                    for (int e = 0; e < ELEMS; e++) below = max(below, key[e] < thr ? key[e] : 0u);
+                    below = wave_max_u32(below);
+                    bool ends_inside = below == 0u;  // (the candidates are all there is)
+                    if (!ends_inside) {
+                        const float pb = round_to_storage<T>(static_cast<float>(static_cast<double>(softmax_term(ordered_to_float(below), M)) * rinv));
+                        ends_inside = order_key(pb) < p_cut;
+                    }
+                    if (!ends_inside) {
                     if (lanes_wanted >= static_cast<uint32_t>(kWave)) break;
+#ifdef VKOP_STAMPS
+                    if (threadIdx.x == 0) atomicAdd(&g_bp_stamps[31], 1ull);
+#endif
                     continue;  // more candidates
+                    }
                 }
             }
         }
@@ -250,6 +275,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             else ov[before] = rowp[idx];  // bit copy (keeps the sign of a zero)
             oi[before] = static_cast<int32_t>(idx);
         }
+        BPS(27);
         return;
     }
     // ---- equal values en masse at the k-th place, or a row of mostly -inf ---------------------------
@@ -405,7 +431,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
 #ifdef VKOP_STAMPS
     if (threadIdx.x == 0) atomicAdd(&g_bp_stamps[30], 1ull);
 #endif
-    BPS(27);
+    BPS(26);
     __syncthreads();  // LDS changes owner
     SelectShared &ex = smem.exact;
     if constexpr (SOFTMAX) {
