@@ -114,6 +114,74 @@ def runtime_api_leg(runs=200):
         return {"error": str(exc)}
 
 
+def timeline_summary(rec, ms_per_step, nlanes, hw_queues):
+    """What the timeline library's log of one timed pass says: records (tag, entry, exit) per logged workgroup,
+    tag = kernel (bit 63: 0 scan, 1 pick) | workgroup << 40 | bits of the call's workspace address (= the lane);
+    clocks in 10 ns.  The scan kernel logs every 16th workgroup and its last 48, the pick kernel all 64."""
+    import numpy as np
+    tag = rec[:, 0]
+    t0 = rec[:, 1].astype(np.int64) * 10
+    t1 = rec[:, 2].astype(np.int64) * 10
+    kind = (tag >> np.uint64(63)).astype(np.int64)
+    lane_id = (tag & np.uint64(0xFFFFFFFFFF)).astype(np.int64)
+    order = np.argsort(t0, kind="stable")
+    kind, lane_id, t0, t1 = kind[order], lane_id[order], t0[order], t1[order]
+    # the timed replays follow the warm-up and the untimed replay after a pause (the gate): the last stretch without one
+    cuts = np.nonzero(np.diff(t0) > 1_000_000)[0]
+    first = int(cuts[-1]) + 1 if len(cuts) else 0
+    kind, lane_id, t0, t1 = kind[first:], lane_id[first:], t0[first:], t1[first:]
+    lanes = sorted(set(lane_id.tolist()))
+    launches = []  # (start, end, lane, kernel)
+    for li, w in enumerate(lanes):
+        for kd in (0, 1):
+            m = np.nonzero((lane_id == w) & (kind == kd))[0]
+            if len(m) == 0:
+                continue
+            # a launch's workgroups enter within a few microseconds of each other; the lane's next launch of the
+            # same kernel enters a whole call later
+            groups = np.split(m, np.nonzero(np.diff(t0[m]) > 4000)[0] + 1)
+            for g in groups:
+                launches.append((int(t0[g].min()), int(t1[g].max()), li, kd))
+    launches.sort()
+    if len(launches) < 8 * nlanes:
+        return {"error": "too few launches in the log", "records": int(len(rec))}
+    # leave the pass's first and last calls out (lanes filling and draining)
+    lo, hi = launches[2 * nlanes][0], launches[-2 * nlanes][0]
+    mid = [l for l in launches if lo <= l[0] < hi]
+    dur = {kd: [(e - s) / 1e3 for s, e, _, k2 in mid if k2 == kd] for kd in (0, 1)}
+    gaps = {"scan_to_pick": [], "pick_to_scan": []}
+    for li in range(len(lanes)):
+        mine = [l for l in mid if l[2] == li]
+        for a, b in zip(mine, mine[1:]):
+            if a[3] != b[3]:
+                gaps["scan_to_pick" if a[3] == 0 else "pick_to_scan"].append((b[0] - a[1]) / 1e3)
+    # how many kernels are running, weighted by time
+    ev = sorted([(s, 1) for s, e, _, _ in mid] + [(e, -1) for s, e, _, _ in mid])
+    conc = {}
+    cur, last = 0, ev[0][0]
+    for t, d in ev:
+        conc[cur] = conc.get(cur, 0) + (t - last)
+        cur, last = cur + d, t
+    total = float(sum(conc.values()))
+    scans = [l for l in mid if l[3] == 0]
+    span = (scans[-1][0] - scans[0][0]) / 1e3
+    mean = lambda v: float(np.mean(v)) if len(v) else None
+    return {
+        "what": "device timestamps logged by the scan and pick kernels themselves (libvkop_hip_timeline.so), one timed pass, "
+                "its first and last calls left out",
+        "calls_in_flight": nlanes, "hw_queues": hw_queues, "lanes_seen": len(lanes),
+        "calls": len(scans), "us_per_call_from_the_log": span / max(1, len(scans) - 1),
+        "us_per_step_by_hip_events_same_run": ms_per_step * 1e3,
+        "scan_kernel_us_first_entry_to_last_exit": {"mean": mean(dur[0]), "p10": float(np.percentile(dur[0], 10)), "p90": float(np.percentile(dur[0], 90))},
+        "pick_kernel_us_first_entry_to_last_exit": {"mean": mean(dur[1]), "p10": float(np.percentile(dur[1], 10)), "p90": float(np.percentile(dur[1], 90))},
+        "pick_workgroup_us_entry_to_exit_mean": float(np.mean((t1 - t0)[(kind == 1) & (t0 >= lo) & (t0 < hi)])) / 1e3,
+        "gap_us_scan_exit_to_pick_entry_same_lane": mean(gaps["scan_to_pick"]),
+        "gap_us_pick_exit_to_next_scan_entry_same_lane": mean(gaps["pick_to_scan"]),
+        "share_of_time_with_n_kernels_running": {str(n): conc[n] / total for n in sorted(conc)},
+        "mean_kernels_running": sum(n * v for n, v in conc.items()) / total,
+    }
+
+
 def cpu_model():
     try:
         for line in open("/proc/cpuinfo"):
@@ -227,6 +295,11 @@ def main():
     ap.add_argument("--eager", action="store_true",
                     help="launch every call from the host instead of replaying recordings (for counter runs under "
                          "rocprofv3 --pmc, which collects per dispatch; the timings of such a run are not the metric)")
+    ap.add_argument("--timeline", action="store_true",
+                    help="run the whole step with the given --hw-queues / --inflight on libvkop_hip_timeline.so (`make -C "
+                         "vkop_amd/csrc timeline`), whose scan and pick kernels log device timestamps per workgroup, and print "
+                         "what the log says about the lanes: each kernel's duration from its first workgroup's entry to its "
+                         "last one's exit, the gaps between a lane's kernels, how many kernels run at the same time")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain device copy of known size (the yardstick for the FETCH_SIZE / "
                          "WRITE_SIZE counters) and print its size")
@@ -246,7 +319,7 @@ def main():
         sys.exit(2)
 
     # (child processes, before this one initialises the GPU)
-    child = args.kernel_legs or args.headline_only
+    child = args.kernel_legs or args.headline_only or args.timeline
     runtime_api = None if (child or args.no_runtime_api or args.workload != "C3") else runtime_api_leg()
     kernel_legs = None
     default_queues = None
@@ -286,6 +359,8 @@ def main():
 
     if args.kernel_legs:
         capi.use_bench_library()
+    if args.timeline:
+        capi.use_timeline_library()
     capi.lib()
     capi.init(0)
     capi.tune("rows.path", args.rows_path)
@@ -494,6 +569,11 @@ def main():
                                     names[1]: (timed(2, len(lanes), 1, True)[0] if path == 2 else timed(2, len(lanes))[0]) * 1e3}
         print(json.dumps({"stage_ms": stage_ms, "stage_overlapped": stage_overlapped,
                           "library": os.path.basename(capi.LIB_PATH)}))
+        return
+    if args.timeline:
+        capi.timeline_records()  # (the log starts here)
+        ms, wall = timed(3, len(lanes))
+        print(json.dumps(timeline_summary(capi.timeline_records(), ms, len(lanes), hw_queues)))
         return
     if args.headline_only:
         ms, wall = timed(3, len(lanes))

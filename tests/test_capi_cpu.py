@@ -80,3 +80,33 @@ def test_workspace_queries_are_pure(lib):
     b = lib.vkop_hip_softmax_topk_workspace_bytes(capi.F32, shape, 2, -1, 50)
     assert a == b and a % 256 == 0
     assert lib.vkop_hip_softmax_topk_workspace_bytes(9, shape, 2, -1, 50) == 0
+
+
+def test_timeline_summary_reads_a_log_of_two_lanes():
+    """bench.py --timeline: the summary of a log made up here -- two lanes, each scan 8 us and pick 6 us with 2 us
+    between them, the lanes half a call apart -- gives back those durations, gaps and the overlap."""
+    import importlib.util
+    import numpy as np
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    recs = []
+    period = 18000  # ns per call of a lane: 8 + 2 + 6 + 2
+    for lane, ws in enumerate((0x1000, 0x2000)):
+        for call in range(40):
+            s0 = 5_000_000 + lane * period // 2 + call * period
+            for wg in (0, 16, 500):        # scan workgroups: enter together, the last leaves after 8 us
+                recs.append(((wg << 40) | ws, (s0 + wg) // 10, (s0 + 7000 + 2 * wg) // 10))
+            p0 = s0 + 8000 + 2000
+            for wg in range(4):            # pick workgroups
+                recs.append(((1 << 63) | (wg << 40) | ws, (p0 + wg) // 10, (p0 + 5000 + 250 * wg + (250 if wg == 3 else 0)) // 10))
+    # (a warm-up stretch long before, which the summary leaves out)
+    recs.append((0x1000, 100, 200))
+    out = bench.timeline_summary(np.array(recs, dtype=np.uint64), 0.009, 2, 8)
+    assert out["lanes_seen"] == 2
+    assert abs(out["scan_kernel_us_first_entry_to_last_exit"]["mean"] - 8.0) < 0.05
+    assert abs(out["pick_kernel_us_first_entry_to_last_exit"]["mean"] - 6.0) < 0.05
+    assert abs(out["gap_us_scan_exit_to_pick_entry_same_lane"] - 2.0) < 0.05
+    assert abs(out["gap_us_pick_exit_to_next_scan_entry_same_lane"] - 2.0) < 0.05
+    assert abs(out["us_per_call_from_the_log"] - 9.0) < 0.05            # two lanes, 18 us a call each
+    assert abs(out["mean_kernels_running"] - 2 * 14.0 / 18.0) < 0.05     # each lane busy 14 of 18 us

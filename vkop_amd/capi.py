@@ -42,6 +42,34 @@ def declared_symbols():
     return sorted(set(re.findall(r"\b(vkop_hip_[a-z0-9_]+)\s*\(", text)))
 
 
+TIMELINE_LIB_PATH = os.path.join(_HERE, "libvkop_hip_timeline.so")
+
+
+def use_timeline_library():
+    """Load libvkop_hip_timeline.so (`make -C vkop_amd/csrc timeline`: the float softmax scan / pick kernels log
+    device timestamps per workgroup) instead of libvkop_hip.so (only before the first lib())."""
+    global LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("the library is loaded already")
+    if not os.path.exists(TIMELINE_LIB_PATH):
+        raise RuntimeError("%s is not built: run `make -C vkop_amd/csrc timeline`" % TIMELINE_LIB_PATH)
+    LIB_PATH = TIMELINE_LIB_PATH
+
+
+def timeline_records(cap=1 << 20):
+    """The timeline library's log since the last call: an array [n, 3] of uint64 (tag, entry, exit); tag = kernel
+    (bit 63: 0 scan, 1 pick) | workgroup << 40 | bits of the call's workspace address; clocks in 10 ns."""
+    import numpy as np
+    fn = lib().vkop_hip_dbg_timeline
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_uint]
+    fn.restype = ctypes.c_int
+    arr = np.zeros((cap, 3), dtype=np.uint64)
+    n = fn(arr.ctypes.data, cap)
+    if n < 0:
+        raise RuntimeError("reading the timeline failed")
+    return arr[:n]
+
+
 def use_bench_library():
     """Load libvkop_hip_bench.so instead of libvkop_hip.so (only before the first lib())."""
     global LIB_PATH
