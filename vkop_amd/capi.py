@@ -30,8 +30,10 @@ class VkopHipError(RuntimeError):
 
 
 def build():
-    """Compile vkop_amd/libvkop_hip.so for gfx950 with hipcc (no GPU needed)."""
+    """Compile vkop_amd/libvkop_hip.so for gfx950 with hipcc (no GPU needed), its benchmark build
+    (libvkop_hip_bench.so) and the build whose headline kernels log a timeline (libvkop_hip_timeline.so)."""
     subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "-B"])
+    subprocess.check_call(["make", "-C", os.path.join(_HERE, "csrc"), "timeline"])
     return LIB_PATH
 
 
