@@ -138,20 +138,21 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
  * precision, x' = fl32(x * scale); out_values / out_indices are the fused
  * softmax -> top-k, largest first, of x', to the bars of vkop_hip_softmax_topk
  * on a tensor holding x' (bit for bit its result on long last-axis rows, where
- * both run the same streaming kernels; to the same bar against an exact softmax elsewhere, where this entry
- * point runs the one-workgroup-per-line kernels).  out_counts (int32 per
+ * both run the same streaming kernels; to the same bar against an exact softmax elsewhere).  out_counts (int32 per
  * row, may be NULL; last axis only) receives the nucleus cut of each row's
  * result for top_p, the number vkop_hip_topp_count gives on out_values.
  * Workspace: vkop_hip_softmax_topk_workspace_bytes().
  * Cost by shape (MI355X, one call at a time): on the long last-axis rows the
  * scan + pick kernels take -- the shapes this entry point is for, e.g.
  * [64,128256] k = 50 -- it costs the plain fused call plus about a tenth
- * (17.2 against 15.5 us).  On every other shape it is correct but runs the
- * one-workgroup-per-line kernels, two passes and an exact select per line and
- * then the count: [256,1000] k = 5 takes 16 us where vkop_hip_softmax_topk
- * takes 5, [64,8192] k = 40 takes 69 us against 9.  A caller with short rows
- * and no temperature is better served by vkop_hip_softmax_topk followed by
- * vkop_hip_topp_count. */
+ * (17.2 against 15.5 us).  Last-axis rows that one workgroup holds (up to
+ * 32768 elements, k up to 408) run that workgroup's kernel with the scale and
+ * the count inside: [64,8192] k = 40 takes 9.6 us (9.4 for the plain fused
+ * call), [256,1000] k = 5 takes 8.9 us (the plain call has a faster one-wave
+ * kernel for such rows: 4.7 us).  What is left -- other axes, k beyond 511 on
+ * long rows -- is correct but runs the one-workgroup-per-line kernels, two
+ * passes and an exact select per line and then the count (tens of
+ * microseconds). */
 int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *out_indices,
                                    int32_t *out_counts, int dtype, const int *shape, int ndim,
                                    int axis, int k, float scale, float top_p, void *workspace,

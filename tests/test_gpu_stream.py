@@ -357,7 +357,9 @@ def test_plain_topk_nan_ranks_first_through_the_scan_pick_pair(ops):
 # ------------------------------------------------------------ sampling variant --
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
-@pytest.mark.parametrize("shape,k", [((16, 128256), 50), ((3, 40000), 7), ((256, 1000), 5), ((2, 33), 33), ((5, 2, 4097), 9)])
+@pytest.mark.parametrize("shape,k", [((16, 128256), 50), ((3, 40000), 7), ((256, 1000), 5), ((2, 33), 33), ((5, 2, 4097), 9),
+                                     ((64, 8192), 40), ((16, 8400), 300), ((40, 4096), 64), ((300, 257), 8), ((7, 20000), 100),
+                                     ((4, 262144), 1024)])
 def test_sampling_variant_against_the_oracle(ops, shape, k, dtype):
     rng = np.random.default_rng(shape[-1] + k)
     x = synth.llm_logits(int(np.prod(shape[:-1])), shape[-1], seed=shape[-1], temperature=1.0).reshape(shape)
@@ -399,10 +401,12 @@ def test_sampling_variant_against_the_oracle(ops, shape, k, dtype):
                 assert np.array_equal(ix.reshape(-1, k)[r], oix.reshape(-1, k)[r]), (what, r)
 
 
-def test_sampling_variant_ties_special_rows_and_errors(ops):
+@pytest.mark.parametrize("n", [50000, 8192, 1000, 8400])
+def test_sampling_variant_ties_special_rows_and_errors(ops, n):
+    """(n = 50000: the scan + pick kernels; the shorter rows: one workgroup, or one wave, per row)"""
     from vkop_amd import capi
     rng = np.random.default_rng(9)
-    x = (np.round(rng.standard_normal((6, 50000)) * 4) / 4).astype(np.float32)   # ties across the cut
+    x = (np.round(rng.standard_normal((6, n)) * 4) / 4).astype(np.float32)   # ties across the cut
     x[1, 10:] = -np.inf                     # fewer elements above -inf than k
     x[2, 77] = np.nan                       # an all-NaN result
     x[3] = 1.5                              # a constant row

@@ -949,7 +949,10 @@ template <typename T, int NT, bool SOFTMAX, int RECS = kMergeRecsMax, bool REDUC
 __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, float *fscratch, double *dscratch,
                                           const T *rowp, T *ov, int32_t *oi, uint32_t n, uint32_t k, uint32_t G,
                                           uint32_t per, uint32_t src_nt, const uint64_t *sums,
-                                          const uint64_t *cand, uint32_t cap_shift) {
+                                          const uint64_t *cand, uint32_t cap_shift, float scale = 1.f,
+                                          int32_t *count_out = nullptr, float top_p = 0.f) {
+    // (scale: the row's elements count times scale -- the candidates' keys are those of the scaled elements
+    // already; count_out, top_p: the nucleus cut of the row's result, finish_row)
     constexpr int NW = NT / kWave;
     constexpr int VEC = Vec128<T>::N;
     constexpr int ES = RECS / NT;  // candidate slots per thread
@@ -1126,6 +1129,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                 store_elem(ov, r, __uint_as_float(0x7FC00000u));
                 oi[r] = static_cast<int32_t>(r);
             }
+            if (count_out != nullptr && tid == 0) *count_out = static_cast<int32_t>(kk);  // (a sum of NaN reaches nothing)
             return;
         }
     }
@@ -1243,7 +1247,7 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                     if (ct <= xlo) continue;  // (same for every thread)
                     const uint32_t c0 = min(b * per, n), c1 = min(c0 + per, n);
                     for (uint32_t j = c0 + tid; j < c1; j += NT) {
-                        const uint32_t key = order_key(load_elem(rowp, j));
+                        const uint32_t key = order_key(scaled(load_elem(rowp, j), scale));
                         if (key >= xlo && key < ct) {
                             const uint32_t pos = atomicAdd(&sh.count, 1u);
                             if (pos < kFastCap) sh.cand[pos] = composite(key, j);
@@ -1258,7 +1262,8 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
                 const uint32_t b = idx / per, off = idx - b * per;
                 return b * src_nw + ((off / VEC) % src_nt) / kWave;
             };
-            finish_row<T, NT, SOFTMAX, REDUCED>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing);
+            finish_row<T, NT, SOFTMAX, REDUCED>(sh, C2, partial, M, s_base, rowp, ov, oi, n, kk, want, wave_of, add_missing, scale,
+                                                count_out, top_p);
             return;
         }
     }
@@ -1270,14 +1275,24 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
     __syncthreads();  // LDS changes owner
     if constexpr (SOFTMAX) {
         // redo the statistics the way the general kernels define them
-        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch);
+        const LineStats st = line_stats<T, NT>(rowp, 0, n, 1, fscratch, dscratch, scale);
         select_topk_line<NT>(exact, n, kk, [&](uint32_t j) {
-            return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
+            return order_key(round_to_storage<T>(softmax_prob(scaled(load_elem(rowp, j), scale), st)));
         });
         for (uint32_t r = tid; r < kk; r += NT) {
             const uint32_t idx = composite_index(exact.sel[r]);
-            store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
+            store_elem(ov, r, softmax_prob(scaled(load_elem(rowp, idx), scale), st));
             oi[r] = static_cast<int32_t>(idx);
+        }
+        if (count_out != nullptr) {
+            // (rare path: the stored values walked in order by the first wave)
+            __syncthreads();
+            if (tid < static_cast<uint32_t>(kWave)) {
+                const uint32_t count = nucleus_count_wave(kk, top_p, [&](uint32_t r) {
+                    return round_to_storage<T>(softmax_prob(scaled(load_elem(rowp, composite_index(exact.sel[r])), scale), st));
+                });
+                if (tid == 0) *count_out = static_cast<int32_t>(count);
+            }
         }
     } else {
         select_topk_line<NT>(exact, n, kk, [&](uint32_t j) { return order_key(load_elem(rowp, j)); });
@@ -1303,10 +1318,20 @@ __device__ __forceinline__ void merge_row(RowsShared &sh, SelectShared &exact, f
 // (a multiple of the vector width, per <= NT * V * vector width, G * per >= n).
 constexpr int kMergeSplit = 0, kMergeByTicket = 1, kMergeLocal = 2;
 
-template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, int MERGE>
+// SAMPLING (a row in one workgroup, softmax variant): every element counts times `scale` (one single-precision
+// multiplication where it is read), and counts, if not null, receives each row's nucleus cut for top_p.
+template <typename T, int NT, int V, bool SOFTMAX, bool ALIGNED, int MERGE, bool SAMPLING = false>
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 && ALIGNED && NT == 256 && MERGE == kMergeSplit ? 5 : 1))) void rows_chunk_kernel(const T *__restrict__ in, T *__restrict__ values,
                                                         int32_t *__restrict__ indices, uint32_t n, uint32_t k,
-                                                        uint32_t G, uint32_t per, RowsWorkspace ws) {
+                                                        uint32_t G, uint32_t per, RowsWorkspace ws, float scale = 1.f,
+                                                        int32_t *__restrict__ counts = nullptr, float top_p = 0.f) {
+    static_assert(!SAMPLING || (SOFTMAX && MERGE == kMergeLocal), "the scaled form exists for rows one workgroup holds");
+    // an element of a loaded vector, as the row counts it
+    auto getq = [&](const Vec128<T> &vec, int c) __attribute__((always_inline)) {
+        float x = vec.get(c);
+        if constexpr (SAMPLING) x = scaled(x, scale);
+        return x;
+    };
     constexpr int VEC = Vec128<T>::N;
     constexpr int NW = NT / kWave;
     constexpr int VPP = kWave / VEC;    // staged vectors a wave unpacks per pass (one element per lane)
@@ -1386,7 +1411,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             for (int i = 0; i < V; i++) {
                 const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
 #pragma unroll
-                for (int c = 0; c < VEC; c++) pm = fmaxf(pm, in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY);
+                for (int c = 0; c < VEC; c++) pm = fmaxf(pm, in_range(ALIGNED ? e0 : e0 + c) ? getq(q[i], c) : -INFINITY);
             }
             const float row_max = block_max_fast<NT>(pm, fscratch);
             ref = (row_max > -INFINITY && row_max < INFINITY) ? row_max : 0.f;
@@ -1399,7 +1424,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             uint32_t vk = 0u;
 #pragma unroll
             for (int c = 0; c < VEC; c++) {
-                xv[c] = in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY;
+                xv[c] = in_range(ALIGNED ? e0 : e0 + c) ? getq(q[i], c) : -INFINITY;
                 vm = fmaxf(vm, xv[c]);
                 if constexpr (!SOFTMAX) vk = max(vk, in_range(ALIGNED ? e0 : e0 + c) ? order_key(xv[c]) : 0u);
             }
@@ -1532,7 +1557,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     Vec128<T> r;
                     r.v = stv[live ? sv : 0u];
                     const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
-                    const float x = r.get(static_cast<int>(lane % VEC));
+                    const float x = getq(r, static_cast<int>(lane % VEC));
                     const uint32_t key = order_key(x);
                     const bool pass = live && idx < c1 && key >= thr_key;
                     const uint64_t mask = __ballot(pass);
@@ -1571,7 +1596,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 for (int i = 0; i < V; i++) {
                     const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
 #pragma unroll
-                    for (int c = 0; c < VEC; c++) ncopy += (in_range(ALIGNED ? e0 : e0 + c) && q[i].get(c) == x0) ? 1u : 0u;
+                    for (int c = 0; c < VEC; c++) ncopy += (in_range(ALIGNED ? e0 : e0 + c) && getq(q[i], c) == x0) ? 1u : 0u;
                 }
                 // (every copy added the same float: taking them out again is exact to the sum's own rounding)
                 if (ncopy != 0u) acc -= static_cast<double>(ncopy) * static_cast<double>(fast_term(x0, ref));
@@ -1591,7 +1616,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
 #pragma unroll
                     for (int c = 0; c < VEC; c++) {
-                        const float x = in_range(ALIGNED ? e0 : e0 + c) ? q[i].get(c) : -INFINITY;
+                        const float x = in_range(ALIGNED ? e0 : e0 + c) ? getq(q[i], c) : -INFINITY;
                         acc += static_cast<double>(fast_term_as<LOCAL>(x, ref));
                     }
                 }
@@ -1623,7 +1648,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
             // kernel waves per SIMD for the sake of this path.)
             auto key_of = [&](int i, int c) {
                 const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-                float x = q[i].get(c);
+                float x = getq(q[i], c);
                 asm volatile("" : "+v"(x));
                 return in_range(ALIGNED ? e0 : e0 + c) ? order_key(x) : 0u;
             };
@@ -1650,7 +1675,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     float vm = INFINITY;  // (a NaN is dropped: it ranks above everything, the others' minimum still holds)
 #pragma unroll
                     for (int c = 0; c < VEC; c++) {
-                        float x = q[i].get(c);
+                        float x = getq(q[i], c);
                         asm volatile("" : "+v"(x));
                         vm = fminf(vm, in_range(ALIGNED ? e0 : e0 + c) ? x : -INFINITY);
                     }
@@ -1733,7 +1758,7 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                     Vec128<T> r;
                     r.v = stv[live ? sv : 0u];
                     const uint32_t idx = ste[live ? sv : 0u] + (lane % VEC);
-                    keys[p] = (live && idx < c1) ? order_key(r.get(static_cast<int>(lane % VEC))) : 0u;
+                    keys[p] = (live && idx < c1) ? order_key(getq(r, static_cast<int>(lane % VEC))) : 0u;
                 }
                 thr = exact_threshold([&](uint32_t trial) {
                     uint32_t c = 0;
@@ -1982,7 +2007,8 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
         BPS(53);
         merge_row<T, NT, SOFTMAX, kLocalCap, true>(smem.fast, smem.exact, fscratch, dscratch, rowp,
                                              values + static_cast<size_t>(row) * k, indices + static_cast<size_t>(row) * k, n, k,
-                                             1u, per, NT, local_ws + kLocalCap, local_ws, ws.cap_shift);
+                                             1u, per, NT, local_ws + kLocalCap, local_ws, ws.cap_shift, SAMPLING ? scale : 1.f,
+                                             (SAMPLING && counts != nullptr) ? counts + row : nullptr, top_p);
         BPS(54);
 #ifdef VKOP_STAMPS
         if (threadIdx.x == 0) {

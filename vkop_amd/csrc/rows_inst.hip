@@ -26,6 +26,38 @@ template <typename T, bool SOFTMAX> bool launch_rows_chunk(const RowsLaunch &a) 
         else VKOP_ROWS_LAUNCH(NT, V, false, kMergeSplit);                                      \
         return true;                                                                           \
     }
+    if constexpr (SOFTMAX) {
+        if (a.sampling) {
+            // a row in one workgroup, every logit times a.scale, the nucleus count beside the result
+            if (a.merge != kMergeLocal) return false;
+#define VKOP_ROWS_SAMPLING(NT, V)                                                                                              \
+    if (a.nt == NT && a.v == V) {                                                                                              \
+        if (a.aligned)                                                                                                         \
+            rows_chunk_kernel<T, NT, V, true, true, kMergeLocal, true>                                                         \
+                <<<blocks, NT, 0, a.stream>>>(in, values, a.indices, a.n, a.k, a.g, a.per, a.ws, a.scale, a.counts, a.top_p);  \
+        else                                                                                                                   \
+            rows_chunk_kernel<T, NT, V, true, false, kMergeLocal, true>                                                        \
+                <<<blocks, NT, 0, a.stream>>>(in, values, a.indices, a.n, a.k, a.g, a.per, a.ws, a.scale, a.counts, a.top_p);  \
+        return true;                                                                                                           \
+    }
+            VKOP_ROWS_SAMPLING(64, 1)
+            VKOP_ROWS_SAMPLING(64, 2)
+            VKOP_ROWS_SAMPLING(64, 4)
+            VKOP_ROWS_SAMPLING(256, 1)
+            VKOP_ROWS_SAMPLING(256, 2)
+            VKOP_ROWS_SAMPLING(256, 4)
+            VKOP_ROWS_SAMPLING(512, 4)
+            VKOP_ROWS_SAMPLING(1024, 4)
+            if constexpr (sizeof(T) == 4) {
+                VKOP_ROWS_SAMPLING(64, 8)
+                VKOP_ROWS_SAMPLING(256, 8)
+                VKOP_ROWS_SAMPLING(512, 8)
+                VKOP_ROWS_SAMPLING(1024, 8)
+            }
+#undef VKOP_ROWS_SAMPLING
+            return false;
+        }
+    }
     // one wave per row (short rows, small k): no barrier costs anything, nothing leaves the wave
 #define VKOP_ROWS_CASE_WAVE(V)                                                 \
     if (a.nt == 64 && a.v == V && a.merge == kMergeLocal) {                    \

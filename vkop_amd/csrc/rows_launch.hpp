@@ -25,6 +25,11 @@ struct RowsLaunch {
     int merge;         // kMergeSplit / kMergeByTicket / kMergeLocal
     RowsWorkspace ws;
     hipStream_t stream;
+    // sampling form (softmax variant, merge == kMergeLocal only): every logit times scale; counts: per-row nucleus cut for top_p, or null
+    bool sampling = false;
+    float scale = 1.f;
+    int32_t *counts = nullptr;
+    float top_p = 0.f;
 };
 
 // Launch of the streaming pair rows_scan_kernel + rows_pick_kernel (kernels_stream.hpp).

@@ -766,7 +766,8 @@ int launch_scan(const T *in, T *values, int32_t *indices, const View &v, int k, 
 
 template <typename T, bool SOFTMAX>
 int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, const RowsCfg &c, void *ws,
-                const RowsLayout &l, hipStream_t st) {
+                const RowsLayout &l, hipStream_t st, bool sampling = false, float scale = 1.f, int32_t *counts = nullptr,
+                float top_p = 0.f) {
     vkop::RowsWorkspace w;
     auto *base = static_cast<unsigned char *>(ws);
     w.tickets = reinterpret_cast<uint32_t *>(base + l.tickets);
@@ -802,6 +803,11 @@ int launch_rows(const T *in, T *values, int32_t *indices, const View &v, int k, 
     }
     a.ws = w;
     a.stream = st;
+    a.sampling = sampling;
+    a.scale = scale;
+    a.counts = counts;
+    a.top_p = top_p;
+    if (sampling && a.merge != vkop::kMergeLocal) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no scaled form of these kernels for this shape");
     const int stages = a.merge != vkop::kMergeSplit ? 1 : measured_stages();
     if (stages & 1) {
         if (!vkop::launch_rows_chunk<T, SOFTMAX>(a))
@@ -1264,6 +1270,14 @@ int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *ou
         if (sc.ok && sc.g2 == 0) {
             const RowsLayout l = rows_layout(v, RowsCfg{}, BigKCfg{}, sc);
             return launch_scan<T, true>(x, values, out_indices, v, k, sc, workspace, l, st, scale, out_counts, top_p);
+        }
+        // a row that one workgroup holds (short rows: a wave): its kernel in the scaled form
+        if (!sc.ok) {
+            const RowsCfg rc = choose_rows_cfg(v, k, dtype);
+            if (rc.ok && rc.g == 1 && rows_cap(k) <= static_cast<uint32_t>(vkop::kLocalCap) && g_rows_fused.load() == 0) {
+                const RowsLayout lr = rows_layout(v, rc);
+                return launch_rows<T, true>(x, values, out_indices, v, k, rc, workspace, lr, st, true, scale, out_counts, top_p);
+            }
         }
         // every other shape: the line kernels on the scaled elements, then the count on their sorted result
         const RowsLayout l = rows_layout(v, RowsCfg{}, BigKCfg{});
