@@ -147,9 +147,9 @@ int vkop_hip_softmax_topk(const void *in, void *out_probs, void *out_values,
  * [64,128256] k = 50 -- it costs the plain fused call plus about a tenth
  * (17.2 against 15.5 us).  Last-axis rows that one workgroup holds (up to
  * 32768 elements, k up to 408) run that workgroup's kernel with the scale and
- * the count inside: [64,8192] k = 40 takes 9.6 us (9.4 for the plain fused
- * call), [256,1000] k = 5 takes 8.9 us (the plain call has a faster one-wave
- * kernel for such rows: 4.7 us).  What is left -- other axes, k beyond 511 on
+ * the count inside, short rows with k up to 32 the one-wave kernel:
+ * [64,8192] k = 40 takes 9.6 us (9.4 for the plain fused call), [256,1000]
+ * k = 5 takes 5.5 us (4.7).  What is left -- other axes, k beyond 511 on
  * long rows -- is correct but runs the one-workgroup-per-line kernels, two
  * passes and an exact select per line and then the count (tens of
  * microseconds). */

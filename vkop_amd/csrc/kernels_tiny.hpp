@@ -32,10 +32,24 @@ namespace vkop {
 
 constexpr int kTinyMaxK = 32;  // (k + 1 candidates, one per lane, and room for a few more)
 
-template <typename T, int V, bool SOFTMAX, bool ALIGNED>
-__global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ in, T *__restrict__ values,
-                                                          int32_t *__restrict__ indices, uint32_t n, uint32_t k,
-                                                          uint32_t smallest = 0) {
+// SAMPLING (softmax variant): every element counts times `scale` (one single-precision multiplication where it is
+// read), and counts, if not null, receives each row's nucleus cut for top_p (the stored values walked in order).
+union TinyShared {
+    uint64_t cand[kWave];
+    SelectShared exact;
+    __device__ TinyShared() {}
+};
+
+// One row by the 64 lanes of the workgroup's only wave (the body of both kernels below).
+template <typename T, int V, bool SOFTMAX, bool ALIGNED, bool SAMPLING>
+__device__ __forceinline__ void tiny_row(TinyShared &smem, float *fscratch, double *dscratch, const T *__restrict__ in,
+                                         T *__restrict__ values, int32_t *__restrict__ indices, uint32_t n, uint32_t k,
+                                         uint32_t smallest, float scale) {
+    static_assert(!SAMPLING || SOFTMAX, "the scaled form belongs to the softmax variant");
+    auto elem_of = [&](float x) __attribute__((always_inline)) {
+        if constexpr (SAMPLING) x = scaled(x, scale);
+        return x;
+    };
     constexpr int VEC = Vec128<T>::N;
     constexpr int ELEMS = V * VEC;
     // smallest (plain top-k only): the k smallest, in increasing order.  Everything below works
@@ -51,13 +65,6 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
         }
         return kx;
     };
-    __shared__ union U {
-        uint64_t cand[kWave];
-        SelectShared exact;
-        __device__ U() {}
-    } smem;
-    __shared__ float fscratch[1];
-    __shared__ double dscratch[1];
     const uint32_t lane = threadIdx.x;
     const uint32_t row = blockIdx.x;
     const T *rowp = in + static_cast<size_t>(row) * n;
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
 #pragma unroll
         for (int c = 0; c < VEC; c++) {
             const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
-            const float x = q[i].get(c);
+            const float x = elem_of(q[i].get(c));
             const bool live = e < n && !(SOFTMAX && x != x);
             key[i * VEC + c] = live ? key_of_value(x) : 0u;
             lmk = max(lmk, key[i * VEC + c]);
@@ -108,7 +115,7 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
 #pragma unroll
             for (int c = 0; c < VEC; c++) {
                 const uint32_t e = (static_cast<uint32_t>(i) * kWave + lane) * VEC + static_cast<uint32_t>(c);
-                if (e < n) acc += static_cast<double>(fast_term_reduced(q[i].get(c), ref));  // (a NaN element makes the sum NaN)
+                if (e < n) acc += static_cast<double>(fast_term_reduced(elem_of(q[i].get(c)), ref));  // (a NaN element makes the sum NaN)
             }
         }
         s_fast = wave_sum_f64_uniform(acc);
@@ -435,13 +442,13 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
     __syncthreads();  // LDS changes owner
     SelectShared &ex = smem.exact;
     if constexpr (SOFTMAX) {
-        const LineStats st = line_stats<T, kWave>(rowp, 0, n, 1, fscratch, dscratch, 1.f);
+        const LineStats st = line_stats<T, kWave>(rowp, 0, n, 1, fscratch, dscratch, SAMPLING ? scale : 1.f);
         select_topk_line<kWave>(ex, n, kk, [&](uint32_t j) {
-            return order_key(round_to_storage<T>(softmax_prob(load_elem(rowp, j), st)));
+            return order_key(round_to_storage<T>(softmax_prob(elem_of(load_elem(rowp, j)), st)));
         });
         for (uint32_t r = lane; r < kk; r += kWave) {
             const uint32_t idx = composite_index(ex.sel[r]);
-            store_elem(ov, r, softmax_prob(load_elem(rowp, idx), st));
+            store_elem(ov, r, softmax_prob(elem_of(load_elem(rowp, idx)), st));
             oi[r] = static_cast<int32_t>(idx);
         }
     } else {
@@ -451,6 +458,37 @@ __global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ 
             ov[r] = rowp[idx];
             oi[r] = static_cast<int32_t>(idx);
         }
+    }
+}
+
+// Launch: one workgroup of 64 threads per row.
+template <typename T, int V, bool SOFTMAX, bool ALIGNED>
+__global__ __launch_bounds__(kWave) void rows_tiny_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                          int32_t *__restrict__ indices, uint32_t n, uint32_t k,
+                                                          uint32_t smallest = 0) {
+    __shared__ TinyShared smem;
+    __shared__ float fscratch[1];
+    __shared__ double dscratch[1];
+    tiny_row<T, V, SOFTMAX, ALIGNED, false>(smem, fscratch, dscratch, in, values, indices, n, k, smallest, 1.f);
+}
+
+// The softmax variant with every element times `scale`, and, if counts is not null, each row's nucleus cut for top_p.
+template <typename T, int V, bool ALIGNED>
+__global__ __launch_bounds__(kWave) void rows_tiny_sampling_kernel(const T *__restrict__ in, T *__restrict__ values,
+                                                                   int32_t *__restrict__ indices, uint32_t n, uint32_t k,
+                                                                   float scale, int32_t *__restrict__ counts, float top_p) {
+    __shared__ TinyShared smem;
+    __shared__ float fscratch[1];
+    __shared__ double dscratch[1];
+    tiny_row<T, V, true, ALIGNED, true>(smem, fscratch, dscratch, in, values, indices, n, k, 0u, scale);
+    if (counts != nullptr) {
+        // the nucleus cut of what was just stored (whichever way the row went): the wave reads its own result
+        // back -- the barrier makes the workgroup's stores visible to it -- and walks it in order
+        __syncthreads();
+        const uint32_t kk = min(k, n);
+        const T *ov = values + static_cast<size_t>(blockIdx.x) * k;
+        const uint32_t count = nucleus_count_wave(kk, top_p, [&](uint32_t r) { return load_elem(ov, r); });
+        if (threadIdx.x == 0) counts[blockIdx.x] = static_cast<int32_t>(count);
     }
 }
 

@@ -99,6 +99,30 @@ template <typename T, bool SOFTMAX> void launch_rows_merge(const RowsLaunch &a) 
 }
 
 template <typename T, bool SOFTMAX> bool launch_rows_tiny(const TinyLaunch &a) {
+    if constexpr (SOFTMAX) {
+        if (a.sampling) {
+#define VKOP_TINY_SAMPLING(V)                                                                          \
+    if (a.v == V) {                                                                                    \
+        if (a.aligned)                                                                                 \
+            rows_tiny_sampling_kernel<T, V, true><<<a.rows, kWave, 0, a.stream>>>(                     \
+                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k,         \
+                a.scale, a.counts, a.top_p);                                                           \
+        else                                                                                           \
+            rows_tiny_sampling_kernel<T, V, false><<<a.rows, kWave, 0, a.stream>>>(                    \
+                static_cast<const T *>(a.in), static_cast<T *>(a.values), a.indices, a.n, a.k,         \
+                a.scale, a.counts, a.top_p);                                                           \
+        return true;                                                                                   \
+    }
+            VKOP_TINY_SAMPLING(1)
+            VKOP_TINY_SAMPLING(2)
+            VKOP_TINY_SAMPLING(4)
+            if constexpr (sizeof(T) == 4) {
+                VKOP_TINY_SAMPLING(8)
+            }
+#undef VKOP_TINY_SAMPLING
+            return false;
+        }
+    }
 #define VKOP_TINY_CASE(V)                                                                              \
     if (a.v == V) {                                                                                    \
         if (a.aligned)                                                                                 \

@@ -67,6 +67,11 @@ struct TinyLaunch {
     bool aligned;
     bool smallest = false;  // plain top-k: the k smallest, increasing
     hipStream_t stream;
+    // sampling form (softmax variant): every logit times scale; counts: per-row nucleus cut for top_p, or null
+    bool sampling = false;
+    float scale = 1.f;
+    int32_t *counts = nullptr;
+    float top_p = 0.f;
 };
 template <typename T, bool SOFTMAX> bool launch_rows_tiny(const TinyLaunch &a);
 extern template bool launch_rows_tiny<float, true>(const TinyLaunch &);

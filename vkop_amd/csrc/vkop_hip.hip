@@ -492,7 +492,7 @@ int choose_tiny_loads(const View &v, int k, int dtype) {
 
 template <typename T, bool SOFTMAX>
 int launch_tiny(const T *in, T *values, int32_t *indices, const View &v, int k, int loads, hipStream_t st,
-                bool smallest = false) {
+                bool smallest = false, bool sampling = false, float scale = 1.f, int32_t *counts = nullptr, float top_p = 0.f) {
     vkop::TinyLaunch a;
     a.in = in;
     a.values = values;
@@ -504,6 +504,10 @@ int launch_tiny(const T *in, T *values, int32_t *indices, const View &v, int k, 
     a.aligned = (reinterpret_cast<uintptr_t>(in) % 16 == 0) && (v.g.n % (16 / sizeof(T)) == 0);
     a.smallest = smallest;
     a.stream = st;
+    a.sampling = sampling;
+    a.scale = scale;
+    a.counts = counts;
+    a.top_p = top_p;
     if (!vkop::launch_rows_tiny<T, SOFTMAX>(a)) return fail(VKOP_HIP_ERR_UNSUPPORTED, "no rows_tiny_kernel for %d loads", loads);
     return launched("rows_tiny_kernel");
 }
@@ -1271,7 +1275,10 @@ int vkop_hip_softmax_topk_sampling(const void *in, void *out_values, int32_t *ou
             const RowsLayout l = rows_layout(v, RowsCfg{}, BigKCfg{}, sc);
             return launch_scan<T, true>(x, values, out_indices, v, k, sc, workspace, l, st, scale, out_counts, top_p);
         }
-        // a row that one workgroup holds (short rows: a wave): its kernel in the scaled form
+        // short rows and a small k: one wave per row, in the scaled form
+        if (const int tiny = choose_tiny_loads(v, k, dtype))
+            return launch_tiny<T, true>(x, values, out_indices, v, k, tiny, st, false, true, scale, out_counts, top_p);
+        // a row that one workgroup holds: its kernel in the scaled form
         if (!sc.ok) {
             const RowsCfg rc = choose_rows_cfg(v, k, dtype);
             if (rc.ok && rc.g == 1 && rows_cap(k) <= static_cast<uint32_t>(vkop::kLocalCap) && g_rows_fused.load() == 0) {
