@@ -110,3 +110,40 @@ def test_timeline_summary_reads_a_log_of_two_lanes():
     assert abs(out["gap_us_pick_exit_to_next_scan_entry_same_lane"] - 2.0) < 0.05
     assert abs(out["us_per_call_from_the_log"] - 9.0) < 0.05            # two lanes, 18 us a call each
     assert abs(out["mean_kernels_running"] - 2 * 14.0 / 18.0) < 0.05     # each lane busy 14 of 18 us
+
+
+def test_route_planner_without_a_gpu(lib):
+    """Which kernels a last-axis top-k / fused call takes is decided on the host (vkop_hip_measure_path: 4 one wave
+    per row, 2 scan + pick, 3 scan + gather + rank, 1 chunk (+ merge), 0 radix select or general kernels;
+    vkop_hip_rows_plan: threads, loads, chunks of the chunk kernel).  The five workloads' routes, the shape that a
+    limit of 8192 blocks had left to the radix select, and the rule that no shape takes chunk + merge over SEVERAL
+    chunks unless vkop_hip_tune asks for it."""
+    F32, F16 = capi.F32, capi.F16
+    assert capi.measure_path(F32, (1, 1000), -1, 5) == 4            # C1
+    assert capi.measure_path(F32, (256, 1000), -1, 5) == 4          # C2
+    assert capi.measure_path(F16, (256, 1000), -1, 5) == 4
+    assert capi.measure_path(F32, (64, 128256), -1, 50) == 2        # C3
+    assert capi.measure_path(F16, (64, 128256), -1, 50) == 2
+    assert capi.measure_path(F32, (8, 262144), -1, 1024) == 3       # C4
+    assert capi.measure_path(F32, (16, 8400), -1, 300) == 1         # C5's select: one workgroup a row
+    assert capi.rows_plan(F32, (16, 8400), -1, 300)[2] == 1
+    assert capi.measure_path(F32, (4, 1048576), -1, 100) == 2       # 16384 blocks a row
+    assert capi.measure_path(F32, (1, 128256), -1, 50) == 2         # a single sequence's logits
+    several = []
+    for dt in (F32, F16):
+        for rows in (1, 8, 16, 17, 64, 1024):
+            for n in list(range(256, 40000, 997)) + [8192, 8193, 8320, 8321, 16384, 32768, 32769, 65536, 131072, 300000, 1 << 20]:
+                for k in (1, 5, 32, 33, 64, 65, 100, 255, 256, 408, 511):
+                    if k > n:
+                        continue
+                    if capi.measure_path(dt, (rows, n), -1, k) == 1 and capi.rows_plan(dt, (rows, n), -1, k)[2] > 1:
+                        several.append((dt, rows, n, k))
+    assert not several, several[:10]
+    try:
+        capi.tune("rows.path", 1)
+        assert capi.measure_path(F32, (64, 128256), -1, 50) == 1 and capi.rows_plan(F32, (64, 128256), -1, 50)[2] > 1
+    finally:
+        capi.tune("rows.path", 0)
+    # the workspace a call is told to bring covers the headline shape with room in the static scratch's 4 MiB
+    need = capi.softmax_topk_workspace_bytes(F32, (64, 128256), -1, 50)
+    assert 64 * 1024 < need <= 4 << 20
