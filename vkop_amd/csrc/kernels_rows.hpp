@@ -435,6 +435,98 @@ template <int NT> __device__ __forceinline__ void block_rank(RowsShared &sh, uin
     __syncthreads();
 }
 
+// The same for a long list (hundreds of candidates: k of 100 and more), where counting all pairs is LDS bandwidth --
+// 1024 threads reading 180 entries each is 4 us on one CU: the candidates are dealt into 256 bins by key
+// (equal steps from the smallest key to the largest), and a candidate's rank is the number of candidates in the
+// bins above its own -- a suffix sum over the bin counts, by one wave -- plus the larger ones in its own bin, which
+// it finds through the bin's list of members (a handful on spread-out data).  A bin with more than kBinnedMax
+// members (values equal en masse; a NaN stretching the range) sends the whole list to block_rank instead.
+// Uses sh.pidx (bin counts, then the bins' fill marks), sh.pkey (where a bin's members start), sh.lane_key (the
+// members, bin by bin from the top), sh.scan_counts: all free until the ranks are known.  Same contract as block_rank.
+constexpr uint32_t kBinnedMin = 64;  // lists up to this long are counted pair by pair
+constexpr uint32_t kBinnedMax = 48;
+template <int NT> __device__ __forceinline__ void block_rank_binned(RowsShared &sh, uint32_t C) {
+    constexpr int NW = NT / kWave;
+    static_assert(kFastMaxK + 1 >= 512 && kFastCap <= 1024, "bin tables in pidx / pkey, members in lane_key");
+    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    if (C <= kBinnedMin) {
+        block_rank<NT>(sh, C);
+        return;
+    }
+    uint32_t *count = sh.pidx, *mark = sh.pidx + 256, *start = sh.pkey, *member = sh.lane_key;
+    // the range of the keys
+    uint32_t kmax = 0, kmin = 0xFFFFFFFFu;
+    for (uint32_t t = tid; t < C; t += NT) {
+        const uint32_t key = static_cast<uint32_t>(sh.cand[t] >> 32);
+        kmax = max(kmax, key);
+        kmin = min(kmin, key);
+    }
+    kmax = wave_max_u32(kmax);
+    kmin = ~wave_max_u32(~kmin);
+    if (lane == 0) {
+        sh.scan_counts[wave] = kmax;
+        sh.scan_counts[16 + wave] = kmin;
+    }
+    for (uint32_t t = tid; t < 256u; t += NT) count[t] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+        kmax = max(kmax, sh.scan_counts[w]);
+        kmin = min(kmin, sh.scan_counts[16 + w]);
+    }
+    const uint32_t range = kmax - kmin;
+    const uint32_t shift = range < 256u ? 0u : 24u - static_cast<uint32_t>(__clz(range));  // (range >> shift) <= 255
+    for (uint32_t t = tid; t < C; t += NT) atomicAdd(&count[(static_cast<uint32_t>(sh.cand[t] >> 32) - kmin) >> shift], 1u);
+    __syncthreads();
+    if (wave == 0) {
+        // lane l takes bins 4 l .. 4 l + 3; start[b] = candidates in the bins above b
+        const uint32_t c0 = count[4 * lane], c1 = count[4 * lane + 1], c2 = count[4 * lane + 2], c3 = count[4 * lane + 3];
+        const uint32_t mine = c0 + c1 + c2 + c3;
+        const uint32_t incl = wave_inclusive_sum_u32(mine);
+        const uint32_t total = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(incl), kWave - 1));
+        const uint32_t above = total - incl;  // in the lanes above this one
+        start[4 * lane + 3] = above;
+        start[4 * lane + 2] = above + c3;
+        start[4 * lane + 1] = above + c3 + c2;
+        start[4 * lane] = above + c3 + c2 + c1;
+        mark[4 * lane + 3] = above;
+        mark[4 * lane + 2] = above + c3;
+        mark[4 * lane + 1] = above + c3 + c2;
+        mark[4 * lane] = above + c3 + c2 + c1;
+        const uint32_t crowd = wave_max_u32(max(max(c0, c1), max(c2, c3)));
+        if (lane == 0) sh.scan_counts[0] = crowd;
+    }
+    __syncthreads();
+    if (sh.scan_counts[0] > kBinnedMax) {  // (the same for every thread)
+        __syncthreads();  // (sh.scan_counts is free again)
+        block_rank<NT>(sh, C);
+        return;
+    }
+    for (uint32_t t = tid; t < C; t += NT) {
+        const uint32_t b = (static_cast<uint32_t>(sh.cand[t] >> 32) - kmin) >> shift;
+        member[atomicAdd(&mark[b], 1u)] = t;
+    }
+    __syncthreads();
+    for (uint32_t t = tid; t < C; t += NT) {
+        const uint64_t mine = sh.cand[t];
+        const uint32_t b = (static_cast<uint32_t>(mine >> 32) - kmin) >> shift;
+        const uint32_t j0 = start[b], j1 = j0 + count[b];
+        uint32_t r = j0;
+        for (uint32_t j = j0; j < j1; j += 4) {  // four members in flight (past the bin's end: the candidate itself, not counted)
+            uint32_t m[4];
+            uint64_t o[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) m[u] = j + u < j1 ? member[j + u] : t;
+#pragma unroll
+            for (int u = 0; u < 4; u++) o[u] = sh.cand[m[u]];
+#pragma unroll
+            for (int u = 0; u < 4; u++) r += (o[u] > mine) ? 1u : 0u;
+        }
+        sh.rank[t] = r;
+    }
+    __syncthreads();
+}
+
 // The same for a list that is followed by zeros up to the power of two P at or above C (a
 // zero ranks behind every candidate), 64 <= P <= NT, sh.rank[0..P) zero: every thread takes
 // P * P / NT entries, two per LDS read, without a test per entry.  Ends with a barrier.
@@ -802,7 +894,7 @@ __device__ __forceinline__ void finish_row(RowsShared &sh, uint32_t C2, bool par
     uint32_t tie_g0 = 0xFFFFFFFFu;  // first rank of a group filled on its own (a tie across the k-th place), if any
     // ---- E. exact ranks; accurate terms for the ranked elements ----------------
     BPS(30);
-    block_rank<NT>(sh, C2);
+    block_rank_binned<NT>(sh, C2);
     BPS(31);
     // only the k+1 largest are used from here on: which other candidates
     // passed the threshold depends on the order the chunks stored theirs in,
