@@ -1946,115 +1946,96 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(sizeof(T) ==
                 }
             }
             BPS(50);
-            // Index of the last equal element to list: elements are in index order by
-            // (vector, wave, lane, position in the vector).
-#pragma unroll
-            for (int i = 0; i < V; i++) {
-                uint32_t ties = 0;
-                if (i < v_used) {
-#pragma unroll
-                    for (int c = 0; c < VEC; c++) ties += static_cast<uint32_t>(__popcll(__ballot(key_of(i, c) == thr)));
-                }
-                if (lane == 0) cs.lane_key[i * NW + wave] = ties;
+            BPS(51);
             }
             drain_stores();  // the first attempt's stores have landed before the same slots are written again
             __syncthreads();  // (and every wave is done with its stage)
-            // exclusive prefix over the (vector, wave) table, one entry per thread: a scan over the lanes of
-            // each of its (at most two) waves, the second adding the first one's total
-            static_assert(V * NW <= 2 * kWave, "the table takes at most two waves");
-            uint32_t mine_before = 0;
+            // The list, straight from the registers -- not through the waves' stages of 64 vectors, which a sorted
+            // row, whose candidates all sit in one wave's elements, would overflow again: everything above thr and,
+            // of the elements equal to it, the first k+1 in index order (the exact turn; at most 2 k + 1 entries) or
+            // all of them (the other turn).  Elements are in index order by (vector, wave, lane, position in the
+            // vector), so three tables with an entry per (vector, wave) say it all: the entry's elements above thr,
+            // its elements equal to thr, and -- from a prefix over those -- how many of the equal ones are still
+            // wanted when the entry begins.  One pass over the registers fills the tables, a second writes; only the
+            // ONE entry that holds the last wanted equal element looks at positions inside itself.
             {
-                const uint32_t val = tid < static_cast<uint32_t>(V * NW) ? cs.lane_key[tid] : 0u;
-                const uint32_t incl = wave_inclusive_sum_u32(val);
-                mine_before = incl - val;
-                if (tid == static_cast<uint32_t>(kWave) - 1u) cs.refine[32] = incl;
-            }
-            __syncthreads();
-            if (tid >= static_cast<uint32_t>(kWave)) mine_before += cs.refine[32];
-            if (tid < static_cast<uint32_t>(V * NW)) cs.lane_key[tid] = mine_before;
-            if (tid == 0) {
-                cs.total = 0;
-                cs.over = 0;
-                cs.thr = 0xFFFFFFFFu;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int i = 0; i < V; i++) {
-                if (i >= v_used) continue;
-                uint32_t pos = cs.lane_key[i * NW + wave];  // equal elements before this wave's vector i
-                bool tie[VEC];
-#pragma unroll
-                for (int c = 0; c < VEC; c++) {
-                    tie[c] = key_of(i, c) == thr;
-                    pos += lanes_below(__ballot(tie[c]));
-                }
-#pragma unroll
-                for (int c = 0; c < VEC; c++) {
-                    if (tie[c]) {
-                        if (pos == want - 1u) cs.thr = e_first + static_cast<uint32_t>(i) * NT * VEC + c;
-                        pos++;
-                    }
-                }
-            }
-            __syncthreads();
-            BPS(51);
-            } else {
-                drain_stores();  // the first attempt's stores have landed before the same slots are written again
-                __syncthreads();
-            }
-            // The list, straight from the registers: at most 2 k + 1 entries (fewer than k+1 above the
-            // value, the first k+1 equal to it), each at a place of its own from counts per (vector,
-            // wave) -- not through the waves' stages of 64 vectors, which a sorted row, whose
-            // candidates all sit in one wave's elements, would overflow again.
-            {
-                const uint32_t idx_limit = exact ? cs.thr : 0xFFFFFFFFu;
-                uint32_t *counts = cs.lane_key + V * NW;  // (behind the table of ties: 2 V NW <= NT words)
-                auto listed = [&](uint32_t kx, uint32_t idx) { return kx > thr || (kx == thr && idx <= idx_limit); };
-                uint32_t wave_total = 0;  // wave-uniform
+                static_assert(3 * V * NW <= NT, "three tables of an entry per (vector, wave)");
+                static_assert(V * NW <= 2 * kWave, "a table takes at most two waves");
+                constexpr uint32_t VN = static_cast<uint32_t>(V * NW);
+                uint32_t *tie_tab = cs.lane_key, *lst_tab = cs.lane_key + VN, *abv_tab = cs.lane_key + 2 * VN;
+                const uint32_t want_ties = exact ? want : 0xFFFFFFFFu;
 #pragma unroll
                 for (int i = 0; i < V; i++) {
-                    const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-                    uint32_t cnt = 0;
+                    uint32_t ties = 0, abv = 0;
                     if (i < v_used) {
 #pragma unroll
-                        for (int c = 0; c < VEC; c++) cnt += static_cast<uint32_t>(__popcll(__ballot(listed(key_of(i, c), e0 + c))));
+                        for (int c = 0; c < VEC; c++) {
+                            const uint32_t kx = key_of(i, c);
+                            ties += static_cast<uint32_t>(__popcll(__ballot(kx == thr)));
+                            abv += static_cast<uint32_t>(__popcll(__ballot(kx > thr)));
+                        }
                     }
-                    if (lane == 0) counts[i * NW + wave] = cnt;
-                    wave_total += cnt;
+                    if (lane == 0) {
+                        tie_tab[i * NW + wave] = ties;
+                        abv_tab[i * NW + wave] = abv;
+                    }
                 }
                 __syncthreads();
-                uint32_t before_mine = 0, mine_cnt = 0;
-                {
-                    mine_cnt = tid < static_cast<uint32_t>(V * NW) ? counts[tid] : 0u;
-                    const uint32_t incl = wave_inclusive_sum_u32(mine_cnt);
-                    before_mine = incl - mine_cnt;
-                    if (tid == static_cast<uint32_t>(kWave) - 1u) cs.refine[32] = incl;
-                }
+                // prefix over the equal ones (a scan over the lanes of each of the table's waves, the second adding
+                // the first one's total), then over what each entry lists
+                const uint32_t mine_ties = tid < VN ? tie_tab[tid] : 0u;
+                const uint32_t mine_abv = tid < VN ? abv_tab[tid] : 0u;
+                const uint32_t incl_t = wave_inclusive_sum_u32(mine_ties);
+                uint32_t ties_before = incl_t - mine_ties;
+                if (tid == static_cast<uint32_t>(kWave) - 1u) cs.refine[32] = incl_t;
                 __syncthreads();
-                if (tid >= static_cast<uint32_t>(kWave)) before_mine += cs.refine[32];
-                if (tid < static_cast<uint32_t>(V * NW)) {
-                    if (tid == static_cast<uint32_t>(V * NW) - 1u) cs.total = before_mine + mine_cnt;
-                    counts[tid] = before_mine;
+                if (tid >= static_cast<uint32_t>(kWave)) ties_before += cs.refine[32];
+                const uint32_t room = want_ties > ties_before ? want_ties - ties_before : 0u;
+                const uint32_t mine_lst = min(mine_ties, room);
+                const uint32_t mine_cnt = tid < VN ? mine_abv + mine_lst : 0u;
+                const uint32_t incl_c = wave_inclusive_sum_u32(mine_cnt);
+                uint32_t before_mine = incl_c - mine_cnt;
+                if (tid == static_cast<uint32_t>(kWave) - 1u) cs.refine[33] = incl_c;
+                __syncthreads();
+                if (tid >= static_cast<uint32_t>(kWave)) before_mine += cs.refine[33];
+                if (tid < VN) {
+                    if (tid == VN - 1u) cs.total = before_mine + mine_cnt;
+                    lst_tab[tid] = mine_lst;
+                    abv_tab[tid] = before_mine;  // (from here on: the entry's first place in the list)
                 }
+                if (tid == 0) cs.over = 0;
                 __syncthreads();
                 if (!exact && cs.total > ws.cap) {  // (the same in every thread: on to the exact cut)
                     __syncthreads();
                     continue;
                 }
+                uint32_t wave_total = 0;  // wave-uniform
 #pragma unroll
                 for (int i = 0; i < V; i++) {
                     if (i >= v_used) continue;
                     const uint32_t e0 = e_first + static_cast<uint32_t>(i) * NT * VEC;
-                    uint32_t pos = counts[i * NW + wave];
+                    const uint32_t n_ties = tie_tab[i * NW + wave], n_lst = lst_tab[i * NW + wave];
+                    uint32_t pos = abv_tab[i * NW + wave];
+                    uint32_t kxs[VEC];
+                    uint32_t tie_at = 0;  // this lane's first equal element's place among the entry's equal ones
+#pragma unroll
+                    for (int c = 0; c < VEC; c++) kxs[c] = key_of(i, c);
+                    const bool partly = n_lst != 0u && n_lst < n_ties;  // (wave-uniform; one entry of a row at most)
+                    if (partly) {
+#pragma unroll
+                        for (int c = 0; c < VEC; c++) tie_at += lanes_below(__ballot(kxs[c] == thr));
+                    }
 #pragma unroll
                     for (int c = 0; c < VEC; c++) {
-                        const uint32_t kx = key_of(i, c);
-                        const bool pass = listed(kx, e0 + c);
+                        const bool tie = kxs[c] == thr;
+                        const bool pass = kxs[c] > thr || (tie && (partly ? tie_at < n_lst : n_lst != 0u));
+                        if (partly && tie) tie_at++;
                         const uint64_t mask = __ballot(pass);
                         if (mask != 0ull) {
                             const uint32_t at = pos + lanes_below(mask);
-                            if (pass && at < ws.cap) publish(cand_out + at, composite(kx, e0 + c));
+                            if (pass && at < ws.cap) publish(cand_out + at, composite(kxs[c], e0 + c));
                             pos += static_cast<uint32_t>(__popcll(mask));
+                            wave_total += static_cast<uint32_t>(__popcll(mask));
                         }
                     }
                 }
