@@ -468,3 +468,25 @@ def test_nan_replacement_on_axes_other_than_the_last(ops, shape, axis):
             assert half_ulp_diff(gotn, expn).max() <= 1
         else:
             assert ulp_diff(gotn, expn).max() <= 2
+
+
+# ------------------------------------------------------------ the benchmark's timeline leg --
+
+def test_bench_timeline_leg_sees_every_lane(ops):
+    """bench.py --timeline (a child process on libvkop_hip_timeline.so, whose scan and pick kernels log their own
+    device timestamps): the summary names as many lanes as calls were in flight, and its per-call time from the
+    log agrees with the HIP-event figure of the same pass."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if not os.path.exists(os.path.join(root, "vkop_amd", "libvkop_hip_timeline.so")):
+        pytest.skip("libvkop_hip_timeline.so is not built (make -C vkop_amd/csrc timeline)")
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--timeline", "--hw-queues", "8", "--inflight", "3",
+                        "--steps", "120", "--warmup", "12"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-500:]
+    out = json.loads([line for line in r.stdout.splitlines() if line.startswith("{")][-1])
+    assert out.get("lanes_seen") == 3, out
+    assert 0.7 < out["us_per_call_from_the_log"] / out["us_per_step_by_hip_events_same_run"] < 1.3, out
+    assert 1.0 < out["mean_kernels_running"] <= 3.2, out
